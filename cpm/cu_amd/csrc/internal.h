@@ -1,0 +1,27 @@
+// Declarations shared between the translation units of libcpmcu_amd (not part of the ABI).
+#pragma once
+#include "common.h"
+
+namespace cpmcu {
+
+// lm_head.hip -- the streaming GEMM with its two epilogues.
+constexpr int kHeadModeStats = 0;
+constexpr int kHeadModeArgmax = 1;
+int launch_head_gemm(const void* hidden, const void* w, int n, int V, int H, int apply_scale, float head_scale,
+                     int mode, void* logits, float* part_a, float* part_b, int* grid_out, int* stride_out,
+                     hipStream_t st);
+int head_max_grid();
+
+// topk.hip -- exact top-k (value descending, ties -> lower index) with an optional fused
+// log-softmax transform whose row statistics come from the GEMM's per-workgroup partials.
+struct TopkStatsSource {
+    const float* part_max;  // [grid][stride] or null: rank the raw values
+    const float* part_sum;
+    int grid, stride;
+    float* row_stats;       // [n][2] out: (max, ln sum)
+};
+int launch_topk(const void* x, int n, int dim, int top, void* val, int32_t* pos, int32_t* ids,
+                const int32_t* token_id_remap, const TopkStatsSource* stats, void* workspace,
+                size_t workspace_bytes, hipStream_t st);
+
+}  // namespace cpmcu

@@ -1,0 +1,413 @@
+// Skinny lm_head GEMMs for gfx950 (MI355X): logits[n, V] = hidden[n, H] . W[V, H]^T with
+// n <= 128 rows, fp16 in, fp32 accumulate, streaming W from HBM exactly once.
+//
+// Two epilogues share one kernel:
+//   * STATS  -- FR-Spec draft head (src/model/linear.cuh:8-37,73-79 as called from
+//     src/model/minicpm4/minicpm4_eagle.cuh:320,366): writes the fp16 logits and, per
+//     workgroup, partial (max, sum exp) of every hidden row for the log-softmax that
+//     follows (src/model/eagle.cuh:29-89).
+//   * ARGMAX -- target head (src/model/linear.cuh:82-101, fp16 pre-scale by head_scale) with
+//     the arg-max of cpmcu/speculative/tree_drafter.py:153,233 fused: per workgroup the best
+//     (value, lowest index) of every hidden row; logits are materialised only on request.
+//
+// The path is HBM-bound (n flop per byte of W), so the design is about keeping many 16-byte
+// loads of W in flight per CU, not about MFMA peak:
+//   * one persistent workgroup of 8 waves per CU; every wave owns whole 16-row blocks of W and
+//     the full K range, so nothing is reduced across waves inside the loop;
+//   * W goes HBM -> registers directly as the A operand of v_mfma_f32_16x16x32_f16 (lane =
+//     (row % 16, k-group): 4 lanes read 64 contiguous bytes of a row, the next k-step the other
+//     half of the 128-byte line), 16 loads in flight per wave, software-pipelined across row
+//     blocks;
+//   * the hidden rows are the B operand, staged once per workgroup in LDS (128 KB for n <= 16,
+//     K-chunked and double-buffered for more rows).
+#include "common.h"
+#include "internal.h"
+
+namespace cpmcu {
+namespace {
+
+constexpr int kHeadWaves = 8;
+constexpr int kHeadThreads = kHeadWaves * 64;
+
+struct HeadParams {
+    const f16* hidden;
+    const f16* w;
+    int n, V, H;
+    int kc;       // K chunk held in one LDS buffer
+    int nch;      // H / kc
+    int npasses;  // row-block passes per workgroup
+    int apply_scale;
+    float head_scale;
+    int mode;
+    f16* logits;          // [n][V] or null
+    float* part_a;        // STATS: max   | ARGMAX: best value      [grid][NB*16]
+    float* part_b;        // STATS: sum   | ARGMAX: best index (int) [grid][NB*16]
+};
+
+template <int NB>
+struct HeadCfg {
+    static constexpr int kKcMax = 2048 / NB;             // halves of K per hidden row per buffer
+    static constexpr int kGroupK = NB <= 4 ? 512 : 256;  // K covered by one prefetch group
+    static constexpr int kDepth = kGroupK / 32;          // 16-byte loads in flight per lane
+    static constexpr int kLdsRowMax = kKcMax * 2 + 16;   // bytes, padded: conflict-free b128 reads
+    static constexpr int kLdsBuf = NB * 16 * kLdsRowMax;
+    static constexpr int kStage = 8;                     // 16-byte staging registers per thread
+};
+
+template <int NB>
+__global__ __launch_bounds__(kHeadThreads) void head_gemm_kernel(HeadParams p) {
+    using C = HeadCfg<NB>;
+    constexpr int PD = C::kDepth;
+    constexpr int GK = C::kGroupK;
+    __shared__ __attribute__((aligned(16))) char lds[2 * C::kLdsBuf];
+    __shared__ float red_a[kHeadWaves][NB * 16];
+    __shared__ float red_b[kHeadWaves][NB * 16];
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    const int l16 = lane & 15;
+    const int kgp = lane >> 4;  // k-group of this lane inside a 32-wide k-step
+    const int G = gridDim.x;
+    const int c = blockIdx.x;
+    const int H = p.H, V = p.V, kc = p.kc, nch = p.nch;
+    const int lds_row = kc * 2 + 16;
+    const bool resident = nch <= 2;
+    const int gpp = H / GK;  // prefetch groups per pass
+    const int total = p.npasses * gpp;
+    const int total_chunks = p.npasses * nch;
+    const f16 sc = (f16)p.head_scale;
+
+    // ---- hidden staging helpers ----
+    const int chunks16 = NB * 16 * kc / 8;  // 16-byte pieces per K chunk
+    f16x8 stage[C::kStage];
+    auto stage_load = [&](int hchunk) {
+#pragma unroll
+        for (int s = 0; s < C::kStage; ++s) {
+            const int i = tid + s * kHeadThreads;
+            if (i < chunks16) {
+                const int row = i / (kc / 8);
+                const int col = (i % (kc / 8)) * 8;
+                f16x8 x;
+                if (row < p.n) {
+                    x = *reinterpret_cast<const f16x8*>(p.hidden + (size_t)row * H + (size_t)hchunk * kc + col);
+                    if (p.apply_scale) {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) x[e] = (f16)((float)x[e] * (float)sc);
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) x[e] = (f16)0.f;
+                }
+                stage[s] = x;
+            }
+        }
+    };
+    auto stage_store = [&](int buf) {
+#pragma unroll
+        for (int s = 0; s < C::kStage; ++s) {
+            const int i = tid + s * kHeadThreads;
+            if (i < chunks16) {
+                const int row = i / (kc / 8);
+                const int col = (i % (kc / 8)) * 8;
+                *reinterpret_cast<f16x8*>(lds + (size_t)buf * C::kLdsBuf + row * lds_row + col * 2) = stage[s];
+            }
+        }
+    };
+
+    // ---- W prefetch: group `it` = (pass, k-group) of this wave's row block ----
+    const int arow_lane = l16;
+    auto row_block = [&](int pass) { return (pass * kHeadWaves + wave) * G + c; };
+    auto load_group = [&](int it, f16x8* buf) {
+        const int pass = it / gpp;
+        const int k0 = (it % gpp) * GK;
+        int row = row_block(pass) * 16 + arow_lane;
+        row = row < V ? row : V - 1;  // clamp: rows past the end are computed and discarded
+        const f16* src = p.w + (size_t)row * H + k0 + kgp * 8;
+#pragma unroll
+        for (int ks = 0; ks < PD; ++ks) buf[ks] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(src + ks * 32));
+    };
+
+    f32x4 acc[NB];
+    // running epilogue state of this lane, per n-block: hidden row nb*16 + l16
+    float ea[NB], eb[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        ea[nb] = -INFINITY;                      // running max / best value
+        eb[nb] = p.mode == kHeadModeStats ? 0.f : __int_as_float(0x7fffffff);  // running sum / best index
+    }
+
+    auto epilogue = [&](int pass) {
+        const int rb = row_block(pass);
+        const int vrow0 = rb * 16 + kgp * 4;  // acc[nb][r] <-> vocab row vrow0 + r, hidden row nb*16 + l16
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            const int hrow = nb * 16 + l16;
+            f16 z[4];
+#pragma unroll
+            for (int r = 0; r < 4; ++r) z[r] = (f16)acc[nb][r];
+            if (hrow < p.n) {
+                if (p.logits) {
+                    f16* dst = p.logits + (size_t)hrow * V + vrow0;
+                    if ((V & 3) == 0 && vrow0 + 3 < V) {
+                        f16x4 zz;
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) zz[r] = z[r];
+                        *reinterpret_cast<f16x4*>(dst) = zz;
+                    } else {
+#pragma unroll
+                        for (int r = 0; r < 4; ++r)
+                            if (vrow0 + r < V) dst[r] = z[r];
+                    }
+                }
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    if (vrow0 + r >= V) continue;
+                    const float x = (float)z[r];
+                    if (p.mode == kHeadModeStats) {
+                        if (x == -INFINITY) continue;  // contributes exp(-inf) = 0
+                        if (x > ea[nb]) {
+                            eb[nb] = eb[nb] * __expf(ea[nb] - x) + 1.f;
+                            ea[nb] = x;
+                        } else {
+                            eb[nb] += __expf(x - ea[nb]);
+                        }
+                    } else {
+                        const int idx = vrow0 + r;
+                        const int bidx = __float_as_int(eb[nb]);
+                        if (x > ea[nb] || (x == ea[nb] && idx < bidx)) {
+                            ea[nb] = x;
+                            eb[nb] = __int_as_float(idx);
+                        }
+                    }
+                }
+            }
+        }
+    };
+
+    // ---- prologue: hidden into LDS ----
+    if (resident) {
+        for (int ch = 0; ch < nch; ++ch) {
+            stage_load(ch);
+            stage_store(ch);
+        }
+        __syncthreads();
+    } else {
+        stage_load(0);
+        stage_store(0);
+    }
+
+    auto compute_group = [&](int it, const f16x8* buf) {
+        const int pass = it / gpp;
+        const int kg = it % gpp;
+        const int k0 = kg * GK;
+        const int chunk = k0 / kc;
+        const int koff = k0 % kc;
+        const int cglobal = pass * nch + chunk;
+        int lbuf;
+        if (resident) {
+            lbuf = chunk;
+        } else {
+            if (koff == 0) {
+                __syncthreads();  // chunk `cglobal` visible; everyone is done with the other buffer
+                if (cglobal + 1 < total_chunks) stage_load((cglobal + 1) % nch);
+            }
+            lbuf = cglobal & 1;
+        }
+        if (kg == 0) {
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) acc[nb][r] = 0.f;
+        }
+        const char* brow = lds + (size_t)lbuf * C::kLdsBuf + l16 * lds_row + (koff + kgp * 8) * 2;
+#pragma unroll
+        for (int ks = 0; ks < PD; ++ks) {
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                const f16x8 b = *reinterpret_cast<const f16x8*>(brow + nb * 16 * lds_row + ks * 64);
+                acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(buf[ks], b, acc[nb], 0, 0, 0);
+            }
+        }
+        if (!resident && koff + GK == kc) {
+            if (cglobal + 1 < total_chunks) stage_store((cglobal + 1) & 1);
+        }
+        if (kg == gpp - 1) epilogue(pass);
+    };
+
+    f16x8 buf_a[PD], buf_b[PD];
+    if (total > 0) load_group(0, buf_a);
+    for (int it = 0; it < total; it += 2) {
+        if (it + 1 < total) load_group(it + 1, buf_b);
+        compute_group(it, buf_a);
+        if (it + 1 < total) {
+            if (it + 2 < total) load_group(it + 2, buf_a);
+            compute_group(it + 1, buf_b);
+        }
+    }
+
+    // ---- reduce the epilogue state: lanes sharing a hidden row, then waves ----
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+        for (int off = 16; off <= 32; off <<= 1) {
+            const float oa = __shfl_xor(ea[nb], off);
+            const float ob = __shfl_xor(eb[nb], off);
+            if (p.mode == kHeadModeStats) {
+                const float m = fmaxf(ea[nb], oa);
+                const float s = (m == -INFINITY) ? 0.f : eb[nb] * __expf(ea[nb] - m) + ob * __expf(oa - m);
+                ea[nb] = m;
+                eb[nb] = s;
+            } else {
+                if (oa > ea[nb] || (oa == ea[nb] && __float_as_int(ob) < __float_as_int(eb[nb]))) {
+                    ea[nb] = oa;
+                    eb[nb] = ob;
+                }
+            }
+        }
+        if (lane < 16) {
+            red_a[wave][nb * 16 + lane] = ea[nb];
+            red_b[wave][nb * 16 + lane] = eb[nb];
+        }
+    }
+    __syncthreads();
+    if (tid < NB * 16) {
+        float a = red_a[0][tid], b = red_b[0][tid];
+        for (int w = 1; w < kHeadWaves; ++w) {
+            const float oa = red_a[w][tid], ob = red_b[w][tid];
+            if (p.mode == kHeadModeStats) {
+                const float m = fmaxf(a, oa);
+                b = (m == -INFINITY) ? 0.f : b * __expf(a - m) + ob * __expf(oa - m);
+                a = m;
+            } else if (oa > a || (oa == a && __float_as_int(ob) < __float_as_int(b))) {
+                a = oa;
+                b = ob;
+            }
+        }
+        p.part_a[(size_t)c * (NB * 16) + tid] = a;
+        p.part_b[(size_t)c * (NB * 16) + tid] = b;
+    }
+}
+
+// Final arg-max over the per-workgroup partials: one block per hidden row.
+__global__ __launch_bounds__(256) void head_argmax_finalize_kernel(const float* part_a, const float* part_b,
+                                                                   int G, int stride, int32_t* gt) {
+    __shared__ float sa[256];
+    __shared__ int sb[256];
+    const int row = blockIdx.x;
+    float a = -INFINITY;
+    int b = 0x7fffffff;
+    for (int c = threadIdx.x; c < G; c += 256) {
+        const float oa = part_a[(size_t)c * stride + row];
+        const int ob = __float_as_int(part_b[(size_t)c * stride + row]);
+        if (oa > a || (oa == a && ob < b)) {
+            a = oa;
+            b = ob;
+        }
+    }
+    sa[threadIdx.x] = a;
+    sb[threadIdx.x] = b;
+    __syncthreads();
+    for (int off = 128; off > 0; off >>= 1) {
+        if (threadIdx.x < off) {
+            const float oa = sa[threadIdx.x + off];
+            const int ob = sb[threadIdx.x + off];
+            if (oa > sa[threadIdx.x] || (oa == sa[threadIdx.x] && ob < sb[threadIdx.x])) {
+                sa[threadIdx.x] = oa;
+                sb[threadIdx.x] = ob;
+            }
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) gt[row] = sb[0];
+}
+
+int g_num_cus = 0;
+
+int num_cus() {
+    if (g_num_cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0)
+            n = 256;
+        g_num_cus = n;
+    }
+    return g_num_cus;
+}
+
+int pick_nb(int n) { return n <= 16 ? 1 : n <= 32 ? 2 : n <= 64 ? 4 : 8; }
+
+}  // namespace
+
+// Shared launcher of the GEMM; returns the grid size used (= number of partial rows) in *grid_out.
+int launch_head_gemm(const void* hidden, const void* w, int n, int V, int H, int apply_scale, float head_scale,
+                     int mode, void* logits, float* part_a, float* part_b, int* grid_out, int* stride_out,
+                     hipStream_t st) {
+    const int NB = pick_nb(n);
+    const int kc_max = 2048 / NB;
+    const int gk = NB <= 4 ? 512 : 256;
+    CPMCU_CHECK_ARG(H >= gk && H % gk == 0, "lm_head: hidden size %d must be a multiple of %d for %d rows", H, gk, n);
+    HeadParams p;
+    p.hidden = (const f16*)hidden;
+    p.w = (const f16*)w;
+    p.n = n;
+    p.V = V;
+    p.H = H;
+    p.kc = H < kc_max ? H : kc_max;
+    CPMCU_CHECK_ARG(H % p.kc == 0, "lm_head: hidden size %d not divisible by the K chunk %d", H, p.kc);
+    p.nch = H / p.kc;
+    p.apply_scale = apply_scale;
+    p.head_scale = head_scale;
+    p.mode = mode;
+    p.logits = (f16*)logits;
+    p.part_a = part_a;
+    p.part_b = part_b;
+    const int nrb = ceil_div(V, 16);
+    int G = num_cus();
+    if (G * kHeadWaves > nrb) G = ceil_div(nrb, kHeadWaves);
+    p.npasses = ceil_div(nrb, G * kHeadWaves);
+    *grid_out = G;
+    *stride_out = NB * 16;
+    switch (NB) {
+        case 1: hipLaunchKernelGGL(head_gemm_kernel<1>, dim3(G), dim3(kHeadThreads), 0, st, p); break;
+        case 2: hipLaunchKernelGGL(head_gemm_kernel<2>, dim3(G), dim3(kHeadThreads), 0, st, p); break;
+        case 4: hipLaunchKernelGGL(head_gemm_kernel<4>, dim3(G), dim3(kHeadThreads), 0, st, p); break;
+        default: hipLaunchKernelGGL(head_gemm_kernel<8>, dim3(G), dim3(kHeadThreads), 0, st, p); break;
+    }
+    CPMCU_LAUNCH_CHECK();
+    return CPMCU_OK;
+}
+
+int head_max_grid() { return 1024; }
+
+}  // namespace cpmcu
+
+using namespace cpmcu;
+
+extern "C" size_t cpmcu_head_workspace_bytes(int n, int V) {
+    if (n <= 0 || V <= 0) return 0;
+    // per-workgroup partials (two float planes) + top-k candidates (see topk.hip)
+    const size_t parts = (size_t)2 * head_max_grid() * 128 * sizeof(float);
+    return align_up(parts, 256) + cpmcu_topk_workspace_bytes(n, V, 32);
+}
+
+extern "C" int cpmcu_lm_head_argmax(const void* hidden, const void* w, int n, int V, int H, int apply_scale,
+                                    float head_scale, void* logits, int32_t* gt, void* workspace,
+                                    size_t workspace_bytes, void* stream) {
+    CPMCU_CHECK_ARG(hidden && w, "lm_head_argmax: null pointer argument");
+    CPMCU_CHECK_ARG(n >= 1 && n <= 128, "lm_head_argmax: n=%d outside [1, 128]", n);
+    CPMCU_CHECK_ARG(V >= 1 && H >= 1, "lm_head_argmax: bad shape V=%d H=%d", V, H);
+    CPMCU_CHECK_ARG(logits || gt, "lm_head_argmax: both outputs are null");
+    CPMCU_CHECK_ARG(workspace && workspace_bytes >= cpmcu_head_workspace_bytes(n, V),
+                    "lm_head_argmax: workspace of %zu bytes needed, %zu given", cpmcu_head_workspace_bytes(n, V), workspace_bytes);
+    hipStream_t st = resolve_stream(stream);
+    float* part_a = (float*)workspace;
+    float* part_b = part_a + (size_t)head_max_grid() * 128;
+    int G = 0, stride = 0;
+    int rc = launch_head_gemm(hidden, w, n, V, H, apply_scale, head_scale, kHeadModeArgmax, logits, part_a, part_b, &G, &stride, st);
+    if (rc != CPMCU_OK) return rc;
+    if (gt) {
+        hipLaunchKernelGGL(head_argmax_finalize_kernel, dim3(n), dim3(256), 0, st, part_a, part_b, G, stride, gt);
+        CPMCU_LAUNCH_CHECK();
+    }
+    return CPMCU_OK;
+}

@@ -1,0 +1,479 @@
+// Host runtime of libcpmcu_amd: error plumbing, the library stream, and the model-level mirror of
+// the reference's pybind module (src/entry.cu:98-534) for the verify/draft path: one process-global
+// model that owns the lm_head, the FR-Spec sub-matrix, the paged KV pools of every layer, one page
+// table and scratch.
+#include <cstdlib>
+#include <cstring>
+#include <map>
+#include <string>
+#include <vector>
+
+#include "common.h"
+#include "internal.h"
+
+namespace cpmcu {
+
+namespace {
+thread_local std::string g_error;
+hipStream_t g_stream = nullptr;
+}  // namespace
+
+void set_error(const char* fmt, ...) {
+    char buf[1024];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof(buf), fmt, ap);
+    va_end(ap);
+    g_error = buf;
+}
+
+hipStream_t resolve_stream(void* stream) {
+    if (stream) return (hipStream_t)stream;
+    if (!g_stream) {
+        // a blocking stream, like the reference's calc_stream (src/utils.cu:19): work on the legacy
+        // default stream is implicitly ordered with it
+        if (hipStreamCreate(&g_stream) != hipSuccess) g_stream = nullptr;
+    }
+    return g_stream;
+}
+
+namespace {
+
+struct PerfEntry {
+    double ms = 0;
+    long count = 0;
+};
+
+struct Model {
+    // base model geometry (init_base_model)
+    bool base = false;
+    float memory_limit = 0.f;
+    int vocab = 0, layers = 0, hidden = 0, q_heads = 0, kv_heads = 0, head_dim = 0;
+    float scale_lmhead = 1.f;
+    // drafter (init_eagle_model / init_minicpm4_eagle_model)
+    bool drafter = false;
+    int num_iter = 0, topk_per_iter = 0, tree_size = 0, frspec_vocab = 0;
+    // storage
+    bool storage = false;
+    int num_pages = 0;
+    f16* lm_head = nullptr;
+    f16* fr_head = nullptr;  // == lm_head when FR-Spec is off
+    int32_t* token_id_remap = nullptr;
+    bool remap_loaded = false, lm_head_loaded = false;
+    std::vector<void*> k_pools, v_pools;
+    void** d_k_pools = nullptr;
+    void** d_v_pools = nullptr;
+    int32_t* block_table = nullptr;
+    void* attn_ws = nullptr;
+    size_t attn_ws_bytes = 0;
+    void* head_ws = nullptr;
+    size_t head_ws_bytes = 0;
+    f16* draft_logits = nullptr;  // [16][frspec_vocab]
+    float* row_stats = nullptr;   // [16][2]
+    int32_t* d_best = nullptr;
+    int32_t* h_best = nullptr;  // pinned
+    uint64_t* chain_mask = nullptr;
+    bool perf = false;
+    std::map<std::string, PerfEntry> perf_log;
+};
+
+Model* g_model = nullptr;
+
+int require_model(bool need_storage) {
+    if (!g_model || !g_model->base) {
+        set_error("no model: call init_base_model first");
+        return CPMCU_ERR_RUNTIME;
+    }
+    if (need_storage && !g_model->storage) {
+        set_error("storage not initialised: call init_storage first");
+        return CPMCU_ERR_RUNTIME;
+    }
+    return CPMCU_OK;
+}
+
+struct PerfScope {
+    const char* label;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    hipStream_t st;
+    PerfScope(const char* l, hipStream_t s) : label(l), st(s) {
+        if (g_model && g_model->perf) {
+            (void)hipEventCreate(&e0);
+            (void)hipEventCreate(&e1);
+            (void)hipEventRecord(e0, st);
+        }
+    }
+    ~PerfScope() {
+        if (e0) {
+            (void)hipEventRecord(e1, st);
+            (void)hipEventSynchronize(e1);  // the reference's timers synchronise on stop too (src/perf.cuh:139-166)
+            float ms = 0;
+            (void)hipEventElapsedTime(&ms, e0, e1);
+            auto& ent = g_model->perf_log[label];
+            ent.ms += ms;
+            ent.count += 1;
+            (void)hipEventDestroy(e0);
+            (void)hipEventDestroy(e1);
+        }
+    }
+};
+
+int check_dtype(int torch_dtype) {
+    if (torch_dtype != 0) {  // 0 = fp16, 1 = bf16 (cpmcu/llm.py:11-14)
+        set_error("dtype %d is not compiled into this library (fp16 only)", torch_dtype);
+        return CPMCU_ERR_RUNTIME;  // std::runtime_error in the reference, src/entry.cu:43,52
+    }
+    return CPMCU_OK;
+}
+
+}  // namespace
+}  // namespace cpmcu
+
+using namespace cpmcu;
+
+extern "C" const char* cpmcu_last_error(void) { return g_error.c_str(); }
+extern "C" const char* cpmcu_version(void) { return "cpmcu_amd 0.1 (gfx950)"; }
+
+extern "C" int cpmcu_init_base_model(float memory_limit, int vocab_size, int num_hidden_layers, int hidden_size,
+                                     int intermediate_size, int num_attention_heads, int num_key_value_heads,
+                                     int head_dim, float rms_norm_eps, int torch_dtype, int chunk_length,
+                                     float scale_embed, float scale_lmhead, float scale_residual) {
+    (void)intermediate_size; (void)rms_norm_eps; (void)chunk_length; (void)scale_embed; (void)scale_residual;
+    int rc = check_dtype(torch_dtype);
+    if (rc) return rc;
+    CPMCU_CHECK_ARG(memory_limit > 0.f && memory_limit <= 1.f, "init_base_model: memory_limit=%g outside (0, 1]", memory_limit);
+    CPMCU_CHECK_ARG(vocab_size > 0 && num_hidden_layers > 0 && hidden_size > 0, "init_base_model: bad model shape");
+    CPMCU_CHECK_ARG(head_dim == kHeadDim, "init_base_model: head_dim=%d, this library is built for %d", head_dim, kHeadDim);
+    CPMCU_CHECK_ARG(num_key_value_heads > 0 && num_attention_heads % num_key_value_heads == 0,
+                    "init_base_model: %d attention heads not a multiple of %d kv heads", num_attention_heads, num_key_value_heads);
+    if (g_model) cpmcu_shutdown();
+    g_model = new Model();
+    Model& m = *g_model;
+    m.base = true;
+    m.memory_limit = memory_limit;
+    m.vocab = vocab_size;
+    m.layers = num_hidden_layers;
+    m.hidden = hidden_size;
+    m.q_heads = num_attention_heads;
+    m.kv_heads = num_key_value_heads;
+    m.head_dim = head_dim;
+    m.scale_lmhead = scale_lmhead;
+    const char* pe = getenv("CPMCU_PERF");
+    m.perf = pe && pe[0] == '1';
+    return CPMCU_OK;
+}
+
+extern "C" int cpmcu_init_eagle_model(int num_layers, int num_iter, int topk_per_iter, int tree_size, int torch_dtype) {
+    return cpmcu_init_minicpm4_eagle_model(num_layers, num_iter, topk_per_iter, tree_size, torch_dtype, 0, 0, 0, 0, 1.f, 1, 1);
+}
+
+extern "C" int cpmcu_init_minicpm4_eagle_model(int num_layers, int num_iter, int topk_per_iter, int tree_size,
+                                               int torch_dtype, int apply_eagle_quant, int group_size,
+                                               int eagle_window_size, int frspec_vocab_size, float residual_scale,
+                                               int use_input_norm, int use_attn_norm) {
+    (void)num_layers; (void)group_size; (void)eagle_window_size; (void)residual_scale; (void)use_input_norm; (void)use_attn_norm;
+    int rc = require_model(false);
+    if (rc) return rc;
+    rc = check_dtype(torch_dtype);
+    if (rc) return rc;
+    if (apply_eagle_quant) {
+        set_error("init_minicpm4_eagle_model: quantised EAGLE layers are outside the verify/draft path");
+        return CPMCU_ERR_UNSUPPORTED;
+    }
+    Model& m = *g_model;
+    CPMCU_CHECK_ARG(!m.storage, "init_minicpm4_eagle_model: storage already initialised");
+    // the reference asserts tree_size <= 64 at this boundary (src/model/minicpm4/minicpm4_eagle.cuh:69)
+    CPMCU_CHECK_ARG(tree_size >= 1 && tree_size <= 64, "init_minicpm4_eagle_model: tree_size=%d outside [1, 64]", tree_size);
+    CPMCU_CHECK_ARG(num_iter >= 1 && topk_per_iter >= 1 && topk_per_iter <= tree_size - 1 && topk_per_iter <= 16,
+                    "init_minicpm4_eagle_model: topk_per_iter=%d must be in [1, min(16, tree_size-1)]", topk_per_iter);
+    CPMCU_CHECK_ARG(frspec_vocab_size >= 0 && frspec_vocab_size <= m.vocab, "init_minicpm4_eagle_model: frspec_vocab_size=%d", frspec_vocab_size);
+    m.drafter = true;
+    m.num_iter = num_iter;
+    m.topk_per_iter = topk_per_iter;
+    m.tree_size = tree_size;
+    m.frspec_vocab = frspec_vocab_size > 0 ? frspec_vocab_size : m.vocab;
+    return CPMCU_OK;
+}
+
+extern "C" int cpmcu_init_storage(int* max_context) {
+    int rc = require_model(false);
+    if (rc) return rc;
+    Model& m = *g_model;
+    CPMCU_CHECK_ARG(!m.storage, "init_storage: already initialised");
+    size_t free_b = 0, total_b = 0;
+    CPMCU_HIP(hipMemGetInfo(&free_b, &total_b));
+    const size_t budget = (size_t)((double)total_b * m.memory_limit);
+    size_t used = 0;
+    auto alloc = [&](void** ptr, size_t bytes) -> int {
+        bytes = align_up(bytes, 256);
+        if (used + bytes > budget || bytes > free_b) {
+            set_error("init_storage: out of memory budget (%zu + %zu > %zu bytes)", used, bytes, budget);
+            return CPMCU_ERR_RUNTIME;
+        }
+        CPMCU_HIP(hipMalloc(ptr, bytes));
+        used += bytes;
+        return CPMCU_OK;
+    };
+    const int max_tree = m.drafter ? m.tree_size : 64;
+    if ((rc = alloc((void**)&m.lm_head, (size_t)m.vocab * m.hidden * 2))) return rc;
+    if (m.drafter && m.frspec_vocab != m.vocab) {
+        if ((rc = alloc((void**)&m.fr_head, (size_t)m.frspec_vocab * m.hidden * 2))) return rc;
+        if ((rc = alloc((void**)&m.token_id_remap, (size_t)m.frspec_vocab * 4))) return rc;
+    } else {
+        m.fr_head = m.lm_head;
+    }
+    m.head_ws_bytes = cpmcu_head_workspace_bytes(128, m.vocab);
+    if ((rc = alloc(&m.head_ws, m.head_ws_bytes))) return rc;
+    if (m.drafter) {
+        if ((rc = alloc((void**)&m.draft_logits, (size_t)16 * m.frspec_vocab * 2))) return rc;
+        if ((rc = alloc((void**)&m.row_stats, 16 * 2 * sizeof(float)))) return rc;
+    }
+    if ((rc = alloc((void**)&m.d_best, 2 * sizeof(int32_t)))) return rc;
+    CPMCU_HIP(hipHostMalloc((void**)&m.h_best, 2 * sizeof(int32_t), hipHostMallocDefault));
+    if ((rc = alloc((void**)&m.chain_mask, 64 * sizeof(uint64_t)))) return rc;
+    {
+        uint64_t rows[64];
+        for (int i = 0; i < 64; ++i) rows[i] = i == 63 ? ~0ull : ((2ull << i) - 1ull);
+        CPMCU_HIP(hipMemcpy(m.chain_mask, rows, sizeof(rows), hipMemcpyHostToDevice));
+    }
+    // KV pools take what is left of the budget, in whole pages (the reference gives the KV cache
+    // all remaining pool memory, src/model/kvcache.cuh:50).
+    const size_t page_bytes = (size_t)m.kv_heads * kPage * kHeadDim * 2;  // one of K/V, one layer
+    const size_t per_page_all = page_bytes * 2 * m.layers + 4;
+    const size_t remaining = budget > used ? budget - used : 0;
+    const size_t free_now = free_b > used ? free_b - used : 0;
+    size_t pages = std::min(remaining, (size_t)(free_now * 0.95)) / per_page_all;
+    if (pages > (1u << 20)) pages = 1u << 20;
+    if (pages < 1) {
+        set_error("init_storage: memory budget leaves no room for a KV page");
+        return CPMCU_ERR_RUNTIME;
+    }
+    // attention scratch is sized once the context bound is known; take it out of the page count
+    m.attn_ws_bytes = cpmcu_tree_attention_workspace_bytes(max_tree, m.q_heads, m.kv_heads, (int)std::min<size_t>(pages * kPage, 1u << 30));
+    const size_t ws_pages = ceil_div((int)(m.attn_ws_bytes / 1024), (int)(per_page_all / 1024)) + 1;
+    if (pages <= ws_pages) {
+        set_error("init_storage: memory budget too small for the attention workspace");
+        return CPMCU_ERR_RUNTIME;
+    }
+    pages -= ws_pages;
+    CPMCU_HIP(hipMalloc(&m.attn_ws, m.attn_ws_bytes));
+    m.num_pages = (int)pages;
+    m.k_pools.assign(m.layers, nullptr);
+    m.v_pools.assign(m.layers, nullptr);
+    for (int l = 0; l < m.layers; ++l) {
+        CPMCU_HIP(hipMalloc(&m.k_pools[l], page_bytes * pages));
+        CPMCU_HIP(hipMalloc(&m.v_pools[l], page_bytes * pages));
+        CPMCU_HIP(hipMemset(m.k_pools[l], 0, page_bytes * pages));
+        CPMCU_HIP(hipMemset(m.v_pools[l], 0, page_bytes * pages));
+    }
+    CPMCU_HIP(hipMalloc((void**)&m.d_k_pools, m.layers * sizeof(void*)));
+    CPMCU_HIP(hipMalloc((void**)&m.d_v_pools, m.layers * sizeof(void*)));
+    CPMCU_HIP(hipMemcpy(m.d_k_pools, m.k_pools.data(), m.layers * sizeof(void*), hipMemcpyHostToDevice));
+    CPMCU_HIP(hipMemcpy(m.d_v_pools, m.v_pools.data(), m.layers * sizeof(void*), hipMemcpyHostToDevice));
+    CPMCU_HIP(hipMalloc((void**)&m.block_table, pages * sizeof(int32_t)));
+    {
+        std::vector<int32_t> ident(pages);
+        for (size_t i = 0; i < pages; ++i) ident[i] = (int32_t)i;
+        CPMCU_HIP(hipMemcpy(m.block_table, ident.data(), pages * sizeof(int32_t), hipMemcpyHostToDevice));
+    }
+    m.storage = true;
+    if (max_context) *max_context = (int)std::min<size_t>(pages * kPage, 0x7fffffff);
+    return CPMCU_OK;
+}
+
+// Extension (no reference counterpart): install a logical -> physical page permutation.
+extern "C" int cpmcu_set_block_table(const int32_t* host_table, int n) {
+    int rc = require_model(true);
+    if (rc) return rc;
+    Model& m = *g_model;
+    CPMCU_CHECK_ARG(host_table && n >= 1 && n <= m.num_pages, "set_block_table: n=%d outside [1, %d]", n, m.num_pages);
+    std::vector<char> seen(m.num_pages, 0);
+    for (int i = 0; i < n; ++i) {
+        CPMCU_CHECK_ARG(host_table[i] >= 0 && host_table[i] < m.num_pages && !seen[host_table[i]],
+                        "set_block_table: entry %d = %d is out of range or repeated", i, host_table[i]);
+        seen[host_table[i]] = 1;
+    }
+    CPMCU_HIP(hipStreamSynchronize(resolve_stream(nullptr)));
+    CPMCU_HIP(hipMemcpy(m.block_table, host_table, n * sizeof(int32_t), hipMemcpyHostToDevice));
+    return CPMCU_OK;
+}
+
+extern "C" int cpmcu_load_model(const char* name, uint64_t host_ptr) {
+    int rc = require_model(true);
+    if (rc) return rc;
+    Model& m = *g_model;
+    CPMCU_CHECK_ARG(name && host_ptr, "load_model: null argument");
+    const std::string nm(name);
+    hipStream_t st = resolve_stream(nullptr);
+    if (nm.rfind("eagle.token_id_remap", 0) == 0) {  // src/model/minicpm4/minicpm4_eagle.cuh:193-194
+        CPMCU_CHECK_ARG(m.drafter && m.token_id_remap, "load_model: %s given but FR-Spec is not configured", name);
+        CPMCU_HIP(hipMemcpy(m.token_id_remap, (const void*)host_ptr, (size_t)m.frspec_vocab * 4, hipMemcpyHostToDevice));
+        m.remap_loaded = true;
+        return CPMCU_OK;
+    }
+    if (nm.rfind("lm_head", 0) == 0) {  // src/model/model.cuh:116-137 routing by prefix
+        CPMCU_HIP(hipMemcpy(m.lm_head, (const void*)host_ptr, (size_t)m.vocab * m.hidden * 2, hipMemcpyHostToDevice));
+        m.lm_head_loaded = true;
+        if (m.fr_head != m.lm_head) {  // src/model/minicpm4/minicpm4_eagle.cuh:215-219
+            if (!m.remap_loaded) {
+                set_error("load_model: eagle.token_id_remap must be loaded before lm_head.weight");
+                return CPMCU_ERR_RUNTIME;
+            }
+            rc = cpmcu_gather_rows(m.lm_head, m.token_id_remap, m.frspec_vocab, m.hidden, m.fr_head, st);
+            if (rc) return rc;
+            CPMCU_HIP(hipStreamSynchronize(st));
+        }
+        return CPMCU_OK;
+    }
+    set_error("Unsupported name: %s (only lm_head.weight and eagle.token_id_remap belong to the verify/draft path)", name);
+    return CPMCU_ERR_INVALID_ARGUMENT;  // std::invalid_argument, src/model/model.cuh:131-135
+}
+
+extern "C" int cpmcu_prefill(int, int, uint64_t, uint64_t, uint64_t) {
+    set_error("prefill runs the dense transformer layers, which are outside the verify/draft path of this library");
+    return CPMCU_ERR_UNSUPPORTED;
+}
+
+extern "C" int cpmcu_decode(int, int, uint64_t, uint64_t, uint64_t, uint64_t, uint64_t, int) {
+    set_error("decode runs the dense transformer layers, which are outside the verify/draft path of this library; "
+              "use decode_attention and decode_lm_head for the parts that are on it");
+    return CPMCU_ERR_UNSUPPORTED;
+}
+
+extern "C" int cpmcu_draft(uint64_t, uint64_t, uint64_t, uint64_t, uint64_t) {
+    set_error("draft runs the EAGLE decoder layer, which is outside the verify/draft path of this library; "
+              "use draft_head for the FR-Spec head + top-k that is on it");
+    return CPMCU_ERR_UNSUPPORTED;
+}
+
+extern "C" int cpmcu_decode_attention(int layer, int input_length, int padded_length, uint64_t q, uint64_t k_new,
+                                      uint64_t v_new, uint64_t cache_length, uint64_t mask_2d, uint64_t out) {
+    int rc = require_model(true);
+    if (rc) return rc;
+    Model& m = *g_model;
+    CPMCU_CHECK_ARG(layer >= 0 && layer < m.layers, "decode_attention: layer %d outside [0, %d)", layer, m.layers);
+    CPMCU_CHECK_ARG(input_length >= 1 && input_length <= 64, "decode_attention: input_length=%d outside [1, 64]", input_length);
+    CPMCU_CHECK_ARG(padded_length >= input_length && padded_length <= m.num_pages * kPage,
+                    "decode_attention: padded_length=%d outside [%d, %d]", padded_length, input_length, m.num_pages * kPage);
+    CPMCU_CHECK_ARG(q && k_new && v_new && cache_length && out, "decode_attention: null pointer argument");
+    hipStream_t st = resolve_stream(nullptr);
+    PerfScope perf("DECODE_ATTN_CORE", st);
+    rc = cpmcu_kv_append(m.k_pools[layer], m.v_pools[layer], m.block_table, (const void*)k_new, (const void*)v_new,
+                         (const int32_t*)cache_length, input_length, m.kv_heads, st);
+    if (rc) return rc;
+    const uint64_t* mask = mask_2d ? (const uint64_t*)mask_2d : m.chain_mask;
+    return cpmcu_tree_attention((const void*)q, m.k_pools[layer], m.v_pools[layer], m.block_table,
+                                (const int32_t*)cache_length, padded_length, mask, 1, input_length, m.q_heads,
+                                m.kv_heads, 1.f / sqrtf((float)kHeadDim), (void*)out, m.attn_ws, m.attn_ws_bytes, 0, st);
+}
+
+extern "C" int cpmcu_decode_lm_head(int input_length, uint64_t hidden, uint64_t logits, uint64_t gt) {
+    int rc = require_model(true);
+    if (rc) return rc;
+    Model& m = *g_model;
+    CPMCU_CHECK_ARG(m.lm_head_loaded, "decode_lm_head: lm_head.weight has not been loaded");
+    hipStream_t st = resolve_stream(nullptr);
+    PerfScope perf("DECODE_LM_HEAD", st);
+    return cpmcu_lm_head_argmax((const void*)hidden, m.lm_head, input_length, m.vocab, m.hidden, 1, m.scale_lmhead,
+                                (void*)logits, (int32_t*)gt, m.head_ws, m.head_ws_bytes, st);
+}
+
+extern "C" int cpmcu_draft_head(int n, uint64_t hidden, uint64_t topk_val, uint64_t topk_pos, uint64_t topk_ids) {
+    int rc = require_model(true);
+    if (rc) return rc;
+    Model& m = *g_model;
+    if (!m.drafter) {
+        set_error("draft_head: no drafter configured");  // src/model/model.cuh:172-173
+        return CPMCU_ERR_RUNTIME;
+    }
+    CPMCU_CHECK_ARG(m.lm_head_loaded, "draft_head: lm_head.weight has not been loaded");
+    hipStream_t st = resolve_stream(nullptr);
+    PerfScope perf("DRAFT_HEAD", st);
+    return cpmcu_frspec_head_topk((const void*)hidden, m.fr_head, m.fr_head != m.lm_head ? m.token_id_remap : nullptr, n,
+                                  m.frspec_vocab, m.hidden, m.topk_per_iter, m.draft_logits, m.row_stats,
+                                  (void*)topk_val, (int32_t*)topk_pos, (int32_t*)topk_ids, m.head_ws, m.head_ws_bytes, st);
+}
+
+extern "C" int cpmcu_verify_and_fix(int num_tokens, uint64_t pred, uint64_t gt, uint64_t position_ids,
+                                    uint64_t cache_length, uint64_t attn_mask, uint64_t tree_parent,
+                                    int* accept_length) {
+    int rc = require_model(true);
+    if (rc) return rc;
+    Model& m = *g_model;
+    if (!m.drafter) {
+        set_error("verify is not supported: no drafter configured");  // src/model/model.cuh:172-173
+        return CPMCU_ERR_RUNTIME;
+    }
+    CPMCU_CHECK_ARG(num_tokens >= 1 && num_tokens <= 64, "verify_and_fix: num_tokens=%d outside [1, 64]", num_tokens);
+    CPMCU_CHECK_ARG(pred && gt && position_ids && cache_length && attn_mask && tree_parent, "verify_and_fix: null pointer argument");
+    hipStream_t st = resolve_stream(nullptr);
+    PerfScope perf("VERIFY_AND_FIX", st);
+    rc = cpmcu_tree_accept(num_tokens, (int32_t*)pred, (const int32_t*)gt, (const int32_t*)position_ids,
+                           (const int32_t*)cache_length, (const uint64_t*)attn_mask, 1, (const int32_t*)tree_parent,
+                           m.d_best, st);
+    if (rc) return rc;
+    // compaction reads the accept length on the device, so the single D2H copy + sync of the step
+    // (src/model/minicpm4/minicpm4_eagle.cuh:400-401) moves to the end
+    rc = cpmcu_kv_compact(m.d_k_pools, m.d_v_pools, m.layers, m.block_table, m.kv_heads, (int32_t*)pred,
+                          (const int32_t*)gt, (const int32_t*)cache_length, m.d_best, num_tokens, st);
+    if (rc) return rc;
+    CPMCU_HIP(hipMemcpyAsync(m.h_best, m.d_best, 2 * sizeof(int32_t), hipMemcpyDeviceToHost, st));
+    CPMCU_HIP(hipStreamSynchronize(st));
+    if (accept_length) *accept_length = m.h_best[0];
+    return CPMCU_OK;
+}
+
+extern "C" int cpmcu_print_perf_summary(void) {
+    if (!g_model) return CPMCU_OK;
+    printf("%-24s %10s %12s %12s\n", "label", "count", "total ms", "avg ms");
+    for (auto& kv : g_model->perf_log)
+        printf("%-24s %10ld %12.3f %12.4f\n", kv.first.c_str(), kv.second.count, kv.second.ms,
+               kv.second.count ? kv.second.ms / kv.second.count : 0.0);
+    size_t free_b = 0, total_b = 0;
+    if (hipMemGetInfo(&free_b, &total_b) == hipSuccess)
+        printf("GPU memory: %.1f MiB used of %.1f MiB\n", (total_b - free_b) / 1048576.0, total_b / 1048576.0);
+    fflush(stdout);
+    return CPMCU_OK;
+}
+
+// Extension: device pointers of the model's storage for harnesses that fill the cache directly.
+extern "C" int cpmcu_model_pointers(int layer, uint64_t* k_pool, uint64_t* v_pool, uint64_t* block_table,
+                                    int* num_pages) {
+    int rc = require_model(true);
+    if (rc) return rc;
+    Model& m = *g_model;
+    CPMCU_CHECK_ARG(layer >= 0 && layer < m.layers, "model_pointers: layer %d outside [0, %d)", layer, m.layers);
+    if (k_pool) *k_pool = (uint64_t)m.k_pools[layer];
+    if (v_pool) *v_pool = (uint64_t)m.v_pools[layer];
+    if (block_table) *block_table = (uint64_t)m.block_table;
+    if (num_pages) *num_pages = m.num_pages;
+    return CPMCU_OK;
+}
+
+extern "C" int cpmcu_synchronize(void) {
+    CPMCU_HIP(hipStreamSynchronize(resolve_stream(nullptr)));
+    return CPMCU_OK;
+}
+
+extern "C" int cpmcu_shutdown(void) {
+    if (!g_model) return CPMCU_OK;
+    Model& m = *g_model;
+    if (g_stream) (void)hipStreamSynchronize(g_stream);
+    if (m.fr_head && m.fr_head != m.lm_head) (void)hipFree(m.fr_head);
+    (void)hipFree(m.lm_head);
+    (void)hipFree(m.token_id_remap);
+    for (void* p : m.k_pools) (void)hipFree(p);
+    for (void* p : m.v_pools) (void)hipFree(p);
+    (void)hipFree(m.d_k_pools);
+    (void)hipFree(m.d_v_pools);
+    (void)hipFree(m.block_table);
+    (void)hipFree(m.attn_ws);
+    (void)hipFree(m.head_ws);
+    (void)hipFree(m.draft_logits);
+    (void)hipFree(m.row_stats);
+    (void)hipFree(m.d_best);
+    (void)hipFree(m.chain_mask);
+    if (m.h_best) (void)hipHostFree(m.h_best);
+    delete g_model;
+    g_model = nullptr;
+    return CPMCU_OK;
+}

@@ -1,0 +1,196 @@
+// Greedy tree acceptance, accepted-path KV compaction and KV append on the paged cache (gfx950).
+//
+// These are byte/integer paths, bound by launch latency (acceptance) and HBM/L2 (compaction moves
+// a * 2L * Hkv * 256 bytes): no matrix cores, just coalesced 16-byte row moves for K and strided
+// 2-byte moves for the transposed V pages.  The accept length never visits the host between the
+// three kernels: compaction reads it from device memory.
+#include "common.h"
+
+namespace cpmcu {
+namespace {
+
+// verify_kernel, src/model/tree_drafter.cuh:5-46, for T <= 128 (W mask words per row).
+__global__ __launch_bounds__(128) void tree_accept_kernel(int T, int W, int32_t* pred, const int32_t* gt,
+                                                          const int32_t* pos, const int32_t* cache_length,
+                                                          const uint64_t* mask, const int32_t* parent,
+                                                          int32_t* best) {
+    __shared__ uint64_t s_correct[2];
+    __shared__ int32_t mx[128], mi[128];
+    const int i = threadIdx.x;
+    const int S = T > 64 ? 128 : 64;  // tournament slots: next_pow2(max(64, T))
+    // :9-20  correct bit i <=> i == 0 or pred[i] == gt[parent[i]]
+    const bool ok = (i == 0) || (i < T && pred[i] == gt[parent[i]]);
+    const uint64_t ballot = __ballot(ok);
+    if ((i & 63) == 0) s_correct[i >> 6] = ballot;
+    __syncthreads();
+    const int P = cache_length[0];
+    // :22-28  a node counts iff every ancestor (its mask row) is correct
+    bool full = i < T;
+    if (full) {
+        for (int w = 0; w < W; ++w) {
+            const uint64_t mw = mask[(size_t)i * W + w];
+            if ((s_correct[w] & mw) != mw) full = false;
+        }
+    }
+    mx[i] = full ? pos[i] - P + 1 : 1;
+    mi[i] = full ? i : 0;
+    __syncthreads();
+    // :30-36  tournament, upper slot wins only when strictly greater
+    for (int off = S >> 1; off > 0; off >>= 1) {
+        if (i < off && mx[i + off] > mx[i]) {
+            mx[i] = mx[i + off];
+            mi[i] = mi[i + off];
+        }
+        __syncthreads();
+    }
+    if (i == 0) {
+        best[0] = mx[0];
+        best[1] = mi[0];
+    }
+    // :42-45  scatter the accepted path (node indices by depth) into pred
+    const int p = mi[0];
+    if (i < T && ((mask[(size_t)p * W + (i >> 6)] >> (i & 63)) & 1ull)) pred[pos[i] - P] = i;
+}
+
+struct CompactParams {
+    void* const* k_pools;
+    void* const* v_pools;
+    const int32_t* block_table;
+    int Hkv;
+    const int32_t* pred;  // path: node indices by depth
+    const int32_t* cache_length;
+    const int32_t* best;
+    int max_accept;
+};
+
+// fix_kvcache_kernel_1/2, src/model/tree_drafter.cuh:48-77, on the paged layout.  One workgroup per
+// (layer, K|V, kv head).  Sources are read into registers before any destination of the same batch
+// is written; batches go in depth order, and because path[d] >= d a later batch never reads a row
+// an earlier batch wrote -- so the reference's staging buffer is not needed.
+__global__ __launch_bounds__(256) void kv_compact_kernel(CompactParams p) {
+    const int g = blockIdx.x % p.Hkv;
+    const int kv = (blockIdx.x / p.Hkv) & 1;
+    const int layer = blockIdx.x / (2 * p.Hkv);
+    const int tid = threadIdx.x;
+    int a = p.best[0];
+    a = a < p.max_accept ? a : p.max_accept;
+    const int P = p.cache_length[0];
+    if (kv == 0) {
+        f16* pool = (f16*)p.k_pools[layer];
+        const int rr = tid >> 4, ch = tid & 15;  // 16 rows x 16 pieces of 16 bytes
+        for (int d0 = 0; d0 < a; d0 += 16) {
+            const int d = d0 + rr;
+            f16x8 x;
+            const bool act = d < a;
+            if (act) {
+                const int ts = P + p.pred[d];
+                const int pg = p.block_table[ts / kPage];
+                x = *reinterpret_cast<const f16x8*>(pool + (((size_t)pg * p.Hkv + g) * kPage + ts % kPage) * kHeadDim + ch * 8);
+            }
+            // the loads above must have returned before any wave overwrites a source row
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            if (act) {
+                const int td = P + d;
+                const int pg = p.block_table[td / kPage];
+                *reinterpret_cast<f16x8*>(pool + (((size_t)pg * p.Hkv + g) * kPage + td % kPage) * kHeadDim + ch * 8) = x;
+            }
+        }
+    } else {
+        f16* pool = (f16*)p.v_pools[layer];
+        const int rr = tid >> 7, dd = tid & 127;  // 2 tokens x 128 dims
+        for (int d0 = 0; d0 < a; d0 += 2) {
+            const int d = d0 + rr;
+            f16 x = (f16)0.f;
+            const bool act = d < a;
+            if (act) {
+                const int ts = P + p.pred[d];
+                const int pg = p.block_table[ts / kPage];
+                x = pool[(((size_t)pg * p.Hkv + g) * kHeadDim + dd) * kPage + v_slot16(ts % kPage)];
+            }
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            __syncthreads();
+            if (act) {
+                const int td = P + d;
+                const int pg = p.block_table[td / kPage];
+                pool[(((size_t)pg * p.Hkv + g) * kHeadDim + dd) * kPage + v_slot16(td % kPage)] = x;
+            }
+        }
+    }
+}
+
+// src/model/tree_drafter.cuh:74-76: pred[d] <- gt[pred[d]] once every cache has been moved.
+__global__ void accepted_ids_kernel(int32_t* pred, const int32_t* gt, const int32_t* best, int max_accept) {
+    int a = best[0];
+    a = a < max_accept ? a : max_accept;
+    const int d = threadIdx.x;
+    int id = 0;
+    if (d < a) id = gt[pred[d]];
+    __syncthreads();
+    if (d < a) pred[d] = id;
+}
+
+// copy_to_kvcache, src/model/attn.cuh:14-21: token t of the T new rows goes to position *kv_len - T + t.
+__global__ __launch_bounds__(256) void kv_append_kernel(f16* k_pool, f16* v_pool, const int32_t* block_table,
+                                                        const f16* k_new, const f16* v_new,
+                                                        const int32_t* kv_len, int T, int Hkv) {
+    const int t = blockIdx.x;
+    const int tok = kv_len[0] - T + t;
+    const int pg = block_table[tok / kPage];
+    const int slot = tok % kPage;
+    const int row_elems = Hkv * kHeadDim;
+    for (int i = threadIdx.x; i < row_elems / 8; i += 256) {  // K: 16-byte pieces
+        const int g = i / (kHeadDim / 8), ch = i % (kHeadDim / 8);
+        *reinterpret_cast<f16x8*>(k_pool + (((size_t)pg * Hkv + g) * kPage + slot) * kHeadDim + ch * 8) =
+            *reinterpret_cast<const f16x8*>(k_new + (size_t)t * row_elems + i * 8);
+    }
+    for (int i = threadIdx.x; i < row_elems; i += 256) {  // V: transposed, one element per dim
+        const int g = i / kHeadDim, dd = i % kHeadDim;
+        v_pool[(((size_t)pg * Hkv + g) * kHeadDim + dd) * kPage + v_slot16(slot)] = v_new[(size_t)t * row_elems + i];
+    }
+}
+
+}  // namespace
+}  // namespace cpmcu
+
+using namespace cpmcu;
+
+extern "C" int cpmcu_tree_accept(int T, int32_t* pred, const int32_t* gt, const int32_t* position_ids,
+                                 const int32_t* cache_length, const uint64_t* attn_mask, int mask_words,
+                                 const int32_t* tree_parent, int32_t* best, void* stream) {
+    CPMCU_CHECK_ARG(pred && gt && position_ids && cache_length && attn_mask && tree_parent && best,
+                    "tree_accept: null pointer argument");
+    CPMCU_CHECK_ARG(T >= 1 && T <= kMaxTree, "tree_accept: tree size %d outside [1, %d]", T, kMaxTree);
+    CPMCU_CHECK_ARG(mask_words >= 1 && mask_words <= 2 && mask_words * 64 >= T,
+                    "tree_accept: mask_words=%d does not cover T=%d", mask_words, T);
+    hipLaunchKernelGGL(tree_accept_kernel, dim3(1), dim3(128), 0, resolve_stream(stream), T, mask_words, pred, gt,
+                       position_ids, cache_length, attn_mask, tree_parent, best);
+    CPMCU_LAUNCH_CHECK();
+    return CPMCU_OK;
+}
+
+extern "C" int cpmcu_kv_compact(void* const* k_pools, void* const* v_pools, int num_layers,
+                                const int32_t* block_table, int Hkv, int32_t* pred, const int32_t* gt,
+                                const int32_t* cache_length, const int32_t* best, int max_accept, void* stream) {
+    CPMCU_CHECK_ARG(k_pools && v_pools && block_table && pred && gt && cache_length && best,
+                    "kv_compact: null pointer argument");
+    CPMCU_CHECK_ARG(num_layers >= 1 && Hkv >= 1, "kv_compact: num_layers=%d Hkv=%d", num_layers, Hkv);
+    CPMCU_CHECK_ARG(max_accept >= 1 && max_accept <= kMaxTree, "kv_compact: max_accept=%d outside [1, %d]", max_accept, kMaxTree);
+    CompactParams p{k_pools, v_pools, block_table, Hkv, pred, cache_length, best, max_accept};
+    hipStream_t st = resolve_stream(stream);
+    hipLaunchKernelGGL(kv_compact_kernel, dim3(num_layers * 2 * Hkv), dim3(256), 0, st, p);
+    CPMCU_LAUNCH_CHECK();
+    hipLaunchKernelGGL(accepted_ids_kernel, dim3(1), dim3(128), 0, st, pred, gt, best, max_accept);
+    CPMCU_LAUNCH_CHECK();
+    return CPMCU_OK;
+}
+
+extern "C" int cpmcu_kv_append(void* k_pool, void* v_pool, const int32_t* block_table, const void* k_new,
+                               const void* v_new, const int32_t* kv_len, int T, int Hkv, void* stream) {
+    CPMCU_CHECK_ARG(k_pool && v_pool && block_table && k_new && v_new && kv_len, "kv_append: null pointer argument");
+    CPMCU_CHECK_ARG(T >= 1 && Hkv >= 1, "kv_append: T=%d Hkv=%d", T, Hkv);
+    hipLaunchKernelGGL(kv_append_kernel, dim3(T), dim3(256), 0, resolve_stream(stream), (f16*)k_pool, (f16*)v_pool,
+                       block_table, (const f16*)k_new, (const f16*)v_new, kv_len, T, Hkv);
+    CPMCU_LAUNCH_CHECK();
+    return CPMCU_OK;
+}

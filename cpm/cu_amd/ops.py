@@ -1,0 +1,159 @@
+"""The operators of the verify/draft path on torch device tensors.
+
+torch only supplies device memory and the current stream; every function here is a thin call into
+``libcpmcu_amd.so`` through the C-ABI (``include/cpmcu_amd.h``).  Nothing falls back to torch math.
+"""
+import ctypes
+import math
+
+import torch
+
+from . import lib as _libmod
+from .kvcache import HEAD_DIM
+
+
+def _lib():
+    return _libmod.get()
+
+
+def _ptr(t):
+    if t is None:
+        return None
+    assert t.is_cuda and t.is_contiguous(), "device-resident contiguous tensor required"
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+_workspaces = {}
+
+
+def _workspace(kind, nbytes, device):
+    key = (kind, device)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def mask_words(T):
+    return (T + 63) // 64
+
+
+def kv_append(cache, layer, k_new, v_new, kv_len):
+    """copy_to_kvcache (src/model/attn.cuh:14-21): rows go to positions [*kv_len - T, *kv_len)."""
+    T = k_new.shape[0]
+    assert k_new.dtype == torch.float16 and v_new.dtype == torch.float16 and kv_len.dtype == torch.int32
+    assert k_new.numel() == T * cache.Hkv * HEAD_DIM and v_new.numel() == k_new.numel()
+    _lib().kv_append(_ptr(cache.k[layer]), _ptr(cache.v[layer]), _ptr(cache.block_table), _ptr(k_new), _ptr(v_new),
+                     _ptr(kv_len), T, cache.Hkv, _stream())
+
+
+def tree_attention(q, cache, layer, kv_len, max_kv_len, mask=None, scale=None, num_splits=0, out=None):
+    """mha_fwd_kvcache with a tree mask (src/flash_attn/flash_api.hpp:292-392) on the paged cache.
+
+    q [T, Hq, 128] fp16; kv_len int32[1] on the device = P + T; mask uint64 [T, W] or None (chain).
+    """
+    T, Hq, D = q.shape
+    assert D == HEAD_DIM and q.dtype == torch.float16 and kv_len.dtype == torch.int32
+    if out is None:
+        out = torch.empty_like(q)
+    W = 0
+    if mask is not None:
+        assert mask.dtype in (torch.uint64, torch.int64)
+        mask = mask.reshape(T, -1)
+        W = mask.shape[1]
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    need = _lib().raw.cpmcu_tree_attention_workspace_bytes(T, Hq, cache.Hkv, int(max_kv_len))
+    ws = _workspace("attn", need, q.device)
+    _lib().tree_attention(_ptr(q), _ptr(cache.k[layer]), _ptr(cache.v[layer]), _ptr(cache.block_table), _ptr(kv_len),
+                          int(max_kv_len), _ptr(mask), W, T, Hq, cache.Hkv, ctypes.c_float(scale), _ptr(out),
+                          _ptr(ws), ws.numel(), int(num_splits), _stream())
+    return out
+
+
+def gather_rows(src, remap):
+    """remap_copy (src/model/tree_drafter.cuh:79-86): dst[r] = src[remap[r]]."""
+    assert src.dtype == torch.float16 and remap.dtype == torch.int32
+    dst = torch.empty((remap.numel(), src.shape[1]), dtype=torch.float16, device=src.device)
+    _lib().gather_rows(_ptr(src), _ptr(remap), remap.numel(), src.shape[1], _ptr(dst), _stream())
+    return dst
+
+
+def frspec_head_topk(hidden, w, token_id_remap, k):
+    """FR-Spec draft head: logits -> log-softmax -> top-k -> full-vocabulary ids.
+
+    Returns dict(logits [n,V] f16 raw, row_stats [n,2] f32 (max, ln sum), val [n,k] f16, pos [n,k] i32, ids [n,k] i32).
+    """
+    n, H = hidden.shape
+    V = w.shape[0]
+    dev = hidden.device
+    logits = torch.empty((n, V), dtype=torch.float16, device=dev)
+    stats = torch.empty((n, 2), dtype=torch.float32, device=dev)
+    val = torch.empty((n, k), dtype=torch.float16, device=dev)
+    pos = torch.empty((n, k), dtype=torch.int32, device=dev)
+    ids = torch.empty((n, k), dtype=torch.int32, device=dev)
+    ws = _workspace("head", _lib().raw.cpmcu_head_workspace_bytes(n, V), dev)
+    _lib().frspec_head_topk(_ptr(hidden), _ptr(w), _ptr(token_id_remap), n, V, H, k, _ptr(logits), _ptr(stats),
+                            _ptr(val), _ptr(pos), _ptr(ids), _ptr(ws), ws.numel(), _stream())
+    return dict(logits=logits, row_stats=stats, val=val, pos=pos, ids=ids)
+
+
+def lm_head_argmax(hidden, w, head_scale=None, want_logits=False, gt=None):
+    """Target head + arg-max (src/model/linear.cuh:82-101 + torch argmax of tree_drafter.py:233)."""
+    n, H = hidden.shape
+    V = w.shape[0]
+    dev = hidden.device
+    logits = torch.empty((n, V), dtype=torch.float16, device=dev) if want_logits else None
+    if gt is None:
+        gt = torch.empty(n, dtype=torch.int32, device=dev)
+    ws = _workspace("head", _lib().raw.cpmcu_head_workspace_bytes(n, V), dev)
+    _lib().lm_head_argmax(_ptr(hidden), _ptr(w), n, V, H, 0 if head_scale is None else 1,
+                          ctypes.c_float(1.0 if head_scale is None else head_scale), _ptr(logits), _ptr(gt),
+                          _ptr(ws), ws.numel(), _stream())
+    return (gt, logits) if want_logits else gt
+
+
+def log_softmax_(x):
+    """In place (src/model/eagle.cuh:29-89); returns row_stats [n,2] (max, ln sum)."""
+    n, dim = x.shape
+    stats = torch.empty((n, 2), dtype=torch.float32, device=x.device)
+    _lib().log_softmax(_ptr(x), n, dim, _ptr(stats), _stream())
+    return stats
+
+
+def topk(x, top):
+    """TopK::prefill (src/model/topk.cuh:255-288): value descending, ties -> lower index."""
+    n, dim = x.shape
+    val = torch.empty((n, top), dtype=torch.float16, device=x.device)
+    pos = torch.empty((n, top), dtype=torch.int32, device=x.device)
+    ws = _workspace("topk", _lib().raw.cpmcu_topk_workspace_bytes(n, dim, top), x.device)
+    _lib().topk(_ptr(x), n, dim, top, _ptr(val), _ptr(pos), _ptr(ws), ws.numel(), _stream())
+    return val, pos
+
+
+def remap(pos, token_id_remap):
+    out = torch.empty_like(pos)
+    _lib().remap(_ptr(pos), pos.numel(), _ptr(token_id_remap), _ptr(out), _stream())
+    return out
+
+
+def tree_accept(pred, gt, position_ids, cache_length, attn_mask, tree_parent, best=None):
+    """verify_kernel (src/model/tree_drafter.cuh:5-46). pred is overwritten with the path; returns best[2]."""
+    T = pred.numel()
+    if best is None:
+        best = torch.empty(2, dtype=torch.int32, device=pred.device)
+    W = attn_mask.numel() // T
+    _lib().tree_accept(T, _ptr(pred), _ptr(gt), _ptr(position_ids), _ptr(cache_length), _ptr(attn_mask), W,
+                       _ptr(tree_parent), _ptr(best), _stream())
+    return best
+
+
+def kv_compact(cache, pred, gt, cache_length, best, max_accept):
+    """fix_kv_cache (src/model/tree_drafter.cuh:48-77) on every layer of the paged cache."""
+    _lib().kv_compact(_ptr(cache.k_ptrs), _ptr(cache.v_ptrs), cache.num_layers, _ptr(cache.block_table), cache.Hkv,
+                      _ptr(pred), _ptr(gt), _ptr(cache_length), _ptr(best), int(max_accept), _stream())

@@ -1,0 +1,259 @@
+/*
+ * libcpmcu_amd -- C-ABI of the MI355X (gfx950) speculative-decoding verify/draft path.
+ *
+ * Two groups of entry points:
+ *
+ *  1. the model-level mirror of the reference's pybind module `cpmcu.C`
+ *     (src/entry.cu:98-534): same names with a `cpmcu_` prefix, same parameter
+ *     lists, `const char*` for the name and `uint64_t` for raw pointers.  State
+ *     is one process-global model, as in the reference (src/entry.cu:98).
+ *
+ *  2. operator-level entry points for the four subsystems of the path, with
+ *     explicit shapes, device pointers and a stream handle.  They have no
+ *     counterpart at the reference's boundary; each cites the reference
+ *     function whose work it does.
+ *
+ * Conventions
+ *   - every function returns a status (CPMCU_OK = 0); on failure the message is
+ *     available from cpmcu_last_error() (thread-local).  The Python shim maps
+ *     CPMCU_ERR_INVALID_ARGUMENT to ValueError and everything else to
+ *     RuntimeError, matching how std::invalid_argument / std::runtime_error
+ *     cross pybind in the reference.
+ *   - "device pointer" = HIP device memory owned by the caller for the duration
+ *     of the call; fp16 tensors are IEEE binary16, row-major unless stated.
+ *   - `stream` is a hipStream_t passed as void*; NULL selects the library's own
+ *     blocking stream (the counterpart of calc_stream, src/utils.cu:6,19).
+ *   - operator-level calls only enqueue work; they never synchronise.
+ *
+ * Paged KV cache layout (this library's own; the reference keeps flat
+ * [budget, kv_heads*head_dim] buffers, src/model/kvcache.cuh:18-25, and its
+ * layout never crosses the boundary):
+ *   page size 256 tokens, head_dim 128.
+ *   K pool  [num_pages][Hkv][256][128] fp16 -- one token's head row is 256 B.
+ *   V pool  [num_pages][Hkv][128][256] fp16 -- transposed (dim-major) so that
+ *           the P.V matrix product reads 8 consecutive tokens per lane; inside
+ *           every aligned group of 16 tokens the slot of token t is
+ *           (t & 3) | ((t & 4) << 1) | ((t & 8) >> 1)   (bits 2 and 3 swapped),
+ *           which is the order in which the MFMA accumulator of Q.K^T hands
+ *           the probabilities to the next MFMA.
+ *   block_table[i] = physical page of logical page i (tokens 256i..256i+255);
+ *   one table serves every layer, each layer has its own K and V pool.
+ */
+#ifndef CPMCU_AMD_H
+#define CPMCU_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CPMCU_OK 0
+#define CPMCU_ERR_INVALID_ARGUMENT 1 /* -> ValueError  (std::invalid_argument in the reference) */
+#define CPMCU_ERR_RUNTIME 2          /* -> RuntimeError (std::runtime_error) */
+#define CPMCU_ERR_UNSUPPORTED 3      /* -> RuntimeError: entry point outside the verify/draft path */
+#define CPMCU_ERR_HIP 4              /* -> RuntimeError: a HIP call failed */
+
+#define CPMCU_PAGE_SIZE 256
+#define CPMCU_HEAD_DIM 128
+#define CPMCU_MAX_TREE 128
+
+const char* cpmcu_last_error(void);
+/* Library version string and the GPU architecture the kernels were built for. */
+const char* cpmcu_version(void);
+
+/* ------------------------------------------------------------------------- */
+/* 1. Model-level mirror of src/entry.cu                                      */
+/* ------------------------------------------------------------------------- */
+
+/* src/entry.cu:100-136 init_base_model.  Records the target-model geometry.
+ * torch_dtype: 0 = fp16 (1 = bf16 is rejected: "dtype not compiled",
+ * src/entry.cu:43,52). */
+int cpmcu_init_base_model(float memory_limit, int vocab_size, int num_hidden_layers, int hidden_size,
+                          int intermediate_size, int num_attention_heads, int num_key_value_heads,
+                          int head_dim, float rms_norm_eps, int torch_dtype, int chunk_length,
+                          float scale_embed, float scale_lmhead, float scale_residual);
+
+/* src/entry.cu:278-301 init_eagle_model. */
+int cpmcu_init_eagle_model(int num_layers, int num_iter, int topk_per_iter, int tree_size, int torch_dtype);
+
+/* src/entry.cu:303-341 init_minicpm4_eagle_model (FR-Spec drafter over the base model). */
+int cpmcu_init_minicpm4_eagle_model(int num_layers, int num_iter, int topk_per_iter, int tree_size,
+                                    int torch_dtype, int apply_eagle_quant, int group_size,
+                                    int eagle_window_size, int frspec_vocab_size, float residual_scale,
+                                    int use_input_norm, int use_attn_norm);
+
+/* src/entry.cu:462-464 init_storage: allocates lm_head, the FR-Spec sub-matrix,
+ * the paged KV pools of every layer, the page table and scratch; writes the
+ * maximum supported context (tokens) to *max_context. */
+int cpmcu_init_storage(int* max_context);
+
+/* src/entry.cu:466-468 load_model: blocking H2D copy of one named tensor from a
+ * HOST pointer.  Names on this path: "lm_head.weight" ([vocab, hidden] fp16),
+ * "eagle.token_id_remap" ([frspec_vocab] int32; must be loaded before
+ * lm_head.weight, src/model/minicpm4/minicpm4_eagle.cuh:193-194,215-219).
+ * Any other name -> CPMCU_ERR_INVALID_ARGUMENT (src/model/model.cuh:131-135). */
+int cpmcu_load_model(const char* name, uint64_t host_ptr);
+
+/* src/entry.cu:470-472 / :474-496 / :498-500.  prefill and decode need the dense
+ * transformer layers and draft needs the EAGLE layer, none of which is part of
+ * this path: they return CPMCU_ERR_UNSUPPORTED.  The parts of decode that are on
+ * the path are cpmcu_decode_attention and cpmcu_decode_lm_head below. */
+int cpmcu_prefill(int input_length, int history_length, uint64_t input, uint64_t position_ids, uint64_t output);
+int cpmcu_decode(int input_length, int padded_length, uint64_t input, uint64_t position_ids,
+                 uint64_t cache_length, uint64_t mask_2d, uint64_t output, int cuda_graph);
+int cpmcu_draft(uint64_t tree_draft_ids, uint64_t tree_position_ids, uint64_t cache_length,
+                uint64_t attn_mask, uint64_t tree_parent);
+
+/* src/entry.cu:502-504 verify_and_fix -> MiniCPM4EagleImpl::verify
+ * (src/model/minicpm4/minicpm4_eagle.cuh:398-418): greedy tree acceptance,
+ * one stream synchronisation, compaction of the accepted rows in the K and V
+ * pools of every layer, pred[0..a) <- accepted token ids.  All pointers are
+ * device pointers; attn_mask has one uint64 per row (num_tokens <= 64, as at the
+ * reference's boundary).  *accept_length receives a. */
+int cpmcu_verify_and_fix(int num_tokens, uint64_t pred, uint64_t gt, uint64_t position_ids,
+                         uint64_t cache_length, uint64_t attn_mask, uint64_t tree_parent,
+                         int* accept_length);
+
+/* src/entry.cu:506-508 print_perf_summary: prints the per-operator event timings
+ * collected when CPMCU_PERF=1 is set in the environment. */
+int cpmcu_print_perf_summary(void);
+
+/* The slice of Attention::decode that is on the path (src/model/attn.cuh:199-229):
+ * append the input_length new K/V rows of `layer` at cache rows
+ * [cache_length - input_length, cache_length) and run tree attention over the
+ * model's paged cache.  cache_length is the device scalar already incremented by
+ * input_length, as cpmcu/llm.py:272 leaves it for the reference's flash call.
+ *   q [input_length][Hq][D], k_new/v_new [input_length][Hkv*D], out like q.
+ * mask_2d: uint64 per row, 0 = causal chain (no tree). */
+int cpmcu_decode_attention(int layer, int input_length, int padded_length, uint64_t q, uint64_t k_new,
+                           uint64_t v_new, uint64_t cache_length, uint64_t mask_2d, uint64_t out);
+
+/* LMHead::prefill on the loaded lm_head (src/model/linear.cuh:82-101,
+ * src/model/model.cuh:164) plus the arg-max the reference leaves to PyTorch
+ * (cpmcu/speculative/tree_drafter.py:153,233).  logits ([>=n][vocab] fp16) and
+ * gt (int32[n]) may each be 0 to skip that output. */
+int cpmcu_decode_lm_head(int input_length, uint64_t hidden, uint64_t logits, uint64_t gt);
+
+/* FR-Spec draft head on the loaded sub-matrix: logits' = hidden . W'^T, log-softmax,
+ * top-k, ids mapped back to the full vocabulary
+ * (src/model/minicpm4/minicpm4_eagle.cuh:319-326,366-368).
+ *   hidden [n][H]; out: topk_val [n][k] fp16 (log-probs), topk_pos [n][k] int32
+ *   (FR-Spec indices), topk_ids [n][k] int32 (full-vocabulary ids). */
+int cpmcu_draft_head(int n, uint64_t hidden, uint64_t topk_val, uint64_t topk_pos, uint64_t topk_ids);
+
+/* No reference counterpart: install a logical -> physical page permutation (host int32[n], a
+ * partial permutation of [0, num_pages)); the default table is the identity. */
+int cpmcu_set_block_table(const int32_t* host_table, int n);
+
+/* No reference counterpart: device addresses of the model's storage, for harnesses that fill the
+ * paged cache directly (any of the outputs may be NULL). */
+int cpmcu_model_pointers(int layer, uint64_t* k_pool, uint64_t* v_pool, uint64_t* block_table, int* num_pages);
+
+/* Synchronise the library's stream. */
+int cpmcu_synchronize(void);
+/* Free everything the global model owns (the reference never frees). */
+int cpmcu_shutdown(void);
+
+/* ------------------------------------------------------------------------- */
+/* 2. Operator-level entry points                                             */
+/* ------------------------------------------------------------------------- */
+
+/* KV append -- copy_to_kvcache, src/model/attn.cuh:14-21,42-47,200.
+ * Writes T new token rows of one layer into the paged pools at token positions
+ * [*kv_len - T, *kv_len).  k_new, v_new: [T][Hkv][128] fp16 row-major.
+ * kv_len: device int32[1], total length after the append. */
+int cpmcu_kv_append(void* k_pool, void* v_pool, const int32_t* block_table, const void* k_new,
+                    const void* v_new, const int32_t* kv_len, int T, int Hkv, void* stream);
+
+/* Bytes of scratch cpmcu_tree_attention needs for these shapes (split-KV partials). */
+size_t cpmcu_tree_attention_workspace_bytes(int T, int Hq, int Hkv, int max_kv_len);
+
+/* Tree-verify attention -- mha_fwd_kvcache with a 2-D tree mask,
+ * src/flash_attn/flash_api.hpp:292-392; kernel body
+ * src/flash_attn/src/flash_fwd_kernel.h:1175-1766; mask src/flash_attn/src/mask.h:139-229;
+ * split merge src/flash_attn/src/flash_fwd_kernel.h:2320-2501.
+ *   q   [T][Hq][128] fp16;  out [T][Hq][128] fp16
+ *   kv_len: device int32[1] = P + T (the true length is read on the device, as
+ *           the reference reads cu_seqlens_k, flash_api.hpp:383-385); the tree
+ *           nodes are the last T tokens, in node order.
+ *   max_kv_len: host upper bound of *kv_len used for the launch geometry (the
+ *           reference's padded_length).
+ *   mask [T][mask_words] uint64: bit j of row i = node i attends tree node j;
+ *           NULL = causal chain.
+ *   scale: softmax scale (1/sqrt(128) in the reference, flash_api.hpp:360).
+ *   workspace: device scratch of at least ..._workspace_bytes(), may be NULL
+ *           when that is 0.
+ *   num_splits_override: 0 = choose from max_kv_len; >0 forces the KV split count. */
+int cpmcu_tree_attention(const void* q, const void* k_pool, const void* v_pool, const int32_t* block_table,
+                         const int32_t* kv_len, int max_kv_len, const uint64_t* mask, int mask_words,
+                         int T, int Hq, int Hkv, float scale, void* out, void* workspace,
+                         size_t workspace_bytes, int num_splits_override, void* stream);
+
+/* remap_copy -- src/model/tree_drafter.cuh:79-86,103-107: dst[r][:] = src[remap[r]][:]. */
+int cpmcu_gather_rows(const void* src, const int32_t* remap, int rows, int dim, void* dst, void* stream);
+
+/* Bytes of scratch the two head operators need. */
+size_t cpmcu_head_workspace_bytes(int n, int V);
+
+/* FR-Spec draft head with fused log-softmax statistics, top-k and id map-back --
+ * Linear::prefill (src/model/linear.cuh:8-37,73-79) + log_softmax
+ * (src/model/eagle.cuh:29-89) + TopK::prefill (src/model/topk.cuh:158-213,255-288)
+ * + remap (src/model/tree_drafter.cuh:88-90).
+ *   hidden [n][H] fp16 (n <= 16); w [V][H] fp16 (the gathered sub-matrix);
+ *   logits [n][V] fp16 scratch/output (raw logits z);
+ *   row_stats [n][2] fp32 output: (max z, ln sum exp(z - max));
+ *   topk_val [n][k] fp16 = f16((z - max) - lnsum); topk_pos [n][k] int32 index into w;
+ *   topk_ids [n][k] int32 = token_id_remap[topk_pos] (token_id_remap NULL -> ids = pos).
+ * Ordering: value descending, ties -> lower index (src/model/topk.cuh:17). k <= 32. */
+int cpmcu_frspec_head_topk(const void* hidden, const void* w, const int32_t* token_id_remap, int n, int V,
+                           int H, int k, void* logits, float* row_stats, void* topk_val, int32_t* topk_pos,
+                           int32_t* topk_ids, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Target head with fused arg-max -- LMHead::prefill (src/model/linear.cuh:82-101;
+ * fp16 pre-scale by head_scale when apply_scale != 0) + torch argmax
+ * (cpmcu/speculative/tree_drafter.py:153,233; lowest index on ties).
+ *   hidden [n][H] fp16 (n <= 128); w [V][H]; logits [n][V] fp16 or NULL (not
+ *   materialised); gt int32[n] or NULL. */
+int cpmcu_lm_head_argmax(const void* hidden, const void* w, int n, int V, int H, int apply_scale,
+                         float head_scale, void* logits, int32_t* gt, void* workspace,
+                         size_t workspace_bytes, void* stream);
+
+/* log_softmax in place -- src/model/eagle.cuh:29-89.  x [n][dim] fp16;
+ * row_stats [n][2] fp32 (max, ln sum) output, may be NULL. */
+int cpmcu_log_softmax(void* x, int n, int dim, float* row_stats, void* stream);
+
+/* TopK::prefill -- src/model/topk.cuh:255-288: per row the `top` largest values,
+ * value descending, ties -> lower index.  top <= min(dim, 128).
+ * workspace: at least cpmcu_topk_workspace_bytes(n, dim, top). */
+size_t cpmcu_topk_workspace_bytes(int n, int dim, int top);
+int cpmcu_topk(const void* x, int n, int dim, int top, void* val, int32_t* pos, void* workspace,
+               size_t workspace_bytes, void* stream);
+
+/* remap -- src/model/tree_drafter.cuh:88-90: out[i] = token_id_remap[in[i]]. */
+int cpmcu_remap(const int32_t* in, int n, const int32_t* token_id_remap, int32_t* out, void* stream);
+
+/* Greedy tree acceptance -- verify_kernel, src/model/tree_drafter.cuh:5-46, extended
+ * to T <= 128 (mask_words = ceil(T/64) uint64 per row; tournament over
+ * next_pow2(max(64, T)) slots, identical to the reference for T <= 64).
+ *   pred int32[T] in: draft ids; out: pred[0..a) = node indices of the accepted
+ *   path in depth order (the reference's scatter, :42-45).
+ *   best int32[2] out: (a, winning node).  cache_length: device int32[1] = P. */
+int cpmcu_tree_accept(int T, int32_t* pred, const int32_t* gt, const int32_t* position_ids,
+                      const int32_t* cache_length, const uint64_t* attn_mask, int mask_words,
+                      const int32_t* tree_parent, int32_t* best, void* stream);
+
+/* Accepted-path compaction -- fix_kv_cache, src/model/tree_drafter.cuh:48-77,97-101.
+ * For every layer l < num_layers and d < a: token P + pred[d] of k_pools[l] /
+ * v_pools[l] moves to token P + d; then pred[d] <- gt[pred[d]] (accepted ids).
+ * a is read on the device from best[0] (no host round trip); max_accept bounds it
+ * for the launch.  k_pools / v_pools: device arrays of num_layers pool pointers. */
+int cpmcu_kv_compact(void* const* k_pools, void* const* v_pools, int num_layers, const int32_t* block_table,
+                     int Hkv, int32_t* pred, const int32_t* gt, const int32_t* cache_length,
+                     const int32_t* best, int max_accept, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

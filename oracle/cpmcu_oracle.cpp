@@ -1,0 +1,352 @@
+// CPU oracle -- TEST INFRASTRUCTURE ONLY (see cpmcu_oracle.h for the contract,
+// the reference citations of every function and what pins each of them).
+//
+// Build: make -C oracle   (g++ -O3 -march=x86-64-v3 -fopenmp, no GPU deps)
+
+#include "cpmcu_oracle.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <limits>
+#include <numeric>
+#include <vector>
+
+#ifdef _OPENMP
+#include <omp.h>
+#endif
+#ifdef __F16C__
+#include <immintrin.h>
+#endif
+
+namespace {
+
+int g_threads = 0;  // 0 = OpenMP default
+
+// ---- software binary16 <-> binary32 (reference implementation; the F16C
+// path below must agree with it bit for bit, which the unit tests check) ----
+inline float half_to_float_sw(uint16_t h) {
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1Fu;
+    uint32_t man = h & 0x3FFu;
+    uint32_t bits;
+    if (exp == 0) {
+        if (man == 0) {
+            bits = sign;
+        } else {  // subnormal: normalise
+            int e = -1;
+            do { man <<= 1; ++e; } while ((man & 0x400u) == 0);
+            bits = sign | ((uint32_t)(127 - 15 - e) << 23) | ((man & 0x3FFu) << 13);
+        }
+    } else if (exp == 31) {
+        bits = sign | 0x7F800000u | (man << 13);
+    } else {
+        bits = sign | ((exp + 112u) << 23) | (man << 13);
+    }
+    float f;
+    std::memcpy(&f, &bits, 4);
+    return f;
+}
+
+inline uint16_t float_to_half_sw(float f) {
+    uint32_t x;
+    std::memcpy(&x, &f, 4);
+    uint16_t sign = (uint16_t)((x >> 16) & 0x8000u);
+    uint32_t absx = x & 0x7FFFFFFFu;
+    if (absx >= 0x7F800000u) {  // inf / nan
+        return (uint16_t)(sign | 0x7C00u | (absx > 0x7F800000u ? 0x200u | ((absx >> 13) & 0x3FFu) : 0u));
+    }
+    if (absx >= 0x477FF000u) {  // >= 65520 rounds to inf
+        return (uint16_t)(sign | 0x7C00u);
+    }
+    if (absx < 0x33000001u) {  // <= 2^-25 rounds to zero (tie at exactly 2^-25 -> even = 0)
+        return sign;
+    }
+    int32_t e = (int32_t)(absx >> 23) - 127;
+    uint32_t m = (absx & 0x7FFFFFu) | 0x800000u;
+    int shift;
+    uint32_t base;
+    if (e < -14) {  // subnormal half: value = m * 2^(e-23), unit = 2^-24
+        shift = 13 + (-14 - e);
+        base = 0;
+    } else {
+        shift = 13;
+        base = ((uint32_t)(e + 15) << 10) - 0x400u;  // hidden bit of m adds 0x400
+    }
+    uint32_t q = m >> shift;
+    uint32_t rem = m & ((1u << shift) - 1u);
+    uint32_t half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (q & 1u))) ++q;
+    return (uint16_t)(sign | (base + q));
+}
+
+inline float h2f(uint16_t h) {
+#ifdef __F16C__
+    return _cvtsh_ss(h);
+#else
+    return half_to_float_sw(h);
+#endif
+}
+inline uint16_t f2h(float f) {
+#ifdef __F16C__
+    return _cvtss_sh(f, _MM_FROUND_TO_NEAREST_INT | _MM_FROUND_NO_EXC);
+#else
+    return float_to_half_sw(f);
+#endif
+}
+
+// dot product with 16 interleaved fp32 partial sums (lane = k mod 16) and a
+// fixed pairwise tree at the end.  n must be a multiple of 16.
+inline float dot16(const float* a, const float* b, int n) {
+    float acc[16];
+    for (int j = 0; j < 16; ++j) acc[j] = 0.f;
+    for (int k = 0; k < n; k += 16) {
+        for (int j = 0; j < 16; ++j) acc[j] = std::fma(a[k + j], b[k + j], acc[j]);
+    }
+    for (int w = 8; w >= 1; w >>= 1)
+        for (int j = 0; j < w; ++j) acc[j] += acc[j + w];
+    return acc[0];
+}
+
+inline float dot_any(const float* a, const float* b, int n) {
+    int n16 = n & ~15;
+    float r = n16 ? dot16(a, b, n16) : 0.f;
+    for (int k = n16; k < n; ++k) r = std::fma(a[k], b[k], r);
+    return r;
+}
+
+inline int threads() {
+#ifdef _OPENMP
+    return g_threads > 0 ? g_threads : omp_get_max_threads();
+#else
+    return 1;
+#endif
+}
+
+}  // namespace
+
+extern "C" {
+
+void orc_f16_to_f32(const uint16_t* in, float* out, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) out[i] = h2f(in[i]);
+}
+void orc_f32_to_f16(const float* in, uint16_t* out, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) out[i] = f2h(in[i]);
+}
+// software versions, exported so the tests can check the F16C path against them
+void orc_f16_to_f32_sw(const uint16_t* in, float* out, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) out[i] = half_to_float_sw(in[i]);
+}
+void orc_f32_to_f16_sw(const float* in, uint16_t* out, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) out[i] = float_to_half_sw(in[i]);
+}
+
+int orc_num_threads(void) { return threads(); }
+void orc_set_num_threads(int n) { g_threads = n; }
+
+// A1 -- src/flash_attn/src/mask.h:139-229, softmax.h:66-91,239-256,
+// flash_fwd_kernel.h:1266,1610-1615, flash_api.hpp:103.
+void orc_tree_attention(const uint16_t* q, const uint16_t* k, const uint16_t* v,
+                        const uint64_t* mask, int T, int P, int Hq, int Hkv, int D,
+                        int mask_words, float scale, uint16_t* out, float* lse) {
+    const int S = P + T;
+    const int group = Hq / Hkv;
+    // flash_api.hpp:103  scale_softmax_log2 = softmax_scale * M_LOG2E
+    const float scale_log2 = scale * (float)M_LOG2E;
+    std::vector<float> kf((size_t)S * D), vf((size_t)S * D);
+    for (int g = 0; g < Hkv; ++g) {
+        for (int c = 0; c < S; ++c) {
+            const uint16_t* kr = k + ((size_t)c * Hkv + g) * D;
+            const uint16_t* vr = v + ((size_t)c * Hkv + g) * D;
+            for (int d = 0; d < D; ++d) {
+                kf[(size_t)c * D + d] = h2f(kr[d]);
+                vf[(size_t)c * D + d] = h2f(vr[d]);
+            }
+        }
+        const int rows = group * T;
+#pragma omp parallel num_threads(threads())
+        {
+            std::vector<float> s(S), qf(D), o(D);
+#pragma omp for schedule(dynamic, 4)
+            for (int r = 0; r < rows; ++r) {
+                const int h = g * group + r / T;  // flash_fwd_kernel.h:1266 kv head = h / group
+                const int i = r % T;
+                const uint16_t* qr = q + ((size_t)i * Hq + h) * D;
+                for (int d = 0; d < D; ++d) qf[d] = h2f(qr[d]);
+                const uint64_t* mrow = mask + (size_t)i * mask_words;
+                float m = -std::numeric_limits<float>::infinity();
+                for (int c = 0; c < S; ++c) {
+                    bool vis = true;
+                    if (c >= P) {  // mask.h:187,194-198 tree bit; :185-186 causal j <= i
+                        int j = c - P;
+                        vis = (j <= i) && ((mrow[j >> 6] >> (j & 63)) & 1ull);
+                    }
+                    if (vis) {
+                        s[c] = dot_any(qf.data(), &kf[(size_t)c * D], D);
+                        m = std::max(m, s[c]);
+                    } else {
+                        s[c] = -std::numeric_limits<float>::infinity();
+                    }
+                }
+                // softmax.h:66-91: exp2f(x*scale_log2 - max*scale_log2); max=-inf -> 0
+                const float max_scaled = (m == -std::numeric_limits<float>::infinity()) ? 0.f : m * scale_log2;
+                float l = 0.f;
+                for (int d = 0; d < D; ++d) o[d] = 0.f;
+                for (int c = 0; c < S; ++c) {
+                    if (s[c] == -std::numeric_limits<float>::infinity()) continue;
+                    float p = exp2f(s[c] * scale_log2 - max_scaled);
+                    l += p;  // row sum uses the fp32 p (softmax.h:157-200)
+                    float ph = h2f(f2h(p));  // flash_fwd_kernel.h:1610 P -> fp16 before P.V
+                    const float* vr = &vf[(size_t)c * D];
+                    for (int d = 0; d < D; ++d) o[d] = std::fma(ph, vr[d], o[d]);
+                }
+                // softmax.h:239-256
+                const bool bad = (l == 0.f || l != l);
+                const float inv = bad ? 1.f : 1.f / l;
+                uint16_t* orow = out + ((size_t)i * Hq + h) * D;
+                for (int d = 0; d < D; ++d) orow[d] = f2h(o[d] * inv);
+                if (lse) lse[(size_t)i * Hq + h] = bad ? std::numeric_limits<float>::infinity() : m * scale + logf(l);
+            }
+        }
+    }
+}
+
+// a7 -- src/model/tree_drafter.cuh:79-86
+void orc_gather_rows(const uint16_t* src, const int32_t* remap, int rows, int dim, uint16_t* dst) {
+#pragma omp parallel for num_threads(threads()) schedule(static)
+    for (int r = 0; r < rows; ++r)
+        std::memcpy(dst + (size_t)r * dim, src + (size_t)remap[r] * dim, (size_t)dim * 2);
+}
+
+// a6 / a11 -- src/model/linear.cuh:8-37,82-101; elementwise.cuh:34-41
+void orc_lm_head(const uint16_t* hid, const uint16_t* w, int n, int V, int H,
+                 int apply_scale, float head_scale, uint16_t* logits) {
+    std::vector<float> hf((size_t)n * H);
+    const float sc = h2f(f2h(head_scale));  // scale is applied as a half (elementwise.cuh:34-41)
+    for (size_t i = 0; i < (size_t)n * H; ++i) {
+        float x = h2f(hid[i]);
+        if (apply_scale) x = h2f(f2h(x * sc));  // linear.cuh:98 fp16 pre-scale
+        hf[i] = x;
+    }
+#pragma omp parallel num_threads(threads())
+    {
+        std::vector<float> wf(H);
+#pragma omp for schedule(static)
+        for (int vv = 0; vv < V; ++vv) {
+            const uint16_t* wr = w + (size_t)vv * H;
+            for (int kk = 0; kk < H; ++kk) wf[kk] = h2f(wr[kk]);
+            for (int r = 0; r < n; ++r)
+                logits[(size_t)r * V + vv] = f2h(dot_any(&hf[(size_t)r * H], wf.data(), H));
+        }
+    }
+}
+
+// a8 -- src/model/eagle.cuh:29-89
+void orc_log_softmax(uint16_t* x, int n, int dim, float* m_out, float* lse_out) {
+    for (int r = 0; r < n; ++r) {
+        uint16_t* row = x + (size_t)r * dim;
+        float m = -std::numeric_limits<float>::infinity();
+        for (int c = 0; c < dim; ++c) m = fmaxf(h2f(row[c]), m);
+        float s = 0.f;
+        for (int c = 0; c < dim; ++c) s += expf(h2f(row[c]) - m);
+        const float ls = logf(s);
+        for (int c = 0; c < dim; ++c) row[c] = f2h(h2f(row[c]) - m - ls);  // eagle.cuh:87
+        if (m_out) m_out[r] = m;
+        if (lse_out) lse_out[r] = ls;
+    }
+}
+
+void orc_log_softmax_apply(uint16_t* x, int n, int dim, const float* m, const float* lse) {
+    for (int r = 0; r < n; ++r) {
+        uint16_t* row = x + (size_t)r * dim;
+        for (int c = 0; c < dim; ++c) row[c] = f2h(h2f(row[c]) - m[r] - lse[r]);
+    }
+}
+
+// a9 -- src/model/topk.cuh:17 ordering: v1 > v2 || (v1 == v2 && pos1 < pos2)
+void orc_topk(const uint16_t* x, int n, int dim, int top, uint16_t* val, int32_t* pos) {
+#pragma omp parallel for num_threads(threads()) schedule(static)
+    for (int r = 0; r < n; ++r) {
+        const uint16_t* row = x + (size_t)r * dim;
+        std::vector<int32_t> idx(dim);
+        std::iota(idx.begin(), idx.end(), 0);
+        auto before = [row](int32_t a, int32_t b) {
+            float va = h2f(row[a]), vb = h2f(row[b]);
+            return va > vb || (va == vb && a < b);
+        };
+        std::partial_sort(idx.begin(), idx.begin() + top, idx.end(), before);
+        for (int j = 0; j < top; ++j) {
+            pos[(size_t)r * top + j] = idx[j];
+            val[(size_t)r * top + j] = row[idx[j]];
+        }
+    }
+}
+
+// a10 -- src/model/tree_drafter.cuh:88-90
+void orc_remap(const int32_t* in, int n, const int32_t* remap, int32_t* out) {
+    for (int i = 0; i < n; ++i) out[i] = remap[in[i]];
+}
+
+// a12 -- cpmcu/speculative/tree_drafter.py:153,233; lowest index on ties
+void orc_argmax(const uint16_t* logits, int n, int V, int32_t* gt) {
+#pragma omp parallel for num_threads(threads()) schedule(static)
+    for (int r = 0; r < n; ++r) {
+        const uint16_t* row = logits + (size_t)r * V;
+        float best = h2f(row[0]);
+        int32_t bi = 0;
+        for (int c = 1; c < V; ++c) {
+            float x = h2f(row[c]);
+            if (x > best) { best = x; bi = c; }
+        }
+        gt[r] = bi;
+    }
+}
+
+// a13 -- src/model/tree_drafter.cuh:5-46
+int orc_tree_accept(int T, int mask_words, const int32_t* pred, const int32_t* gt,
+                    const int32_t* pos, int P, const uint64_t* mask, const int32_t* parent,
+                    int32_t* best, int32_t* path) {
+    uint64_t correct[4] = {1ull, 0, 0, 0};  // :9 bit 0 always set
+    for (int i = 1; i < T; ++i)             // :10 pred[i] == gt[tree_parent[i]]
+        if (pred[i] == gt[parent[i]]) correct[i >> 6] |= 1ull << (i & 63);
+    int S = 64;
+    while (S < T) S <<= 1;
+    std::vector<int32_t> mx(S), mi(S);
+    for (int i = 0; i < S; ++i) {           // :22-28
+        bool full = i < T;
+        if (full) {
+            for (int w = 0; w < mask_words; ++w) {
+                uint64_t mw = mask[(size_t)i * mask_words + w];
+                if ((correct[w] & mw) != mw) { full = false; break; }
+            }
+        }
+        if (full) { mx[i] = pos[i] - P + 1; mi[i] = i; }
+        else      { mx[i] = 1;              mi[i] = 0; }
+    }
+    for (int off = S / 2; off > 0; off >>= 1)  // :30-36 strictly-greater tournament
+        for (int i = 0; i < off; ++i)
+            if (mx[i + off] > mx[i]) { mx[i] = mx[i + off]; mi[i] = mi[i + off]; }
+    best[0] = mx[0];
+    best[1] = mi[0];
+    const int p = mi[0];
+    for (int i = 0; i < T; ++i)                // :42-45
+        if ((mask[(size_t)p * mask_words + (i >> 6)] >> (i & 63)) & 1ull) path[pos[i] - P] = i;
+    return mx[0];
+}
+
+// a14 -- src/model/tree_drafter.cuh:48-77
+void orc_kv_compact(uint16_t* const* caches, int num_caches, int row_halves, int P, int a,
+                    const int32_t* path, const int32_t* gt, int32_t* ids_out) {
+    std::vector<uint16_t> tmp((size_t)a * row_halves);
+    for (int c = 0; c < num_caches; ++c) {
+        uint16_t* cache = caches[c];
+        for (int d = 0; d < a; ++d)  // kernel_1: stage
+            std::memcpy(&tmp[(size_t)d * row_halves], cache + (size_t)(P + path[d]) * row_halves, (size_t)row_halves * 2);
+        for (int d = 0; d < a; ++d)  // kernel_2: write back
+            std::memcpy(cache + (size_t)(P + d) * row_halves, &tmp[(size_t)d * row_halves], (size_t)row_halves * 2);
+    }
+    if (ids_out)
+        for (int d = 0; d < a; ++d) ids_out[d] = gt[path[d]];  // :74-76
+}
+
+}  // extern "C"

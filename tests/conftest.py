@@ -1,0 +1,31 @@
+import os
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+
+
+@pytest.fixture(scope="session")
+def orc():
+    """The CPU oracle (test infrastructure): built on demand with g++."""
+    import oracle
+    return oracle
+
+
+@pytest.fixture(scope="session")
+def gpu():
+    """torch + the HIP library on cuda:0; skips (never falls back) when there is no GPU."""
+    import torch
+    if not torch.cuda.is_available():
+        pytest.skip("no GPU in this environment")
+    from cpm.cu_amd import lib
+    lib.get()  # raises ImportError if libcpmcu_amd.so is missing: no fallback
+    torch.cuda.set_device(0)
+    return torch

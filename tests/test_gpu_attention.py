@@ -1,0 +1,131 @@
+"""GPU parity of the tree-verify attention and KV append kernels against the CPU oracle.
+
+Every call goes through the C-ABI (cpm.cu_amd.ops -> ctypes -> libcpmcu_amd.so).  Tolerance of the
+path for fp16 outputs: max-abs 2e-2 and max-rel 1e-2 (see tests/util.py).
+"""
+import numpy as np
+import pytest
+
+from cpm.cu_amd import synth
+from util import assert_close_f16, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+HQ, HKV, D = 32, 2, 128
+
+
+def _case(torch, orc, tree, P, seed, page_perm=True, splits=0, use_mask=True, extra_pages=2, q_std=1.0):
+    from cpm.cu_amd import ops
+    from cpm.cu_amd.kvcache import PagedKVCache
+    T = tree.T
+    S = P + T
+    q = synth.normal_f16((T, HQ, D), seed, 1, q_std)
+    k = synth.normal_f16((S, HKV, D), seed, 2)
+    v = synth.normal_f16((S, HKV, D), seed, 3)
+    npages = (S + 255) // 256 + extra_pages
+    table = synth.rng(seed, 4).permutation(npages).astype(np.int32) if page_perm else np.arange(npages, dtype=np.int32)
+    # stale garbage (incl. NaN bit patterns) in unused slots must not leak into the result
+    cache = PagedKVCache(1, HKV, npages, block_table=table, fill=float("nan"))
+    cache.write_logical(0, 0, to_dev(torch, k), to_dev(torch, v))
+    kv_len = torch.tensor([S], dtype=torch.int32, device="cuda")
+    mask = tree.mask if use_mask else None
+    out = ops.tree_attention(to_dev(torch, q), cache, 0, kv_len, S, None if mask is None else to_dev(torch, mask),
+                             num_splits=splits)
+    torch.cuda.synchronize()
+    ref_mask = tree.mask if use_mask else synth.chain_tree(T).mask
+    ref = orc.tree_attention(q, k, v, ref_mask, P)
+    return to_np(out), ref
+
+
+@pytest.mark.parametrize("splits", [1, 2, 5, 0])
+def test_c1_plumbing_case(gpu, orc, splits):
+    """Config 1: 16-node tree (depth 4, top-k 4), 1024-token prefix, 32 q / 2 kv heads."""
+    tree = synth.eagle_tree(4, 4, 16, seed=0)
+    out, ref = _case(gpu, orc, tree, 1024, seed=0, splits=splits)
+    assert_close_f16(out, ref, "attention c1 splits=%d" % splits)
+
+
+@pytest.mark.parametrize("P,T,seed", [(0, 16, 1), (1, 7, 2), (63, 33, 3), (64, 64, 4), (255, 60, 5), (257, 60, 6),
+                                      (700, 1, 7), (500, 128, 8), (2049, 100, 9)])
+def test_ragged_shapes(gpu, orc, P, T, seed):
+    """Prefix lengths around tile/page boundaries, empty prefix, one-node tree, two-word masks."""
+    tree = synth.random_tree(T, seed, max_children=5, max_depth=10)
+    for splits in (1, 3):
+        out, ref = _case(gpu, orc, tree, P, seed, splits=splits)
+        assert_close_f16(out, ref, "attention P=%d T=%d splits=%d" % (P, T, splits))
+
+
+def test_chain_without_mask(gpu, orc):
+    """mask == NULL means a causal chain (the reference's mask_2d = nullptr decode path)."""
+    tree = synth.chain_tree(24)
+    out, ref = _case(gpu, orc, tree, 300, seed=11, use_mask=False)
+    assert_close_f16(out, ref, "attention chain")
+
+
+def test_c2_shape_one_layer(gpu, orc):
+    """Config 2 shape (60-node EAGLE tree, 4096-token prefix), one layer, default split choice."""
+    tree = synth.eagle_tree(6, 10, 60, seed=0)
+    out, ref = _case(gpu, orc, tree, 4096, seed=12)
+    assert_close_f16(out, ref, "attention c2")
+
+
+def test_split_count_invariance(gpu, orc):
+    """The result may depend on the split count only through fp16 rounding of P."""
+    tree = synth.eagle_tree(6, 10, 60, seed=3)
+    outs = [_case(gpu, orc, tree, 1500, seed=13, splits=s)[0] for s in (1, 4, 24)]
+    for o in outs[1:]:
+        assert_close_f16(o, outs[0], "split invariance", atol=4e-3, rtol=4e-3)
+
+
+def test_non_ancestor_perturbation(gpu, orc):
+    """Row i must not change when K/V of a tree node outside its mask is perturbed."""
+    from cpm.cu_amd import ops
+    from cpm.cu_amd.kvcache import PagedKVCache
+    torch = gpu
+    tree = synth.eagle_tree(6, 10, 60, seed=5)
+    T, P = tree.T, 777
+    S = P + T
+    q = to_dev(torch, synth.normal_f16((T, HQ, D), 21, 1))
+    k = to_dev(torch, synth.normal_f16((S, HKV, D), 21, 2))
+    v = to_dev(torch, synth.normal_f16((S, HKV, D), 21, 3))
+    npages = (S + 255) // 256
+    kv_len = torch.tensor([S], dtype=torch.int32, device="cuda")
+    mask = to_dev(torch, tree.mask)
+    cache = PagedKVCache(1, HKV, npages)
+    cache.write_logical(0, 0, k, v)
+    base = ops.tree_attention(q, cache, 0, kv_len, S, mask).clone()
+    victim = 17
+    k2, v2 = k.clone(), v.clone()
+    k2[P + victim] += 3.0
+    v2[P + victim] -= 5.0
+    cache.write_logical(0, 0, k2, v2)
+    pert = ops.tree_attention(q, cache, 0, kv_len, S, mask)
+    torch.cuda.synchronize()
+    sees = np.array([(int(tree.mask[i, victim // 64]) >> (victim % 64)) & 1 for i in range(T)], bool)
+    base, pert = to_np(base), to_np(pert)
+    assert np.array_equal(base[~sees], pert[~sees]), "rows that do not see the node changed"
+    assert not np.array_equal(base[sees], pert[sees])
+
+
+def test_kv_append_matches_logical_write(gpu):
+    """copy_to_kvcache: the HIP append equals an index-based write, across a page boundary."""
+    from cpm.cu_amd import ops
+    from cpm.cu_amd.kvcache import PagedKVCache
+    torch = gpu
+    T, P = 60, 4096 - 23
+    npages = 20
+    table = synth.rng(31, 4).permutation(npages).astype(np.int32)
+    a = PagedKVCache(2, HKV, npages, block_table=table)
+    b = PagedKVCache(2, HKV, npages, block_table=table)
+    for layer in range(2):
+        k = to_dev(torch, synth.normal_f16((T, HKV, D), 31, 10 + layer))
+        v = to_dev(torch, synth.normal_f16((T, HKV, D), 31, 20 + layer))
+        kv_len = torch.tensor([P + T], dtype=torch.int32, device="cuda")
+        ops.kv_append(a, layer, k, v, kv_len)
+        b.write_logical(layer, P, k, v)
+    torch.cuda.synchronize()
+    for layer in range(2):
+        assert torch.equal(a.k[layer], b.k[layer])
+        assert torch.equal(a.v[layer], b.v[layer])
+        kk, vv = a.read_logical(layer, P, T)
+        assert kk.abs().sum() > 0 and vv.abs().sum() > 0
