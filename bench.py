@@ -1,0 +1,317 @@
+#!/usr/bin/env python3
+"""Benchmark of the speculative-decoding verify step on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2_verify_4k]
+
+One "step" = one pass of the verify hot path over one batch of synthetic MiniCPM4-8B-shaped input,
+with every input already resident in HBM: for each of the 32 layers append the 60 tree rows' K/V and
+run tree-masked attention over the paged cache (4096-token prefix + 60 tree rows), then the target
+lm_head (73448 x 4096) with fused arg-max, greedy tree acceptance and accepted-path KV compaction in
+all layers.  The step is captured once into a HIP graph (the reference replays a CUDA graph for
+decode as well) and replayed; exactly K replays are timed between synchronisations.
+
+Prints ONE JSON line.  `value` is microseconds per step (lower is better).  `roofline` is for the
+kernel that takes the largest share of the step; `kernels` lists all of them; `contexts` gives the
+step time at 4K / 32K / 128K context; `cpu_baseline` is the CPU oracle timed on this host on a
+bounded sample of the same workload (a reported baseline only).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
+
+
+def parse_args():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c2_verify_4k")
+    ap.add_argument("--splits", type=int, default=0, help="force the KV split count of tree attention (0 = auto)")
+    ap.add_argument("--no-contexts", action="store_true", help="skip the 32K / 128K context step timings")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    ap.add_argument("--accept-depth", type=int, default=3, help="draft tokens the rigged tree gets accepted")
+    return ap.parse_args()
+
+
+class Workload:
+    """Synthetic tensors of one configuration, resident on the GPU."""
+
+    def __init__(self, torch, name, accept_depth, seed=0):
+        import numpy as np
+        from cpm.cu_amd import synth
+        from cpm.cu_amd.kvcache import PagedKVCache
+        cfg = dict(synth.CONFIGS[name])
+        shp = synth.MINICPM4_8B
+        self.name, self.cfg, self.shape = name, cfg, shp
+        L, P, T = cfg["layers"], cfg["prefix"], cfg["T"]
+        Hq, Hkv, D, H, V = shp["q_heads"], shp["kv_heads"], shp["head_dim"], shp["hidden"], shp["vocab"]
+        self.L, self.P, self.T = L, P, T
+        dev = torch.device("cuda:0")
+        g = torch.Generator(device=dev)
+        g.manual_seed(seed)
+        S = P + T
+        npages = (S + 255) // 256 + 1
+        table = synth.rng(seed, 4).permutation(npages).astype(np.int32)  # seeded page-table permutation
+        self.cache = PagedKVCache(L, Hkv, npages, device=dev, block_table=table)
+        for l in range(L):  # ~N(0,1) prefix K/V, written page by page in the kernels' layout
+            self.cache.k[l].normal_(generator=g)
+            self.cache.v[l].normal_(generator=g)
+        rn = lambda *s, std=1.0: (torch.randn(*s, device=dev, dtype=torch.float32, generator=g) * std).to(torch.float16)
+        self.q = [rn(T, Hq, D) for _ in range(L)]
+        self.k_new = [rn(T, Hkv, D) for _ in range(L)]
+        self.v_new = [rn(T, Hkv, D) for _ in range(L)]
+        self.hidden = rn(T, H)
+        self.w = rn(V, H, std=0.02)
+        self.tree = synth.eagle_tree(cfg["num_iter"], cfg["topk"], T, seed)
+        tm = torch.from_numpy(self.tree.mask.view(np.int64)).to(dev)
+        self.mask = tm
+        self.parent = torch.from_numpy(self.tree.parent).to(dev)
+        self.pos = torch.from_numpy(self.tree.positions(P)).to(dev)
+        self.accept_depth = min(accept_depth, int(self.tree.depth.max()))
+        self.draft_ids = None  # rigged from the target arg-max once it is known
+        self.attn_out = [torch.empty(T, Hq, D, dtype=torch.float16, device=dev) for _ in range(L)]
+
+    def rig_draft(self, torch, gt_np):
+        from cpm.cu_amd import synth
+        pred, self.leaf = synth.draft_ids_for_accept(self.tree, gt_np, self.accept_depth, self.shape["vocab"], 1)
+        self.draft_np = pred
+        self.draft_ids = torch.from_numpy(pred).cuda()
+
+    def flops_attention_layer(self):
+        s = self.shape
+        return 4.0 * s["q_heads"] * self.T * s["head_dim"] * (self.P + self.T)
+
+    def bytes_attention_layer(self):
+        s = self.shape
+        return 2.0 * (self.P + self.T) * s["kv_heads"] * s["head_dim"] * 2 + 2.0 * self.T * s["q_heads"] * s["head_dim"] * 2
+
+    def bytes_target_head(self):
+        s = self.shape
+        return s["vocab"] * s["hidden"] * 2.0 + self.T * s["hidden"] * 2.0 + self.T * 4.0
+
+
+def timed_replays(torch, fn, steps, warmup, use_graph):
+    """Capture fn() once (unless disabled), run `warmup` untimed and exactly `steps` timed calls."""
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        fn()  # eager once: allocates workspaces outside capture
+        stream.synchronize()
+        run = fn
+        if use_graph:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                fn()
+            run = graph.replay
+        for _ in range(warmup):
+            run()
+        stream.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record(stream)
+        for _ in range(steps):
+            run()
+        e1.record(stream)
+        stream.synchronize()
+        torch.cuda.synchronize()
+        wall_ms = (time.perf_counter() - t0) * 1e3
+        ev_ms = e0.elapsed_time(e1)
+    return ev_ms / steps, wall_ms / steps
+
+
+def cpu_baseline(torch, wl, layers_sampled=2):
+    """CPU oracle on a bounded sample: `layers_sampled` attention layers + the full target head +
+    acceptance + compaction of those layers; the per-step figure scales the attention part to 32 layers."""
+    import numpy as np
+    import oracle
+    P, T = wl.P, wl.T
+    S = P + T
+    ks, vs, qs = [], [], []
+    for l in range(layers_sampled):
+        k, v = wl.cache.read_logical(l, 0, S)
+        ks.append(k.cpu().numpy())
+        vs.append(v.cpu().numpy())
+        qs.append(wl.q[l].cpu().numpy())
+    hid = wl.hidden.cpu().numpy()
+    w = wl.w.cpu().numpy()
+    t0 = time.perf_counter()
+    for l in range(layers_sampled):
+        oracle.tree_attention(qs[l], ks[l], vs[l], wl.tree.mask, P)
+    t_attn = (time.perf_counter() - t0) / layers_sampled
+    t0 = time.perf_counter()
+    gt = oracle.argmax(oracle.lm_head(hid, w))
+    t_head = time.perf_counter() - t0
+    t0 = time.perf_counter()
+    a, node, path = oracle.tree_accept(wl.draft_np, gt, wl.tree.positions(P), P, wl.tree.mask, wl.tree.parent)
+    flat = [x.reshape(S, -1).copy() for l in range(layers_sampled) for x in (ks[l], vs[l])]
+    ids = oracle.kv_compact(flat, P, path, gt)
+    t_tail = time.perf_counter() - t0
+    step_us = (t_attn * wl.L + t_head + t_tail) * 1e6
+    return dict(value=round(step_us, 1), unit="us/step", cores=oracle.num_threads(), kind="port",
+                sample="%d of %d attention layers timed (x%d extrapolated) + full target head/arg-max + acceptance + compaction; "
+                       "attention %.1f ms/layer, head %.1f ms" % (layers_sampled, wl.L, wl.L, t_attn * 1e3, t_head * 1e3)), (a, ids, gt)
+
+
+def main():
+    args = parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path is measured on one GPU; --gpus %d is not supported (nothing in it is sharded)" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+    import numpy as np
+    import torch
+    from cpm.cu_amd import lib, ops
+    from cpm.cu_amd.driver import VerifyStep
+    lib.get()  # fails loudly without the HIP library
+    torch.cuda.set_device(0)
+    use_graph = not args.no_graph
+
+    wl = Workload(torch, args.workload, args.accept_depth)
+    vs = VerifyStep(wl.cache, wl.w, wl.mask, wl.parent, wl.pos, wl.P)
+    # target arg-max once, to rig the draft ids for the chosen accept length
+    gt = ops.lm_head_argmax(wl.hidden, wl.w)
+    torch.cuda.synchronize()
+    wl.rig_draft(torch, gt.cpu().numpy())
+
+    def full_step():
+        vs.enqueue(wl.q, wl.k_new, wl.v_new, wl.hidden, wl.draft_ids, attn_out=wl.attn_out, splits=args.splits)
+
+    ms_step, wall_ms = timed_replays(torch, full_step, args.steps, args.warmup, use_graph)
+    a_gpu, ids_gpu = vs.result()
+
+    # ---- per-operator timings (same inputs, each operator alone, graph-replayed) ----
+    reps = max(5, args.steps // 5)
+
+    def attn_all_layers():
+        for l in range(wl.L):
+            ops.tree_attention(wl.q[l], wl.cache, l, vs.kv_len, vs.max_kv_len, wl.mask, num_splits=args.splits, out=wl.attn_out[l])
+
+    def append_all_layers():
+        for l in range(wl.L):
+            ops.kv_append(wl.cache, l, wl.k_new[l], wl.v_new[l], vs.kv_len)
+
+    def head_only():
+        ops.lm_head_argmax(wl.hidden, wl.w, gt=vs.gt)
+
+    def accept_compact():
+        vs.pred.copy_(wl.draft_ids)
+        ops.tree_accept(vs.pred, vs.gt, wl.pos, vs.cache_length, wl.mask, wl.parent, best=vs.best)
+        ops.kv_compact(wl.cache, vs.pred, vs.gt, vs.cache_length, vs.best, wl.T)
+
+    ms_attn = timed_replays(torch, attn_all_layers, reps, 2, use_graph)[0] / wl.L
+    ms_append = timed_replays(torch, append_all_layers, reps, 2, use_graph)[0] / wl.L
+    ms_head = timed_replays(torch, head_only, reps, 2, use_graph)[0]
+    ms_tail = timed_replays(torch, accept_compact, reps, 2, use_graph)[0]
+
+    attn_tflops = wl.flops_attention_layer() / (ms_attn * 1e-3) / 1e12
+    attn_gbs = wl.bytes_attention_layer() / (ms_attn * 1e-3) / 1e9
+    head_gbs = wl.bytes_target_head() / (ms_head * 1e-3) / 1e9
+    kernels = [
+        dict(kernel="tree_attn_split_kernel+tree_attn_combine_kernel", launches_per_step=wl.L, us_per_launch=round(ms_attn * 1e3, 2),
+             bound="mfma", achieved=round(attn_tflops, 2), peak=MFMA_F16_PEAK_TFLOPS, unit="TFLOP/s",
+             frac=round(attn_tflops / MFMA_F16_PEAK_TFLOPS, 4), hbm_gbs=round(attn_gbs, 1), traffic=None),
+        dict(kernel="head_gemm_kernel<4>+head_argmax_finalize_kernel", launches_per_step=1, us_per_launch=round(ms_head * 1e3, 2),
+             bound="hbm", achieved=round(head_gbs, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(head_gbs / HBM_PEAK_GBS, 4),
+             traffic=None),
+        dict(kernel="kv_append_kernel", launches_per_step=wl.L, us_per_launch=round(ms_append * 1e3, 2), bound="hbm",
+             achieved=None, peak=HBM_PEAK_GBS, unit="GB/s", frac=None, traffic=None),
+        dict(kernel="tree_accept_kernel+kv_compact_kernel+accepted_ids_kernel", launches_per_step=1,
+             us_per_launch=round(ms_tail * 1e3, 2), bound="hbm", achieved=None, peak=HBM_PEAK_GBS, unit="GB/s", frac=None, traffic=None),
+    ]
+    dominant = max(kernels, key=lambda k: k["us_per_launch"] * k["launches_per_step"])
+    roofline = {k: dominant[k] for k in ("bound", "achieved", "peak", "unit", "frac", "traffic")}
+    roofline["kernel"] = dominant["kernel"]
+    roofline["us_per_launch"] = dominant["us_per_launch"]
+
+    # ---- FR-Spec draft head (config 3 shape), reported beside the verify step ----
+    from cpm.cu_amd import synth
+    remap = torch.from_numpy(synth.frspec_remap(wl.shape["vocab"], wl.shape["frspec_vocab"], 0)).cuda()
+    w_sub = ops.gather_rows(wl.w, remap)
+    hid10 = wl.hidden[:10].contiguous()
+    ms_fr = timed_replays(torch, lambda: ops.frspec_head_topk(hid10, w_sub, remap, 10), reps, 2, use_graph)[0]
+    fr_bytes = wl.shape["frspec_vocab"] * wl.shape["hidden"] * 2.0 + 10 * wl.shape["hidden"] * 2.0 + 10 * 10 * 6.0
+    fr_gbs = fr_bytes / (ms_fr * 1e-3) / 1e9
+    frspec = dict(kernel="head_gemm_kernel<1>+topk_chunk_kernel+topk_merge_kernel", us_per_call=round(ms_fr * 1e3, 2), bound="hbm",
+                  achieved=round(fr_gbs, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(fr_gbs / HBM_PEAK_GBS, 4))
+    del w_sub
+
+    # ---- CPU oracle on the host cores + parity of the step's integer results ----
+    cpu = None
+    parity = None
+    if not args.no_cpu_baseline:
+        import oracle
+        cpu, (a_cpu, ids_cpu, gt_cpu) = cpu_baseline(torch, wl)
+        gt_gpu = vs.gt.cpu().numpy()
+        a_st, _, path_st = oracle.tree_accept(wl.draft_np, gt_gpu, wl.tree.positions(wl.P), wl.P, wl.tree.mask, wl.tree.parent)
+        parity = dict(accept_length_gpu=a_gpu, accept_length_oracle=int(a_cpu),
+                      ids_equal_oracle=bool(a_gpu == a_cpu and np.array_equal(ids_gpu, ids_cpu)),
+                      staged_equal=bool(a_gpu == a_st and np.array_equal(ids_gpu, gt_gpu[path_st])),
+                      argmax_rows_equal=int((gt_gpu == gt_cpu).sum()), rows=int(wl.T))
+
+    # ---- the same step at longer contexts ----
+    contexts = {str(wl.P): round(ms_step * 1e3, 1)}
+    ctx_attn = {str(wl.P): round(ms_attn * 1e3, 2)}
+    if not args.no_contexts and args.workload == "c2_verify_4k":
+        w_keep, hid_keep = wl.w, wl.hidden
+        del vs, wl
+        torch.cuda.empty_cache()
+        for name in ("c4_verify_32k", "c4_verify_128k"):
+            w2 = Workload.__new__(Workload)
+            Workload.__init__(w2, torch, name, args.accept_depth)
+            w2.w, w2.hidden = w_keep, hid_keep  # same head
+            v2 = VerifyStep(w2.cache, w2.w, w2.mask, w2.parent, w2.pos, w2.P)
+            w2.rig_draft(torch, gt.cpu().numpy())
+            n = max(3, args.steps // 5)
+            ms2 = timed_replays(torch, lambda: v2.enqueue(w2.q, w2.k_new, w2.v_new, w2.hidden, w2.draft_ids, attn_out=w2.attn_out,
+                                                          splits=args.splits), n, 2, use_graph)[0]
+
+            def attn2():
+                for l in range(w2.L):
+                    ops.tree_attention(w2.q[l], w2.cache, l, v2.kv_len, v2.max_kv_len, w2.mask, num_splits=args.splits, out=w2.attn_out[l])
+            ms_a2 = timed_replays(torch, attn2, n, 2, use_graph)[0] / w2.L
+            contexts[str(w2.P)] = round(ms2 * 1e3, 1)
+            ctx_attn[str(w2.P)] = dict(us_per_layer=round(ms_a2 * 1e3, 2),
+                                       tflops=round(w2.flops_attention_layer() / (ms_a2 * 1e-3) / 1e12, 1),
+                                       frac_mfma=round(w2.flops_attention_layer() / (ms_a2 * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4))
+            del v2, w2
+            torch.cuda.empty_cache()
+
+    out = {
+        "metric": "verify us/step @8B shape, 60-node tree, 4K ctx",
+        "value": round(ms_step * 1e3, 1),
+        "unit": "us/step",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_step, 5),
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": args.workload + ": 32 layers x (KV append + tree attention, 32q/2kv heads, d128, 4096-token paged prefix + "
+                               "60-node tree) + target head 73448x4096 with arg-max + tree acceptance + KV compaction",
+                   "batch": 1, "graph_replay": use_graph, "kv_splits": args.splits or "auto"},
+        "wall_ms_per_step": round(wall_ms, 5),
+        "roofline": roofline,
+        "kernels": kernels,
+        "frspec_head": frspec,
+        "contexts_us_per_step": contexts,
+        "attention_by_context": ctx_attn,
+        "cpu_baseline": cpu,
+        "parity": parity,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

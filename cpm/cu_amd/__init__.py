@@ -13,4 +13,6 @@ interface for that path:
 
 There is no CPU fallback: importing ``lib`` without the built shared library raises.
 """
+import torch  # noqa: F401,E402  -- first, so the shared library binds to the HIP runtime torch loads
+
 __all__ = ["lib", "ops", "kvcache", "synth", "driver"]
