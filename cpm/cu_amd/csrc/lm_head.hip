@@ -76,6 +76,11 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_kernel(HeadParams p) {
     const int gpp = H / GK;  // prefetch groups per pass
     const int total = p.npasses * gpp;
     const int total_chunks = p.npasses * nch;
+    // Every workgroup (and, when all of hidden is LDS-resident, every wave) walks K from a different
+    // starting chunk.  All rows of W are H*2 bytes apart, so waves that swept K in lockstep would
+    // keep hitting addresses with the same low bits -- the same few HBM channels -- at any instant.
+    const int rotc = resident ? 0 : c % nch;
+    const int rotg = resident ? (c * kHeadWaves + wave) % gpp : rotc * (kc / GK);
     const f16 sc = (f16)p.head_scale;
 
     // ---- hidden staging helpers ----
@@ -120,7 +125,7 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_kernel(HeadParams p) {
     auto row_block = [&](int pass) { return (pass * kHeadWaves + wave) * G + c; };
     auto load_group = [&](int it, f16x8* buf) {
         const int pass = it / gpp;
-        const int k0 = (it % gpp) * GK;
+        const int k0 = ((it % gpp + rotg) % gpp) * GK;
         int row = row_block(pass) * 16 + arow_lane;
         row = row < V ? row : V - 1;  // clamp: rows past the end are computed and discarded
         const f16* src = p.w + (size_t)row * H + k0 + kgp * 8;
@@ -193,24 +198,24 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_kernel(HeadParams p) {
         }
         __syncthreads();
     } else {
-        stage_load(0);
+        stage_load(rotc);
         stage_store(0);
     }
 
     auto compute_group = [&](int it, const f16x8* buf) {
         const int pass = it / gpp;
-        const int kg = it % gpp;
-        const int k0 = kg * GK;
-        const int chunk = k0 / kc;
+        const int kg = it % gpp;                     // position in this wave's K walk
+        const int k0 = ((kg + rotg) % gpp) * GK;     // actual K offset (rotated by whole chunks)
+        const int chunk = (kg * GK) / kc;            // sequential chunk number of the walk
         const int koff = k0 % kc;
         const int cglobal = pass * nch + chunk;
         int lbuf;
         if (resident) {
-            lbuf = chunk;
+            lbuf = k0 / kc;
         } else {
             if (koff == 0) {
                 __syncthreads();  // chunk `cglobal` visible; everyone is done with the other buffer
-                if (cglobal + 1 < total_chunks) stage_load((cglobal + 1) % nch);
+                if (cglobal + 1 < total_chunks) stage_load(((cglobal + 1) % nch + rotc) % nch);
             }
             lbuf = cglobal & 1;
         }

@@ -20,6 +20,15 @@
 //  * V pages are stored transposed and 16-token interleaved (see
 //    include/cpmcu_amd.h) so the A operand of O^T = V^T.P^T is one 16-byte LDS
 //    read per lane.
+//  * K/V tiles (64 keys, 32 KB) go HBM/L2 -> LDS with direct-to-LDS loads
+//    (global_load_lds_dwordx4) into a 4-stage ring, XOR-swizzled through the
+//    choice of the global address each lane fetches, so no registers are spent
+//    on staging and two tiles are always in flight behind the two being
+//    consumed.
+//  * A workgroup is 8 waves = 2 KV groups x 4 row waves over the same 128
+//    packed rows: the groups take alternate tiles of the ring (two independent
+//    instruction streams per SIMD) and are merged through LDS at the end -- half
+//    the partial traffic of splitting the same work over two workgroups.
 //  * Workgroups are mapped so that all M-tiles that stream the same KV range
 //    land on the same XCD (workgroup id modulo 8) and share its L2.
 #include "common.h"
@@ -27,14 +36,22 @@
 namespace cpmcu {
 namespace {
 
-constexpr int kTileN = 64;                     // keys per LDS tile
-constexpr int kWaves = 4;                      // waves per workgroup
-constexpr int kRowsPerWave = 32;               // packed query rows per wave (one MFMA N block)
-constexpr int kRowsPerWg = kWaves * kRowsPerWave;
+constexpr int kTileN = 64;                  // keys per LDS tile
+constexpr int kRowWaves = 4;                // row waves per KV group
+constexpr int kGroups = 2;                  // KV groups per workgroup
+constexpr int kWaves = kRowWaves * kGroups;
+constexpr int kRowsPerWave = 32;            // packed query rows per wave (one MFMA N block)
+constexpr int kRowsPerWg = kRowWaves * kRowsPerWave;
 constexpr int kThreads = kWaves * 64;
-constexpr int kKRowBytes = kHeadDim * 2 + 16;  // padded K row in LDS: conflict-free b128 reads
-constexpr int kVRowBytes = kTileN * 2 + 16;    // padded V^T row in LDS
+constexpr int kStages = 4;
+constexpr int kKTileBytes = kTileN * kHeadDim * 2;  // 16 KB, row = one key (256 B)
+constexpr int kVTileBytes = kHeadDim * kTileN * 2;  // 16 KB, row = one dim (128 B)
+constexpr int kStageBytes = kKTileBytes + kVTileBytes;
+constexpr int kMaxPagesPerSplit = 1024;
+constexpr int kMaxSplits = 64;
 constexpr int kXcds = 8;
+
+typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
 struct AttnParams {
     const f16* q;
@@ -46,10 +63,16 @@ struct AttnParams {
     int mask_words;
     int T, Hq, Hkv, group;
     int num_splits, num_mtiles, rows_pad;
+    int ntiles_max;  // ceil(max_kv_len / 64): the split partition is fixed by the host-side bound
     float scale_log2;
     f16* out;
-    float* o_part;   // [Hkv][num_splits][rows_pad][128]
-    float* ml_part;  // [Hkv][num_splits][rows_pad][2]  (max * scale_log2, sum)
+    // Split partials in the accumulator's own layout, so that both the split kernel's stores and the
+    // combine kernel's loads are whole 1 KB wave transactions:
+    //   o_part  [Hkv][num_splits][num_mtiles][row wave][16 quads][64 lanes] x float4
+    //           quad q = db * 4 + rq of lane (qcol, hf) holds O[row = rw*32 + qcol][d = db*32 + rq*8 + hf*4 + 0..3]
+    //   ml_part [Hkv][num_splits][rows_pad] x float2 (max * scale_log2, sum)
+    float* o_part;
+    float* ml_part;
 };
 
 __device__ inline f16x8 zero8() {
@@ -59,71 +82,55 @@ __device__ inline f16x8 zero8() {
     return z;
 }
 
-struct TileRegs {
-    f16x8 k[4];
-    f16x8 v[4];
-};
+// Swizzled LDS byte offsets inside one stage.  K: row = key (16 pieces of 16 B), piece index is
+// XORed with key % 16.  V^T: row = dim (8 pieces), XORed with (dim / 2) % 8 -- even and odd rows
+// already sit in different bank halves.  Both make the 16-byte MFMA operand reads conflict-free.
+__device__ inline int k_lds_off(int key, int piece) { return key * 256 + ((piece ^ (key & 15)) << 4); }
+__device__ inline int v_lds_off(int d, int piece) { return kKTileBytes + d * 128 + ((piece ^ ((d >> 1) & 7)) << 4); }
 
-// Global -> registers for one 64-key tile.  Keys at or beyond S are zero-filled
-// (stale or never-written page memory must not reach the MFMAs: 0 * NaN = NaN).
-__device__ inline void load_tile(const AttnParams& p, int g, int tile, int S, int tid, TileRegs& r) {
-    const int c0 = tile * kTileN;
-    const int page = p.block_table[c0 / kPage];
-    const int slot0 = c0 % kPage;
+// One direct-to-LDS load: every lane fetches 16 bytes from its own global address and the wave's
+// 1 KB lands at `lds_dst` (wave-uniform) in lane order.  Written as inline assembly on purpose: the
+// completion of these loads is tracked by hand (s_waitcnt vmcnt before the workgroup barrier that
+// publishes a stage), which lets the next tiles stay in flight while the current ones are consumed;
+// with the compiler builtin every LDS read would first wait for all of them.
+__device__ inline void load_to_lds16(const void* gptr, const char* lds_dst) {
+    const uint32_t lds_addr = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)lds_dst);
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gptr), "s"(lds_addr) : "memory", "m0");
+}
+
+// Issues this thread's four 16-byte direct-to-LDS loads of one tile (2 for K, 2 for V^T).  Each
+// wave-level instruction fills 1 KB of LDS in lane order; the swizzle is applied on the global side.
+__device__ inline void issue_tile(const AttnParams& p, int g, int tile, int page, char* stage, int wave, int lane) {
+    const int slot0 = (tile * kTileN) % kPage;
     const f16* kbase = p.k_pool + (((size_t)page * p.Hkv + g) * kPage + slot0) * kHeadDim;
     const f16* vbase = p.v_pool + ((size_t)page * p.Hkv + g) * kHeadDim * kPage + slot0;
-    const bool partial = c0 + kTileN > S;
 #pragma unroll
-    for (int ps = 0; ps < 4; ++ps) {
-        const int key = ps * 16 + (tid >> 4);
-        const int chunk = tid & 15;
-        if (!partial || c0 + key < S)
-            r.k[ps] = *reinterpret_cast<const f16x8*>(kbase + (size_t)key * kHeadDim + chunk * 8);
-        else
-            r.k[ps] = zero8();
-    }
-#pragma unroll
-    for (int ps = 0; ps < 4; ++ps) {
-        const int d = ps * 32 + (tid >> 3);
-        const int chunk = tid & 7;
-        f16x8 v = *reinterpret_cast<const f16x8*>(vbase + (size_t)d * kPage + chunk * 8);
-        if (partial) {
-#pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const int key = v_slot16(chunk * 8 + e);  // storage slot -> token within the tile
-                if (c0 + key >= S) v[e] = (f16)0.f;
-            }
+    for (int qq = 0; qq < 2; ++qq) {
+        const int inst = wave + kWaves * qq;  // 16 KB / 1 KB = 16 instructions per operand, 2 per wave
+        {
+            const int key = inst * 4 + (lane >> 4);
+            const int piece = (lane & 15) ^ (key & 15);
+            load_to_lds16(kbase + (size_t)key * kHeadDim + piece * 8, stage + inst * 1024);
         }
-        r.v[ps] = v;
+        {
+            const int d = inst * 8 + (lane >> 3);
+            const int piece = (lane & 7) ^ ((d >> 1) & 7);
+            load_to_lds16(vbase + (size_t)d * kPage + piece * 8, stage + kKTileBytes + inst * 1024);
+        }
     }
 }
 
-__device__ inline void store_tile(char* lds_k, char* lds_v, int tid, const TileRegs& r) {
-#pragma unroll
-    for (int ps = 0; ps < 4; ++ps) {
-        const int key = ps * 16 + (tid >> 4);
-        const int chunk = tid & 15;
-        *reinterpret_cast<f16x8*>(lds_k + key * kKRowBytes + chunk * 16) = r.k[ps];
-    }
-#pragma unroll
-    for (int ps = 0; ps < 4; ++ps) {
-        const int d = ps * 32 + (tid >> 3);
-        const int chunk = tid & 7;
-        *reinterpret_cast<f16x8*>(lds_v + d * kVRowBytes + chunk * 16) = r.v[ps];
-    }
-}
-
-__global__ __launch_bounds__(kThreads) void tree_attn_split_kernel(AttnParams p) {
-    __shared__ __attribute__((aligned(16))) char lds_k[kTileN * kKRowBytes];
-    __shared__ __attribute__((aligned(16))) char lds_v[kHeadDim * kVRowBytes];
+__global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams p) {
+    __shared__ __attribute__((aligned(1024))) char ring[kStages * kStageBytes];
+    __shared__ int32_t s_pages[kMaxPagesPerSplit];
 
     // XCD-aware work mapping: consecutive workgroup ids go to consecutive XCDs, so
     // id % 8 picks the XCD; all M-tiles of one (split, kv head) pair share an XCD.
     const int wg = blockIdx.x;
     const int xcd = wg % kXcds;
-    const int j = wg / kXcds;
-    const int sh = xcd + kXcds * (j / p.num_mtiles);
-    const int mt = j % p.num_mtiles;
+    const int jj = wg / kXcds;
+    const int sh = xcd + kXcds * (jj / p.num_mtiles);
+    const int mt = jj % p.num_mtiles;
     if (sh >= p.num_splits * p.Hkv) return;
     const int g = sh % p.Hkv;
     const int split = sh / p.Hkv;
@@ -131,21 +138,17 @@ __global__ __launch_bounds__(kThreads) void tree_attn_split_kernel(AttnParams p)
     const int tid = threadIdx.x;
     const int wave = tid >> 6;
     const int lane = tid & 63;
+    const int grp = wave / kRowWaves;  // KV group: takes tiles grp, grp + 2, ...
+    const int rw = wave % kRowWaves;
     const int qcol = lane & 31;
     const int hf = lane >> 5;
 
-    const int S = p.kv_len[0];
-    const int P = S - p.T;
-    const int ntiles = (S + kTileN - 1) / kTileN;
-    const int tps = (ntiles + p.num_splits - 1) / p.num_splits;
-    const int t0 = split * tps;
-    const int t1 = min(ntiles, t0 + tps);
-
-    const int R = mt * kRowsPerWg + wave * kRowsPerWave + qcol;  // packed row
+    const int R = mt * kRowsPerWg + rw * kRowsPerWave + qcol;  // packed row
     const bool row_ok = R < p.group * p.T;
     const int node = row_ok ? R / p.group : 0;
     const int head = g * p.group + (row_ok ? R % p.group : 0);
 
+    // Loads that do not depend on the KV length go first.
     // Q as the B operand of S^T = K.Q^T: lane (qcol, hf) holds d = 16*ks + 8*hf + [0,8).
     f16x8 qreg[8];
     {
@@ -171,6 +174,34 @@ __global__ __launch_bounds__(kThreads) void tree_attn_split_kernel(AttnParams p)
         mw1 &= c1;
     }
 
+    // The split's tile range is fixed by the host-side bound, so the page ids can be fetched without
+    // waiting for the device-side length; the length only clips the range.
+    const int t0 = (int)(((long long)split * p.ntiles_max) / p.num_splits);
+    const int t1_max = (int)(((long long)(split + 1) * p.ntiles_max) / p.num_splits);
+    const int pg0 = (t0 * kTileN) / kPage;
+    if (t1_max > t0) {
+        const int npg = ((t1_max * kTileN - 1) / kPage) - pg0 + 1;
+        for (int i = tid; i < npg; i += kThreads) s_pages[i] = p.block_table[pg0 + i];
+    }
+    const int S = p.kv_len[0];
+    const int P = S - p.T;
+    const int ntiles = (S + kTileN - 1) / kTileN;
+    const int t1 = min(t1_max, ntiles);
+    const int n = max(t1 - t0, 0);
+    const int npairs = (n + 1) / 2;
+    __syncthreads();
+
+    auto issue_pair = [&](int pair) {
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+            const int i = pair * 2 + e;
+            if (i < n) {
+                const int tile = t0 + i;
+                issue_tile(p, g, tile, s_pages[(tile * kTileN) / kPage - pg0], ring + (i % kStages) * kStageBytes, wave, lane);
+            }
+        }
+    };
+
     f32x16 oacc[4];
 #pragma unroll
     for (int db = 0; db < 4; ++db)
@@ -179,88 +210,179 @@ __global__ __launch_bounds__(kThreads) void tree_attn_split_kernel(AttnParams p)
     float m_run = -INFINITY;  // running row max (raw score units)
     float l_run = 0.f;        // this lane's share of the row sum
 
-    TileRegs regs;
-    if (t0 < t1) load_tile(p, g, t0, S, tid, regs);
+    if (npairs > 0) issue_pair(0);
+    if (npairs > 1) issue_pair(1);
 
-    for (int t = t0; t < t1; ++t) {
-        __syncthreads();  // previous tile fully consumed
-        store_tile(lds_k, lds_v, tid, regs);
-        __syncthreads();
-        if (t + 1 < t1) load_tile(p, g, t + 1, S, tid, regs);  // prefetch under the MFMAs
-
-        // ---- S^T = K.Q^T : two 32-key blocks ----
-        f32x16 sacc[2];
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) sacc[kb][r] = 0.f;
-            const char* krow = lds_k + (kb * 32 + qcol) * kKRowBytes + hf * 16;
-#pragma unroll
-            for (int ks = 0; ks < 8; ++ks) {
-                const f16x8 a = *reinterpret_cast<const f16x8*>(krow + ks * 32);
-                sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, qreg[ks], sacc[kb], 0, 0, 0);
-            }
+    for (int pair = 0; pair < npairs; ++pair) {
+        // Wait for this pair's tiles.  Pair p+1 is issued right after the barrier of iteration p, so
+        // nothing newer is outstanding here -- except in iteration 0, where pair 1 (4 loads per
+        // thread and tile, issued in the prologue) may stay in flight.
+        if (pair == 0 && npairs > 1) {
+            if (n >= 4) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+        } else {
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
-        // sacc[kb][r] is the score of key  c0 + kb*32 + 8*(r/4) + 4*hf + r%4  for query qcol.
+        __syncthreads();  // every thread's pieces have landed; the previous pair's stages are free
+        if (pair >= 1 && pair + 1 < npairs) issue_pair(pair + 1);
+
+        const int i = pair * 2 + grp;  // this group's tile of the pair
+        const int t = t0 + i;
         const int c0 = t * kTileN;
-        if (c0 + kTileN > P) {  // tile touches tree columns or the end of the stream
+        char* stage = ring + (i % kStages) * kStageBytes;
+        // The tile that holds position S-1 may extend past it: stale page contents there must not
+        // reach the MFMA (0 * NaN = NaN), so the V^T columns of tokens >= S are zeroed in LDS.  K
+        // needs nothing: the scores of those keys are replaced (not scaled) by -inf below.
+        const bool pair_has_tail = (t0 + pair * 2) * kTileN + 2 * kTileN > S;  // uniform over the workgroup
+        if (pair_has_tail) {
+            for (int e = 0; e < 2; ++e) {
+                const int ie = pair * 2 + e;
+                const int ce = (t0 + ie) * kTileN;
+                if (ie < n && ce + kTileN > S) {
+                    char* st = ring + (ie % kStages) * kStageBytes;
+                    for (int x = tid; x < kHeadDim * kTileN; x += kThreads) {
+                        const int d = x >> 6, slot = x & 63;
+                        if (ce + v_slot16(slot) >= S)
+                            *reinterpret_cast<f16*>(st + v_lds_off(d, slot >> 3) + (slot & 7) * 2) = (f16)0.f;
+                    }
+                }
+            }
+            __syncthreads();
+        }
+        if (i < n) {
+            // ---- S^T = K.Q^T : two 32-key blocks.  All 16 operand reads are issued before the first
+            // MFMA: LDS returns in order, so MFMA i only waits for read i. ----
+            f32x16 sacc[2];
+            {
+                f16x8 kf[16];
+#pragma unroll
+                for (int ks = 0; ks < 8; ++ks)
+#pragma unroll
+                    for (int kb = 0; kb < 2; ++kb)
+                        kf[ks * 2 + kb] = *reinterpret_cast<const f16x8*>(stage + k_lds_off(kb * 32 + qcol, 2 * ks + hf));
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) sacc[kb][r] = 0.f;
+#pragma unroll
+                for (int ks = 0; ks < 8; ++ks)
+#pragma unroll
+                    for (int kb = 0; kb < 2; ++kb)  // two independent accumulation chains, interleaved
+                        sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[ks * 2 + kb], qreg[ks], sacc[kb], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            // sacc[kb][r] is the score of key  c0 + kb*32 + 8*(r/4) + 4*hf + r%4  for query qcol.
+            if (c0 + kTileN > P) {  // tile touches tree columns or the end of the stream
+                // 64-bit visibility word of this tile for the lane's query: bit x <-> key c0 + x.  Prefix
+                // keys are visible; tree key P + j is visible iff bit j of the node's mask row is set
+                // (the causal bound already cleared every bit above the node, hence at or beyond T).
+                const int sh = P - c0;  // < 64 here; negative once the tile starts inside the tree
+                uint64_t tmask;
+                if (sh >= 0) {
+                    tmask = (mw0 << sh) | (sh > 0 ? ((1ull << sh) - 1ull) : 0ull);
+                } else {
+                    const int tt = -sh;
+                    tmask = tt < 64 ? ((mw0 >> tt) | (mw1 << (64 - tt))) : (tt < 128 ? (mw1 >> (tt - 64)) : 0ull);
+                }
+                const uint64_t tm = tmask >> (4 * hf);
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        const bool vis = (tm >> (kb * 32 + 8 * (r >> 2) + (r & 3))) & 1ull;
+                        sacc[kb][r] = vis ? sacc[kb][r] : -INFINITY;
+                    }
+            }
+            // ---- online softmax (one query column per lane) ----
+            float tmax = sacc[0][0];
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, sacc[kb][r]);
+            tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
+            const float m_new = fmaxf(m_run, tmax);
+            const float m_scaled = (m_new == -INFINITY) ? 0.f : m_new * p.scale_log2;
+            const float alpha = __builtin_amdgcn_exp2f(m_run * p.scale_log2 - m_scaled);
+            m_run = m_new;
+            float psum = 0.f;
+            f16x8 pb[4];  // P^T as B operand: k-step j holds keys 16*j + {4hf..4hf+3, 8+4hf..8+4hf+3}
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
-                    const int c = c0 + kb * 32 + 8 * (r >> 2) + 4 * hf + (r & 3);
-                    const int jn = c - P;
-                    bool vis = true;
-                    if (jn >= 0) {
-                        const uint64_t w = jn < 64 ? mw0 : mw1;
-                        vis = jn < p.T && ((w >> (jn & 63)) & 1ull);
-                    }
-                    if (!vis) sacc[kb][r] = -INFINITY;
+                    const float pv = __builtin_amdgcn_exp2f(sacc[kb][r] * p.scale_log2 - m_scaled);
+                    psum += pv;                              // row sum keeps the fp32 value
+                    pb[kb * 2 + (r >> 3)][r & 7] = (f16)pv;  // P is rounded to fp16 before P.V
                 }
-        }
-        // ---- online softmax (one query column per lane) ----
-        float tmax = sacc[0][0];
+            l_run = l_run * alpha + psum;
+            if (__any(alpha != 1.f)) {  // skipped when no lane's running max moved
 #pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
+                for (int db = 0; db < 4; ++db)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, sacc[kb][r]);
-        tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
-        const float m_new = fmaxf(m_run, tmax);
-        const float m_scaled = (m_new == -INFINITY) ? 0.f : m_new * p.scale_log2;
-        const float alpha = __builtin_amdgcn_exp2f(m_run * p.scale_log2 - m_scaled);
-        m_run = m_new;
-        float psum = 0.f;
-        f16x8 pb[4];  // P^T as B operand: k-step jj holds keys 16*jj + {4hf..4hf+3, 8+4hf..8+4hf+3}
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const float pv = __builtin_amdgcn_exp2f(sacc[kb][r] * p.scale_log2 - m_scaled);
-                psum += pv;                                // row sum keeps the fp32 value
-                pb[kb * 2 + (r >> 3)][r & 7] = (f16)pv;    // P is rounded to fp16 before P.V
+                    for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
             }
-        l_run = l_run * alpha + psum;
-#pragma unroll
-        for (int db = 0; db < 4; ++db)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
 
-        // ---- O^T += V^T.P^T ----
+            // ---- O^T += V^T.P^T ----
+            {
+                f16x8 vf[16];
 #pragma unroll
-        for (int db = 0; db < 4; ++db) {
-            const char* vrow = lds_v + (db * 32 + qcol) * kVRowBytes + hf * 16;
+                for (int j = 0; j < 4; ++j)
 #pragma unroll
-            for (int jj = 0; jj < 4; ++jj) {
-                const f16x8 a = *reinterpret_cast<const f16x8*>(vrow + jj * 32);
-                oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, pb[jj], oacc[db], 0, 0, 0);
+                    for (int db = 0; db < 4; ++db)
+                        vf[j * 4 + db] = *reinterpret_cast<const f16x8*>(stage + v_lds_off(db * 32 + qcol, 2 * j + hf));
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int db = 0; db < 4; ++db)  // four independent accumulation chains, interleaved
+                        oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[j * 4 + db], pb[j], oacc[db], 0, 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
     }
 
+    // ---- merge the two KV groups through LDS (lane-private layout: [row wave][value][lane]) ----
+    __syncthreads();  // ring no longer read
+    f32x4* xch = reinterpret_cast<f32x4*>(ring);           // [row wave][17 quads][64 lanes]
+    const int xbase = rw * 17 * 64 + lane;
+    if (grp == 1) {
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+#pragma unroll
+            for (int rq = 0; rq < 4; ++rq) {
+                f32x4 o;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = oacc[db][rq * 4 + e];
+                xch[xbase + (db * 4 + rq) * 64] = o;
+            }
+        xch[xbase + 16 * 64] = f32x4{m_run, l_run, 0.f, 0.f};
+    }
+    __syncthreads();
+    if (grp == 1) return;
+    {
+        const f32x4 ml1 = xch[xbase + 16 * 64];
+        const float m1 = ml1[0], l1 = ml1[1];
+        const float m_new = fmaxf(m_run, m1);
+        const float m_scaled = (m_new == -INFINITY) ? 0.f : m_new * p.scale_log2;
+        const float a0 = __builtin_amdgcn_exp2f(m_run * p.scale_log2 - m_scaled);
+        const float a1 = __builtin_amdgcn_exp2f(m1 * p.scale_log2 - m_scaled);
+#pragma unroll
+        for (int db = 0; db < 4; ++db)
+#pragma unroll
+            for (int rq = 0; rq < 4; ++rq) {
+                const f32x4 o = xch[xbase + (db * 4 + rq) * 64];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) oacc[db][rq * 4 + e] = oacc[db][rq * 4 + e] * a0 + o[e] * a1;
+            }
+        l_run = l_run * a0 + l1 * a1;
+        m_run = m_new;
+    }
+
     // oacc[db][r] is O[query qcol][d = db*32 + 8*(r/4) + 4*hf + r%4], unnormalised.
     const float l_tot = l_run + __shfl_xor(l_run, 32);
-    if (!row_ok) return;
     if (p.num_splits == 1) {
+        if (!row_ok) return;
         const float inv = (l_tot == 0.f || l_tot != l_tot) ? 1.f : 1.f / l_tot;
         f16* orow = p.out + ((size_t)node * p.Hq + head) * kHeadDim;
 #pragma unroll
@@ -274,7 +396,8 @@ __global__ __launch_bounds__(kThreads) void tree_attn_split_kernel(AttnParams p)
             }
     } else {
         const size_t prow = ((size_t)g * p.num_splits + split) * p.rows_pad + R;
-        float* op = p.o_part + prow * kHeadDim;
+        f32x4* op = reinterpret_cast<f32x4*>(p.o_part) +
+                    ((((size_t)g * p.num_splits + split) * p.num_mtiles + mt) * kRowWaves + rw) * 16 * 64 + lane;
 #pragma unroll
         for (int db = 0; db < 4; ++db)
 #pragma unroll
@@ -282,9 +405,9 @@ __global__ __launch_bounds__(kThreads) void tree_attn_split_kernel(AttnParams p)
                 f32x4 o;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) o[e] = oacc[db][rq * 4 + e];
-                *reinterpret_cast<f32x4*>(op + db * 32 + rq * 8 + hf * 4) = o;
+                __builtin_nontemporal_store(o, &op[(db * 4 + rq) * 64]);  // streamed: nothing left to flush at kernel end
             }
-        if (hf == 0) {
+        if (hf == 0 && row_ok) {
             p.ml_part[prow * 2 + 0] = (m_run == -INFINITY) ? -INFINITY : m_run * p.scale_log2;
             p.ml_part[prow * 2 + 1] = l_tot;
         }
@@ -294,57 +417,76 @@ __global__ __launch_bounds__(kThreads) void tree_attn_split_kernel(AttnParams p)
 // Merge of the split partials: M = max_s m_s, L = sum_s l_s 2^(m_s - M),
 // O = sum_s 2^(m_s - M) O_s / L  -- the log-sum-exp merge of
 // src/flash_attn/src/flash_fwd_kernel.h:2392-2472 in base-2 form.
-// One thread per (packed row, 8 output dims).
+// One thread per (packed row, 4 output dims).  The statistics and the O partials of up to 16 splits
+// are all requested before any is used, so the kernel pays one memory round trip, not one per split.
+constexpr int kCombineBatch = 16;
 __global__ __launch_bounds__(256) void tree_attn_combine_kernel(AttnParams p) {
-    const int rows = p.group * p.T;
+    // thread -> (kv head, M-tile, row wave, quad, lane) in the partial layout's own order
     const int idx = blockIdx.x * 256 + threadIdx.x;
-    const int row_all = idx >> 4;  // over Hkv * rows
-    const int dchunk = idx & 15;
-    if (row_all >= p.Hkv * rows) return;
-    const int g = row_all / rows;
-    const int R = row_all % rows;
+    const int lane = idx & 63;
+    const int quad = (idx >> 6) & 15;
+    const int rw = (idx >> 10) & (kRowWaves - 1);
+    const int gm = idx >> 12;  // g * num_mtiles + mt   (kRowWaves * 16 * 64 = 4096 threads per M-tile)
+    if (gm >= p.Hkv * p.num_mtiles) return;
+    const int g = gm / p.num_mtiles, mt = gm % p.num_mtiles;
+    const int qcol = lane & 31, hf = lane >> 5;
+    const int R = mt * kRowsPerWg + rw * kRowsPerWave + qcol;
+    if (R >= p.group * p.T) return;
     const int node = R / p.group;
     const int head = g * p.group + R % p.group;
+    const int d0 = (quad >> 2) * 32 + (quad & 3) * 8 + hf * 4;
+    const float2* ml = reinterpret_cast<const float2*>(p.ml_part) + (size_t)g * p.num_splits * p.rows_pad + R;
+    const f32x4* op = reinterpret_cast<const f32x4*>(p.o_part) +
+                      ((((size_t)g * p.num_splits) * p.num_mtiles + mt) * kRowWaves + rw) * 16 * 64 + quad * 64 + lane;
+    const size_t ml_stride = (size_t)p.rows_pad;
+    const size_t o_stride = (size_t)p.num_mtiles * kRowWaves * 16 * 64;
 
-    float M = -INFINITY;
-    for (int s = 0; s < p.num_splits; ++s) {
-        const size_t prow = ((size_t)g * p.num_splits + s) * p.rows_pad + R;
-        const float l = p.ml_part[prow * 2 + 1];
-        if (l > 0.f) M = fmaxf(M, p.ml_part[prow * 2 + 0]);
-    }
-    float acc[8];
+    float M = -INFINITY, L = 0.f;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < p.num_splits; s0 += kCombineBatch) {
+        float2 v[kCombineBatch];
+        f32x4 o[kCombineBatch];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
-    float L = 0.f;
-    for (int s = 0; s < p.num_splits; ++s) {
-        const size_t prow = ((size_t)g * p.num_splits + s) * p.rows_pad + R;
-        const float l = p.ml_part[prow * 2 + 1];
-        if (!(l > 0.f)) continue;  // empty split: its O partial was never meaningful
-        const float w = __builtin_amdgcn_exp2f(p.ml_part[prow * 2 + 0] - M);
-        L += w * l;
-        const f32x4* op = reinterpret_cast<const f32x4*>(p.o_part + prow * kHeadDim + dchunk * 8);
-        const f32x4 a = op[0], b = op[1];
+        for (int u = 0; u < kCombineBatch; ++u) {
+            const int s = min(s0 + u, p.num_splits - 1);  // clamp: repeats are ignored below
+            v[u] = ml[s * ml_stride];
+            o[u] = op[s * o_stride];
+        }
+        float Mb = M;
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            acc[e] += w * a[e];
-            acc[4 + e] += w * b[e];
+        for (int u = 0; u < kCombineBatch; ++u)
+            if (s0 + u < p.num_splits && v[u].y > 0.f) Mb = fmaxf(Mb, v[u].x);
+        if (Mb == -INFINITY) continue;  // nothing but empty splits so far
+        const float resc = __builtin_amdgcn_exp2f(M - Mb);  // 0 when M was -inf
+        L *= resc;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] *= resc;
+        M = Mb;
+#pragma unroll
+        for (int u = 0; u < kCombineBatch; ++u) {
+            // an empty split (l == 0) has no meaningful O partial: select it away, never scale it
+            if (!(s0 + u < p.num_splits && v[u].y > 0.f)) continue;
+            const float w = __builtin_amdgcn_exp2f(v[u].x - M);
+            L += w * v[u].y;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[e] += w * o[u][e];
         }
     }
     const float inv = (L == 0.f || L != L) ? 1.f : 1.f / L;
-    f16x8 o;
+    f16x4 o;
 #pragma unroll
-    for (int e = 0; e < 8; ++e) o[e] = (f16)(acc[e] * inv);
-    *reinterpret_cast<f16x8*>(p.out + ((size_t)node * p.Hq + head) * kHeadDim + dchunk * 8) = o;
+    for (int e = 0; e < 4; ++e) o[e] = (f16)(acc[e] * inv);
+    *reinterpret_cast<f16x4*>(p.out + ((size_t)node * p.Hq + head) * kHeadDim + d0) = o;
 }
 
 int choose_splits(int T, int group, int Hkv, int max_kv_len) {
     const int num_mtiles = ceil_div(group * T, kRowsPerWg);
     const int ntiles = ceil_div(max_kv_len, kTileN);
-    // Aim for ~one workgroup per CU (256 CUs); every split needs at least one tile.
+    // One workgroup per CU (256 CUs); every split should get at least one tile per KV group.
     int splits = 256 / (num_mtiles * Hkv);
     if (splits < 1) splits = 1;
-    if (splits > ntiles) splits = ntiles;
-    if (splits > 64) splits = 64;
+    if (splits > ntiles / 2) splits = ntiles / 2 > 0 ? ntiles / 2 : 1;
+    if (splits > kMaxSplits) splits = kMaxSplits;
     return splits;
 }
 
@@ -354,13 +496,13 @@ int choose_splits(int T, int group, int Hkv, int max_kv_len) {
 using namespace cpmcu;
 
 extern "C" size_t cpmcu_tree_attention_workspace_bytes(int T, int Hq, int Hkv, int max_kv_len) {
+    (void)max_kv_len;
     if (T <= 0 || Hkv <= 0 || Hq <= 0 || Hq % Hkv) return 0;
     const int group = Hq / Hkv;
     const int num_mtiles = ceil_div(group * T, kRowsPerWg);
     const int rows_pad = num_mtiles * kRowsPerWg;
     // sized for the largest split count the library ever picks, so an override fits too
-    const size_t splits = 64;
-    return align_up((size_t)Hkv * splits * rows_pad * (kHeadDim + 2) * sizeof(float), 256);
+    return align_up((size_t)Hkv * kMaxSplits * rows_pad * (kHeadDim + 2) * sizeof(float), 256);
 }
 
 extern "C" int cpmcu_tree_attention(const void* q, const void* k_pool, const void* v_pool,
@@ -374,7 +516,8 @@ extern "C" int cpmcu_tree_attention(const void* q, const void* k_pool, const voi
     CPMCU_CHECK_ARG(max_kv_len >= T, "tree_attention: max_kv_len=%d < T=%d", max_kv_len, T);
     CPMCU_CHECK_ARG(mask == nullptr || mask_words == ceil_div(T, 64) || (mask_words == 1 && T <= 64),
                     "tree_attention: mask_words=%d does not match T=%d", mask_words, T);
-    CPMCU_CHECK_ARG(num_splits_override >= 0 && num_splits_override <= 64, "tree_attention: num_splits_override=%d outside [0, 64]", num_splits_override);
+    CPMCU_CHECK_ARG(num_splits_override >= 0 && num_splits_override <= kMaxSplits,
+                    "tree_attention: num_splits_override=%d outside [0, %d]", num_splits_override, kMaxSplits);
     const int group = Hq / Hkv;
     AttnParams p;
     p.q = (const f16*)q;
@@ -391,6 +534,11 @@ extern "C" int cpmcu_tree_attention(const void* q, const void* k_pool, const voi
     p.num_mtiles = ceil_div(group * T, kRowsPerWg);
     p.rows_pad = p.num_mtiles * kRowsPerWg;
     p.num_splits = num_splits_override > 0 ? num_splits_override : choose_splits(T, group, Hkv, max_kv_len);
+    // a split keeps the physical page ids of its range in LDS
+    const int min_splits = ceil_div(ceil_div(max_kv_len, kPage) + 2, kMaxPagesPerSplit - 2);
+    if (p.num_splits < min_splits) p.num_splits = min_splits;
+    CPMCU_CHECK_ARG(p.num_splits <= kMaxSplits, "tree_attention: max_kv_len=%d is beyond the supported context", max_kv_len);
+    p.ntiles_max = ceil_div(max_kv_len, kTileN);
     p.scale_log2 = scale * 1.4426950408889634f;
     p.out = (f16*)out;
     p.o_part = nullptr;
@@ -409,7 +557,7 @@ extern "C" int cpmcu_tree_attention(const void* q, const void* k_pool, const voi
     hipLaunchKernelGGL(tree_attn_split_kernel, dim3(grid), dim3(kThreads), 0, st, p);
     CPMCU_LAUNCH_CHECK();
     if (p.num_splits > 1) {
-        const int threads_total = Hkv * group * T * 16;
+        const int threads_total = Hkv * p.num_mtiles * kRowWaves * 16 * 64;
         hipLaunchKernelGGL(tree_attn_combine_kernel, dim3(ceil_div(threads_total, 256)), dim3(256), 0, st, p);
         CPMCU_LAUNCH_CHECK();
     }
