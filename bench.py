@@ -5,7 +5,7 @@
 
 One "step" = one pass of the verify hot path over one batch of synthetic MiniCPM4-8B-shaped input,
 with every input already resident in HBM: for each of the 32 layers append the 60 tree rows' K/V and
-run tree-masked attention over the paged cache (4096-token prefix + 60 tree rows), then the target
+run tree-masked attention (one fused kernel + the split merge) over the paged cache (4096-token prefix + 60 tree rows), then the target
 lm_head (73448 x 4096) with fused arg-max, greedy tree acceptance and accepted-path KV compaction in
 all layers.  The step is captured once into a HIP graph (the reference replays a CUDA graph for
 decode as well) and replayed; exactly K replays are timed between synchronisations.
@@ -191,26 +191,25 @@ def main():
     # ---- per-operator timings (same inputs, each operator alone, graph-replayed) ----
     reps = max(5, args.steps // 5)
 
-    def attn_all_layers():
+    def attn_all_layers():  # with the KV append of the tree rows fused in, as in the step
         for l in range(wl.L):
-            ops.tree_attention(wl.q[l], wl.cache, l, vs.kv_len, vs.max_kv_len, wl.mask, num_splits=args.splits, out=wl.attn_out[l])
-
-    def append_all_layers():
-        for l in range(wl.L):
-            ops.kv_append(wl.cache, l, wl.k_new[l], wl.v_new[l], vs.kv_len)
+            ops.tree_attention(wl.q[l], wl.cache, l, vs.kv_len, vs.max_kv_len, wl.mask, num_splits=args.splits, out=wl.attn_out[l],
+                               k_new=wl.k_new[l], v_new=wl.v_new[l])
 
     def head_only():
         ops.lm_head_argmax(wl.hidden, wl.w, gt=vs.gt)
 
+    TAIL_REP = 8  # several repetitions per graph, so that the graph launch itself does not dominate
+
     def accept_compact():
-        vs.pred.copy_(wl.draft_ids)
-        ops.tree_accept(vs.pred, vs.gt, wl.pos, vs.cache_length, wl.mask, wl.parent, best=vs.best)
-        ops.kv_compact(wl.cache, vs.pred, vs.gt, vs.cache_length, vs.best, wl.T)
+        for _ in range(TAIL_REP):
+            vs.pred.copy_(wl.draft_ids)
+            ops.tree_accept(vs.pred, vs.gt, wl.pos, vs.cache_length, wl.mask, wl.parent, best=vs.best)
+            ops.kv_compact(wl.cache, vs.pred, vs.gt, vs.cache_length, vs.best, wl.T)
 
     ms_attn = timed_replays(torch, attn_all_layers, reps, 2, use_graph)[0] / wl.L
-    ms_append = timed_replays(torch, append_all_layers, reps, 2, use_graph)[0] / wl.L
     ms_head = timed_replays(torch, head_only, reps, 2, use_graph)[0]
-    ms_tail = timed_replays(torch, accept_compact, reps, 2, use_graph)[0]
+    ms_tail = timed_replays(torch, accept_compact, reps, 2, use_graph)[0] / TAIL_REP
 
     attn_tflops = wl.flops_attention_layer() / (ms_attn * 1e-3) / 1e12
     attn_gbs = wl.bytes_attention_layer() / (ms_attn * 1e-3) / 1e9
@@ -222,8 +221,6 @@ def main():
         dict(kernel="head_gemm_kernel<4>+head_argmax_finalize_kernel", launches_per_step=1, us_per_launch=round(ms_head * 1e3, 2),
              bound="hbm", achieved=round(head_gbs, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(head_gbs / HBM_PEAK_GBS, 4),
              traffic=None),
-        dict(kernel="kv_append_kernel", launches_per_step=wl.L, us_per_launch=round(ms_append * 1e3, 2), bound="hbm",
-             achieved=None, peak=HBM_PEAK_GBS, unit="GB/s", frac=None, traffic=None),
         dict(kernel="tree_accept_kernel+kv_compact_kernel+accepted_ids_kernel", launches_per_step=1,
              us_per_launch=round(ms_tail * 1e3, 2), bound="hbm", achieved=None, peak=HBM_PEAK_GBS, unit="GB/s", frac=None, traffic=None),
     ]
@@ -276,7 +273,8 @@ def main():
 
             def attn2():
                 for l in range(w2.L):
-                    ops.tree_attention(w2.q[l], w2.cache, l, v2.kv_len, v2.max_kv_len, w2.mask, num_splits=args.splits, out=w2.attn_out[l])
+                    ops.tree_attention(w2.q[l], w2.cache, l, v2.kv_len, v2.max_kv_len, w2.mask, num_splits=args.splits, out=w2.attn_out[l],
+                                       k_new=w2.k_new[l], v_new=w2.v_new[l])
             ms_a2 = timed_replays(torch, attn2, n, 2, use_graph)[0] / w2.L
             contexts[str(w2.P)] = round(ms2 * 1e3, 1)
             ctx_attn[str(w2.P)] = dict(us_per_layer=round(ms_a2 * 1e3, 2),

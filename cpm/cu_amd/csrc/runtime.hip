@@ -357,13 +357,12 @@ extern "C" int cpmcu_decode_attention(int layer, int input_length, int padded_le
     CPMCU_CHECK_ARG(q && k_new && v_new && cache_length && out, "decode_attention: null pointer argument");
     hipStream_t st = resolve_stream(nullptr);
     PerfScope perf("DECODE_ATTN_CORE", st);
-    rc = cpmcu_kv_append(m.k_pools[layer], m.v_pools[layer], m.block_table, (const void*)k_new, (const void*)v_new,
-                         (const int32_t*)cache_length, input_length, m.kv_heads, st);
-    if (rc) return rc;
+    // KV append (src/model/attn.cuh:200) is fused into the attention kernel
     const uint64_t* mask = mask_2d ? (const uint64_t*)mask_2d : m.chain_mask;
     return cpmcu_tree_attention((const void*)q, m.k_pools[layer], m.v_pools[layer], m.block_table,
-                                (const int32_t*)cache_length, padded_length, mask, 1, input_length, m.q_heads,
-                                m.kv_heads, 1.f / sqrtf((float)kHeadDim), (void*)out, m.attn_ws, m.attn_ws_bytes, 0, st);
+                                (const int32_t*)cache_length, padded_length, (const void*)k_new, (const void*)v_new, mask, 1,
+                                input_length, m.q_heads, m.kv_heads, 1.f / sqrtf((float)kHeadDim), (void*)out, m.attn_ws,
+                                m.attn_ws_bytes, 0, st);
 }
 
 extern "C" int cpmcu_decode_lm_head(int input_length, uint64_t hidden, uint64_t logits, uint64_t gt) {

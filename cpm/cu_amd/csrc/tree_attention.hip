@@ -59,6 +59,10 @@ struct AttnParams {
     const f16* v_pool;
     const int32_t* block_table;
     const int32_t* kv_len;
+    const f16* k_new;  // [T][Hkv][128] rows of the tree nodes to append, or null: already in the cache
+    const f16* v_new;
+    f16* k_pool_w;     // writable aliases of the pools (used only when k_new is set)
+    f16* v_pool_w;
     const uint64_t* mask;
     int mask_words;
     int T, Hq, Hkv, group;
@@ -230,16 +234,61 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
         const int t = t0 + i;
         const int c0 = t * kTileN;
         char* stage = ring + (i % kStages) * kStageBytes;
-        // The tile that holds position S-1 may extend past it: stale page contents there must not
-        // reach the MFMA (0 * NaN = NaN), so the V^T columns of tokens >= S are zeroed in LDS.  K
-        // needs nothing: the scores of those keys are replaced (not scaled) by -inf below.
-        const bool pair_has_tail = (t0 + pair * 2) * kTileN + 2 * kTileN > S;  // uniform over the workgroup
-        if (pair_has_tail) {
+        // Fix-ups of landed tiles, in LDS (uniform over the workgroup: only the pairs that reach the
+        // tree region or the end of the stream pay for them):
+        //  * fused KV append (copy_to_kvcache, src/model/attn.cuh:14-21,200): when the T new rows are
+        //    handed in, they replace whatever the cache held at positions [P, S) -- every workgroup
+        //    patches its own LDS copy, and the M-tile-0 workgroup of the split also writes the rows
+        //    into the paged pools;
+        //  * the tile that holds position S-1 may extend past it: stale page contents there must not
+        //    reach the MFMA (0 * NaN = NaN), so the V^T columns of tokens >= S are zeroed.  K needs
+        //    nothing: the scores of those keys are replaced (not scaled) by -inf below.
+        const int pair_end = (t0 + pair * 2) * kTileN + 2 * kTileN;
+        const bool pair_needs_fix = pair_end > S || (p.k_new != nullptr && pair_end > P);
+        if (pair_needs_fix) {
             for (int e = 0; e < 2; ++e) {
                 const int ie = pair * 2 + e;
                 const int ce = (t0 + ie) * kTileN;
-                if (ie < n && ce + kTileN > S) {
-                    char* st = ring + (ie % kStages) * kStageBytes;
+                if (ie >= n) continue;
+                char* st = ring + (ie % kStages) * kStageBytes;
+                const bool append = p.k_new != nullptr && ce + kTileN > P;
+                if (append) {
+                    // K rows: 16 pieces of 16 bytes per key
+                    for (int x = tid; x < kTileN * 16; x += kThreads) {
+                        const int key = x >> 4, piece = x & 15;
+                        const int c = ce + key;
+                        if (c >= P && c < S) {
+                            const f16x8 val = *reinterpret_cast<const f16x8*>(p.k_new + ((size_t)(c - P) * p.Hkv + g) * kHeadDim + piece * 8);
+                            *reinterpret_cast<f16x8*>(st + k_lds_off(key, piece)) = val;
+                            if (mt == 0) {
+                                const int pg = s_pages[c / kPage - pg0];
+                                *reinterpret_cast<f16x8*>(p.k_pool_w + (((size_t)pg * p.Hkv + g) * kPage + c % kPage) * kHeadDim + piece * 8) = val;
+                            }
+                        }
+                    }
+                }
+                if (append) {
+                    // V rows: one 16-byte piece (8 dims) of one new row per thread, scattered into the
+                    // transposed tile (and pool) as 2-byte elements
+                    for (int x = tid; x < kTileN * 16; x += kThreads) {
+                        const int key = x >> 4, piece = x & 15;
+                        const int c = ce + key;
+                        if (c >= P && c < S) {
+                            const f16x8 val = *reinterpret_cast<const f16x8*>(p.v_new + ((size_t)(c - P) * p.Hkv + g) * kHeadDim + piece * 8);
+                            const int slot = v_slot16(key);  // storage slot of this token inside the tile
+#pragma unroll
+                            for (int e = 0; e < 8; ++e)
+                                *reinterpret_cast<f16*>(st + v_lds_off(piece * 8 + e, slot >> 3) + (slot & 7) * 2) = val[e];
+                            if (mt == 0) {
+                                const int pg = s_pages[c / kPage - pg0];
+                                f16* dst = p.v_pool_w + (((size_t)pg * p.Hkv + g) * kHeadDim + piece * 8) * kPage + v_slot16(c % kPage);
+#pragma unroll
+                                for (int e = 0; e < 8; ++e) dst[(size_t)e * kPage] = val[e];
+                            }
+                        }
+                    }
+                }
+                if (ce + kTileN > S) {
                     for (int x = tid; x < kHeadDim * kTileN; x += kThreads) {
                         const int d = x >> 6, slot = x & 63;
                         if (ce + v_slot16(slot) >= S)
@@ -505,8 +554,9 @@ extern "C" size_t cpmcu_tree_attention_workspace_bytes(int T, int Hq, int Hkv, i
     return align_up((size_t)Hkv * kMaxSplits * rows_pad * (kHeadDim + 2) * sizeof(float), 256);
 }
 
-extern "C" int cpmcu_tree_attention(const void* q, const void* k_pool, const void* v_pool,
+extern "C" int cpmcu_tree_attention(const void* q, void* k_pool, void* v_pool,
                                     const int32_t* block_table, const int32_t* kv_len, int max_kv_len,
+                                    const void* k_new, const void* v_new,
                                     const uint64_t* mask, int mask_words, int T, int Hq, int Hkv,
                                     float scale, void* out, void* workspace, size_t workspace_bytes,
                                     int num_splits_override, void* stream) {
@@ -525,6 +575,11 @@ extern "C" int cpmcu_tree_attention(const void* q, const void* k_pool, const voi
     p.v_pool = (const f16*)v_pool;
     p.block_table = block_table;
     p.kv_len = kv_len;
+    CPMCU_CHECK_ARG((k_new == nullptr) == (v_new == nullptr), "tree_attention: k_new and v_new must be given together");
+    p.k_new = (const f16*)k_new;
+    p.v_new = (const f16*)v_new;
+    p.k_pool_w = (f16*)k_pool;
+    p.v_pool_w = (f16*)v_pool;
     p.mask = mask;
     p.mask_words = mask ? mask_words : 0;
     p.T = T;

@@ -3,8 +3,8 @@
 One verify step, as the reference drives it (cpmcu/speculative/tree_drafter.py:222-250 around
 cpmcu/llm.py:263-283), restricted to the operators that are on the path:
 
-    for every layer:  append the T tree rows' K/V at cache rows [P, P+T)   (src/model/attn.cuh:200)
-                      tree attention of the T queries over P + T keys      (src/model/attn.cuh:204-229)
+    for every layer:  append the T tree rows' K/V at cache rows [P, P+T)   (src/model/attn.cuh:200)   } one fused
+                      tree attention of the T queries over P + T keys      (src/model/attn.cuh:204-229) } kernel
     target head on the T hidden rows + arg-max  -> gt                      (src/model/model.cuh:164, tree_drafter.py:233)
     greedy acceptance -> (a, path)                                         (src/model/tree_drafter.cuh:5-46)
     compaction of the accepted rows in every layer, pred[:a] <- ids        (src/model/tree_drafter.cuh:48-77)
@@ -42,9 +42,10 @@ class VerifyStep:
         hidden [T,H]; draft_ids int32[T].  Results: self.best (a, node), self.pred[:a] accepted ids."""
         c = self.cache
         for l in range(c.num_layers):
-            ops.kv_append(c, l, k_new_layers[l], v_new_layers[l], self.kv_len)
             out = None if attn_out is None else attn_out[l]
-            o = ops.tree_attention(q_layers[l], c, l, self.kv_len, self.max_kv_len, self.mask, num_splits=splits, out=out)
+            # the KV append of the T tree rows is fused into the attention kernel
+            o = ops.tree_attention(q_layers[l], c, l, self.kv_len, self.max_kv_len, self.mask, num_splits=splits, out=out,
+                                   k_new=k_new_layers[l], v_new=v_new_layers[l])
             if attn_out is None:
                 self.attn_out = o
         ops.lm_head_argmax(hidden, self.w, head_scale=self.head_scale, gt=self.gt)

@@ -52,10 +52,13 @@ def kv_append(cache, layer, k_new, v_new, kv_len):
                      _ptr(kv_len), T, cache.Hkv, _stream())
 
 
-def tree_attention(q, cache, layer, kv_len, max_kv_len, mask=None, scale=None, num_splits=0, out=None):
+def tree_attention(q, cache, layer, kv_len, max_kv_len, mask=None, scale=None, num_splits=0, out=None,
+                   k_new=None, v_new=None):
     """mha_fwd_kvcache with a tree mask (src/flash_attn/flash_api.hpp:292-392) on the paged cache.
 
     q [T, Hq, 128] fp16; kv_len int32[1] on the device = P + T; mask uint64 [T, W] or None (chain).
+    k_new / v_new [T, Hkv, 128]: the tree rows' K/V; when given the kernel appends them to the cache
+    itself (src/model/attn.cuh:200) instead of expecting them there.
     """
     T, Hq, D = q.shape
     assert D == HEAD_DIM and q.dtype == torch.float16 and kv_len.dtype == torch.int32
@@ -70,8 +73,12 @@ def tree_attention(q, cache, layer, kv_len, max_kv_len, mask=None, scale=None, n
         scale = 1.0 / math.sqrt(D)
     need = _lib().raw.cpmcu_tree_attention_workspace_bytes(T, Hq, cache.Hkv, int(max_kv_len))
     ws = _workspace("attn", need, q.device)
+    if k_new is not None:
+        assert k_new.dtype == torch.float16 and v_new.dtype == torch.float16
+        assert k_new.numel() == T * cache.Hkv * HEAD_DIM and v_new.numel() == k_new.numel()
     _lib().tree_attention(_ptr(q), _ptr(cache.k[layer]), _ptr(cache.v[layer]), _ptr(cache.block_table), _ptr(kv_len),
-                          int(max_kv_len), _ptr(mask), W, T, Hq, cache.Hkv, ctypes.c_float(scale), _ptr(out),
+                          int(max_kv_len), _ptr(k_new), _ptr(v_new), _ptr(mask), W, T, Hq, cache.Hkv,
+                          ctypes.c_float(scale), _ptr(out),
                           _ptr(ws), ws.numel(), int(num_splits), _stream())
     return out
 

@@ -178,18 +178,25 @@ size_t cpmcu_tree_attention_workspace_bytes(int T, int Hq, int Hkv, int max_kv_l
  *   kv_len: device int32[1] = P + T (the true length is read on the device, as
  *           the reference reads cu_seqlens_k, flash_api.hpp:383-385); the tree
  *           nodes are the last T tokens, in node order.
- *   max_kv_len: host upper bound of *kv_len used for the launch geometry (the
- *           reference's padded_length).
+ *   max_kv_len: host upper bound of *kv_len used for the launch geometry and the
+ *           split partition (the reference's padded_length); keep it tight (within
+ *           a few hundred tokens of *kv_len).  block_table must have an entry for
+ *           every page below ceil(max_kv_len / 256).
+ *   k_new, v_new: [T][Hkv][128] fp16 rows of the T tree nodes, or both NULL.  When
+ *           given, the kernel performs the KV append of src/model/attn.cuh:14-21,200
+ *           itself: the rows are used for positions [*kv_len - T, *kv_len) and are
+ *           written into the pools, so no separate cpmcu_kv_append call is needed.
+ *           When NULL the rows must already be in the cache.
  *   mask [T][mask_words] uint64: bit j of row i = node i attends tree node j;
  *           NULL = causal chain.
  *   scale: softmax scale (1/sqrt(128) in the reference, flash_api.hpp:360).
  *   workspace: device scratch of at least ..._workspace_bytes(), may be NULL
  *           when that is 0.
  *   num_splits_override: 0 = choose from max_kv_len; >0 forces the KV split count. */
-int cpmcu_tree_attention(const void* q, const void* k_pool, const void* v_pool, const int32_t* block_table,
-                         const int32_t* kv_len, int max_kv_len, const uint64_t* mask, int mask_words,
-                         int T, int Hq, int Hkv, float scale, void* out, void* workspace,
-                         size_t workspace_bytes, int num_splits_override, void* stream);
+int cpmcu_tree_attention(const void* q, void* k_pool, void* v_pool, const int32_t* block_table,
+                         const int32_t* kv_len, int max_kv_len, const void* k_new, const void* v_new,
+                         const uint64_t* mask, int mask_words, int T, int Hq, int Hkv, float scale, void* out,
+                         void* workspace, size_t workspace_bytes, int num_splits_override, void* stream);
 
 /* remap_copy -- src/model/tree_drafter.cuh:79-86,103-107: dst[r][:] = src[remap[r]][:]. */
 int cpmcu_gather_rows(const void* src, const int32_t* remap, int rows, int dim, void* dst, void* stream);

@@ -129,3 +129,40 @@ def test_kv_append_matches_logical_write(gpu):
         assert torch.equal(a.v[layer], b.v[layer])
         kk, vv = a.read_logical(layer, P, T)
         assert kk.abs().sum() > 0 and vv.abs().sum() > 0
+
+
+@pytest.mark.parametrize("P,T,splits", [(1024, 16, 0), (4096 - 23, 60, 0), (250, 60, 1), (0, 16, 1), (700, 128, 3), (63, 64, 2)])
+def test_fused_append_equals_append_then_attend(gpu, orc, P, T, splits):
+    """Handing the tree rows' K/V to the attention kernel (fused copy_to_kvcache) must give the same
+    output as appending first, and must leave the same cache behind -- stale garbage at [P, S) included."""
+    from cpm.cu_amd import ops
+    from cpm.cu_amd.kvcache import PagedKVCache
+    torch = gpu
+    tree = synth.random_tree(T, P + T, max_children=5, max_depth=10)
+    S = P + T
+    seed = 41 + P
+    q = synth.normal_f16((T, HQ, D), seed, 1)
+    k = synth.normal_f16((S, HKV, D), seed, 2)
+    v = synth.normal_f16((S, HKV, D), seed, 3)
+    npages = (S + 255) // 256 + 1
+    table = synth.rng(seed, 4).permutation(npages).astype(np.int32)
+    kv_len = torch.tensor([S], dtype=torch.int32, device="cuda")
+    mask = to_dev(torch, tree.mask)
+    # reference path: append kernel, then attention
+    a = PagedKVCache(1, HKV, npages, block_table=table, fill=float("nan"))
+    if P:
+        a.write_logical(0, 0, to_dev(torch, k[:P]), to_dev(torch, v[:P]))
+    ops.kv_append(a, 0, to_dev(torch, k[P:]), to_dev(torch, v[P:]), kv_len)
+    out_a = ops.tree_attention(to_dev(torch, q), a, 0, kv_len, S, mask, num_splits=splits)
+    # fused path on a cache whose tree region holds NaN garbage
+    b = PagedKVCache(1, HKV, npages, block_table=table, fill=float("nan"))
+    if P:
+        b.write_logical(0, 0, to_dev(torch, k[:P]), to_dev(torch, v[:P]))
+    out_b = ops.tree_attention(to_dev(torch, q), b, 0, kv_len, S, mask, num_splits=splits,
+                               k_new=to_dev(torch, k[P:]), v_new=to_dev(torch, v[P:]))
+    torch.cuda.synchronize()
+    assert torch.equal(out_a, out_b)
+    assert_close_f16(to_np(out_b), orc.tree_attention(q, k, v, tree.mask, P), "fused append attention")
+    kb, vb = b.read_logical(0, 0, S)
+    assert np.array_equal(to_np(kb).view(np.uint16), k.view(np.uint16))
+    assert np.array_equal(to_np(vb).view(np.uint16), v.view(np.uint16))
