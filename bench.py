@@ -39,6 +39,9 @@ def parse_args():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--accept-depth", type=int, default=3, help="draft tokens the rigged tree gets accepted")
+    ap.add_argument("--traffic-probe", action="store_true",
+                    help="also run a plain 256 MiB device copy three times: the known-size kernel that scales "
+                         "rocprofv3's FETCH_SIZE / WRITE_SIZE counters")
     return ap.parse_args()
 
 
@@ -174,6 +177,14 @@ def main():
     lib.get()  # fails loudly without the HIP library
     torch.cuda.set_device(0)
     use_graph = not args.no_graph
+
+    if args.traffic_probe:
+        src = torch.full((256 << 20,), 7, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     wl = Workload(torch, args.workload, args.accept_depth)
     vs = VerifyStep(wl.cache, wl.w, wl.mask, wl.parent, wl.pos, wl.P)

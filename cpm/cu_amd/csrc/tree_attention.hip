@@ -72,7 +72,7 @@ struct AttnParams {
     f16* out;
     // Split partials in the accumulator's own layout, so that both the split kernel's stores and the
     // combine kernel's loads are whole 1 KB wave transactions:
-    //   o_part  [Hkv][num_splits][num_mtiles][row wave][16 quads][64 lanes] x float4
+    //   o_part  [Hkv][num_splits][num_mtiles][row wave][16 quads][64 lanes] x 4 halves (normalised O)
     //           quad q = db * 4 + rq of lane (qcol, hf) holds O[row = rw*32 + qcol][d = db*32 + rq*8 + hf*4 + 0..3]
     //   ml_part [Hkv][num_splits][rows_pad] x float2 (max * scale_log2, sum)
     float* o_part;
@@ -445,15 +445,19 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
             }
     } else {
         const size_t prow = ((size_t)g * p.num_splits + split) * p.rows_pad + R;
-        f32x4* op = reinterpret_cast<f32x4*>(p.o_part) +
+        // Partials leave the kernel normalised (O / l) and rounded to fp16 -- the precision of the
+        // final output -- which halves the dominant extra HBM traffic of the split design; (max, l)
+        // stay fp32.  The reference keeps fp32 partials; the difference is far inside the tolerance.
+        const float inv = (l_tot == 0.f || l_tot != l_tot) ? 0.f : 1.f / l_tot;
+        f16x4* op = reinterpret_cast<f16x4*>(p.o_part) +
                     ((((size_t)g * p.num_splits + split) * p.num_mtiles + mt) * kRowWaves + rw) * 16 * 64 + lane;
 #pragma unroll
         for (int db = 0; db < 4; ++db)
 #pragma unroll
             for (int rq = 0; rq < 4; ++rq) {
-                f32x4 o;
+                f16x4 o;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) o[e] = oacc[db][rq * 4 + e];
+                for (int e = 0; e < 4; ++e) o[e] = (f16)(oacc[db][rq * 4 + e] * inv);
                 __builtin_nontemporal_store(o, &op[(db * 4 + rq) * 64]);  // streamed: nothing left to flush at kernel end
             }
         if (hf == 0 && row_ok) {
@@ -464,7 +468,7 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
 }
 
 // Merge of the split partials: M = max_s m_s, L = sum_s l_s 2^(m_s - M),
-// O = sum_s 2^(m_s - M) O_s / L  -- the log-sum-exp merge of
+// O = sum_s l_s 2^(m_s - M) (O_s / l_s) / L  -- the log-sum-exp merge of
 // src/flash_attn/src/flash_fwd_kernel.h:2392-2472 in base-2 form.
 // One thread per (packed row, 4 output dims).  The statistics and the O partials of up to 16 splits
 // are all requested before any is used, so the kernel pays one memory round trip, not one per split.
@@ -485,7 +489,7 @@ __global__ __launch_bounds__(256) void tree_attn_combine_kernel(AttnParams p) {
     const int head = g * p.group + R % p.group;
     const int d0 = (quad >> 2) * 32 + (quad & 3) * 8 + hf * 4;
     const float2* ml = reinterpret_cast<const float2*>(p.ml_part) + (size_t)g * p.num_splits * p.rows_pad + R;
-    const f32x4* op = reinterpret_cast<const f32x4*>(p.o_part) +
+    const f16x4* op = reinterpret_cast<const f16x4*>(p.o_part) +
                       ((((size_t)g * p.num_splits) * p.num_mtiles + mt) * kRowWaves + rw) * 16 * 64 + quad * 64 + lane;
     const size_t ml_stride = (size_t)p.rows_pad;
     const size_t o_stride = (size_t)p.num_mtiles * kRowWaves * 16 * 64;
@@ -494,7 +498,7 @@ __global__ __launch_bounds__(256) void tree_attn_combine_kernel(AttnParams p) {
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
     for (int s0 = 0; s0 < p.num_splits; s0 += kCombineBatch) {
         float2 v[kCombineBatch];
-        f32x4 o[kCombineBatch];
+        f16x4 o[kCombineBatch];
 #pragma unroll
         for (int u = 0; u < kCombineBatch; ++u) {
             const int s = min(s0 + u, p.num_splits - 1);  // clamp: repeats are ignored below
@@ -515,10 +519,10 @@ __global__ __launch_bounds__(256) void tree_attn_combine_kernel(AttnParams p) {
         for (int u = 0; u < kCombineBatch; ++u) {
             // an empty split (l == 0) has no meaningful O partial: select it away, never scale it
             if (!(s0 + u < p.num_splits && v[u].y > 0.f)) continue;
-            const float w = __builtin_amdgcn_exp2f(v[u].x - M);
-            L += w * v[u].y;
+            const float w = __builtin_amdgcn_exp2f(v[u].x - M) * v[u].y;  // partials are stored normalised
+            L += w;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) acc[e] += w * o[u][e];
+            for (int e = 0; e < 4; ++e) acc[e] += w * (float)o[u][e];
         }
     }
     const float inv = (L == 0.f || L != L) ? 1.f : 1.f / L;
@@ -599,7 +603,7 @@ extern "C" int cpmcu_tree_attention(const void* q, void* k_pool, void* v_pool,
     p.o_part = nullptr;
     p.ml_part = nullptr;
     if (p.num_splits > 1) {
-        const size_t o_bytes = (size_t)Hkv * p.num_splits * p.rows_pad * kHeadDim * sizeof(float);
+        const size_t o_bytes = align_up((size_t)Hkv * p.num_splits * p.rows_pad * kHeadDim * sizeof(f16), 256);
         const size_t ml_bytes = (size_t)Hkv * p.num_splits * p.rows_pad * 2 * sizeof(float);
         CPMCU_CHECK_ARG(workspace && workspace_bytes >= o_bytes + ml_bytes,
                         "tree_attention: workspace of %zu bytes needed, %zu given", o_bytes + ml_bytes, workspace_bytes);
