@@ -27,6 +27,17 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
+# HBM bytes per launch on c2_verify_4k with the automatic split count, from rocprofv3's FETCH_SIZE and
+# WRITE_SIZE counters (KiB per dispatch, one counter per run, eager launches), each scaled by what the
+# same counter read for a plain 256 MiB copy (x2.000 and x1.000): the table and the two commands are in
+# profiles/verify_step_hbm_traffic.md.  Counters cannot be read from inside this process, so the figures
+# are carried here as constants and are reported only for the workload they were measured on.
+MEASURED_TRAFFIC_KIB = {
+    "tree_attn_split_kernel+tree_attn_combine_kernel": 6482 + 9518 + 8722 + 480,
+    "head_gemm_kernel<4>+head_argmax_finalize_kernel": 608804 + 128 + 1064 + 2,
+    "tree_accept_kernel+kv_compact_kernel+accepted_ids_kernel": 6 + 1125 + 320 + 2,
+}
+
 
 def parse_args():
     ap = argparse.ArgumentParser()
@@ -235,6 +246,10 @@ def main():
         dict(kernel="tree_accept_kernel+kv_compact_kernel+accepted_ids_kernel", launches_per_step=1,
              us_per_launch=round(ms_tail * 1e3, 2), bound="hbm", achieved=None, peak=HBM_PEAK_GBS, unit="GB/s", frac=None, traffic=None),
     ]
+    if args.workload == "c2_verify_4k" and args.splits == 0:
+        for k in kernels:
+            k["traffic"] = MEASURED_TRAFFIC_KIB[k["kernel"]] * 1024
+            k["traffic_unit"] = "bytes/launch"
     dominant = max(kernels, key=lambda k: k["us_per_launch"] * k["launches_per_step"])
     roofline = {k: dominant[k] for k in ("bound", "achieved", "peak", "unit", "frac", "traffic")}
     roofline["kernel"] = dominant["kernel"]
