@@ -25,10 +25,11 @@
 //    choice of the global address each lane fetches, so no registers are spent
 //    on staging and two tiles are always in flight behind the two being
 //    consumed.
-//  * A workgroup is 8 waves = 2 KV groups x 4 row waves over the same 128
-//    packed rows: the groups take alternate tiles of the ring (two independent
-//    instruction streams per SIMD) and are merged through LDS at the end -- half
-//    the partial traffic of splitting the same work over two workgroups.
+//  * A workgroup is 8 waves.  For short contexts they are 2 KV groups x 4 row
+//    waves over the same 128 packed rows: the groups take alternate tiles of
+//    the ring and are merged through LDS at the end -- half the partial traffic
+//    of splitting the same work over two workgroups.  For long contexts they
+//    are 8 row waves over 256 packed rows, every tile feeding all of them.
 //  * Workgroups are mapped so that all M-tiles that stream the same KV range
 //    land on the same XCD (workgroup id modulo 8) and share its L2.
 #include "common.h"
@@ -37,12 +38,15 @@ namespace cpmcu {
 namespace {
 
 constexpr int kTileN = 64;                  // keys per LDS tile
-constexpr int kRowWaves = 4;                // row waves per KV group
-constexpr int kGroups = 2;                  // KV groups per workgroup
-constexpr int kWaves = kRowWaves * kGroups;
+constexpr int kWaves = 8;                   // waves per workgroup = KV groups x row waves
 constexpr int kRowsPerWave = 32;            // packed query rows per wave (one MFMA N block)
-constexpr int kRowsPerWg = kRowWaves * kRowsPerWave;
 constexpr int kThreads = kWaves * 64;
+// The kernel comes in two shapes (template parameter G = KV groups per workgroup):
+//   G = 2: 4 row waves (128 packed rows) x 2 KV groups that take alternate tiles and are merged through
+//          LDS at the end.  More (KV head, M-tile) units, so fewer splits fill the GPU: short contexts.
+//   G = 1: 8 row waves (256 packed rows) on every tile.  Each tile fetched feeds twice the rows and
+//          three tiles are in flight behind the one being consumed: long contexts.
+constexpr int rows_per_wg(int G) { return (kWaves / G) * kRowsPerWave; }
 constexpr int kStages = 4;
 constexpr int kKTileBytes = kTileN * kHeadDim * 2;  // 16 KB, row = one key (256 B)
 constexpr int kVTileBytes = kHeadDim * kTileN * 2;  // 16 KB, row = one dim (128 B)
@@ -50,6 +54,7 @@ constexpr int kStageBytes = kKTileBytes + kVTileBytes;
 constexpr int kMaxPagesPerSplit = 1024;
 constexpr int kMaxSplits = 64;
 constexpr int kXcds = 8;
+constexpr float kLazyLog2 = 8.f;  // slack of the lazily updated softmax reference, in log2 units
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
@@ -72,8 +77,8 @@ struct AttnParams {
     f16* out;
     // Split partials in the accumulator's own layout, so that both the split kernel's stores and the
     // combine kernel's loads are whole 1 KB wave transactions:
-    //   o_part  [Hkv][num_splits][num_mtiles][row wave][16 quads][64 lanes] x 4 halves (normalised O)
-    //           quad q = db * 4 + rq of lane (qcol, hf) holds O[row = rw*32 + qcol][d = db*32 + rq*8 + hf*4 + 0..3]
+    //   o_part  [Hkv][num_splits][rows_pad / 32 row blocks][16 quads][64 lanes] x 4 halves (normalised O)
+    //           quad q = db * 4 + rq of lane (qcol, hf) holds O[row = block*32 + qcol][d = db*32 + rq*8 + hf*4 + 0..3]
     //   ml_part [Hkv][num_splits][rows_pad] x float2 (max * scale_log2, sum)
     float* o_part;
     float* ml_part;
@@ -97,34 +102,42 @@ __device__ inline int v_lds_off(int d, int piece) { return kKTileBytes + d * 128
 // completion of these loads is tracked by hand (s_waitcnt vmcnt before the workgroup barrier that
 // publishes a stage), which lets the next tiles stay in flight while the current ones are consumed;
 // with the compiler builtin every LDS read would first wait for all of them.
-__device__ inline void load_to_lds16(const void* gptr, const char* lds_dst) {
+__device__ inline void load_to_lds16(const void* base, uint32_t byte_off, const char* lds_dst) {
     const uint32_t lds_addr = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)lds_dst);
-    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gptr), "s"(lds_addr) : "memory", "m0");
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(byte_off), "s"(base), "s"(lds_addr) : "memory", "m0");
+}
+
+// Per-thread byte offsets of its pieces inside a K tile and a V^T tile of a page (second piece of each:
+// + 32 keys = 8192 bytes for K, + 64 dims = 64 * 512 bytes for V^T; the swizzle terms do not change).
+__device__ inline uint32_t k_piece_off(int wave, int lane) {
+    const int key = wave * 4 + (lane >> 4);
+    const int piece = (lane & 15) ^ (key & 15);
+    return (uint32_t)(key * kHeadDim + piece * 8) * 2u;
+}
+__device__ inline uint32_t v_piece_off(int wave, int lane) {
+    const int d = wave * 8 + (lane >> 3);
+    const int piece = (lane & 7) ^ ((d >> 1) & 7);
+    return (uint32_t)(d * kPage + piece * 8) * 2u;
 }
 
 // Issues this thread's four 16-byte direct-to-LDS loads of one tile (2 for K, 2 for V^T).  Each
 // wave-level instruction fills 1 KB of LDS in lane order; the swizzle is applied on the global side.
-__device__ inline void issue_tile(const AttnParams& p, int g, int tile, int page, char* stage, int wave, int lane) {
+// Everything but the two per-thread offsets is wave-uniform, so the address arithmetic is scalar.
+__device__ inline void issue_tile(const AttnParams& p, int g, int tile, int page, char* stage, int wave, uint32_t koff, uint32_t voff) {
     const int slot0 = (tile * kTileN) % kPage;
-    const f16* kbase = p.k_pool + (((size_t)page * p.Hkv + g) * kPage + slot0) * kHeadDim;
-    const f16* vbase = p.v_pool + ((size_t)page * p.Hkv + g) * kHeadDim * kPage + slot0;
-#pragma unroll
-    for (int qq = 0; qq < 2; ++qq) {
-        const int inst = wave + kWaves * qq;  // 16 KB / 1 KB = 16 instructions per operand, 2 per wave
-        {
-            const int key = inst * 4 + (lane >> 4);
-            const int piece = (lane & 15) ^ (key & 15);
-            load_to_lds16(kbase + (size_t)key * kHeadDim + piece * 8, stage + inst * 1024);
-        }
-        {
-            const int d = inst * 8 + (lane >> 3);
-            const int piece = (lane & 7) ^ ((d >> 1) & 7);
-            load_to_lds16(vbase + (size_t)d * kPage + piece * 8, stage + kKTileBytes + inst * 1024);
-        }
-    }
+    const char* kbase = reinterpret_cast<const char*>(p.k_pool + (((size_t)page * p.Hkv + g) * kPage + slot0) * kHeadDim);
+    const char* vbase = reinterpret_cast<const char*>(p.v_pool + ((size_t)page * p.Hkv + g) * kHeadDim * kPage + slot0);
+    load_to_lds16(kbase, koff, stage + wave * 1024);
+    load_to_lds16(vbase, voff, stage + kKTileBytes + wave * 1024);
+    load_to_lds16(kbase + 32 * kHeadDim * 2, koff, stage + (wave + kWaves) * 1024);
+    load_to_lds16(vbase + 64 * kPage * 2, voff, stage + kKTileBytes + (wave + kWaves) * 1024);
 }
 
+template <int G>
 __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams p) {
+    constexpr int kRowWaves = kWaves / G;
+    constexpr int kRowsPerWg = kRowWaves * kRowsPerWave;
+    constexpr int kDepth = kStages / G - 1;  // iterations in flight behind the one being consumed
     __shared__ __attribute__((aligned(1024))) char ring[kStages * kStageBytes];
     __shared__ int32_t s_pages[kMaxPagesPerSplit];
 
@@ -142,7 +155,7 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
     const int tid = threadIdx.x;
     const int wave = tid >> 6;
     const int lane = tid & 63;
-    const int grp = wave / kRowWaves;  // KV group: takes tiles grp, grp + 2, ...
+    const int grp = wave / kRowWaves;  // KV group: takes tiles grp, grp + G, ...
     const int rw = wave % kRowWaves;
     const int qcol = lane & 31;
     const int hf = lane >> 5;
@@ -192,16 +205,19 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
     const int ntiles = (S + kTileN - 1) / kTileN;
     const int t1 = min(t1_max, ntiles);
     const int n = max(t1 - t0, 0);
-    const int npairs = (n + 1) / 2;
+    const int niter = (n + G - 1) / G;  // one iteration consumes G tiles, one per KV group
     __syncthreads();
 
-    auto issue_pair = [&](int pair) {
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    const uint32_t koff = k_piece_off(wave, lane), voff = v_piece_off(wave, lane);
+    auto issue_iter = [&](int it) {
 #pragma unroll
-        for (int e = 0; e < 2; ++e) {
-            const int i = pair * 2 + e;
+        for (int e = 0; e < G; ++e) {
+            const int i = it * G + e;
             if (i < n) {
                 const int tile = t0 + i;
-                issue_tile(p, g, tile, s_pages[(tile * kTileN) / kPage - pg0], ring + (i % kStages) * kStageBytes, wave, lane);
+                const int page = __builtin_amdgcn_readfirstlane(s_pages[(tile * kTileN) / kPage - pg0]);
+                issue_tile(p, g, tile, page, ring + (i % kStages) * kStageBytes, wave_u, koff, voff);
             }
         }
     };
@@ -211,26 +227,38 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
     for (int db = 0; db < 4; ++db)
 #pragma unroll
         for (int r = 0; r < 16; ++r) oacc[db][r] = 0.f;
-    float m_run = -INFINITY;  // running row max (raw score units)
+    // Online softmax state of this lane's query row.  m_ref is the exponent reference in log2 units
+    // (score * scale * log2 e): probabilities are computed as 2^(s - m_ref).  It follows the running
+    // row maximum lazily -- it is raised (and O, l rescaled) only when a tile's maximum exceeds it by
+    // more than kLazyLog2, so the rescale of the 64 accumulator registers is rare; meanwhile
+    // probabilities may reach 2^kLazyLog2, far inside fp16 and fp32 range.  O / l does not depend
+    // on the reference.
+    float m_ref = -INFINITY;
     float l_run = 0.f;        // this lane's share of the row sum
 
-    if (npairs > 0) issue_pair(0);
-    if (npairs > 1) issue_pair(1);
+#pragma unroll
+    for (int d = 0; d <= kDepth; ++d)
+        if (d < niter) issue_iter(d);
 
-    for (int pair = 0; pair < npairs; ++pair) {
-        // Wait for this pair's tiles.  Pair p+1 is issued right after the barrier of iteration p, so
-        // nothing newer is outstanding here -- except in iteration 0, where pair 1 (4 loads per
-        // thread and tile, issued in the prologue) may stay in flight.
-        if (pair == 0 && npairs > 1) {
-            if (n >= 4) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
-            else asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-        } else {
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    for (int it = 0; it < niter; ++it) {
+        // Wait for this iteration's tiles.  The prologue issued iterations 0..kDepth and iteration
+        // j >= 1 issues iteration j + kDepth right after its barrier, so the tiles issued so far are
+        // those of iterations <= max(it - 1, 0) + kDepth; the ones beyond this iteration (4 loads per
+        // thread and tile, returned in order) may stay in flight.
+        {
+            const int issued = min(n, (max(it - 1, 0) + kDepth + 1) * G);
+            const int needed = min(n, (it + 1) * G);
+            switch (issued - needed) {
+                case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+                case 1: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
+                case 2: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+                default: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
+            }
         }
-        __syncthreads();  // every thread's pieces have landed; the previous pair's stages are free
-        if (pair >= 1 && pair + 1 < npairs) issue_pair(pair + 1);
+        __syncthreads();  // every thread's pieces have landed; the previous iteration's stages are free
+        if (it >= 1 && it + kDepth < niter) issue_iter(it + kDepth);
 
-        const int i = pair * 2 + grp;  // this group's tile of the pair
+        const int i = it * G + grp;  // this group's tile of the iteration
         const int t = t0 + i;
         const int c0 = t * kTileN;
         char* stage = ring + (i % kStages) * kStageBytes;
@@ -243,11 +271,11 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
         //  * the tile that holds position S-1 may extend past it: stale page contents there must not
         //    reach the MFMA (0 * NaN = NaN), so the V^T columns of tokens >= S are zeroed.  K needs
         //    nothing: the scores of those keys are replaced (not scaled) by -inf below.
-        const int pair_end = (t0 + pair * 2) * kTileN + 2 * kTileN;
-        const bool pair_needs_fix = pair_end > S || (p.k_new != nullptr && pair_end > P);
-        if (pair_needs_fix) {
-            for (int e = 0; e < 2; ++e) {
-                const int ie = pair * 2 + e;
+        const int iter_end = (t0 + it * G) * kTileN + G * kTileN;
+        const bool iter_needs_fix = iter_end > S || (p.k_new != nullptr && iter_end > P);
+        if (iter_needs_fix) {
+            for (int e = 0; e < G; ++e) {
+                const int ie = it * G + e;
                 const int ce = (t0 + ie) * kTileN;
                 if (ie >= n) continue;
                 char* st = ring + (ie % kStages) * kStageBytes;
@@ -349,11 +377,18 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, sacc[kb][r]);
-            tmax = fmaxf(tmax, __shfl_xor(tmax, 32));
-            const float m_new = fmaxf(m_run, tmax);
-            const float m_scaled = (m_new == -INFINITY) ? 0.f : m_new * p.scale_log2;
-            const float alpha = __builtin_amdgcn_exp2f(m_run * p.scale_log2 - m_scaled);
-            m_run = m_new;
+            tmax = fmaxf(tmax, __shfl_xor(tmax, 32)) * p.scale_log2;  // scale > 0
+            if (__any(tmax > m_ref + kLazyLog2)) {  // some row's maximum moved far: re-reference all rows
+                const float m_new = fmaxf(m_ref, tmax);
+                const float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_ref - m_new);
+                m_ref = m_new;
+                l_run *= alpha;
+#pragma unroll
+                for (int db = 0; db < 4; ++db)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
+            }
+            const float m_scaled = (m_ref == -INFINITY) ? 0.f : m_ref;
             float psum = 0.f;
             f16x8 pb[4];  // P^T as B operand: k-step j holds keys 16*j + {4hf..4hf+3, 8+4hf..8+4hf+3}
 #pragma unroll
@@ -361,16 +396,21 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const float pv = __builtin_amdgcn_exp2f(sacc[kb][r] * p.scale_log2 - m_scaled);
-                    psum += pv;                              // row sum keeps the fp32 value
                     pb[kb * 2 + (r >> 3)][r & 7] = (f16)pv;  // P is rounded to fp16 before P.V
                 }
-            l_run = l_run * alpha + psum;
-            if (__any(alpha != 1.f)) {  // skipped when no lane's running max moved
+            // Row sum of the rounded probabilities, two per instruction (fp32 accumulation): the
+            // denominator then weighs exactly the values the numerator's MFMA sees.
+            {
+                const f16x2 ones = {(f16)1.f, (f16)1.f};
 #pragma unroll
-                for (int db = 0; db < 4; ++db)
+                for (int j = 0; j < 4; ++j)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) oacc[db][r] *= alpha;
+                    for (int e = 0; e < 4; ++e) {
+                        const f16x2 pp = {pb[j][2 * e], pb[j][2 * e + 1]};
+                        psum = __builtin_amdgcn_fdot2(pp, ones, psum, false);
+                    }
             }
+            l_run += psum;
 
             // ---- O^T += V^T.P^T ----
             {
@@ -392,6 +432,7 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
     }
 
     // ---- merge the two KV groups through LDS (lane-private layout: [row wave][value][lane]) ----
+    if constexpr (G == 2) {
     __syncthreads();  // ring no longer read
     f32x4* xch = reinterpret_cast<f32x4*>(ring);           // [row wave][17 quads][64 lanes]
     const int xbase = rw * 17 * 64 + lane;
@@ -405,17 +446,17 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
                 for (int e = 0; e < 4; ++e) o[e] = oacc[db][rq * 4 + e];
                 xch[xbase + (db * 4 + rq) * 64] = o;
             }
-        xch[xbase + 16 * 64] = f32x4{m_run, l_run, 0.f, 0.f};
+        xch[xbase + 16 * 64] = f32x4{m_ref, l_run, 0.f, 0.f};
     }
     __syncthreads();
     if (grp == 1) return;
     {
         const f32x4 ml1 = xch[xbase + 16 * 64];
         const float m1 = ml1[0], l1 = ml1[1];
-        const float m_new = fmaxf(m_run, m1);
-        const float m_scaled = (m_new == -INFINITY) ? 0.f : m_new * p.scale_log2;
-        const float a0 = __builtin_amdgcn_exp2f(m_run * p.scale_log2 - m_scaled);
-        const float a1 = __builtin_amdgcn_exp2f(m1 * p.scale_log2 - m_scaled);
+        const float m_new = fmaxf(m_ref, m1);
+        const float m_scaled = (m_new == -INFINITY) ? 0.f : m_new;
+        const float a0 = __builtin_amdgcn_exp2f(m_ref - m_scaled);
+        const float a1 = __builtin_amdgcn_exp2f(m1 - m_scaled);
 #pragma unroll
         for (int db = 0; db < 4; ++db)
 #pragma unroll
@@ -425,7 +466,8 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
                 for (int e = 0; e < 4; ++e) oacc[db][rq * 4 + e] = oacc[db][rq * 4 + e] * a0 + o[e] * a1;
             }
         l_run = l_run * a0 + l1 * a1;
-        m_run = m_new;
+        m_ref = m_new;
+    }
     }
 
     // oacc[db][r] is O[query qcol][d = db*32 + 8*(r/4) + 4*hf + r%4], unnormalised.
@@ -461,7 +503,7 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
                 __builtin_nontemporal_store(o, &op[(db * 4 + rq) * 64]);  // streamed: nothing left to flush at kernel end
             }
         if (hf == 0 && row_ok) {
-            p.ml_part[prow * 2 + 0] = (m_run == -INFINITY) ? -INFINITY : m_run * p.scale_log2;
+            p.ml_part[prow * 2 + 0] = m_ref;
             p.ml_part[prow * 2 + 1] = l_tot;
         }
     }
@@ -474,25 +516,25 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
 // are all requested before any is used, so the kernel pays one memory round trip, not one per split.
 constexpr int kCombineBatch = 16;
 __global__ __launch_bounds__(256) void tree_attn_combine_kernel(AttnParams p) {
-    // thread -> (kv head, M-tile, row wave, quad, lane) in the partial layout's own order
+    // thread -> (kv head, 32-row block, quad, lane) in the partial layout's own order
     const int idx = blockIdx.x * 256 + threadIdx.x;
     const int lane = idx & 63;
     const int quad = (idx >> 6) & 15;
-    const int rw = (idx >> 10) & (kRowWaves - 1);
-    const int gm = idx >> 12;  // g * num_mtiles + mt   (kRowWaves * 16 * 64 = 4096 threads per M-tile)
-    if (gm >= p.Hkv * p.num_mtiles) return;
-    const int g = gm / p.num_mtiles, mt = gm % p.num_mtiles;
+    const int nrb = p.rows_pad / kRowsPerWave;  // 32-row blocks per kv head (16 * 64 = 1024 threads each)
+    const int grb = idx >> 10;
+    if (grb >= p.Hkv * nrb) return;
+    const int g = grb / nrb, rb = grb % nrb;
     const int qcol = lane & 31, hf = lane >> 5;
-    const int R = mt * kRowsPerWg + rw * kRowsPerWave + qcol;
+    const int R = rb * kRowsPerWave + qcol;
     if (R >= p.group * p.T) return;
     const int node = R / p.group;
     const int head = g * p.group + R % p.group;
     const int d0 = (quad >> 2) * 32 + (quad & 3) * 8 + hf * 4;
     const float2* ml = reinterpret_cast<const float2*>(p.ml_part) + (size_t)g * p.num_splits * p.rows_pad + R;
     const f16x4* op = reinterpret_cast<const f16x4*>(p.o_part) +
-                      ((((size_t)g * p.num_splits) * p.num_mtiles + mt) * kRowWaves + rw) * 16 * 64 + quad * 64 + lane;
+                      (((size_t)g * p.num_splits) * nrb + rb) * 16 * 64 + quad * 64 + lane;
     const size_t ml_stride = (size_t)p.rows_pad;
-    const size_t o_stride = (size_t)p.num_mtiles * kRowWaves * 16 * 64;
+    const size_t o_stride = (size_t)nrb * 16 * 64;
 
     float M = -INFINITY, L = 0.f;
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
@@ -532,15 +574,27 @@ __global__ __launch_bounds__(256) void tree_attn_combine_kernel(AttnParams p) {
     *reinterpret_cast<f16x4*>(p.out + ((size_t)node * p.Hq + head) * kHeadDim + d0) = o;
 }
 
-int choose_splits(int T, int group, int Hkv, int max_kv_len) {
-    const int num_mtiles = ceil_div(group * T, kRowsPerWg);
+int choose_splits(int T, int group, int Hkv, int max_kv_len, int G) {
+    const int num_mtiles = ceil_div(group * T, rows_per_wg(G));
     const int ntiles = ceil_div(max_kv_len, kTileN);
     // One workgroup per CU (256 CUs); every split should get at least one tile per KV group.
     int splits = 256 / (num_mtiles * Hkv);
     if (splits < 1) splits = 1;
-    if (splits > ntiles / 2) splits = ntiles / 2 > 0 ? ntiles / 2 : 1;
+    if (splits > ntiles / G) splits = ntiles / G > 0 ? ntiles / G : 1;
     if (splits > kMaxSplits) splits = kMaxSplits;
     return splits;
+}
+
+// KV groups per workgroup.  The 256-row shape pays off once every workgroup of a full-GPU launch has
+// a long enough run of tiles to amortise its larger split count (twice the partials to merge).
+// CPMCU_ATTN_KV_GROUPS=1|2 in the environment overrides the choice (tests exercise both shapes).
+constexpr int kLongContextTiles = 256;
+int choose_groups(int max_kv_len) {
+    if (const char* e = getenv("CPMCU_ATTN_KV_GROUPS")) {
+        if (e[0] == '1' && e[1] == 0) return 1;
+        if (e[0] == '2' && e[1] == 0) return 2;
+    }
+    return ceil_div(max_kv_len, kTileN) >= kLongContextTiles ? 1 : 2;
 }
 
 }  // namespace
@@ -552,8 +606,7 @@ extern "C" size_t cpmcu_tree_attention_workspace_bytes(int T, int Hq, int Hkv, i
     (void)max_kv_len;
     if (T <= 0 || Hkv <= 0 || Hq <= 0 || Hq % Hkv) return 0;
     const int group = Hq / Hkv;
-    const int num_mtiles = ceil_div(group * T, kRowsPerWg);
-    const int rows_pad = num_mtiles * kRowsPerWg;
+    const int rows_pad = align_up(group * T, rows_per_wg(1));  // the larger padding of the two kernel shapes
     // sized for the largest split count the library ever picks, so an override fits too
     return align_up((size_t)Hkv * kMaxSplits * rows_pad * (kHeadDim + 2) * sizeof(float), 256);
 }
@@ -590,9 +643,10 @@ extern "C" int cpmcu_tree_attention(const void* q, void* k_pool, void* v_pool,
     p.Hq = Hq;
     p.Hkv = Hkv;
     p.group = group;
-    p.num_mtiles = ceil_div(group * T, kRowsPerWg);
-    p.rows_pad = p.num_mtiles * kRowsPerWg;
-    p.num_splits = num_splits_override > 0 ? num_splits_override : choose_splits(T, group, Hkv, max_kv_len);
+    const int G = choose_groups(max_kv_len);
+    p.num_mtiles = ceil_div(group * T, rows_per_wg(G));
+    p.rows_pad = p.num_mtiles * rows_per_wg(G);
+    p.num_splits = num_splits_override > 0 ? num_splits_override : choose_splits(T, group, Hkv, max_kv_len, G);
     // a split keeps the physical page ids of its range in LDS
     const int min_splits = ceil_div(ceil_div(max_kv_len, kPage) + 2, kMaxPagesPerSplit - 2);
     if (p.num_splits < min_splits) p.num_splits = min_splits;
@@ -613,10 +667,11 @@ extern "C" int cpmcu_tree_attention(const void* q, void* k_pool, void* v_pool,
     hipStream_t st = resolve_stream(stream);
     const int nsh = p.num_splits * Hkv;
     const int grid = kXcds * ceil_div(nsh, kXcds) * p.num_mtiles;
-    hipLaunchKernelGGL(tree_attn_split_kernel, dim3(grid), dim3(kThreads), 0, st, p);
+    if (G == 1) hipLaunchKernelGGL(tree_attn_split_kernel<1>, dim3(grid), dim3(kThreads), 0, st, p);
+    else hipLaunchKernelGGL(tree_attn_split_kernel<2>, dim3(grid), dim3(kThreads), 0, st, p);
     CPMCU_LAUNCH_CHECK();
     if (p.num_splits > 1) {
-        const int threads_total = Hkv * p.num_mtiles * kRowWaves * 16 * 64;
+        const int threads_total = Hkv * (p.rows_pad / kRowsPerWave) * 16 * 64;
         hipLaunchKernelGGL(tree_attn_combine_kernel, dim3(ceil_div(threads_total, 256)), dim3(256), 0, st, p);
         CPMCU_LAUNCH_CHECK();
     }

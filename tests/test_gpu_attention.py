@@ -14,6 +14,14 @@ pytestmark = pytest.mark.gpu
 HQ, HKV, D = 32, 2, 128
 
 
+@pytest.fixture(autouse=True, params=["2", "1"], ids=["groups2", "groups1"])
+def kv_groups(request, monkeypatch):
+    """Every test of this module runs on both shapes of the split kernel (2 KV groups x 128 rows and
+    1 x 256 rows per workgroup); without the override the library picks by context length."""
+    monkeypatch.setenv("CPMCU_ATTN_KV_GROUPS", request.param)
+    return request.param
+
+
 def _case(torch, orc, tree, P, seed, page_perm=True, splits=0, use_mask=True, extra_pages=2, q_std=1.0):
     from cpm.cu_amd import ops
     from cpm.cu_amd.kvcache import PagedKVCache
