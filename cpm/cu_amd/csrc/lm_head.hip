@@ -54,6 +54,103 @@ struct HeadCfg {
     static constexpr int kStage = 8;                     // 16-byte staging registers per thread
 };
 
+// Folds one finished 16-row block of W (acc[nb][r] <-> vocab row vrow0 + r, hidden row nb*16 + l16) into
+// the lane's running epilogue state and writes its logits when asked to.
+template <int NB>
+__device__ inline void head_epilogue(const HeadParams& p, const f32x4 (&acc)[NB], int vrow0, int l16, float (&ea)[NB], float (&eb)[NB]) {
+    const int V = p.V;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        const int hrow = nb * 16 + l16;
+        f16 z[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) z[r] = (f16)acc[nb][r];
+        if (hrow < p.n) {
+            if (p.logits) {
+                f16* dst = p.logits + (size_t)hrow * V + vrow0;
+                if ((V & 3) == 0 && vrow0 + 3 < V) {
+                    f16x4 zz;
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) zz[r] = z[r];
+                    *reinterpret_cast<f16x4*>(dst) = zz;
+                } else {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (vrow0 + r < V) dst[r] = z[r];
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                if (vrow0 + r >= V) continue;
+                const float x = (float)z[r];
+                if (p.mode == kHeadModeStats) {
+                    if (x == -INFINITY) continue;  // contributes exp(-inf) = 0
+                    if (x > ea[nb]) {
+                        eb[nb] = eb[nb] * __expf(ea[nb] - x) + 1.f;
+                        ea[nb] = x;
+                    } else {
+                        eb[nb] += __expf(x - ea[nb]);
+                    }
+                } else {
+                    const int idx = vrow0 + r;
+                    const int bidx = __float_as_int(eb[nb]);
+                    if (x > ea[nb] || (x == ea[nb] && idx < bidx)) {
+                        ea[nb] = x;
+                        eb[nb] = __int_as_float(idx);
+                    }
+                }
+            }
+        }
+    }
+}
+
+// Reduces the epilogue state over the lanes that share a hidden row, then over the waves, and writes
+// the workgroup's partials.
+template <int NB>
+__device__ inline void head_finish(const HeadParams& p, float (&ea)[NB], float (&eb)[NB], float (*red_a)[NB * 16], float (*red_b)[NB * 16],
+                                   int tid, int wave, int lane, int c) {
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+#pragma unroll
+        for (int off = 16; off <= 32; off <<= 1) {
+            const float oa = __shfl_xor(ea[nb], off);
+            const float ob = __shfl_xor(eb[nb], off);
+            if (p.mode == kHeadModeStats) {
+                const float m = fmaxf(ea[nb], oa);
+                const float s = (m == -INFINITY) ? 0.f : eb[nb] * __expf(ea[nb] - m) + ob * __expf(oa - m);
+                ea[nb] = m;
+                eb[nb] = s;
+            } else {
+                if (oa > ea[nb] || (oa == ea[nb] && __float_as_int(ob) < __float_as_int(eb[nb]))) {
+                    ea[nb] = oa;
+                    eb[nb] = ob;
+                }
+            }
+        }
+        if (lane < 16) {
+            red_a[wave][nb * 16 + lane] = ea[nb];
+            red_b[wave][nb * 16 + lane] = eb[nb];
+        }
+    }
+    __syncthreads();
+    if (tid < NB * 16) {
+        float a = red_a[0][tid], b = red_b[0][tid];
+        for (int w = 1; w < kHeadWaves; ++w) {
+            const float oa = red_a[w][tid], ob = red_b[w][tid];
+            if (p.mode == kHeadModeStats) {
+                const float m = fmaxf(a, oa);
+                b = (m == -INFINITY) ? 0.f : b * __expf(a - m) + ob * __expf(oa - m);
+                a = m;
+            } else if (oa > a || (oa == a && __float_as_int(ob) < __float_as_int(b))) {
+                a = oa;
+                b = ob;
+            }
+        }
+        p.part_a[(size_t)c * (NB * 16) + tid] = a;
+        p.part_b[(size_t)c * (NB * 16) + tid] = b;
+    }
+}
+
 template <int NB>
 __global__ __launch_bounds__(kHeadThreads) void head_gemm_kernel(HeadParams p) {
     using C = HeadCfg<NB>;
@@ -142,53 +239,7 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_kernel(HeadParams p) {
         eb[nb] = p.mode == kHeadModeStats ? 0.f : __int_as_float(0x7fffffff);  // running sum / best index
     }
 
-    auto epilogue = [&](int pass) {
-        const int rb = row_block(pass);
-        const int vrow0 = rb * 16 + kgp * 4;  // acc[nb][r] <-> vocab row vrow0 + r, hidden row nb*16 + l16
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-            const int hrow = nb * 16 + l16;
-            f16 z[4];
-#pragma unroll
-            for (int r = 0; r < 4; ++r) z[r] = (f16)acc[nb][r];
-            if (hrow < p.n) {
-                if (p.logits) {
-                    f16* dst = p.logits + (size_t)hrow * V + vrow0;
-                    if ((V & 3) == 0 && vrow0 + 3 < V) {
-                        f16x4 zz;
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) zz[r] = z[r];
-                        *reinterpret_cast<f16x4*>(dst) = zz;
-                    } else {
-#pragma unroll
-                        for (int r = 0; r < 4; ++r)
-                            if (vrow0 + r < V) dst[r] = z[r];
-                    }
-                }
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    if (vrow0 + r >= V) continue;
-                    const float x = (float)z[r];
-                    if (p.mode == kHeadModeStats) {
-                        if (x == -INFINITY) continue;  // contributes exp(-inf) = 0
-                        if (x > ea[nb]) {
-                            eb[nb] = eb[nb] * __expf(ea[nb] - x) + 1.f;
-                            ea[nb] = x;
-                        } else {
-                            eb[nb] += __expf(x - ea[nb]);
-                        }
-                    } else {
-                        const int idx = vrow0 + r;
-                        const int bidx = __float_as_int(eb[nb]);
-                        if (x > ea[nb] || (x == ea[nb] && idx < bidx)) {
-                            ea[nb] = x;
-                            eb[nb] = __int_as_float(idx);
-                        }
-                    }
-                }
-            }
-        }
-    };
+    auto epilogue = [&](int pass) { head_epilogue<NB>(p, acc, row_block(pass) * 16 + kgp * 4, l16, ea, eb); };
 
     // ---- prologue: hidden into LDS ----
     if (resident) {
@@ -251,47 +302,139 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_kernel(HeadParams p) {
         }
     }
 
-    // ---- reduce the epilogue state: lanes sharing a hidden row, then waves ----
+    head_finish<NB>(p, ea, eb, red_a, red_b, tid, wave, lane, c);
+}
+
+// More than 16 hidden rows do not fit LDS for the whole K range.  This kernel walks K in chunks in the
+// OUTER loop: a chunk of all hidden rows (64 KB) is brought into LDS by direct-to-LDS loads, double
+// buffered, and every wave then streams that K range of each of its row blocks of W, keeping one
+// accumulator set per row block (NP row blocks per sweep over K).  The workgroup synchronises once
+// per chunk, not once per (row block, chunk), so the waves' W streams run free in between.
+//   LDS layout of a chunk: [hidden row][KC halves], unpadded; the 16-byte piece index is XORed with
+//   row % 16 (applied through the global address each DMA lane fetches), which makes the B-operand
+//   reads (16 rows x one piece per 16 lanes) conflict-free.
+template <int NB, int NP, int KC, int NBUF>  // KC = halves of K per chunk, NBUF = W register buffers
+__global__ __launch_bounds__(kHeadThreads) void head_gemm_chunked_kernel(HeadParams p) {
+    constexpr int PD = KC / 32;              // 16-byte W loads in flight per lane and buffer
+    constexpr int ROWB = KC * 2;
+    constexpr int BUF = NB * 16 * ROWB;
+    constexpr int PR = KC / 8;               // 16-byte pieces per hidden row chunk
+    constexpr int NINST = BUF / 1024 / kHeadWaves;  // 1 KB DMA instructions per wave and chunk
+    static_assert(NP % NBUF == 0, "the W buffers rotate with the row-block index");
+    __shared__ __attribute__((aligned(1024))) char lds[2 * BUF];
+    __shared__ float red_a[kHeadWaves][NB * 16];
+    __shared__ float red_b[kHeadWaves][NB * 16];
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    const int l16 = lane & 15;
+    const int kgp = lane >> 4;
+    const int G = gridDim.x;
+    const int c = blockIdx.x;
+    const int H = p.H, V = p.V;
+    const int nch = H / KC;
+    const int nsweeps = (p.npasses + NP - 1) / NP;
+    const int total_q = nsweeps * nch;
+    const int rotc = c % nch;  // workgroups start their K walk at different chunks (HBM channel spread)
+    const f16 sc = (f16)p.head_scale;
+
+    auto chunk_of = [&](int q) { return (q % nch + rotc) % nch; };
+    // hidden chunk q -> LDS buffer q & 1 (asynchronous; completion is awaited with vmcnt below)
+    auto issue_hidden = [&](int q) {
+        const int k0 = chunk_of(q) * KC;
+#pragma unroll
+        for (int j = 0; j < NINST; ++j) {
+            const int inst = wave * NINST + j;
+            const int row = inst * (64 / PR) + lane / PR;
+            const int piece = (lane % PR) ^ (row & 15);
+            const int rc = row < p.n ? row : p.n - 1;  // rows past n: any valid data, their results are dropped
+            const f16* src = p.hidden + (size_t)rc * H + k0 + piece * 8;
+            const uint32_t dst = __builtin_amdgcn_readfirstlane(
+                (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)(lds + (q & 1) * BUF + inst * 1024));
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(dst) : "memory", "m0");
+        }
+    };
+    auto row_block = [&](int pass) { return (pass * kHeadWaves + wave) * G + c; };
+    auto load_w = [&](int q, int pl, f16x8* buf) {
+        const int pass = (q / nch) * NP + pl;
+        if (pass >= p.npasses) return;
+        int row = row_block(pass) * 16 + l16;
+        row = row < V ? row : V - 1;  // clamp: rows past the end are computed and discarded
+        const f16* src = p.w + (size_t)row * H + chunk_of(q) * KC + kgp * 8;
+#pragma unroll
+        for (int ks = 0; ks < PD; ++ks) buf[ks] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(src + ks * 32));
+    };
+
+    f32x4 acc[NP][NB];
+    float ea[NB], eb[NB];
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
+        ea[nb] = -INFINITY;
+        eb[nb] = p.mode == kHeadModeStats ? 0.f : __int_as_float(0x7fffffff);
+    }
+    const int xl = (kgp ^ (l16 & 3)) << 4, hi = l16 >> 2;
+
+    // W groups are requested NBUF - 1 steps ahead of their use (a step = one row block x one chunk).
+    f16x8 bufs[NBUF][PD];
+    issue_hidden(0);
 #pragma unroll
-        for (int off = 16; off <= 32; off <<= 1) {
-            const float oa = __shfl_xor(ea[nb], off);
-            const float ob = __shfl_xor(eb[nb], off);
-            if (p.mode == kHeadModeStats) {
-                const float m = fmaxf(ea[nb], oa);
-                const float s = (m == -INFINITY) ? 0.f : eb[nb] * __expf(ea[nb] - m) + ob * __expf(oa - m);
-                ea[nb] = m;
-                eb[nb] = s;
-            } else {
-                if (oa > ea[nb] || (oa == ea[nb] && __float_as_int(ob) < __float_as_int(eb[nb]))) {
-                    ea[nb] = oa;
-                    eb[nb] = ob;
+    for (int s0 = 0; s0 < NBUF - 1; ++s0) load_w(s0 / NP, s0 % NP, bufs[s0 % NBUF]);  // NBUF - 1 <= NP
+    for (int q = 0; q < total_q; ++q) {
+        const int ch = q % nch;
+        if (ch == 0) {
+#pragma unroll
+            for (int pl = 0; pl < NP; ++pl)
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) acc[pl][nb][r] = 0.f;
+        }
+        // Chunk q was requested one iteration ago; the only memory operations issued after it that
+        // may still be in flight are the loads of the NBUF - 1 W groups prefetched last (returns are in order).
+        asm volatile("s_waitcnt vmcnt(%0)" : : "n"((NBUF - 1) * PD) : "memory");
+        if (p.apply_scale) {  // fp16 pre-scale of the hidden rows (src/model/linear.cuh:82-101): own pieces, in place
+#pragma unroll
+            for (int j = 0; j < NINST; ++j) {
+                f16x8* px = reinterpret_cast<f16x8*>(lds + (q & 1) * BUF + (wave * NINST + j) * 1024 + lane * 16);
+                f16x8 x = *px;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x[e] = (f16)((float)x[e] * (float)sc);
+                *px = x;
+            }
+        }
+        __syncthreads();  // chunk q visible to all waves; all waves are done with the other buffer
+        if (q + 1 < total_q) issue_hidden(q + 1);
+        const char* base = lds + (q & 1) * BUF + l16 * ROWB + xl;
+#pragma unroll
+        for (int pl = 0; pl < NP; ++pl) {
+            {
+                constexpr int kA = NBUF - 1;
+                const int pn = pl + kA;
+                if (pn < NP) load_w(q, pn, bufs[pn % NBUF]);
+                else if (q + 1 < total_q) load_w(q + 1, pn - NP, bufs[(pn - NP) % NBUF]);
+            }
+            if ((q / nch) * NP + pl < p.npasses) {
+#pragma unroll
+                for (int ks = 0; ks < PD; ++ks) {
+                    const char* bk = base + ((ks ^ hi) << 6);
+#pragma unroll
+                    for (int nb = 0; nb < NB; ++nb) {
+                        const f16x8 b = *reinterpret_cast<const f16x8*>(bk + nb * 16 * ROWB);
+                        acc[pl][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bufs[pl % NBUF][ks], b, acc[pl][nb], 0, 0, 0);
+                    }
                 }
             }
         }
-        if (lane < 16) {
-            red_a[wave][nb * 16 + lane] = ea[nb];
-            red_b[wave][nb * 16 + lane] = eb[nb];
-        }
-    }
-    __syncthreads();
-    if (tid < NB * 16) {
-        float a = red_a[0][tid], b = red_b[0][tid];
-        for (int w = 1; w < kHeadWaves; ++w) {
-            const float oa = red_a[w][tid], ob = red_b[w][tid];
-            if (p.mode == kHeadModeStats) {
-                const float m = fmaxf(a, oa);
-                b = (m == -INFINITY) ? 0.f : b * __expf(a - m) + ob * __expf(oa - m);
-                a = m;
-            } else if (oa > a || (oa == a && __float_as_int(ob) < __float_as_int(b))) {
-                a = oa;
-                b = ob;
+        if (ch == nch - 1) {
+#pragma unroll
+            for (int pl = 0; pl < NP; ++pl) {
+                const int pass = (q / nch) * NP + pl;
+                if (pass < p.npasses) head_epilogue<NB>(p, acc[pl], row_block(pass) * 16 + kgp * 4, l16, ea, eb);
             }
         }
-        p.part_a[(size_t)c * (NB * 16) + tid] = a;
-        p.part_b[(size_t)c * (NB * 16) + tid] = b;
     }
+    head_finish<NB>(p, ea, eb, red_a, red_b, tid, wave, lane, c);
 }
 
 // Final arg-max over the per-workgroup partials: one block per hidden row.
@@ -372,11 +515,20 @@ int launch_head_gemm(const void* hidden, const void* w, int n, int V, int H, int
     p.npasses = ceil_div(nrb, G * kHeadWaves);
     *grid_out = G;
     *stride_out = NB * 16;
-    switch (NB) {
-        case 1: hipLaunchKernelGGL(head_gemm_kernel<1>, dim3(G), dim3(kHeadThreads), 0, st, p); break;
-        case 2: hipLaunchKernelGGL(head_gemm_kernel<2>, dim3(G), dim3(kHeadThreads), 0, st, p); break;
-        case 4: hipLaunchKernelGGL(head_gemm_kernel<4>, dim3(G), dim3(kHeadThreads), 0, st, p); break;
-        default: hipLaunchKernelGGL(head_gemm_kernel<8>, dim3(G), dim3(kHeadThreads), 0, st, p); break;
+    const int kc_chunked = 512;
+    if (p.nch <= 2 || H % kc_chunked != 0) {  // all hidden rows fit LDS for the whole K range (or an odd H)
+        switch (NB) {
+            case 1: hipLaunchKernelGGL(head_gemm_kernel<1>, dim3(G), dim3(kHeadThreads), 0, st, p); break;
+            case 2: hipLaunchKernelGGL(head_gemm_kernel<2>, dim3(G), dim3(kHeadThreads), 0, st, p); break;
+            case 4: hipLaunchKernelGGL(head_gemm_kernel<4>, dim3(G), dim3(kHeadThreads), 0, st, p); break;
+            default: hipLaunchKernelGGL(head_gemm_kernel<8>, dim3(G), dim3(kHeadThreads), 0, st, p); break;
+        }
+    } else {
+        switch (NB) {
+            case 2: hipLaunchKernelGGL((head_gemm_chunked_kernel<2, 4, 512, 2>), dim3(G), dim3(kHeadThreads), 0, st, p); break;
+            case 4: hipLaunchKernelGGL((head_gemm_chunked_kernel<4, 4, 128, 4>), dim3(G), dim3(kHeadThreads), 0, st, p); break;
+            default: hipLaunchKernelGGL((head_gemm_chunked_kernel<8, 2, 128, 2>), dim3(G), dim3(kHeadThreads), 0, st, p); break;
+        }
     }
     CPMCU_LAUNCH_CHECK();
     return CPMCU_OK;
