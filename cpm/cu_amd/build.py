@@ -20,7 +20,7 @@ LIB_PATH = os.path.join(HERE, "libcpmcu_amd.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 ARCH = "gfx950"
 
-HIP_SOURCES = ["runtime.hip", "tree_attention.hip", "lm_head.hip", "topk.hip", "tree_accept.hip"]
+HIP_SOURCES = ["runtime.hip", "tree_attention.hip", "lm_head.hip", "topk.hip", "tree_accept.hip", "draft_tree.hip"]
 HEADERS = ["common.h", "internal.h"]
 
 # packed fp32 VALU ops stay off for every device translation unit

@@ -1,0 +1,210 @@
+// Draft-tree construction around the FR-Spec head for gfx950: the tree bookkeeping of the
+// reference's draft() (src/model/minicpm4/minicpm4_eagle.cuh:319-393) as three single-workgroup
+// kernels that keep all state on the device:
+//   begin  -- d = 0: record the first k candidates, init_tree (src/model/eagle.cuh:91-93);
+//   extend -- d >= 1: cumsum (eagle.cuh:103-106), history append, top-k over k*k -> k,
+//             set_parent / update_tree (eagle.cuh:95-101), id remap (eagle.cuh:121-127) and the row
+//             indices the hidden-state gather needs (remap_hidden, eagle.cuh:108-115);
+//   finish -- top-(T-1) over the whole history, build_dynamic_tree (eagle.cuh:188-214) and the id
+//             remap of the chosen nodes.
+// The reference spends about ten launches and a device-to-host copy per iteration on these; here
+// the prefix length is read from device memory, so building the tree needs no host round trip.
+// Selection uses the same 64-bit keys as the top-k kernels (value descending, lower index first).
+#include "common.h"
+#include "topk_keys.h"
+
+namespace cpmcu {
+namespace {
+
+constexpr int kMaxK = 32;        // topk_per_iter
+constexpr int kMaxTried = kTopkThreads * kPerThread;  // history entries one workgroup can rank
+
+struct DraftState {
+    uint16_t* tried_val;    // [total] fp16 bits
+    int32_t* tried_pos;     // [total]
+    int32_t* tried_parent;  // [k * (num_iter - 1)]
+    uint64_t* mask;         // [k] eagle_mask_2d
+    uint16_t* cum;          // [k] running log-prob of the k live nodes
+};
+
+__host__ __device__ inline size_t draft_state_layout(int k, int num_iter, size_t* off_pos, size_t* off_parent, size_t* off_mask,
+                                                     size_t* off_cum) {
+    const size_t total = (size_t)k + (size_t)(num_iter - 1) * k * k;
+    size_t o = (total * 2 + 15) / 16 * 16;
+    *off_pos = o;
+    o += total * 4;
+    *off_parent = o;
+    o += (size_t)k * (num_iter > 1 ? num_iter - 1 : 1) * 4;
+    o = (o + 15) / 16 * 16;
+    *off_mask = o;
+    o += (size_t)k * 8;
+    *off_cum = o;
+    o += (size_t)k * 2;
+    return (o + 255) / 256 * 256;
+}
+
+inline DraftState draft_state(void* state, int k, int num_iter) {
+    size_t op, opar, om, oc;
+    draft_state_layout(k, num_iter, &op, &opar, &om, &oc);
+    char* b = (char*)state;
+    return DraftState{(uint16_t*)b, (int32_t*)(b + op), (int32_t*)(b + opar), (uint64_t*)(b + om), (uint16_t*)(b + oc)};
+}
+
+__global__ void draft_begin_kernel(DraftState s, int k, const uint16_t* val, const int32_t* pos, const int32_t* remap,
+                                   int32_t* next_ids, uint64_t* mask_out) {
+    const int i = threadIdx.x;
+    if (i >= k) return;
+    s.tried_val[i] = val[i];
+    s.tried_pos[i] = pos[i];
+    s.cum[i] = val[i];
+    s.mask[i] = 1ull << i;
+    if (mask_out) mask_out[i] = 1ull << i;
+    next_ids[i] = remap ? remap[pos[i]] : pos[i];
+}
+
+__global__ __launch_bounds__(kTopkThreads) void draft_extend_kernel(DraftState s, int k, int d, uint16_t* val, const int32_t* pos,
+                                                                    const int32_t* remap, int32_t* next_ids, int32_t* parent_rows,
+                                                                    uint64_t* mask_out) {
+    __shared__ int32_t s_sel[kMaxK];
+    __shared__ uint16_t s_val[kMaxK];
+    __shared__ uint64_t s_oldmask[kMaxK];
+    const int tid = threadIdx.x;
+    const int kk = k * k;
+    const int base = k + (d - 1) * kk;
+    if (tid < k) s_oldmask[tid] = s.mask[tid];
+    uint64_t keys[kPerThread];
+#pragma unroll
+    for (int e = 0; e < kPerThread; ++e) {
+        const int x = tid * kPerThread + e;
+        uint64_t key = 0;
+        if (x < kk) {
+            const float c = (float)__builtin_bit_cast(f16, s.cum[x / k]);
+            const f16 v = (f16)((float)__builtin_bit_cast(f16, val[x]) + c);  // half += half, rounded to half
+            const uint16_t bits = __builtin_bit_cast(uint16_t, v);
+            val[x] = bits;
+            s.tried_val[base + x] = bits;
+            s.tried_pos[base + x] = pos[x];
+            key = make_key(bits, x);
+        }
+        keys[e] = key;
+    }
+    select_topk(keys, k, [&](int round, uint64_t key) {
+        s_sel[round] = key_index(key);
+        s_val[round] = key_bits(key);
+    });
+    // select_topk ends with a barrier: s_sel / s_val / s_oldmask are visible
+    if (tid < k) {
+        const int p2 = s_sel[tid];
+        s.tried_parent[(d - 1) * k + tid] = p2 + base;
+        const uint64_t m = s_oldmask[p2 / k] | (1ull << (k * d + tid));
+        s.mask[tid] = m;
+        if (mask_out) mask_out[tid] = m;
+        if (parent_rows) parent_rows[tid] = p2 / k;
+        const int32_t fr = pos[p2];
+        next_ids[tid] = remap ? remap[fr] : fr;
+        s.cum[tid] = s_val[tid];
+    }
+}
+
+__global__ __launch_bounds__(kTopkThreads) void draft_finish_kernel(DraftState s, int k, int num_iter, int T, const int32_t* cache_length,
+                                                                    const int32_t* remap, int32_t* ids_out, int32_t* tree_pos,
+                                                                    uint64_t* tree_mask, int32_t* tree_parent) {
+    __shared__ int32_t s_sel[kMaxTree];
+    __shared__ int32_t s_reverse[kMaxTried];
+    const int tid = threadIdx.x;
+    const int kk = k * k;
+    const int total = k + (num_iter - 1) * kk;
+    const int W = (T + 63) / 64;
+    uint64_t keys[kPerThread];
+#pragma unroll
+    for (int e = 0; e < kPerThread; ++e) {
+        const int x = tid * kPerThread + e;
+        keys[e] = x < total ? make_key(s.tried_val[x], x) : 0;
+    }
+    for (int x = tid; x < total; x += kTopkThreads) s_reverse[x] = 0;  // a parent that was not selected maps to the root
+    select_topk(keys, T - 1, [&](int round, uint64_t key) { s_sel[round] = key_index(key); });
+    if (tid >= 1 && tid < T) {
+        const int p = s_sel[tid - 1];
+        s_reverse[p] = tid;
+        const int32_t fr = s.tried_pos[p];
+        ids_out[tid] = remap ? remap[fr] : fr;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        const int P = cache_length[0];
+        for (int w = 0; w < W; ++w) tree_mask[w] = 0;
+        tree_mask[0] = 1;
+        tree_pos[0] = P;
+        tree_parent[0] = 0;
+        for (int i = 1; i < T; ++i) {  // parents come before children: cumulative log-probs fall along a path
+            int p = s_sel[i - 1];
+            tree_pos[i] = P + (p < k ? 1 : (p - k) / kk + 2);
+            if (p < k) {
+                p = -1;
+            } else {
+                p -= k;
+                p = p < kk ? p / k : s.tried_parent[(p - kk) / k];
+            }
+            const int parent = p == -1 ? 0 : s_reverse[p];
+            tree_parent[i] = parent;
+            for (int w = 0; w < W; ++w) tree_mask[(size_t)i * W + w] = tree_mask[(size_t)parent * W + w];
+            tree_mask[(size_t)i * W + (i >> 6)] |= 1ull << (i & 63);
+        }
+    }
+}
+
+int check_shape(const char* what, int k, int num_iter) {
+    CPMCU_CHECK_ARG(k >= 1 && k <= kMaxK, "%s: k=%d outside [1, %d]", what, k, kMaxK);
+    CPMCU_CHECK_ARG(num_iter >= 1 && k * num_iter <= 64, "%s: k * num_iter = %d does not fit the 64-bit draft mask", what, k * num_iter);
+    CPMCU_CHECK_ARG((size_t)k + (size_t)(num_iter - 1) * k * k <= (size_t)kMaxTried, "%s: history of %d entries exceeds %d", what,
+                    k + (num_iter - 1) * k * k, kMaxTried);
+    return CPMCU_OK;
+}
+
+}  // namespace
+}  // namespace cpmcu
+
+using namespace cpmcu;
+
+extern "C" size_t cpmcu_draft_tree_state_bytes(int k, int num_iter) {
+    if (k < 1 || num_iter < 1) return 0;
+    size_t a, b, c, d;
+    return draft_state_layout(k, num_iter, &a, &b, &c, &d);
+}
+
+extern "C" int cpmcu_draft_tree_begin(void* state, int k, int num_iter, const void* topk_val, const int32_t* topk_pos,
+                                      const int32_t* token_id_remap, int32_t* next_ids, uint64_t* draft_mask, void* stream) {
+    CPMCU_CHECK_ARG(state && topk_val && topk_pos && next_ids, "draft_tree_begin: null pointer argument");
+    if (int rc = check_shape("draft_tree_begin", k, num_iter)) return rc;
+    hipLaunchKernelGGL(draft_begin_kernel, dim3(1), dim3(64), 0, resolve_stream(stream), draft_state(state, k, num_iter), k,
+                       (const uint16_t*)topk_val, topk_pos, token_id_remap, next_ids, draft_mask);
+    CPMCU_LAUNCH_CHECK();
+    return CPMCU_OK;
+}
+
+extern "C" int cpmcu_draft_tree_extend(void* state, int k, int num_iter, int d, void* topk_val, const int32_t* topk_pos,
+                                       const int32_t* token_id_remap, int32_t* next_ids, int32_t* parent_rows,
+                                       uint64_t* draft_mask, void* stream) {
+    CPMCU_CHECK_ARG(state && topk_val && topk_pos && next_ids, "draft_tree_extend: null pointer argument");
+    if (int rc = check_shape("draft_tree_extend", k, num_iter)) return rc;
+    CPMCU_CHECK_ARG(d >= 1 && d < num_iter, "draft_tree_extend: iteration d=%d outside [1, %d)", d, num_iter);
+    hipLaunchKernelGGL(draft_extend_kernel, dim3(1), dim3(kTopkThreads), 0, resolve_stream(stream), draft_state(state, k, num_iter), k, d,
+                       (uint16_t*)topk_val, topk_pos, token_id_remap, next_ids, parent_rows, draft_mask);
+    CPMCU_LAUNCH_CHECK();
+    return CPMCU_OK;
+}
+
+extern "C" int cpmcu_draft_tree_finish(void* state, int k, int num_iter, int tree_size, const int32_t* cache_length,
+                                       const int32_t* token_id_remap, int32_t* tree_draft_ids, int32_t* tree_position_ids,
+                                       uint64_t* tree_attn_mask, int32_t* tree_parent, void* stream) {
+    CPMCU_CHECK_ARG(state && cache_length && tree_draft_ids && tree_position_ids && tree_attn_mask && tree_parent,
+                    "draft_tree_finish: null pointer argument");
+    if (int rc = check_shape("draft_tree_finish", k, num_iter)) return rc;
+    const int total = k + (num_iter - 1) * k * k;
+    CPMCU_CHECK_ARG(tree_size >= 2 && tree_size <= kMaxTree && tree_size - 1 <= total,
+                    "draft_tree_finish: tree_size=%d outside [2, min(%d, history %d + 1)]", tree_size, kMaxTree, total);
+    hipLaunchKernelGGL(draft_finish_kernel, dim3(1), dim3(kTopkThreads), 0, resolve_stream(stream), draft_state(state, k, num_iter), k,
+                       num_iter, tree_size, cache_length, token_id_remap, tree_draft_ids, tree_position_ids, tree_attn_mask, tree_parent);
+    CPMCU_LAUNCH_CHECK();
+    return CPMCU_OK;
+}

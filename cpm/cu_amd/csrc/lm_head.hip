@@ -321,6 +321,7 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_chunked_kernel(HeadPar
     constexpr int PR = KC / 8;               // 16-byte pieces per hidden row chunk
     constexpr int NINST = BUF / 1024 / kHeadWaves;  // 1 KB DMA instructions per wave and chunk
     static_assert(NP % NBUF == 0, "the W buffers rotate with the row-block index");
+    static_assert(NBUF >= 2 && NBUF <= 4 && 3 * PD <= 63, "vmcnt immediates below");
     __shared__ __attribute__((aligned(1024))) char lds[2 * BUF];
     __shared__ float red_a[kHeadWaves][NB * 16];
     __shared__ float red_b[kHeadWaves][NB * 16];
@@ -356,9 +357,11 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_chunked_kernel(HeadPar
         }
     };
     auto row_block = [&](int pass) { return (pass * kHeadWaves + wave) * G + c; };
+    int groups_since_dma = 0;  // W groups requested after the newest hidden chunk request
     auto load_w = [&](int q, int pl, f16x8* buf) {
         const int pass = (q / nch) * NP + pl;
         if (pass >= p.npasses) return;
+        ++groups_since_dma;
         int row = row_block(pass) * 16 + l16;
         row = row < V ? row : V - 1;  // clamp: rows past the end are computed and discarded
         const f16* src = p.w + (size_t)row * H + chunk_of(q) * KC + kgp * 8;
@@ -390,9 +393,16 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_chunked_kernel(HeadPar
 #pragma unroll
                     for (int r = 0; r < 4; ++r) acc[pl][nb][r] = 0.f;
         }
-        // Chunk q was requested one iteration ago; the only memory operations issued after it that
-        // may still be in flight are the loads of the NBUF - 1 W groups prefetched last (returns are in order).
-        asm volatile("s_waitcnt vmcnt(%0)" : : "n"((NBUF - 1) * PD) : "memory");
+        // Chunk q was requested one iteration ago.  Memory operations return in order, so it has landed
+        // once at most the W groups requested after it -- and never more than the NBUF - 1 that are
+        // prefetched ahead -- are still in flight.  (Row blocks past the end request nothing, so the
+        // number of groups behind the chunk varies.)
+        switch (groups_since_dma < NBUF - 1 ? groups_since_dma : NBUF - 1) {
+            case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+            case 1: asm volatile("s_waitcnt vmcnt(%0)" : : "n"(PD) : "memory"); break;
+            case 2: asm volatile("s_waitcnt vmcnt(%0)" : : "n"(2 * PD) : "memory"); break;
+            default: asm volatile("s_waitcnt vmcnt(%0)" : : "n"(3 * PD) : "memory"); break;
+        }
         if (p.apply_scale) {  // fp16 pre-scale of the hidden rows (src/model/linear.cuh:82-101): own pieces, in place
 #pragma unroll
             for (int j = 0; j < NINST; ++j) {
@@ -404,7 +414,10 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_chunked_kernel(HeadPar
             }
         }
         __syncthreads();  // chunk q visible to all waves; all waves are done with the other buffer
-        if (q + 1 < total_q) issue_hidden(q + 1);
+        if (q + 1 < total_q) {
+            issue_hidden(q + 1);
+            groups_since_dma = 0;
+        }
         const char* base = lds + (q & 1) * BUF + l16 * ROWB + xl;
 #pragma unroll
         for (int pl = 0; pl < NP; ++pl) {

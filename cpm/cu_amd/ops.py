@@ -164,3 +164,50 @@ def kv_compact(cache, pred, gt, cache_length, best, max_accept):
     """fix_kv_cache (src/model/tree_drafter.cuh:48-77) on every layer of the paged cache."""
     _lib().kv_compact(_ptr(cache.k_ptrs), _ptr(cache.v_ptrs), cache.num_layers, _ptr(cache.block_table), cache.Hkv,
                       _ptr(pred), _ptr(gt), _ptr(cache_length), _ptr(best), int(max_accept), _stream())
+
+
+class DraftTree:
+    """Tree bookkeeping of the drafter (src/model/minicpm4/minicpm4_eagle.cuh:319-393) on the device.
+
+    One object per draft model; ``begin`` / ``extend`` / ``finish`` are one kernel each and never
+    synchronise, so a whole draft can be enqueued (or graph-captured) without a host round trip.
+    """
+
+    def __init__(self, k, num_iter, token_id_remap=None, device="cuda"):
+        self.k, self.num_iter = int(k), int(num_iter)
+        self.remap = token_id_remap
+        nbytes = _lib().raw.cpmcu_draft_tree_state_bytes(self.k, self.num_iter)
+        self.state = torch.zeros(max(nbytes, 256), dtype=torch.uint8, device=device)
+        self.next_ids = torch.empty(self.k, dtype=torch.int32, device=device)
+        self.parent_rows = torch.empty(self.k, dtype=torch.int32, device=device)
+        self.draft_mask = torch.empty(self.k, dtype=torch.int64, device=device)
+
+    def begin(self, topk_val, topk_pos):
+        """topk_val fp16[k], topk_pos int32[k] (first row). Returns next_ids [k]."""
+        assert topk_val.dtype == torch.float16 and topk_pos.dtype == torch.int32 and topk_val.numel() == self.k
+        _lib().draft_tree_begin(_ptr(self.state), self.k, self.num_iter, _ptr(topk_val), _ptr(topk_pos), _ptr(self.remap),
+                                _ptr(self.next_ids), _ptr(self.draft_mask), _stream())
+        return self.next_ids
+
+    def extend(self, d, topk_val, topk_pos):
+        """topk_val fp16[k,k] (cumulated in place), topk_pos int32[k,k] of iteration d >= 1.
+        Returns (next_ids [k], parent_rows [k], draft_mask [k])."""
+        assert topk_val.dtype == torch.float16 and topk_pos.dtype == torch.int32 and topk_val.numel() == self.k * self.k
+        _lib().draft_tree_extend(_ptr(self.state), self.k, self.num_iter, int(d), _ptr(topk_val), _ptr(topk_pos), _ptr(self.remap),
+                                 _ptr(self.next_ids), _ptr(self.parent_rows), _ptr(self.draft_mask), _stream())
+        return self.next_ids, self.parent_rows, self.draft_mask
+
+    def finish(self, tree_size, cache_length, tree_draft_ids=None):
+        """cache_length int32[1] on the device = P.  Returns (ids [T] -- entry 0 untouched --, positions [T],
+        mask [T, W] as int64 bit patterns, parent [T])."""
+        T = int(tree_size)
+        dev = self.state.device
+        W = mask_words(T)
+        if tree_draft_ids is None:
+            tree_draft_ids = torch.full((T,), -1, dtype=torch.int32, device=dev)
+        pos = torch.empty(T, dtype=torch.int32, device=dev)
+        mask = torch.empty((T, W), dtype=torch.int64, device=dev)
+        parent = torch.empty(T, dtype=torch.int32, device=dev)
+        _lib().draft_tree_finish(_ptr(self.state), self.k, self.num_iter, T, _ptr(cache_length), _ptr(self.remap),
+                                 _ptr(tree_draft_ids), _ptr(pos), _ptr(mask), _ptr(parent), _stream())
+        return tree_draft_ids, pos, mask, parent

@@ -166,3 +166,17 @@ CONFIGS = {
     "c4_verify_128k": dict(layers=32, prefix=131072, T=60, num_iter=6, topk=10, seed=0),
     "c5_wide_32k": dict(layers=32, prefix=32768, T=128, num_iter=8, topk=16, seed=0),
 }
+
+
+def draft_topk_rows(n, k, vocab, seed, stream=0, dyadic=False):
+    """Synthetic top-k output of the draft head for n rows: log-probs <= 0 in descending order
+    (fp16) and distinct positions per row.  dyadic=True draws multiples of 1/64 in (-4, 0], whose
+    sums along a draft path stay exact in fp16."""
+    g = rng(seed, 200 + stream)
+    if dyadic:
+        val = -(g.integers(0, 256, size=(n, k)).astype(np.float32) / 64.0)
+    else:
+        val = -np.abs(g.standard_normal((n, k)).astype(np.float32)) * 2.0
+    val = -np.sort(-val, axis=1)
+    pos = np.stack([g.choice(vocab, size=k, replace=False) for _ in range(n)]).astype(np.int32)
+    return val.astype(np.float16), pos

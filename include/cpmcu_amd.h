@@ -260,6 +260,35 @@ int cpmcu_kv_compact(void* const* k_pools, void* const* v_pools, int num_layers,
                      int Hkv, int32_t* pred, const int32_t* gt, const int32_t* cache_length,
                      const int32_t* best, int max_accept, void* stream);
 
+/* ---- Draft-tree construction around the FR-Spec head (the tree bookkeeping of draft()) ----
+ * src/model/minicpm4/minicpm4_eagle.cuh:319-393 with src/model/eagle.cuh:91-106,121-127,188-214.
+ * k = topk_per_iter (<= 32), num_iter iterations (k * num_iter <= 64: the draft mask is one
+ * uint64 per live node, as in the reference).  `state` is a caller-owned device buffer of
+ * cpmcu_draft_tree_state_bytes(k, num_iter) bytes that holds tried_history_val / _pos / _parent,
+ * eagle_mask_2d and the running log-probs between the calls of one draft.
+ *   begin  (d = 0, :319-332): topk_val fp16[k] / topk_pos int32[k] = top-k of the first row's
+ *          log-probs.  next_ids int32[k] out: the ids to embed next (mapped through
+ *          token_id_remap unless it is NULL).  draft_mask uint64[k] out (may be NULL).
+ *   extend (d >= 1, :367-382): topk_val fp16[k][k] (in/out: the row's running log-prob is added,
+ *          rounded to fp16 -- cumsum, eagle.cuh:103-106) / topk_pos int32[k][k].  Out: next_ids
+ *          [k], parent_rows int32[k] (row of the previous hidden states each new node continues:
+ *          remap_hidden's index, may be NULL), draft_mask [k] for the next draft-layer attention.
+ *   finish (:385-393): selects the tree_size - 1 best candidates of the history and writes
+ *          tree_draft_ids[1..tree_size) (entry 0, the root token, is the caller's),
+ *          tree_position_ids [tree_size] (P + depth; P read from the device scalar
+ *          cache_length[0] -- the reference copies it to the host first, :305),
+ *          tree_attn_mask [tree_size][ceil(tree_size/64)], tree_parent [tree_size].
+ * Ordering everywhere: value descending, equal values -> lower index (src/model/topk.cuh:17). */
+size_t cpmcu_draft_tree_state_bytes(int k, int num_iter);
+int cpmcu_draft_tree_begin(void* state, int k, int num_iter, const void* topk_val, const int32_t* topk_pos,
+                           const int32_t* token_id_remap, int32_t* next_ids, uint64_t* draft_mask, void* stream);
+int cpmcu_draft_tree_extend(void* state, int k, int num_iter, int d, void* topk_val, const int32_t* topk_pos,
+                            const int32_t* token_id_remap, int32_t* next_ids, int32_t* parent_rows,
+                            uint64_t* draft_mask, void* stream);
+int cpmcu_draft_tree_finish(void* state, int k, int num_iter, int tree_size, const int32_t* cache_length,
+                            const int32_t* token_id_remap, int32_t* tree_draft_ids, int32_t* tree_position_ids,
+                            uint64_t* tree_attn_mask, int32_t* tree_parent, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

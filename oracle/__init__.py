@@ -44,6 +44,9 @@ def _load():
         "orc_argmax": (None, [c_p, i32, i32, c_p]),
         "orc_tree_accept": (i32, [i32, i32, c_p, c_p, c_p, i32, c_p, c_p, c_p, c_p]),
         "orc_kv_compact": (None, [c_p, i32, i32, i32, i32, c_p, c_p, c_p]),
+        "orc_draft_tree_begin": (None, [i32, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p]),
+        "orc_draft_tree_extend": (None, [i32, i32, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p]),
+        "orc_draft_tree_finish": (None, [i32, i32, i32, i32, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p]),
     }
     for name, (res, args) in sigs.items():
         fn = getattr(lib, name)
@@ -199,3 +202,46 @@ def kv_compact(caches, P, path, gt):
     ids = np.empty(a, np.int32)
     _lib.orc_kv_compact(ptrs, len(caches), row_halves, int(P), a, _p(path), _p(gt), _p(ids))
     return ids
+
+
+class DraftTree:
+    """Tree bookkeeping of the drafter (src/model/minicpm4/minicpm4_eagle.cuh:319-393) on host arrays."""
+
+    def __init__(self, k, num_iter, token_id_remap=None):
+        self.k, self.num_iter = int(k), int(num_iter)
+        total = k + (num_iter - 1) * k * k
+        self.remap = None if token_id_remap is None else _c(token_id_remap, np.int32)
+        self.tried_val = np.zeros(total, np.float16)
+        self.tried_pos = np.zeros(total, np.int32)
+        self.tried_parent = np.zeros(max(1, k * (num_iter - 1)), np.int32)
+        self.cum = np.zeros(k, np.float16)
+        self.mask = np.zeros(k, np.uint64)
+
+    def begin(self, val, pos):
+        """val, pos [k] -> next_ids [k]."""
+        val, pos = _c(val, np.float16), _c(pos, np.int32)
+        ids = np.empty(self.k, np.int32)
+        _lib.orc_draft_tree_begin(self.k, _p(val), _p(pos), _p(self.remap), _p(self.tried_val), _p(self.tried_pos),
+                                  _p(self.cum), _p(self.mask), _p(ids))
+        return ids
+
+    def extend(self, d, val, pos):
+        """val, pos [k, k] of iteration d >= 1 -> (next_ids [k], parent_rows [k], cumulated val [k, k])."""
+        val = np.array(val, dtype=np.float16, order="C", copy=True)
+        pos = _c(pos, np.int32)
+        ids = np.empty(self.k, np.int32)
+        rows = np.empty(self.k, np.int32)
+        _lib.orc_draft_tree_extend(self.k, int(d), _p(val), _p(pos), _p(self.remap), _p(self.tried_val), _p(self.tried_pos),
+                                   _p(self.tried_parent), _p(self.cum), _p(self.mask), _p(ids), _p(rows))
+        return ids, rows, val
+
+    def finish(self, T, P):
+        """-> (ids [T] with ids[0] = -1, positions [T], mask [T, W], parent [T])."""
+        W = (T + 63) // 64
+        ids = np.full(T, -1, np.int32)
+        tpos = np.empty(T, np.int32)
+        tmask = np.zeros((T, W), np.uint64)
+        tpar = np.empty(T, np.int32)
+        _lib.orc_draft_tree_finish(self.k, self.num_iter, int(T), int(P), _p(self.remap), _p(self.tried_val), _p(self.tried_pos),
+                                   _p(self.tried_parent), _p(ids), _p(tpos), _p(tmask), _p(tpar))
+        return ids, tpos, tmask, tpar

@@ -349,4 +349,76 @@ void orc_kv_compact(uint16_t* const* caches, int num_caches, int row_halves, int
         for (int d = 0; d < a; ++d) ids_out[d] = gt[path[d]];  // :74-76
 }
 
+// f1 -- d = 0 of draft(): src/model/minicpm4/minicpm4_eagle.cuh:319-332, init_tree src/model/eagle.cuh:91-93
+void orc_draft_tree_begin(int k, const uint16_t* val, const int32_t* pos, const int32_t* token_id_remap,
+                          uint16_t* tried_val, int32_t* tried_pos, uint16_t* cum, uint64_t* mask, int32_t* next_ids) {
+    for (int i = 0; i < k; ++i) {
+        tried_val[i] = val[i];                                     // :323
+        tried_pos[i] = pos[i];                                     // :324
+        next_ids[i] = token_id_remap ? token_id_remap[pos[i]] : pos[i];  // :325-329
+        cum[i] = val[i];                                           // :330 topk_func_2->topk_val
+        mask[i] = 1ull << i;                                       // eagle.cuh:92
+    }
+}
+
+// f1 -- iteration d >= 1: src/model/minicpm4/minicpm4_eagle.cuh:367-382
+void orc_draft_tree_extend(int k, int d, uint16_t* val, const int32_t* pos, const int32_t* token_id_remap,
+                           uint16_t* tried_val, int32_t* tried_pos, int32_t* tried_parent, uint16_t* cum,
+                           uint64_t* mask, int32_t* next_ids, int32_t* parent_rows) {
+    const int kk = k * k;
+    const int base = k + (d - 1) * kk;
+    for (int i = 0; i < k; ++i)  // cumsum, eagle.cuh:103-106: half += half, rounded to half
+        for (int j = 0; j < k; ++j) val[i * k + j] = f2h(h2f(val[i * k + j]) + h2f(cum[i]));
+    for (int x = 0; x < kk; ++x) {  // :370-371
+        tried_val[base + x] = val[x];
+        tried_pos[base + x] = pos[x];
+    }
+    std::vector<uint16_t> v2(k);
+    std::vector<int32_t> p2(k);
+    orc_topk(val, 1, kk, k, v2.data(), p2.data());  // :372
+    std::vector<uint64_t> tmp(mask, mask + k);      // :374
+    for (int i = 0; i < k; ++i) {
+        tried_parent[(d - 1) * k + i] = p2[i] + base;               // :375, eagle.cuh:95-97
+        mask[i] = tmp[p2[i] / k] | (1ull << (k * d + i));           // :376, eagle.cuh:99-101
+        parent_rows[i] = p2[i] / k;                                 // :377 remap_hidden's row
+        const int32_t fr = pos[p2[i]];                              // :378-382, eagle.cuh:121-127
+        next_ids[i] = token_id_remap ? token_id_remap[fr] : fr;
+        cum[i] = v2[i];
+    }
+}
+
+// f1 -- final selection and tree: src/model/minicpm4/minicpm4_eagle.cuh:385-393, eagle.cuh:188-214
+void orc_draft_tree_finish(int k, int num_iter, int T, int P, const int32_t* token_id_remap,
+                           const uint16_t* tried_val, const int32_t* tried_pos, const int32_t* tried_parent,
+                           int32_t* ids_out, int32_t* tree_pos, uint64_t* tree_mask, int32_t* tree_parent) {
+    const int kk = k * k;
+    const int total = k + (num_iter - 1) * kk;
+    const int W = (T + 63) / 64;
+    std::vector<uint16_t> v3(T - 1);
+    std::vector<int32_t> sel(T - 1);
+    orc_topk(tried_val, 1, total, T - 1, v3.data(), sel.data());  // :385
+    std::vector<int32_t> reverse(total, 0);
+    for (int i = 1; i < T; ++i) reverse[sel[i - 1]] = i;          // eagle.cuh:191-193
+    for (int w = 0; w < W; ++w) tree_mask[w] = 0;
+    tree_mask[0] = 1;                                             // :196
+    tree_pos[0] = P;                                              // :197
+    tree_parent[0] = 0;
+    for (int i = 1; i < T; ++i) {
+        int p = sel[i - 1];
+        tree_pos[i] = P + (p < k ? 1 : (p - k) / kk + 2);         // :200
+        if (p < k) {
+            p = -1;
+        } else {
+            p -= k;
+            p = p < kk ? p / k : tried_parent[(p - kk) / k];      // :203-211
+        }
+        const int parent = p == -1 ? 0 : reverse[p];              // :212
+        tree_parent[i] = parent;
+        for (int w = 0; w < W; ++w) tree_mask[(size_t)i * W + w] = tree_mask[(size_t)parent * W + w];  // :214
+        tree_mask[(size_t)i * W + (i >> 6)] |= 1ull << (i & 63);  // :201
+        const int32_t fr = tried_pos[sel[i - 1]];                 // :389-393
+        ids_out[i] = token_id_remap ? token_id_remap[fr] : fr;
+    }
+}
+
 }  // extern "C"

@@ -136,6 +136,34 @@ int orc_tree_accept(int T, int mask_words, const int32_t* pred, const int32_t* g
 void orc_kv_compact(uint16_t* const* caches, int num_caches, int row_halves, int P, int a,
                     const int32_t* path, const int32_t* gt, int32_t* ids_out);
 
+/* ---- f1: draft-tree construction around the FR-Spec head ----
+ * src/model/minicpm4/minicpm4_eagle.cuh:319-393 (the tree bookkeeping of draft()), with
+ * src/model/eagle.cuh:91-101 (init_tree, set_parent, update_tree), :103-106 (cumsum),
+ * :121-127 (remap_id), :188-214 (build_dynamic_tree).  k = topk_per_iter.
+ * State arrays (caller-owned): tried_val/tried_pos [k + (num_iter-1) k^2], tried_parent
+ * [k (num_iter-1)], cum [k] (running log-prob of the k live nodes), mask [k] (eagle_mask_2d).
+ *   begin : d = 0 (:319-332).  val/pos [k] = top-k of the first row's log-probs.
+ *   extend: d >= 1 (:367-382).  val [k][k] (modified: += cum of its row, rounded to fp16),
+ *           pos [k][k]; outputs next_ids [k], parent_rows [k] (= selected / k, the row gather
+ *           of remap_hidden :376), updated cum, mask, tried_*.
+ *   finish: (:385-393) top-(T-1) of tried_val, build_dynamic_tree with pos_offset = P,
+ *           ids_out[1..T) = (remap of) tried_pos[selected]; ids_out[0] is left alone.
+ *           mask_words = ceil(T/64) words per mask row (the reference has one).
+ *           A selected node whose parent was not selected gets parent 0 (the reference reads an
+ *           uninitialised slot there; it cannot happen while log-probs are <= 0).
+ * token_id_remap may be NULL (frspec_vocab_size == vocab_size, :327-329,:378-382,:389-393).
+ * pinned by: an independent reconstruction with explicit node records (ancestor sets by
+ * walking parents, depths, exact cumulative sums on dyadic inputs), hand-worked 2-iteration
+ * case; parity with the reference's bits unpinned. */
+void orc_draft_tree_begin(int k, const uint16_t* val, const int32_t* pos, const int32_t* token_id_remap,
+                          uint16_t* tried_val, int32_t* tried_pos, uint16_t* cum, uint64_t* mask, int32_t* next_ids);
+void orc_draft_tree_extend(int k, int d, uint16_t* val, const int32_t* pos, const int32_t* token_id_remap,
+                           uint16_t* tried_val, int32_t* tried_pos, int32_t* tried_parent, uint16_t* cum,
+                           uint64_t* mask, int32_t* next_ids, int32_t* parent_rows);
+void orc_draft_tree_finish(int k, int num_iter, int T, int P, const int32_t* token_id_remap,
+                           const uint16_t* tried_val, const int32_t* tried_pos, const int32_t* tried_parent,
+                           int32_t* ids_out, int32_t* tree_pos, uint64_t* tree_mask, int32_t* tree_parent);
+
 #ifdef __cplusplus
 }
 #endif
