@@ -34,6 +34,8 @@
 //    land on the same XCD (workgroup id modulo 8) and share its L2.
 #include "common.h"
 
+#include <type_traits>
+
 namespace cpmcu {
 namespace {
 
@@ -52,6 +54,7 @@ constexpr int kKTileBytes = kTileN * kHeadDim * 2;  // 16 KB, row = one key (256
 constexpr int kVTileBytes = kHeadDim * kTileN * 2;  // 16 KB, row = one dim (128 B)
 constexpr int kStageBytes = kKTileBytes + kVTileBytes;
 constexpr int kMaxPagesPerSplit = 1024;
+constexpr int kVStageRows = 64;  // appended V rows staged in LDS ahead of their transposition
 constexpr int kMaxSplits = 64;
 constexpr int kXcds = 8;
 constexpr float kLazyLog2 = 8.f;  // slack of the lazily updated softmax reference, in log2 units
@@ -107,6 +110,12 @@ __device__ inline void load_to_lds16(const void* base, uint32_t byte_off, const 
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(byte_off), "s"(base), "s"(lds_addr) : "memory", "m0");
 }
 
+// Same, with a full per-lane address (used where lanes of one instruction read from different buffers).
+__device__ inline void load_to_lds16_v(const void* gptr, const char* lds_dst) {
+    const uint32_t lds_addr = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)lds_dst);
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gptr), "s"(lds_addr) : "memory", "m0");
+}
+
 // Per-thread byte offsets of its pieces inside a K tile and a V^T tile of a page (second piece of each:
 // + 32 keys = 8192 bytes for K, + 64 dims = 64 * 512 bytes for V^T; the swizzle terms do not change).
 __device__ inline uint32_t k_piece_off(int wave, int lane) {
@@ -133,6 +142,26 @@ __device__ inline void issue_tile(const AttnParams& p, int g, int tile, int page
     load_to_lds16(vbase + 64 * kPage * 2, voff, stage + kKTileBytes + (wave + kWaves) * 1024);
 }
 
+// The same for a tile that reaches the rows being appended: keys at positions [P, S) take their K
+// pieces straight from k_new (same 16-byte pieces, so the fused append costs K nothing); V^T comes
+// from the pool as usual and is patched in LDS afterwards.
+__device__ inline void issue_tile_append(const AttnParams& p, int g, int tile, int page, char* stage, int wave, int lane, uint32_t koff,
+                                         uint32_t voff, int P, int S) {
+    const int slot0 = (tile * kTileN) % kPage;
+    const char* kbase = reinterpret_cast<const char*>(p.k_pool + (((size_t)page * p.Hkv + g) * kPage + slot0) * kHeadDim);
+    const char* vbase = reinterpret_cast<const char*>(p.v_pool + ((size_t)page * p.Hkv + g) * kHeadDim * kPage + slot0);
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int key = h * 32 + wave * 4 + (lane >> 4);
+        const int c = tile * kTileN + key;
+        const int piece = (lane & 15) ^ (key & 15);
+        const char* src = kbase + h * (32 * kHeadDim * 2) + koff;
+        if (c >= P && c < S) src = reinterpret_cast<const char*>(p.k_new + ((size_t)(c - P) * p.Hkv + g) * kHeadDim + piece * 8);
+        load_to_lds16_v(src, stage + (wave + kWaves * h) * 1024);
+        load_to_lds16(vbase + h * (64 * kPage * 2), voff, stage + kKTileBytes + (wave + kWaves * h) * 1024);
+    }
+}
+
 template <int G>
 __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams p) {
     constexpr int kRowWaves = kWaves / G;
@@ -140,6 +169,7 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
     constexpr int kDepth = kStages / G - 1;  // iterations in flight behind the one being consumed
     __shared__ __attribute__((aligned(1024))) char ring[kStages * kStageBytes];
     __shared__ int32_t s_pages[kMaxPagesPerSplit];
+    __shared__ __attribute__((aligned(1024))) char vstage[kVStageRows * kHeadDim * 2];  // first appended V rows, row-major
 
     // XCD-aware work mapping: consecutive workgroup ids go to consecutive XCDs, so
     // id % 8 picks the XCD; all M-tiles of one (split, kv head) pair share an XCD.
@@ -193,8 +223,12 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
 
     // The split's tile range is fixed by the host-side bound, so the page ids can be fetched without
     // waiting for the device-side length; the length only clips the range.
-    const int t0 = (int)(((long long)split * p.ntiles_max) / p.num_splits);
-    const int t1_max = (int)(((long long)(split + 1) * p.ntiles_max) / p.num_splits);
+    // With the fused append the last split also patches the appended rows into its tiles, which costs
+    // about as much as an iteration: the partition counts two tiles' worth of extra work at the end
+    // of the stream, so that split gets fewer real tiles.
+    const int vtiles = p.ntiles_max + (p.k_new != nullptr && p.num_splits > 1 ? 2 : 0);
+    const int t0 = min((int)(((long long)split * vtiles) / p.num_splits), p.ntiles_max);
+    const int t1_max = min((int)(((long long)(split + 1) * vtiles) / p.num_splits), p.ntiles_max);
     const int pg0 = (t0 * kTileN) / kPage;
     if (t1_max > t0) {
         const int npg = ((t1_max * kTileN - 1) / kPage) - pg0 + 1;
@@ -217,7 +251,10 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
             if (i < n) {
                 const int tile = t0 + i;
                 const int page = __builtin_amdgcn_readfirstlane(s_pages[(tile * kTileN) / kPage - pg0]);
-                issue_tile(p, g, tile, page, ring + (i % kStages) * kStageBytes, wave_u, koff, voff);
+                if (p.k_new != nullptr && (tile + 1) * kTileN > P)
+                    issue_tile_append(p, g, tile, page, ring + (i % kStages) * kStageBytes, wave_u, lane, koff, voff, P, S);
+                else
+                    issue_tile(p, g, tile, page, ring + (i % kStages) * kStageBytes, wave_u, koff, voff);
             }
         }
     };
@@ -236,6 +273,17 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
     float m_ref = -INFINITY;
     float l_run = 0.f;        // this lane's share of the row sum
 
+    // A workgroup whose range reaches the tree region transposes the appended V rows into its tiles.
+    // The first kVStageRows of them are requested into LDS now -- the oldest loads, so the first wait
+    // below covers them -- and the latency of reading v_new stays off the critical path.
+    if (p.k_new != nullptr && (t0 + n) * kTileN > P) {
+#pragma unroll
+        for (int qq = 0; qq < 2; ++qq) {
+            const int inst = wave_u + kWaves * qq;
+            const int r = min(inst * 4 + (lane >> 4), p.T - 1);
+            load_to_lds16_v(p.v_new + ((size_t)r * p.Hkv + g) * kHeadDim + (lane & 15) * 8, vstage + inst * 1024);
+        }
+    }
 #pragma unroll
     for (int d = 0; d <= kDepth; ++d)
         if (d < niter) issue_iter(d);
@@ -280,48 +328,57 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
                 if (ie >= n) continue;
                 char* st = ring + (ie % kStages) * kStageBytes;
                 const bool append = p.k_new != nullptr && ce + kTileN > P;
-                if (append) {
-                    // K rows: 16 pieces of 16 bytes per key
+                const int pg = append ? s_pages[(ce + kTileN - 1) / kPage - pg0] : 0;  // a tile lies inside one page
+                if (append && mt == 0) {
+                    // K is already in the tile (fetched from k_new): the M-tile-0 workgroup copies the new
+                    // rows' 16-byte pieces on to the pool.
                     for (int x = tid; x < kTileN * 16; x += kThreads) {
                         const int key = x >> 4, piece = x & 15;
                         const int c = ce + key;
-                        if (c >= P && c < S) {
-                            const f16x8 val = *reinterpret_cast<const f16x8*>(p.k_new + ((size_t)(c - P) * p.Hkv + g) * kHeadDim + piece * 8);
-                            *reinterpret_cast<f16x8*>(st + k_lds_off(key, piece)) = val;
-                            if (mt == 0) {
-                                const int pg = s_pages[c / kPage - pg0];
-                                *reinterpret_cast<f16x8*>(p.k_pool_w + (((size_t)pg * p.Hkv + g) * kPage + c % kPage) * kHeadDim + piece * 8) = val;
-                            }
-                        }
+                        if (c >= P && c < S)
+                            *reinterpret_cast<f16x8*>(p.k_pool_w + (((size_t)pg * p.Hkv + g) * kPage + c % kPage) * kHeadDim + piece * 8) =
+                                *reinterpret_cast<const f16x8*>(st + k_lds_off(key, piece));
                     }
                 }
-                if (append) {
-                    // V rows: one 16-byte piece (8 dims) of one new row per thread, scattered into the
-                    // transposed tile (and pool) as 2-byte elements
-                    for (int x = tid; x < kTileN * 16; x += kThreads) {
-                        const int key = x >> 4, piece = x & 15;
-                        const int c = ce + key;
-                        if (c >= P && c < S) {
-                            const f16x8 val = *reinterpret_cast<const f16x8*>(p.v_new + ((size_t)(c - P) * p.Hkv + g) * kHeadDim + piece * 8);
-                            const int slot = v_slot16(key);  // storage slot of this token inside the tile
+                if (append || ce + kTileN > S) {
+                    // V^T, one 16-byte piece (8 token slots of one dim) per thread, read-modify-write:
+                    // slots of appended tokens take the value from the staged row-major copy (the
+                    // transposition), slots at or beyond S become zero, the others keep the pool's value.
+                    // Trees of more than kVStageRows nodes read the rows beyond the staging area from
+                    // v_new; the choice is uniform, so the usual case issues no global load here.
+                    auto patch_v = [&](auto all_staged_c) {
+                        constexpr bool kAllStaged = decltype(all_staged_c)::value;
+                        for (int x = tid; x < kHeadDim * 8; x += kThreads) {
+                            const int d = x & (kHeadDim - 1), sg = x >> 7;
+                            f16x8* pp = reinterpret_cast<f16x8*>(st + v_lds_off(d, sg));
+                            f16x8 cur = *pp;
+                            bool has_new = false;
+                            // all eight staged values are read unconditionally (clamped index) and selected
+                            // afterwards: conditional reads would each wait for their own LDS round trip
+                            f16 nv[8];
 #pragma unroll
-                            for (int e = 0; e < 8; ++e)
-                                *reinterpret_cast<f16*>(st + v_lds_off(piece * 8 + e, slot >> 3) + (slot & 7) * 2) = val[e];
-                            if (mt == 0) {
-                                const int pg = s_pages[c / kPage - pg0];
-                                f16* dst = p.v_pool_w + (((size_t)pg * p.Hkv + g) * kHeadDim + piece * 8) * kPage + v_slot16(c % kPage);
-#pragma unroll
-                                for (int e = 0; e < 8; ++e) dst[(size_t)e * kPage] = val[e];
+                            for (int j = 0; j < 8; ++j) {
+                                const int r = min(max(ce + v_slot16(sg * 8 + j) - P, 0), kAllStaged ? p.T - 1 : kVStageRows - 1);
+                                nv[j] = reinterpret_cast<const f16*>(vstage)[r * kHeadDim + d];
                             }
+#pragma unroll
+                            for (int j = 0; j < 8; ++j) {
+                                const int c = ce + v_slot16(sg * 8 + j);
+                                if (append && c >= P && c < S) {
+                                    if (kAllStaged || c - P < kVStageRows) cur[j] = nv[j];
+                                    else cur[j] = p.v_new[((size_t)(c - P) * p.Hkv + g) * kHeadDim + d];
+                                    has_new = true;
+                                } else if (c >= S) {
+                                    cur[j] = (f16)0.f;
+                                }
+                            }
+                            *pp = cur;
+                            if (has_new && mt == 0)  // the same 8 slots are 16 contiguous bytes of the pool's page row
+                                *reinterpret_cast<f16x8*>(p.v_pool_w + (((size_t)pg * p.Hkv + g) * kHeadDim + d) * kPage + ce % kPage + sg * 8) = cur;
                         }
-                    }
-                }
-                if (ce + kTileN > S) {
-                    for (int x = tid; x < kHeadDim * kTileN; x += kThreads) {
-                        const int d = x >> 6, slot = x & 63;
-                        if (ce + v_slot16(slot) >= S)
-                            *reinterpret_cast<f16*>(st + v_lds_off(d, slot >> 3) + (slot & 7) * 2) = (f16)0.f;
-                    }
+                    };
+                    if (p.T <= kVStageRows) patch_v(std::true_type{});
+                    else patch_v(std::false_type{});
                 }
             }
             __syncthreads();

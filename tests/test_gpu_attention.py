@@ -142,7 +142,8 @@ def test_kv_append_matches_logical_write(gpu):
 @pytest.mark.parametrize("P,T,splits", [(1024, 16, 0), (4096 - 23, 60, 0), (250, 60, 1), (0, 16, 1), (700, 128, 3), (63, 64, 2)])
 def test_fused_append_equals_append_then_attend(gpu, orc, P, T, splits):
     """Handing the tree rows' K/V to the attention kernel (fused copy_to_kvcache) must give the same
-    output as appending first, and must leave the same cache behind -- stale garbage at [P, S) included."""
+    output as appending first (up to the rounding of a different split partition), and must leave
+    exactly the same cache behind -- stale garbage at [P, S) included."""
     from cpm.cu_amd import ops
     from cpm.cu_amd.kvcache import PagedKVCache
     torch = gpu
@@ -169,7 +170,9 @@ def test_fused_append_equals_append_then_attend(gpu, orc, P, T, splits):
     out_b = ops.tree_attention(to_dev(torch, q), b, 0, kv_len, S, mask, num_splits=splits,
                                k_new=to_dev(torch, k[P:]), v_new=to_dev(torch, v[P:]))
     torch.cuda.synchronize()
-    assert torch.equal(out_a, out_b)
+    # the fused call partitions the KV stream differently (the appending split gets fewer tiles), so the
+    # two outputs agree to the fp16 rounding of the split partials, not bit for bit
+    assert_close_f16(to_np(out_b), to_np(out_a), "fused vs unfused append", atol=4e-3, rtol=4e-3)
     assert_close_f16(to_np(out_b), orc.tree_attention(q, k, v, tree.mask, P), "fused append attention")
     kb, vb = b.read_logical(0, 0, S)
     assert np.array_equal(to_np(kb).view(np.uint16), k.view(np.uint16))
