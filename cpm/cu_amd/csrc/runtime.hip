@@ -360,7 +360,7 @@ extern "C" int cpmcu_decode_attention(int layer, int input_length, int padded_le
     // KV append (src/model/attn.cuh:200) is fused into the attention kernel
     const uint64_t* mask = mask_2d ? (const uint64_t*)mask_2d : m.chain_mask;
     return cpmcu_tree_attention((const void*)q, m.k_pools[layer], m.v_pools[layer], m.block_table,
-                                (const int32_t*)cache_length, padded_length, (const void*)k_new, (const void*)v_new, mask, 1,
+                                (const int32_t*)cache_length, padded_length, (const void*)k_new, (const void*)v_new, mask, 1, 0,
                                 input_length, m.q_heads, m.kv_heads, 1.f / sqrtf((float)kHeadDim), (void*)out, m.attn_ws,
                                 m.attn_ws_bytes, 0, st);
 }

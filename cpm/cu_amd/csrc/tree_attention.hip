@@ -73,6 +73,7 @@ struct AttnParams {
     f16* v_pool_w;
     const uint64_t* mask;
     int mask_words;
+    int mask_k_range;  // trailing key columns the mask bits refer to (>= T; = T for the verify tree)
     int T, Hq, Hkv, group;
     int num_splits, num_mtiles, rows_pad;
     int ntiles_max;  // ceil(max_kv_len / 64): the split partition is fixed by the host-side bound
@@ -215,8 +216,10 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
         mw1 = ~0ull;
     }
     {
-        const uint64_t c0 = node >= 63 ? ~0ull : ((2ull << node) - 1ull);
-        const uint64_t c1 = node >= 127 ? ~0ull : (node < 64 ? 0ull : ((2ull << (node - 64)) - 1ull));
+        // mask column of the query's own key: the causal bound keeps columns up to and including it
+        const int own = p.mask_k_range - p.T + node;
+        const uint64_t c0 = own >= 63 ? ~0ull : ((2ull << own) - 1ull);
+        const uint64_t c1 = own >= 127 ? ~0ull : (own < 64 ? 0ull : ((2ull << (own - 64)) - 1ull));
         mw0 &= c0;
         mw1 &= c1;
     }
@@ -235,7 +238,8 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
         for (int i = tid; i < npg; i += kThreads) s_pages[i] = p.block_table[pg0 + i];
     }
     const int S = p.kv_len[0];
-    const int P = S - p.T;
+    const int P = S - p.T;              // the T query tokens are the last T keys
+    const int Pm = S - p.mask_k_range;  // first key column governed by the mask bits (mask.h: mask_k_begin)
     const int ntiles = (S + kTileN - 1) / kTileN;
     const int t1 = min(t1_max, ntiles);
     const int n = max(t1 - t0, 0);
@@ -407,11 +411,11 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
                 __builtin_amdgcn_sched_barrier(0);
             }
             // sacc[kb][r] is the score of key  c0 + kb*32 + 8*(r/4) + 4*hf + r%4  for query qcol.
-            if (c0 + kTileN > P) {  // tile touches tree columns or the end of the stream
+            if (c0 + kTileN > Pm) {  // tile touches masked columns or the end of the stream
                 // 64-bit visibility word of this tile for the lane's query: bit x <-> key c0 + x.  Prefix
                 // keys are visible; tree key P + j is visible iff bit j of the node's mask row is set
                 // (the causal bound already cleared every bit above the node, hence at or beyond T).
-                const int sh = P - c0;  // < 64 here; negative once the tile starts inside the tree
+                const int sh = Pm - c0;  // < 64 here; negative once the tile starts inside the masked range
                 uint64_t tmask;
                 if (sh >= 0) {
                     tmask = (mw0 << sh) | (sh > 0 ? ((1ull << sh) - 1ull) : 0ull);
@@ -671,15 +675,18 @@ extern "C" size_t cpmcu_tree_attention_workspace_bytes(int T, int Hq, int Hkv, i
 extern "C" int cpmcu_tree_attention(const void* q, void* k_pool, void* v_pool,
                                     const int32_t* block_table, const int32_t* kv_len, int max_kv_len,
                                     const void* k_new, const void* v_new,
-                                    const uint64_t* mask, int mask_words, int T, int Hq, int Hkv,
+                                    const uint64_t* mask, int mask_words, int mask_k_range, int T, int Hq, int Hkv,
                                     float scale, void* out, void* workspace, size_t workspace_bytes,
                                     int num_splits_override, void* stream) {
     CPMCU_CHECK_ARG(q && k_pool && v_pool && block_table && kv_len && out, "tree_attention: null pointer argument");
     CPMCU_CHECK_ARG(T >= 1 && T <= kMaxTree, "tree_attention: T=%d outside [1, %d]", T, kMaxTree);
     CPMCU_CHECK_ARG(Hkv >= 1 && Hq >= Hkv && Hq % Hkv == 0, "tree_attention: Hq=%d must be a multiple of Hkv=%d", Hq, Hkv);
     CPMCU_CHECK_ARG(max_kv_len >= T, "tree_attention: max_kv_len=%d < T=%d", max_kv_len, T);
-    CPMCU_CHECK_ARG(mask == nullptr || mask_words == ceil_div(T, 64) || (mask_words == 1 && T <= 64),
-                    "tree_attention: mask_words=%d does not match T=%d", mask_words, T);
+    if (mask_k_range == 0 || mask == nullptr) mask_k_range = T;
+    CPMCU_CHECK_ARG(mask_k_range >= T && mask_k_range <= kMaxTree && mask_k_range <= max_kv_len,
+                    "tree_attention: mask_k_range=%d outside [T=%d, min(%d, max_kv_len)]", mask_k_range, T, kMaxTree);
+    CPMCU_CHECK_ARG(mask == nullptr || mask_words == ceil_div(mask_k_range, 64) || (mask_words == 1 && mask_k_range <= 64),
+                    "tree_attention: mask_words=%d does not match mask_k_range=%d", mask_words, mask_k_range);
     CPMCU_CHECK_ARG(num_splits_override >= 0 && num_splits_override <= kMaxSplits,
                     "tree_attention: num_splits_override=%d outside [0, %d]", num_splits_override, kMaxSplits);
     const int group = Hq / Hkv;
@@ -696,6 +703,7 @@ extern "C" int cpmcu_tree_attention(const void* q, void* k_pool, void* v_pool,
     p.v_pool_w = (f16*)v_pool;
     p.mask = mask;
     p.mask_words = mask ? mask_words : 0;
+    p.mask_k_range = mask_k_range;
     p.T = T;
     p.Hq = Hq;
     p.Hkv = Hkv;

@@ -41,7 +41,7 @@ SIGNATURES = {
     "cpmcu_shutdown": (c_int, []),
     "cpmcu_kv_append": (c_int, [_P, _P, _P, _P, _P, _P, c_int, c_int, _P]),
     "cpmcu_tree_attention_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
-    "cpmcu_tree_attention": (c_int, [_P, _P, _P, _P, _P, c_int, _P, _P, _P, c_int, c_int, c_int, c_int, c_float, _P, _P, c_size_t, c_int, _P]),
+    "cpmcu_tree_attention": (c_int, [_P, _P, _P, _P, _P, c_int, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_float, _P, _P, c_size_t, c_int, _P]),
     "cpmcu_gather_rows": (c_int, [_P, _P, c_int, c_int, _P, _P]),
     "cpmcu_head_workspace_bytes": (c_size_t, [c_int, c_int]),
     "cpmcu_frspec_head_topk": (c_int, [_P, _P, _P, c_int, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, c_size_t, _P]),

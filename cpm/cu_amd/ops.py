@@ -53,12 +53,13 @@ def kv_append(cache, layer, k_new, v_new, kv_len):
 
 
 def tree_attention(q, cache, layer, kv_len, max_kv_len, mask=None, scale=None, num_splits=0, out=None,
-                   k_new=None, v_new=None):
+                   k_new=None, v_new=None, mask_k_range=0):
     """mha_fwd_kvcache with a tree mask (src/flash_attn/flash_api.hpp:292-392) on the paged cache.
 
     q [T, Hq, 128] fp16; kv_len int32[1] on the device = P + T; mask uint64 [T, W] or None (chain).
     k_new / v_new [T, Hkv, 128]: the tree rows' K/V; when given the kernel appends them to the cache
     itself (src/model/attn.cuh:200) instead of expecting them there.
+    mask_k_range (0 = T): number of trailing keys the mask bits refer to; k*d for the drafter's layers.
     """
     T, Hq, D = q.shape
     assert D == HEAD_DIM and q.dtype == torch.float16 and kv_len.dtype == torch.int32
@@ -77,7 +78,7 @@ def tree_attention(q, cache, layer, kv_len, max_kv_len, mask=None, scale=None, n
         assert k_new.dtype == torch.float16 and v_new.dtype == torch.float16
         assert k_new.numel() == T * cache.Hkv * HEAD_DIM and v_new.numel() == k_new.numel()
     _lib().tree_attention(_ptr(q), _ptr(cache.k[layer]), _ptr(cache.v[layer]), _ptr(cache.block_table), _ptr(kv_len),
-                          int(max_kv_len), _ptr(k_new), _ptr(v_new), _ptr(mask), W, T, Hq, cache.Hkv,
+                          int(max_kv_len), _ptr(k_new), _ptr(v_new), _ptr(mask), W, int(mask_k_range), T, Hq, cache.Hkv,
                           ctypes.c_float(scale), _ptr(out),
                           _ptr(ws), ws.numel(), int(num_splits), _stream())
     return out

@@ -187,15 +187,22 @@ size_t cpmcu_tree_attention_workspace_bytes(int T, int Hq, int Hkv, int max_kv_l
  *           itself: the rows are used for positions [*kv_len - T, *kv_len) and are
  *           written into the pools, so no separate cpmcu_kv_append call is needed.
  *           When NULL the rows must already be in the cache.
- *   mask [T][mask_words] uint64: bit j of row i = node i attends tree node j;
- *           NULL = causal chain.
+ *   mask [T][mask_words] uint64, mask_k_range: bit j of row i = query i attends the key at
+ *           position *kv_len - mask_k_range + j; keys before that are all visible, and the
+ *           causal bound (query i sees keys up to its own position *kv_len - T + i) applies
+ *           as well (src/flash_attn/src/mask.h:185-203).  mask_k_range = T (or 0, which means
+ *           T) is the verify tree (bit j = tree node j); mask_k_range = k * d > T is the
+ *           drafter's own attention over its previous d - 1 rounds of k draft tokens
+ *           (Mask(eagle_mask_2d, k, k * d), src/model/minicpm4/minicpm4_eagle.cuh:359).
+ *           mask = NULL: causal chain.  mask_words = ceil(mask_k_range / 64).
  *   scale: softmax scale (1/sqrt(128) in the reference, flash_api.hpp:360).
  *   workspace: device scratch of at least ..._workspace_bytes(), may be NULL
  *           when that is 0.
  *   num_splits_override: 0 = choose from max_kv_len; >0 forces the KV split count. */
 int cpmcu_tree_attention(const void* q, void* k_pool, void* v_pool, const int32_t* block_table,
                          const int32_t* kv_len, int max_kv_len, const void* k_new, const void* v_new,
-                         const uint64_t* mask, int mask_words, int T, int Hq, int Hkv, float scale, void* out,
+                         const uint64_t* mask, int mask_words, int mask_k_range, int T, int Hq, int Hkv, float scale,
+                         void* out,
                          void* workspace, size_t workspace_bytes, int num_splits_override, void* stream);
 
 /* remap_copy -- src/model/tree_drafter.cuh:79-86,103-107: dst[r][:] = src[remap[r]][:]. */

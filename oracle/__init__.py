@@ -34,7 +34,7 @@ def _load():
         "orc_f32_to_f16_sw": (None, [c_p, c_p, i64]),
         "orc_num_threads": (i32, []),
         "orc_set_num_threads": (None, [i32]),
-        "orc_tree_attention": (None, [c_p, c_p, c_p, c_p, i32, i32, i32, i32, i32, i32, f32, c_p, c_p]),
+        "orc_tree_attention": (None, [c_p, c_p, c_p, c_p, i32, i32, i32, i32, i32, i32, i32, f32, c_p, c_p]),
         "orc_gather_rows": (None, [c_p, c_p, i32, i32, c_p]),
         "orc_lm_head": (None, [c_p, c_p, i32, i32, i32, i32, f32, c_p]),
         "orc_log_softmax": (None, [c_p, i32, i32, c_p, c_p]),
@@ -93,8 +93,9 @@ def mask_words(T):
     return (T + 63) // 64
 
 
-def tree_attention(q, k, v, mask, P, scale=None, return_lse=False):
-    """q [T,Hq,D] f16; k,v [P+T,Hkv,D] f16; mask [T,W] uint64 -> out [T,Hq,D] f16."""
+def tree_attention(q, k, v, mask, P, scale=None, return_lse=False, mask_k_range=None):
+    """q [T,Hq,D] f16; k,v [P+T,Hkv,D] f16; mask [T,W] uint64 -> out [T,Hq,D] f16.
+    mask_k_range (default T): number of trailing key columns the mask bits refer to."""
     q = _c(q, np.float16)
     k = _c(k, np.float16)
     v = _c(v, np.float16)
@@ -107,7 +108,9 @@ def tree_attention(q, k, v, mask, P, scale=None, return_lse=False):
         scale = 1.0 / np.sqrt(D)
     out = np.empty((T, Hq, D), np.float16)
     lse = np.empty((T, Hq), np.float32)
-    _lib.orc_tree_attention(_p(q), _p(k), _p(v), _p(mask), T, P, Hq, Hkv, D, W,
+    R = T if mask_k_range is None else int(mask_k_range)
+    assert T <= R <= S and W == (R + 63) // 64 or (W == 1 and R <= 64)
+    _lib.orc_tree_attention(_p(q), _p(k), _p(v), _p(mask), T, P, Hq, Hkv, D, W, R,
                             ctypes.c_float(scale), _p(out), _p(lse))
     return (out, lse) if return_lse else out
 

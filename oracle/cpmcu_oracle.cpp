@@ -148,8 +148,9 @@ void orc_set_num_threads(int n) { g_threads = n; }
 // flash_fwd_kernel.h:1266,1610-1615, flash_api.hpp:103.
 void orc_tree_attention(const uint16_t* q, const uint16_t* k, const uint16_t* v,
                         const uint64_t* mask, int T, int P, int Hq, int Hkv, int D,
-                        int mask_words, float scale, uint16_t* out, float* lse) {
+                        int mask_words, int mask_k_range, float scale, uint16_t* out, float* lse) {
     const int S = P + T;
+    const int Pm = S - mask_k_range;  // mask.h: mask_k_begin = seqlen_k - mask_k_range
     const int group = Hq / Hkv;
     // flash_api.hpp:103  scale_softmax_log2 = softmax_scale * M_LOG2E
     const float scale_log2 = scale * (float)M_LOG2E;
@@ -177,10 +178,11 @@ void orc_tree_attention(const uint16_t* q, const uint16_t* k, const uint16_t* v,
                 float m = -std::numeric_limits<float>::infinity();
                 for (int c = 0; c < S; ++c) {
                     bool vis = true;
-                    if (c >= P) {  // mask.h:187,194-198 tree bit; :185-186 causal j <= i
-                        int j = c - P;
-                        vis = (j <= i) && ((mrow[j >> 6] >> (j & 63)) & 1ull);
+                    if (c >= Pm) {  // mask.h:187,194-198 mask bit of column c - mask_k_begin
+                        int j = c - Pm;
+                        vis = (mrow[j >> 6] >> (j & 63)) & 1ull;
                     }
+                    if (c > P + i) vis = false;  // mask.h:185-186,199-203 causal: col < row + 1 + seqlen_k - seqlen_q
                     if (vis) {
                         s[c] = dot_any(qf.data(), &kf[(size_t)c * D], D);
                         m = std::max(m, s[c]);

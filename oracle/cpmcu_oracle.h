@@ -48,9 +48,13 @@ void orc_set_num_threads(int n);
  *
  *   q    [T][Hq][D]          fp16
  *   k,v  [P+T][Hkv][D]       fp16, flat logical caches (row = token)
- *   mask [T][mask_words]     bit j of row i (word j/64, bit j%64): node i
- *                            attends tree node j.  The causal bound j <= i is
- *                            applied as well (mask.h:185-186,207-211).
+ *   mask [T][mask_words]     bit j of row i (word j/64, bit j%64): query i
+ *                            attends the key at column P + T - mask_k_range + j
+ *                            (mask_k_range >= T trailing columns are governed
+ *                            by the mask; = T for the verify tree, = k*d for
+ *                            the draft layers, minicpm4_eagle.cuh:359).  The
+ *                            causal bound column <= P + i is applied as well
+ *                            (mask.h:185-186,207-211).
  *   out  [T][Hq][D]          fp16
  *   lse  [T][Hq]             fp32 or NULL: max*scale + ln(sum)
  * One global row max (no blocking); the blocked/split evaluation of the
@@ -61,7 +65,7 @@ void orc_set_num_threads(int n);
  * mapping. */
 void orc_tree_attention(const uint16_t* q, const uint16_t* k, const uint16_t* v,
                         const uint64_t* mask, int T, int P, int Hq, int Hkv, int D,
-                        int mask_words, float scale, uint16_t* out, float* lse);
+                        int mask_words, int mask_k_range, float scale, uint16_t* out, float* lse);
 
 /* ---- a7: load-time gather of the frequency-ranked rows ----
  * src/model/tree_drafter.cuh:79-86,103-107:  dst[r][:] = src[remap[r]][:].

@@ -177,3 +177,41 @@ def test_fused_append_equals_append_then_attend(gpu, orc, P, T, splits):
     kb, vb = b.read_logical(0, 0, S)
     assert np.array_equal(to_np(kb).view(np.uint16), k.view(np.uint16))
     assert np.array_equal(to_np(vb).view(np.uint16), v.view(np.uint16))
+
+
+def _draft_layer_case(k, d, P0, seed):
+    """Inputs of the drafter's own attention in round d (src/model/minicpm4/minicpm4_eagle.cuh:359):
+    k queries (the newest k draft tokens) over P0 prefix tokens + k*d draft tokens, with
+    Mask(eagle_mask_2d, k, k*d): bit j of row i refers to draft token j of the k*d."""
+    import oracle
+    vocab = 300
+    t = oracle.DraftTree(k, d + 1)
+    v, p = synth.draft_topk_rows(1, k, vocab, seed, 0)
+    t.begin(v[0], p[0])
+    for it in range(1, d):
+        v, p = synth.draft_topk_rows(k, k, vocab, seed, it)
+        t.extend(it, v, p)
+    mask = t.mask.copy().reshape(k, 1)  # the mask the round-d attention uses: bits over k*d columns
+    S = P0 + k * d
+    q = synth.normal_f16((k, HQ, D), seed, 1)
+    kk = synth.normal_f16((S, HKV, D), seed, 2)
+    vv = synth.normal_f16((S, HKV, D), seed, 3)
+    return mask, q, kk, vv, S
+
+
+@pytest.mark.parametrize("k,d,P0,seed", [(10, 1, 500, 1), (10, 3, 500, 2), (10, 6, 4096, 3), (4, 5, 61, 4), (8, 8, 0, 5)])
+def test_draft_layer_mask_range(gpu, orc, k, d, P0, seed):
+    """mask_k_range = k*d > T = k: the mask bits cover more key columns than there are queries."""
+    from cpm.cu_amd import ops
+    from cpm.cu_amd.kvcache import PagedKVCache
+    torch = gpu
+    mask, q, kk, vv, S = _draft_layer_case(k, d, P0, seed)
+    npages = (S + 255) // 256 + 1
+    cache = PagedKVCache(1, HKV, npages, fill=float("nan"))
+    cache.write_logical(0, 0, to_dev(torch, kk[:S - k]), to_dev(torch, vv[:S - k]))
+    kv_len = torch.tensor([S], dtype=torch.int32, device="cuda")
+    out = ops.tree_attention(to_dev(torch, q), cache, 0, kv_len, S, to_dev(torch, mask), mask_k_range=k * d,
+                             k_new=to_dev(torch, kk[S - k:]), v_new=to_dev(torch, vv[S - k:]))
+    torch.cuda.synchronize()
+    ref = orc.tree_attention(q, kk, vv, mask, S - k, mask_k_range=k * d)
+    assert_close_f16(to_np(out), ref, "draft-layer attention k=%d d=%d" % (k, d))

@@ -305,3 +305,30 @@ def test_compaction_is_a_row_permutation(orc):
             assert np.array_equal(c[:P], b[:P])                                  # prefix untouched
             assert np.array_equal(c[P:P + len(path)], b[P + np.array(path)])     # dst[P+d] = src[P+path[d]]
             assert np.array_equal(c[P + len(path):], b[P + len(path):])          # the rest is not written
+
+
+def test_attention_mask_range_wider_than_queries(orc):
+    """mask_k_range > T (the drafter's own attention, src/model/minicpm4/minicpm4_eagle.cuh:359) against torch's
+    CPU scaled_dot_product_attention with an explicit boolean mask built from the definition: key
+    column c is visible to query i iff c <= P + i and (c < S - R or bit c - (S - R) of mask[i])."""
+    import torch
+    g = synth.rng(5, 55)
+    T, R, P, Hq, Hkv, D = 5, 20, 37, 4, 2, 32
+    S = P + T
+    q = g.standard_normal((T, Hq, D)).astype(np.float16)
+    k = g.standard_normal((S, Hkv, D)).astype(np.float16)
+    v = g.standard_normal((S, Hkv, D)).astype(np.float16)
+    bits = g.integers(0, 2, size=(T, R)).astype(np.uint64)
+    for i in range(T):
+        bits[i, R - T + i] = 1  # a query always sees its own key
+    mask = np.array([[sum(int(bits[i, j]) << j for j in range(R))] for i in range(T)], np.uint64)
+    out = orc.tree_attention(q, k, v, mask, P, mask_k_range=R).astype(np.float32)
+    vis = np.zeros((T, S), bool)
+    for i in range(T):
+        for c in range(S):
+            vis[i, c] = c <= P + i and (c < S - R or bool(bits[i, c - (S - R)]))
+    qt = torch.from_numpy(q.astype(np.float32)).permute(1, 0, 2)                          # [Hq, T, D]
+    kt = torch.from_numpy(k.astype(np.float32)).permute(1, 0, 2).repeat_interleave(Hq // Hkv, 0)
+    vt = torch.from_numpy(v.astype(np.float32)).permute(1, 0, 2).repeat_interleave(Hq // Hkv, 0)
+    ref = torch.nn.functional.scaled_dot_product_attention(qt, kt, vt, attn_mask=torch.from_numpy(vis)).permute(1, 0, 2).numpy()
+    assert np.abs(out - ref).max() < 5e-3
