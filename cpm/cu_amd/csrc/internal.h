@@ -7,7 +7,7 @@ namespace cpmcu {
 // lm_head.hip -- the streaming GEMM with its two epilogues.
 constexpr int kHeadModeStats = 0;
 constexpr int kHeadModeArgmax = 1;
-int launch_head_gemm(const void* hidden, const void* w, int n, int V, int H, int apply_scale, float head_scale,
+int launch_head_gemm(const void* hidden, const void* w, int w_layout, int n, int V, int H, int apply_scale, float head_scale,
                      int mode, void* logits, float* part_a, float* part_b, int* grid_out, int* stride_out,
                      hipStream_t st);
 int head_max_grid();

@@ -39,6 +39,7 @@ struct HeadParams {
     int apply_scale;
     float head_scale;
     int mode;
+    int w_tiled;  // W is stored as MFMA operand tiles: [16-row block][32-column step][lane][8 halves]
     f16* logits;          // [n][V] or null
     float* part_a;        // STATS: max   | ARGMAX: best value      [grid][NB*16]
     float* part_b;        // STATS: sum   | ARGMAX: best index (int) [grid][NB*16]
@@ -223,6 +224,14 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_kernel(HeadParams p) {
     auto load_group = [&](int it, f16x8* buf) {
         const int pass = it / gpp;
         const int k0 = ((it % gpp + rotg) % gpp) * GK;
+        if (p.w_tiled) {  // one contiguous KB per instruction, consecutive steps consecutive in memory
+            int rb = row_block(pass);
+            rb = rb * 16 < V ? rb : (V - 1) / 16;
+            const f16* src = p.w + ((size_t)rb * (H / 32) + k0 / 32) * 512 + lane * 8;
+#pragma unroll
+            for (int ks = 0; ks < PD; ++ks) buf[ks] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(src + ks * 512));
+            return;
+        }
         int row = row_block(pass) * 16 + arow_lane;
         row = row < V ? row : V - 1;  // clamp: rows past the end are computed and discarded
         const f16* src = p.w + (size_t)row * H + k0 + kgp * 8;
@@ -362,6 +371,14 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_chunked_kernel(HeadPar
         const int pass = (q / nch) * NP + pl;
         if (pass >= p.npasses) return;
         ++groups_since_dma;
+        if (p.w_tiled) {  // one contiguous KB per instruction, consecutive steps consecutive in memory
+            int rb = row_block(pass);
+            rb = rb * 16 < V ? rb : (V - 1) / 16;
+            const f16* src = p.w + ((size_t)rb * (H / 32) + chunk_of(q) * (KC / 32)) * 512 + lane * 8;
+#pragma unroll
+            for (int ks = 0; ks < PD; ++ks) buf[ks] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(src + ks * 512));
+            return;
+        }
         int row = row_block(pass) * 16 + l16;
         row = row < V ? row : V - 1;  // clamp: rows past the end are computed and discarded
         const f16* src = p.w + (size_t)row * H + chunk_of(q) * KC + kgp * 8;
@@ -500,9 +517,10 @@ int pick_nb(int n) { return n <= 16 ? 1 : n <= 32 ? 2 : n <= 64 ? 4 : 8; }
 }  // namespace
 
 // Shared launcher of the GEMM; returns the grid size used (= number of partial rows) in *grid_out.
-int launch_head_gemm(const void* hidden, const void* w, int n, int V, int H, int apply_scale, float head_scale,
+int launch_head_gemm(const void* hidden, const void* w, int w_layout, int n, int V, int H, int apply_scale, float head_scale,
                      int mode, void* logits, float* part_a, float* part_b, int* grid_out, int* stride_out,
                      hipStream_t st) {
+    CPMCU_CHECK_ARG(w_layout == CPMCU_W_ROW_MAJOR || w_layout == CPMCU_W_TILED, "lm_head: unknown weight layout %d", w_layout);
     const int NB = pick_nb(n);
     const int kc_max = 2048 / NB;
     const int gk = NB <= 4 ? 512 : 256;
@@ -519,6 +537,7 @@ int launch_head_gemm(const void* hidden, const void* w, int n, int V, int H, int
     p.apply_scale = apply_scale;
     p.head_scale = head_scale;
     p.mode = mode;
+    p.w_tiled = w_layout == CPMCU_W_TILED;
     p.logits = (f16*)logits;
     p.part_a = part_a;
     p.part_b = part_b;
@@ -560,7 +579,41 @@ extern "C" size_t cpmcu_head_workspace_bytes(int n, int V) {
     return align_up(parts, 256) + cpmcu_topk_workspace_bytes(n, V, 32);
 }
 
-extern "C" int cpmcu_lm_head_argmax(const void* hidden, const void* w, int n, int V, int H, int apply_scale,
+// Re-tiles a [V][H] row-major weight matrix (optionally gathering rows through `row_remap`, which fuses
+// remap_copy, src/model/tree_drafter.cuh:79-86) into MFMA operand order: one workgroup per 16-row block.
+__global__ __launch_bounds__(256) void head_weight_tile_kernel(const f16x8* __restrict__ w, const int32_t* __restrict__ row_remap, int V,
+                                                               int H, f16x8* __restrict__ out) {
+    const int rb = blockIdx.x;
+    const int steps = H / 32;
+    for (int x = threadIdx.x; x < steps * 64; x += 256) {
+        const int ks = x >> 6, lane = x & 63;
+        const int row = rb * 16 + (lane & 15);
+        f16x8 v;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) v[e] = (f16)0.f;
+        if (row < V) {
+            const size_t src_row = row_remap ? (size_t)row_remap[row] : (size_t)row;
+            v = w[(src_row * H + ks * 32 + (lane >> 4) * 8) / 8];
+        }
+        out[((size_t)rb * steps + ks) * 64 + lane] = v;
+    }
+}
+
+extern "C" size_t cpmcu_head_weight_tiled_bytes(int V, int H) {
+    if (V <= 0 || H <= 0) return 0;
+    return (size_t)ceil_div(V, 16) * 16 * H * sizeof(f16);
+}
+
+extern "C" int cpmcu_head_weight_tile(const void* w, const int32_t* row_remap, int V, int H, void* w_tiled, void* stream) {
+    CPMCU_CHECK_ARG(w && w_tiled && w != w_tiled, "head_weight_tile: null or aliased pointer argument");
+    CPMCU_CHECK_ARG(V >= 1 && H >= 32 && H % 32 == 0, "head_weight_tile: V=%d, H=%d must be a positive multiple of 32", V, H);
+    hipLaunchKernelGGL(head_weight_tile_kernel, dim3(ceil_div(V, 16)), dim3(256), 0, resolve_stream(stream), (const f16x8*)w, row_remap, V, H,
+                       (f16x8*)w_tiled);
+    CPMCU_LAUNCH_CHECK();
+    return CPMCU_OK;
+}
+
+extern "C" int cpmcu_lm_head_argmax(const void* hidden, const void* w, int w_layout, int n, int V, int H, int apply_scale,
                                     float head_scale, void* logits, int32_t* gt, void* workspace,
                                     size_t workspace_bytes, void* stream) {
     CPMCU_CHECK_ARG(hidden && w, "lm_head_argmax: null pointer argument");
@@ -573,7 +626,7 @@ extern "C" int cpmcu_lm_head_argmax(const void* hidden, const void* w, int n, in
     float* part_a = (float*)workspace;
     float* part_b = part_a + (size_t)head_max_grid() * 128;
     int G = 0, stride = 0;
-    int rc = launch_head_gemm(hidden, w, n, V, H, apply_scale, head_scale, kHeadModeArgmax, logits, part_a, part_b, &G, &stride, st);
+    int rc = launch_head_gemm(hidden, w, w_layout, n, V, H, apply_scale, head_scale, kHeadModeArgmax, logits, part_a, part_b, &G, &stride, st);
     if (rc != CPMCU_OK) return rc;
     if (gt) {
         hipLaunchKernelGGL(head_argmax_finalize_kernel, dim3(n), dim3(256), 0, st, part_a, part_b, G, stride, gt);

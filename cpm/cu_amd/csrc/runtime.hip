@@ -214,9 +214,9 @@ extern "C" int cpmcu_init_storage(int* max_context) {
         return CPMCU_OK;
     };
     const int max_tree = m.drafter ? m.tree_size : 64;
-    if ((rc = alloc((void**)&m.lm_head, (size_t)m.vocab * m.hidden * 2))) return rc;
+    if ((rc = alloc((void**)&m.lm_head, cpmcu_head_weight_tiled_bytes(m.vocab, m.hidden)))) return rc;  // kept in tiled layout
     if (m.drafter && m.frspec_vocab != m.vocab) {
-        if ((rc = alloc((void**)&m.fr_head, (size_t)m.frspec_vocab * m.hidden * 2))) return rc;
+        if ((rc = alloc((void**)&m.fr_head, cpmcu_head_weight_tiled_bytes(m.frspec_vocab, m.hidden)))) return rc;
         if ((rc = alloc((void**)&m.token_id_remap, (size_t)m.frspec_vocab * 4))) return rc;
     } else {
         m.fr_head = m.lm_head;
@@ -311,17 +311,29 @@ extern "C" int cpmcu_load_model(const char* name, uint64_t host_ptr) {
         return CPMCU_OK;
     }
     if (nm.rfind("lm_head", 0) == 0) {  // src/model/model.cuh:116-137 routing by prefix
-        CPMCU_HIP(hipMemcpy(m.lm_head, (const void*)host_ptr, (size_t)m.vocab * m.hidden * 2, hipMemcpyHostToDevice));
-        m.lm_head_loaded = true;
-        if (m.fr_head != m.lm_head) {  // src/model/minicpm4/minicpm4_eagle.cuh:215-219
-            if (!m.remap_loaded) {
-                set_error("load_model: eagle.token_id_remap must be loaded before lm_head.weight");
-                return CPMCU_ERR_RUNTIME;
-            }
-            rc = cpmcu_gather_rows(m.lm_head, m.token_id_remap, m.frspec_vocab, m.hidden, m.fr_head, st);
-            if (rc) return rc;
-            CPMCU_HIP(hipStreamSynchronize(st));
+        if (m.fr_head != m.lm_head && !m.remap_loaded) {
+            set_error("load_model: eagle.token_id_remap must be loaded before lm_head.weight");
+            return CPMCU_ERR_RUNTIME;
         }
+        // The row-major matrix only passes through a staging buffer: both heads are kept in the tiled
+        // layout their kernels stream fastest; the FR-Spec gather (remap_copy,
+        // src/model/minicpm4/minicpm4_eagle.cuh:215-219) is fused into its re-tiling.
+        void* staging = nullptr;
+        CPMCU_HIP(hipMalloc(&staging, (size_t)m.vocab * m.hidden * 2));
+        rc = CPMCU_OK;
+        if (hipMemcpy(staging, (const void*)host_ptr, (size_t)m.vocab * m.hidden * 2, hipMemcpyHostToDevice) != hipSuccess) {
+            set_error("load_model: copy of lm_head.weight to the device failed");
+            rc = CPMCU_ERR_HIP;
+        }
+        if (!rc) rc = cpmcu_head_weight_tile(staging, nullptr, m.vocab, m.hidden, m.lm_head, st);
+        if (!rc && m.fr_head != m.lm_head) rc = cpmcu_head_weight_tile(staging, m.token_id_remap, m.frspec_vocab, m.hidden, m.fr_head, st);
+        if (!rc && hipStreamSynchronize(st) != hipSuccess) {
+            set_error("load_model: re-tiling of lm_head.weight failed");
+            rc = CPMCU_ERR_HIP;
+        }
+        (void)hipFree(staging);
+        if (rc) return rc;
+        m.lm_head_loaded = true;
         return CPMCU_OK;
     }
     set_error("Unsupported name: %s (only lm_head.weight and eagle.token_id_remap belong to the verify/draft path)", name);
@@ -372,7 +384,7 @@ extern "C" int cpmcu_decode_lm_head(int input_length, uint64_t hidden, uint64_t 
     CPMCU_CHECK_ARG(m.lm_head_loaded, "decode_lm_head: lm_head.weight has not been loaded");
     hipStream_t st = resolve_stream(nullptr);
     PerfScope perf("DECODE_LM_HEAD", st);
-    return cpmcu_lm_head_argmax((const void*)hidden, m.lm_head, input_length, m.vocab, m.hidden, 1, m.scale_lmhead,
+    return cpmcu_lm_head_argmax((const void*)hidden, m.lm_head, CPMCU_W_TILED, input_length, m.vocab, m.hidden, 1, m.scale_lmhead,
                                 (void*)logits, (int32_t*)gt, m.head_ws, m.head_ws_bytes, st);
 }
 
@@ -387,7 +399,7 @@ extern "C" int cpmcu_draft_head(int n, uint64_t hidden, uint64_t topk_val, uint6
     CPMCU_CHECK_ARG(m.lm_head_loaded, "draft_head: lm_head.weight has not been loaded");
     hipStream_t st = resolve_stream(nullptr);
     PerfScope perf("DRAFT_HEAD", st);
-    return cpmcu_frspec_head_topk((const void*)hidden, m.fr_head, m.fr_head != m.lm_head ? m.token_id_remap : nullptr, n,
+    return cpmcu_frspec_head_topk((const void*)hidden, m.fr_head, CPMCU_W_TILED, m.fr_head != m.lm_head ? m.token_id_remap : nullptr, n,
                                   m.frspec_vocab, m.hidden, m.topk_per_iter, m.draft_logits, m.row_stats,
                                   (void*)topk_val, (int32_t*)topk_pos, (int32_t*)topk_ids, m.head_ws, m.head_ws_bytes, st);
 }

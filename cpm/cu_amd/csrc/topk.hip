@@ -256,7 +256,7 @@ extern "C" int cpmcu_gather_rows(const void* src, const int32_t* remap, int rows
     return CPMCU_OK;
 }
 
-extern "C" int cpmcu_frspec_head_topk(const void* hidden, const void* w, const int32_t* token_id_remap, int n, int V,
+extern "C" int cpmcu_frspec_head_topk(const void* hidden, const void* w, int w_layout, const int32_t* token_id_remap, int n, int V,
                                       int H, int k, void* logits, float* row_stats, void* topk_val,
                                       int32_t* topk_pos, int32_t* topk_ids, void* workspace, size_t workspace_bytes,
                                       void* stream) {
@@ -270,7 +270,7 @@ extern "C" int cpmcu_frspec_head_topk(const void* hidden, const void* w, const i
     float* part_b = part_a + (size_t)head_max_grid() * 128;
     const size_t parts_bytes = align_up((size_t)2 * head_max_grid() * 128 * sizeof(float), 256);
     int G = 0, stride = 0;
-    int rc = launch_head_gemm(hidden, w, n, V, H, 0, 1.f, kHeadModeStats, logits, part_a, part_b, &G, &stride, st);
+    int rc = launch_head_gemm(hidden, w, w_layout, n, V, H, 0, 1.f, kHeadModeStats, logits, part_a, part_b, &G, &stride, st);
     if (rc != CPMCU_OK) return rc;
     TopkStatsSource src{part_a, part_b, G, stride, row_stats};
     return launch_topk(logits, n, V, k, topk_val, topk_pos, topk_ids, token_id_remap, &src,

@@ -92,13 +92,41 @@ def gather_rows(src, remap):
     return dst
 
 
+W_ROW_MAJOR, W_TILED = 0, 1
+
+
+class TiledWeight:
+    """A head weight matrix in MFMA operand order (CPMCU_W_TILED): built once, streamed ~20 % faster."""
+
+    def __init__(self, data, V, H):
+        self.data, self.V, self.H = data, int(V), int(H)
+        self.shape = (self.V, self.H)
+
+
+def tile_head_weight(w, row_remap=None):
+    """[*, H] row-major fp16 -> TiledWeight of V rows; with row_remap (int32 [V]) row r is w[row_remap[r]]
+    (remap_copy, src/model/tree_drafter.cuh:79-86, fused with the re-tiling)."""
+    assert w.dtype == torch.float16 and w.is_contiguous()
+    H = w.shape[1]
+    V = w.shape[0] if row_remap is None else row_remap.numel()
+    out = torch.empty(_lib().raw.cpmcu_head_weight_tiled_bytes(V, H) // 2, dtype=torch.float16, device=w.device)
+    _lib().head_weight_tile(_ptr(w), _ptr(row_remap), V, H, _ptr(out), _stream())
+    return TiledWeight(out, V, H)
+
+
+def _weight(w):
+    if isinstance(w, TiledWeight):
+        return w.data, W_TILED, w.V
+    return w, W_ROW_MAJOR, w.shape[0]
+
+
 def frspec_head_topk(hidden, w, token_id_remap, k):
     """FR-Spec draft head: logits -> log-softmax -> top-k -> full-vocabulary ids.
 
     Returns dict(logits [n,V] f16 raw, row_stats [n,2] f32 (max, ln sum), val [n,k] f16, pos [n,k] i32, ids [n,k] i32).
     """
     n, H = hidden.shape
-    V = w.shape[0]
+    w, layout, V = _weight(w)
     dev = hidden.device
     logits = torch.empty((n, V), dtype=torch.float16, device=dev)
     stats = torch.empty((n, 2), dtype=torch.float32, device=dev)
@@ -106,7 +134,7 @@ def frspec_head_topk(hidden, w, token_id_remap, k):
     pos = torch.empty((n, k), dtype=torch.int32, device=dev)
     ids = torch.empty((n, k), dtype=torch.int32, device=dev)
     ws = _workspace("head", _lib().raw.cpmcu_head_workspace_bytes(n, V), dev)
-    _lib().frspec_head_topk(_ptr(hidden), _ptr(w), _ptr(token_id_remap), n, V, H, k, _ptr(logits), _ptr(stats),
+    _lib().frspec_head_topk(_ptr(hidden), _ptr(w), layout, _ptr(token_id_remap), n, V, H, k, _ptr(logits), _ptr(stats),
                             _ptr(val), _ptr(pos), _ptr(ids), _ptr(ws), ws.numel(), _stream())
     return dict(logits=logits, row_stats=stats, val=val, pos=pos, ids=ids)
 
@@ -114,13 +142,13 @@ def frspec_head_topk(hidden, w, token_id_remap, k):
 def lm_head_argmax(hidden, w, head_scale=None, want_logits=False, gt=None):
     """Target head + arg-max (src/model/linear.cuh:82-101 + torch argmax of tree_drafter.py:233)."""
     n, H = hidden.shape
-    V = w.shape[0]
+    w, layout, V = _weight(w)
     dev = hidden.device
     logits = torch.empty((n, V), dtype=torch.float16, device=dev) if want_logits else None
     if gt is None:
         gt = torch.empty(n, dtype=torch.int32, device=dev)
     ws = _workspace("head", _lib().raw.cpmcu_head_workspace_bytes(n, V), dev)
-    _lib().lm_head_argmax(_ptr(hidden), _ptr(w), n, V, H, 0 if head_scale is None else 1,
+    _lib().lm_head_argmax(_ptr(hidden), _ptr(w), layout, n, V, H, 0 if head_scale is None else 1,
                           ctypes.c_float(1.0 if head_scale is None else head_scale), _ptr(logits), _ptr(gt),
                           _ptr(ws), ws.numel(), _stream())
     return (gt, logits) if want_logits else gt

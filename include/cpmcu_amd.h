@@ -208,6 +208,20 @@ int cpmcu_tree_attention(const void* q, void* k_pool, void* v_pool, const int32_
 /* remap_copy -- src/model/tree_drafter.cuh:79-86,103-107: dst[r][:] = src[remap[r]][:]. */
 int cpmcu_gather_rows(const void* src, const int32_t* remap, int rows, int dim, void* dst, void* stream);
 
+/* Weight layouts of the two head operators (w_layout).
+ * CPMCU_W_ROW_MAJOR: [V][H] fp16 as the reference keeps it (src/model/linear.cuh:39-47).
+ * CPMCU_W_TILED: the same numbers in MFMA operand order, [ceil(V/16)][H/32][64 lanes][8 halves]
+ *   (rows beyond V are zero): a wave's 16-row block is one contiguous stream of H*32 bytes, which
+ *   the GPU reads ~20 % faster than 16 strided rows.  Built once at load time by
+ *   cpmcu_head_weight_tile; logits are identical for both layouts. */
+#define CPMCU_W_ROW_MAJOR 0
+#define CPMCU_W_TILED 1
+size_t cpmcu_head_weight_tiled_bytes(int V, int H);
+/* w [*][H] fp16 row-major -> w_tiled (cpmcu_head_weight_tiled_bytes(V, H) bytes, must not alias w).
+ * Row r of the result is row row_remap[r] of w when row_remap is given (this is remap_copy,
+ * src/model/tree_drafter.cuh:79-86, fused with the re-tiling), else row r.  H % 32 == 0. */
+int cpmcu_head_weight_tile(const void* w, const int32_t* row_remap, int V, int H, void* w_tiled, void* stream);
+
 /* Bytes of scratch the two head operators need. */
 size_t cpmcu_head_workspace_bytes(int n, int V);
 
@@ -215,22 +229,22 @@ size_t cpmcu_head_workspace_bytes(int n, int V);
  * Linear::prefill (src/model/linear.cuh:8-37,73-79) + log_softmax
  * (src/model/eagle.cuh:29-89) + TopK::prefill (src/model/topk.cuh:158-213,255-288)
  * + remap (src/model/tree_drafter.cuh:88-90).
- *   hidden [n][H] fp16 (n <= 16); w [V][H] fp16 (the gathered sub-matrix);
+ *   hidden [n][H] fp16 (n <= 16); w: the gathered sub-matrix, V rows, in layout w_layout;
  *   logits [n][V] fp16 scratch/output (raw logits z);
  *   row_stats [n][2] fp32 output: (max z, ln sum exp(z - max));
  *   topk_val [n][k] fp16 = f16((z - max) - lnsum); topk_pos [n][k] int32 index into w;
  *   topk_ids [n][k] int32 = token_id_remap[topk_pos] (token_id_remap NULL -> ids = pos).
  * Ordering: value descending, ties -> lower index (src/model/topk.cuh:17). k <= 32. */
-int cpmcu_frspec_head_topk(const void* hidden, const void* w, const int32_t* token_id_remap, int n, int V,
+int cpmcu_frspec_head_topk(const void* hidden, const void* w, int w_layout, const int32_t* token_id_remap, int n, int V,
                            int H, int k, void* logits, float* row_stats, void* topk_val, int32_t* topk_pos,
                            int32_t* topk_ids, void* workspace, size_t workspace_bytes, void* stream);
 
 /* Target head with fused arg-max -- LMHead::prefill (src/model/linear.cuh:82-101;
  * fp16 pre-scale by head_scale when apply_scale != 0) + torch argmax
  * (cpmcu/speculative/tree_drafter.py:153,233; lowest index on ties).
- *   hidden [n][H] fp16 (n <= 128); w [V][H]; logits [n][V] fp16 or NULL (not
+ *   hidden [n][H] fp16 (n <= 128); w: V rows in layout w_layout; logits [n][V] fp16 or NULL (not
  *   materialised); gt int32[n] or NULL. */
-int cpmcu_lm_head_argmax(const void* hidden, const void* w, int n, int V, int H, int apply_scale,
+int cpmcu_lm_head_argmax(const void* hidden, const void* w, int w_layout, int n, int V, int H, int apply_scale,
                          float head_scale, void* logits, int32_t* gt, void* workspace,
                          size_t workspace_bytes, void* stream);
 

@@ -208,3 +208,36 @@ def test_log_softmax_operator(gpu, orc):
     staged = orc.log_softmax_apply(x, stats[:, 0], stats[:, 1])
     assert np.array_equal(to_np(d).view(np.uint16), staged.view(np.uint16))
     assert_close_f16(to_np(d), lp_ref, "log_softmax", atol=2e-2, rtol=1e-2)
+
+
+@pytest.mark.parametrize("n,V,H", [(60, 1000 + 7, 512), (10, 4096, 1024), (24, 530, 2048), (128, 2000, 512), (1, 16, 512)])
+def test_tiled_weight_layout_gives_identical_logits(gpu, orc, n, V, H):
+    """The tiled layout holds the same numbers in another order and the kernels accumulate them in the
+    same order, so logits and arg-max are bit-identical to the row-major layout; both match the oracle."""
+    from cpm.cu_amd import ops
+    torch = gpu
+    hid = synth.normal_f16((n, H), V + n, 1)
+    w = synth.normal_f16((V, H), V + n, 2, std=0.05)
+    d_hid, d_w = to_dev(torch, hid), to_dev(torch, w)
+    gt_r, z_r = ops.lm_head_argmax(d_hid, d_w, want_logits=True)
+    gt_t, z_t = ops.lm_head_argmax(d_hid, ops.tile_head_weight(d_w), want_logits=True)
+    torch.cuda.synchronize()
+    assert torch.equal(z_r, z_t) and torch.equal(gt_r, gt_t)
+    assert_close_f16(to_np(z_t), orc.lm_head(hid, w), "tiled target logits")
+
+
+def test_tiled_frspec_head_with_fused_gather(gpu, orc):
+    """tile_head_weight with a row map == gather_rows followed by tiling == the row-major sub-matrix."""
+    from cpm.cu_amd import ops
+    torch = gpu
+    V, Vs, H, n, k = 3000, 1024 + 8, 512, 10, 10
+    hid = synth.normal_f16((n, H), 91, 1)
+    w = synth.normal_f16((V, H), 91, 2, std=0.05)
+    remap = synth.frspec_remap(V, Vs, 91)
+    d_hid, d_w, d_remap = to_dev(torch, hid), to_dev(torch, w), to_dev(torch, remap)
+    a = ops.frspec_head_topk(d_hid, ops.gather_rows(d_w, d_remap), d_remap, k)
+    b = ops.frspec_head_topk(d_hid, ops.tile_head_weight(d_w, d_remap), d_remap, k)
+    torch.cuda.synchronize()
+    for key in ("logits", "row_stats", "val", "pos", "ids"):
+        assert torch.equal(a[key], b[key]), key
+    assert_close_f16(to_np(b["logits"]), orc.lm_head(hid, orc.gather_rows(w, remap)), "tiled FR-Spec logits")
