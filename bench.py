@@ -34,7 +34,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 # are carried here as constants and are reported only for the workload they were measured on.
 MEASURED_TRAFFIC_KIB = {
     "tree_attn_split_kernel+tree_attn_combine_kernel": 6372 + 8494 + 8718 + 480,
-    "head_gemm_chunked_kernel<4,4,128,4>+head_argmax_finalize_kernel": 608804 + 128 + 1064 + 2,
+    "head_gemm_chunked_kernel<4,4,256,4>+head_argmax_finalize_kernel": 608804 + 128 + 1064 + 2,
     "tree_accept_kernel+kv_compact_kernel+accepted_ids_kernel": 6 + 1125 + 320 + 2,
 }
 
@@ -245,7 +245,7 @@ def main():
         dict(kernel="tree_attn_split_kernel+tree_attn_combine_kernel", launches_per_step=wl.L, us_per_launch=round(ms_attn * 1e3, 2),
              bound="mfma", achieved=round(attn_tflops, 2), peak=MFMA_F16_PEAK_TFLOPS, unit="TFLOP/s",
              frac=round(attn_tflops / MFMA_F16_PEAK_TFLOPS, 4), hbm_gbs=round(attn_gbs, 1), traffic=None),
-        dict(kernel="head_gemm_chunked_kernel<4,4,128,4>+head_argmax_finalize_kernel", launches_per_step=1, us_per_launch=round(ms_head * 1e3, 2),
+        dict(kernel="head_gemm_chunked_kernel<4,4,256,4>+head_argmax_finalize_kernel", launches_per_step=1, us_per_launch=round(ms_head * 1e3, 2),
              bound="hbm", achieved=round(head_gbs, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(head_gbs / HBM_PEAK_GBS, 4),
              traffic=None),
         dict(kernel="tree_accept_kernel+kv_compact_kernel+accepted_ids_kernel", launches_per_step=1,
@@ -271,7 +271,7 @@ def main():
     ms_fr = timed_replays(torch, fr_head, reps, 2, use_graph)[0] / HEAD_REP
     fr_bytes = wl.shape["frspec_vocab"] * wl.shape["hidden"] * 2.0 + 10 * wl.shape["hidden"] * 2.0 + 10 * 10 * 6.0
     fr_gbs = fr_bytes / (ms_fr * 1e-3) / 1e9
-    frspec = dict(kernel="head_gemm_kernel<1>+topk_chunk_kernel+topk_merge_kernel", us_per_call=round(ms_fr * 1e3, 2), bound="hbm",
+    frspec = dict(kernel="head_gemm_chunked_kernel<1,4,256,4>+topk_chunk_kernel+topk_merge_kernel", us_per_call=round(ms_fr * 1e3, 2), bound="hbm",
                   achieved=round(fr_gbs, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(fr_gbs / HBM_PEAK_GBS, 4))
     del w_sub
 

@@ -547,18 +547,18 @@ int launch_head_gemm(const void* hidden, const void* w, int w_layout, int n, int
     p.npasses = ceil_div(nrb, G * kHeadWaves);
     *grid_out = G;
     *stride_out = NB * 16;
-    const int kc_chunked = 512;
-    if (p.nch <= 2 || H % kc_chunked != 0) {  // all hidden rows fit LDS for the whole K range (or an odd H)
+    if (H % 256 != 0) {  // odd hidden sizes: every wave walks whole rows, hidden rows resident or chunked per row block
         switch (NB) {
             case 1: hipLaunchKernelGGL(head_gemm_kernel<1>, dim3(G), dim3(kHeadThreads), 0, st, p); break;
             case 2: hipLaunchKernelGGL(head_gemm_kernel<2>, dim3(G), dim3(kHeadThreads), 0, st, p); break;
             case 4: hipLaunchKernelGGL(head_gemm_kernel<4>, dim3(G), dim3(kHeadThreads), 0, st, p); break;
             default: hipLaunchKernelGGL(head_gemm_kernel<8>, dim3(G), dim3(kHeadThreads), 0, st, p); break;
         }
-    } else {
+    } else {  // shapes chosen by measurement on MI355X (73448 x 4096 and 32768 x 4096 heads)
         switch (NB) {
-            case 2: hipLaunchKernelGGL((head_gemm_chunked_kernel<2, 4, 512, 2>), dim3(G), dim3(kHeadThreads), 0, st, p); break;
-            case 4: hipLaunchKernelGGL((head_gemm_chunked_kernel<4, 4, 128, 4>), dim3(G), dim3(kHeadThreads), 0, st, p); break;
+            case 1: hipLaunchKernelGGL((head_gemm_chunked_kernel<1, 4, 256, 4>), dim3(G), dim3(kHeadThreads), 0, st, p); break;
+            case 2: hipLaunchKernelGGL((head_gemm_chunked_kernel<2, 4, 256, 4>), dim3(G), dim3(kHeadThreads), 0, st, p); break;
+            case 4: hipLaunchKernelGGL((head_gemm_chunked_kernel<4, 4, 256, 4>), dim3(G), dim3(kHeadThreads), 0, st, p); break;
             default: hipLaunchKernelGGL((head_gemm_chunked_kernel<8, 2, 128, 2>), dim3(G), dim3(kHeadThreads), 0, st, p); break;
         }
     }
