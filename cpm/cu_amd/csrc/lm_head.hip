@@ -547,18 +547,27 @@ int launch_head_gemm(const void* hidden, const void* w, int w_layout, int n, int
     p.npasses = ceil_div(nrb, G * kHeadWaves);
     *grid_out = G;
     *stride_out = NB * 16;
-    if (H % 256 != 0) {  // odd hidden sizes: every wave walks whole rows, hidden rows resident or chunked per row block
+    // Kernel shapes chosen by measurement on MI355X (73448 x 4096 and 32768 x 4096 heads).
+    if (H % 256 != 0 || (!p.w_tiled && p.nch <= 2)) {
+        // every wave walks whole rows; hidden rows LDS-resident (<= 16 rows) or chunked per row block.
+        // Best for row-major weights with <= 16 rows (1 KB runs per row), and the fallback for odd H.
         switch (NB) {
             case 1: hipLaunchKernelGGL(head_gemm_kernel<1>, dim3(G), dim3(kHeadThreads), 0, st, p); break;
             case 2: hipLaunchKernelGGL(head_gemm_kernel<2>, dim3(G), dim3(kHeadThreads), 0, st, p); break;
             case 4: hipLaunchKernelGGL(head_gemm_kernel<4>, dim3(G), dim3(kHeadThreads), 0, st, p); break;
             default: hipLaunchKernelGGL(head_gemm_kernel<8>, dim3(G), dim3(kHeadThreads), 0, st, p); break;
         }
-    } else {  // shapes chosen by measurement on MI355X (73448 x 4096 and 32768 x 4096 heads)
+    } else if (p.w_tiled) {
         switch (NB) {
             case 1: hipLaunchKernelGGL((head_gemm_chunked_kernel<1, 4, 256, 4>), dim3(G), dim3(kHeadThreads), 0, st, p); break;
             case 2: hipLaunchKernelGGL((head_gemm_chunked_kernel<2, 4, 256, 4>), dim3(G), dim3(kHeadThreads), 0, st, p); break;
             case 4: hipLaunchKernelGGL((head_gemm_chunked_kernel<4, 4, 256, 4>), dim3(G), dim3(kHeadThreads), 0, st, p); break;
+            default: hipLaunchKernelGGL((head_gemm_chunked_kernel<8, 2, 128, 2>), dim3(G), dim3(kHeadThreads), 0, st, p); break;
+        }
+    } else {
+        switch (NB) {
+            case 2: hipLaunchKernelGGL((head_gemm_chunked_kernel<2, 4, 512, 2>), dim3(G), dim3(kHeadThreads), 0, st, p); break;
+            case 4: hipLaunchKernelGGL((head_gemm_chunked_kernel<4, 4, 128, 4>), dim3(G), dim3(kHeadThreads), 0, st, p); break;
             default: hipLaunchKernelGGL((head_gemm_chunked_kernel<8, 2, 128, 2>), dim3(G), dim3(kHeadThreads), 0, st, p); break;
         }
     }

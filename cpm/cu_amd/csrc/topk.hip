@@ -50,8 +50,9 @@ __global__ __launch_bounds__(kTopkThreads) void topk_chunk_kernel(TopkParams p) 
     const int tid = threadIdx.x;
     float m = 0.f, lse = 0.f;
     if (LOGSOFTMAX) {
-        // row statistics from the GEMM's per-workgroup (max, sum exp(z - max)) partials
-        __shared__ float sm[kTopkThreads], ss[kTopkThreads];
+        // row statistics from the GEMM's per-workgroup (max, sum exp(z - max)) partials: in-wave by
+        // shuffles, then across the four waves through LDS
+        __shared__ float sm[kTopkThreads / 64], ss[kTopkThreads / 64];
         float a = -INFINITY, b = 0.f;
         for (int c = tid; c < p.grid; c += kTopkThreads) {
             const float oa = p.part_max[(size_t)c * p.stride + row];
@@ -60,20 +61,28 @@ __global__ __launch_bounds__(kTopkThreads) void topk_chunk_kernel(TopkParams p) 
             b = (mm == -INFINITY) ? 0.f : b * expf(a - mm) + ob * expf(oa - mm);
             a = mm;
         }
-        sm[tid] = a;
-        ss[tid] = b;
-        __syncthreads();
-        for (int off = kTopkThreads / 2; off > 0; off >>= 1) {
-            if (tid < off) {
-                const float a0 = sm[tid], a1 = sm[tid + off];
-                const float mm = fmaxf(a0, a1);
-                ss[tid] = (mm == -INFINITY) ? 0.f : ss[tid] * expf(a0 - mm) + ss[tid + off] * expf(a1 - mm);
-                sm[tid] = mm;
-            }
-            __syncthreads();
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const float oa = __shfl_xor(a, off), ob = __shfl_xor(b, off);
+            const float mm = fmaxf(a, oa);
+            b = (mm == -INFINITY) ? 0.f : b * expf(a - mm) + ob * expf(oa - mm);
+            a = mm;
         }
-        m = sm[0];
-        lse = logf(ss[0]);
+        if ((tid & 63) == 0) {
+            sm[tid >> 6] = a;
+            ss[tid >> 6] = b;
+        }
+        __syncthreads();
+        a = sm[0];
+        b = ss[0];
+#pragma unroll
+        for (int w = 1; w < kTopkThreads / 64; ++w) {
+            const float mm = fmaxf(a, sm[w]);
+            b = (mm == -INFINITY) ? 0.f : b * expf(a - mm) + ss[w] * expf(sm[w] - mm);
+            a = mm;
+        }
+        m = a;
+        lse = logf(b);
         if (chunk == 0 && tid == 0 && p.row_stats) {
             p.row_stats[row * 2 + 0] = m;
             p.row_stats[row * 2 + 1] = lse;

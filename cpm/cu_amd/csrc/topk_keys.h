@@ -40,10 +40,13 @@ __device__ inline uint64_t wave_max_u64(uint64_t v) {
 }
 
 // k rounds of workgroup-wide max over the keys held in registers; round j's winner goes to
-// emit(j, key).  Keys equal to 0 are empty slots.
+// emit(j, key), called by thread 0.  Keys equal to 0 are empty slots.  One barrier per round: the
+// per-wave maxima alternate between two LDS buffers, so a wave that runs ahead into the next round
+// writes the other buffer (it cannot get two rounds ahead: the barrier in between needs every wave).
+// Ends with a barrier, so whatever emit stored in LDS is visible to the workgroup afterwards.
 template <typename Emit>
 __device__ inline void select_topk(uint64_t (&keys)[kPerThread], int top, Emit emit) {
-    __shared__ uint64_t wave_best[kTopkThreads / 64];
+    __shared__ uint64_t wave_best[2][kTopkThreads / 64];
     const int wave = threadIdx.x >> 6;
     const int lane = threadIdx.x & 63;
     for (int round = 0; round < top; ++round) {
@@ -51,19 +54,20 @@ __device__ inline void select_topk(uint64_t (&keys)[kPerThread], int top, Emit e
 #pragma unroll
         for (int e = 0; e < kPerThread; ++e) mine = keys[e] > mine ? keys[e] : mine;
         const uint64_t wbest = wave_max_u64(mine);
-        if (lane == 0) wave_best[wave] = wbest;
+        uint64_t* wb = wave_best[round & 1];
+        if (lane == 0) wb[wave] = wbest;
         __syncthreads();
-        uint64_t best = wave_best[0];
+        uint64_t best = wb[0];
 #pragma unroll
-        for (int w = 1; w < kTopkThreads / 64; ++w) best = wave_best[w] > best ? wave_best[w] : best;
+        for (int w = 1; w < kTopkThreads / 64; ++w) best = wb[w] > best ? wb[w] : best;
         if (best != 0 && mine == best) {
 #pragma unroll
             for (int e = 0; e < kPerThread; ++e)
                 if (keys[e] == best) keys[e] = 0;
         }
         if (threadIdx.x == 0) emit(round, best);
-        __syncthreads();
     }
+    __syncthreads();
 }
 
 }  // namespace cpmcu

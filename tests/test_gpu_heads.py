@@ -211,9 +211,10 @@ def test_log_softmax_operator(gpu, orc):
 
 
 @pytest.mark.parametrize("n,V,H", [(60, 1000 + 7, 512), (10, 4096, 1024), (24, 530, 2048), (128, 2000, 512), (1, 16, 512)])
-def test_tiled_weight_layout_gives_identical_logits(gpu, orc, n, V, H):
-    """The tiled layout holds the same numbers in another order and the kernels accumulate them in the
-    same order, so logits and arg-max are bit-identical to the row-major layout; both match the oracle."""
+def test_tiled_weight_layout_gives_the_same_logits(gpu, orc, n, V, H):
+    """The tiled layout holds the same numbers in another order.  The kernels chosen for the two layouts
+    may walk K in different chunk sizes, so the fp32 sums can differ in their last bits: logits agree
+    to an fp16 ulp, the arg-max wherever the top two are further apart than that, both match the oracle."""
     from cpm.cu_amd import ops
     torch = gpu
     hid = synth.normal_f16((n, H), V + n, 1)
@@ -222,8 +223,12 @@ def test_tiled_weight_layout_gives_identical_logits(gpu, orc, n, V, H):
     gt_r, z_r = ops.lm_head_argmax(d_hid, d_w, want_logits=True)
     gt_t, z_t = ops.lm_head_argmax(d_hid, ops.tile_head_weight(d_w), want_logits=True)
     torch.cuda.synchronize()
-    assert torch.equal(z_r, z_t) and torch.equal(gt_r, gt_t)
-    assert_close_f16(to_np(z_t), orc.lm_head(hid, w), "tiled target logits")
+    assert_close_f16(to_np(z_t), to_np(z_r), "tiled vs row-major logits", atol=8e-3, rtol=2e-3)
+    ref = orc.lm_head(hid, w)
+    assert_close_f16(to_np(z_t), ref, "tiled target logits")
+    top2 = np.sort(ref.astype(np.float32), axis=1)[:, -2:]
+    clear = (top2[:, 1] - top2[:, 0]) > 2e-2
+    assert np.array_equal(to_np(gt_t)[clear], to_np(gt_r)[clear]) and np.array_equal(to_np(gt_t)[clear], orc.argmax(ref)[clear])
 
 
 def test_tiled_frspec_head_with_fused_gather(gpu, orc):
@@ -238,6 +243,12 @@ def test_tiled_frspec_head_with_fused_gather(gpu, orc):
     a = ops.frspec_head_topk(d_hid, ops.gather_rows(d_w, d_remap), d_remap, k)
     b = ops.frspec_head_topk(d_hid, ops.tile_head_weight(d_w, d_remap), d_remap, k)
     torch.cuda.synchronize()
-    for key in ("logits", "row_stats", "val", "pos", "ids"):
-        assert torch.equal(a[key], b[key]), key
-    assert_close_f16(to_np(b["logits"]), orc.lm_head(hid, orc.gather_rows(w, remap)), "tiled FR-Spec logits")
+    ref = orc.lm_head(hid, orc.gather_rows(w, remap))
+    assert_close_f16(to_np(b["logits"]), to_np(a["logits"]), "tiled vs row-major FR-Spec logits", atol=8e-3, rtol=2e-3)
+    assert_close_f16(to_np(b["logits"]), ref, "tiled FR-Spec logits")
+    # staged exactness of the tiled path: the oracle ranks the device's own logits and statistics
+    st = to_np(b["row_stats"])
+    lp = orc.log_softmax_apply(to_np(b["logits"]), st[:, 0], st[:, 1])
+    val_s, pos_s = orc.topk(lp, k)
+    assert np.array_equal(to_np(b["pos"]), pos_s) and np.array_equal(to_np(b["val"]).view(np.uint16), val_s.view(np.uint16))
+    assert np.array_equal(to_np(b["ids"]), remap[pos_s])
