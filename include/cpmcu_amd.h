@@ -213,7 +213,8 @@ int cpmcu_gather_rows(const void* src, const int32_t* remap, int rows, int dim, 
  * CPMCU_W_TILED: the same numbers in MFMA operand order, [ceil(V/16)][H/32][64 lanes][8 halves]
  *   (rows beyond V are zero): a wave's 16-row block is one contiguous stream of H*32 bytes, which
  *   the GPU reads ~20 % faster than 16 strided rows.  Built once at load time by
- *   cpmcu_head_weight_tile; logits are identical for both layouts. */
+ *   cpmcu_head_weight_tile.  Logits of the two layouts agree to fp16 rounding of the same fp32
+ *   sums taken in a different order (the K-chunking chosen per layout differs). */
 #define CPMCU_W_ROW_MAJOR 0
 #define CPMCU_W_TILED 1
 size_t cpmcu_head_weight_tiled_bytes(int V, int H);
