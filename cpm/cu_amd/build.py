@@ -21,7 +21,7 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 ARCH = "gfx950"
 
 HIP_SOURCES = ["runtime.hip", "tree_attention.hip", "lm_head.hip", "topk.hip", "tree_accept.hip", "draft_tree.hip"]
-HEADERS = ["common.h", "internal.h"]
+HEADERS = sorted(f for f in os.listdir(CSRC) if f.endswith(".h"))
 
 # packed fp32 VALU ops stay off for every device translation unit
 HIP_FLAGS = [

@@ -128,6 +128,223 @@ __global__ __launch_bounds__(kTopkThreads) void topk_merge_kernel(TopkParams p) 
     select_topk(keys, p.top, [&](int round, uint64_t key) { emit_final<LOGSOFTMAX>(p, row, round, key); });
 }
 
+// One-launch top-k for rows of at most kRowMaxDim elements: one 1024-thread workgroup per row keeps
+// the whole row in registers, two values per register as order-preserving 16-bit images of the raw
+// input ("raw images": bits ^ (sign ? 0xFFFF : 0x8000); -0 is one below +0 here, which every bound
+// below allows for).
+//   1. a lower bound of the k-th largest value: every wave takes the k-th largest of its 64
+//      per-lane maxima (bisection over the 16 bits with ballots, no barrier); the largest of the 16
+//      wave results has at least k elements at or above it, and on anything but tie-heavy data only
+//      a few hundred;
+//   2. fused log-softmax: ranking is on f16((z - max) - ln sum), a monotone map of z that merges
+//      neighbours, so the bound moves down by four ulps of the mapped bound -- every z that can map
+//      to the same fp16 value or above stays a candidate -- and only candidates are mapped;
+//   3. candidates go to LDS as exact 64-bit keys; each counts the candidates with a larger key:
+//      that count IS its output slot.
+// More than kRowCap candidates (rows dominated by one value): k rounds of a workgroup-wide maximum
+// over the register-resident values instead, each round taking the largest key below the previous winner.
+constexpr int kRowThreads = 1024;
+constexpr int kRowWaves = kRowThreads / 64;
+constexpr int kRowPieces = 4;                          // 16-byte pieces per thread
+constexpr int kRowElems = kRowPieces * 8;
+constexpr int kRowMaxDim = kRowThreads * kRowElems;    // 32768
+constexpr int kRowCap = kRowThreads;                   // candidate keys held in LDS
+constexpr int kRowMaxTop = 64;                         // the wave-level bound needs k <= 64 lanes
+
+typedef int16_t s16x2 __attribute__((ext_vector_type(2)));
+typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
+
+template <bool LOGSOFTMAX>
+__global__ __launch_bounds__(kRowThreads) void topk_row_kernel(TopkParams p) {
+    __shared__ uint64_t cand[kRowCap];
+    __shared__ int rank[kRowCap];
+    __shared__ uint64_t wave_best[2][kRowWaves];
+    __shared__ float row_m_lse[2];
+    __shared__ uint32_t wave_kth[kRowWaves];
+    __shared__ int ncand;
+    const int row = blockIdx.x;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int npieces = p.dim >> 3;
+    const uint4* xr = (const uint4*)(p.x + (size_t)row * p.dim);
+    // slots beyond the row read as 0xFFFF, whose raw image is 0: below every bound that is used
+    uint4 raw[kRowPieces];
+#pragma unroll
+    for (int j = 0; j < kRowPieces; ++j) {
+        const int pc = j * kRowThreads + tid;
+        raw[j] = pc < npieces ? xr[pc] : make_uint4(~0u, ~0u, ~0u, ~0u);
+    }
+    if (tid == 0) ncand = 0;
+    rank[tid] = 0;
+    if (LOGSOFTMAX && wave == 0) {
+        // row statistics from the GEMM's per-workgroup (max, sum exp(z - max)) partials, one wave
+        float a = -INFINITY, b = 0.f;
+        for (int c = lane; c < p.grid; c += 64) {
+            const float oa = p.part_max[(size_t)c * p.stride + row];
+            const float ob = p.part_sum[(size_t)c * p.stride + row];
+            const float mm = fmaxf(a, oa);
+            b = (mm == -INFINITY) ? 0.f : b * expf(a - mm) + ob * expf(oa - mm);
+            a = mm;
+        }
+        const float wm = wave_max_f32(a);
+        b = wave_sum_f32((a == -INFINITY) ? 0.f : b * expf(a - wm));
+        if (lane == 0) {
+            const float l = logf(b);
+            row_m_lse[0] = wm;
+            row_m_lse[1] = l;
+            if (p.row_stats) {
+                p.row_stats[row * 2 + 0] = wm;
+                p.row_stats[row * 2 + 1] = l;
+            }
+        }
+    }
+    // raw images, two per register
+    uint32_t img[kRowElems / 2];
+    u16x2 lmax2 = {0, 0};
+#pragma unroll
+    for (int j = 0; j < kRowPieces; ++j) {
+        const uint32_t w4[4] = {raw[j].x, raw[j].y, raw[j].z, raw[j].w};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const s16x2 sx = __builtin_bit_cast(s16x2, w4[q]);
+            const uint32_t sign = __builtin_bit_cast(uint32_t, sx >> 15);
+            const uint32_t o = w4[q] ^ (sign | 0x80008000u);
+            img[j * 4 + q] = o;
+            lmax2 = __builtin_elementwise_max(lmax2, __builtin_bit_cast(u16x2, o));
+        }
+    }
+    const uint32_t lmax = lmax2[0] > lmax2[1] ? lmax2[0] : lmax2[1];
+    // k-th largest of this wave's lane maxima (0 when fewer than k lanes hold anything), two bits a step
+    uint32_t kth = 0;
+    for (int bit = 14; bit >= 0; bit -= 2) {
+        const uint32_t c1 = kth | (1u << bit), c2 = kth | (2u << bit), c3 = kth | (3u << bit);
+        const int n1 = __popcll(__ballot(lmax >= c1)), n2 = __popcll(__ballot(lmax >= c2)), n3 = __popcll(__ballot(lmax >= c3));
+        kth = n3 >= p.top ? c3 : n2 >= p.top ? c2 : n1 >= p.top ? c1 : kth;
+    }
+    if (lane == 0) wave_kth[wave] = kth;
+    __syncthreads();
+    uint32_t bound = wave_kth[0];
+#pragma unroll
+    for (int w = 1; w < kRowWaves; ++w) bound = wave_kth[w] > bound ? wave_kth[w] : bound;
+    uint32_t lo = bound > 0 ? bound - 1 : 0;  // candidates: raw image >= lo
+    float m = 0.f, lse = 0.f;
+    if (LOGSOFTMAX) {
+        m = row_m_lse[0];
+        lse = row_m_lse[1];
+        if (bound > 0) {
+            const uint16_t zb = (uint16_t)((bound & 0x8000u) ? (bound ^ 0x8000u) : (bound ^ 0xFFFFu));
+            const float zl = (float)__builtin_bit_cast(f16, zb);
+            const f16 y = (f16)((zl - m) - lse);
+            const int e = (__builtin_bit_cast(uint16_t, y) >> 10) & 31;
+            const float zlo = zl - 4.f * ldexpf(1.f, e ? e - 25 : -24);
+            lo = 0;
+            if (e != 31 && zlo == zlo && fabsf(zlo) <= 65504.f) {  // finite mapped bound, representable lower bound
+                const uint16_t lb = __builtin_bit_cast(uint16_t, (f16)zlo);
+                const uint32_t o = (uint32_t)(lb ^ ((lb & 0x8000u) ? 0xFFFFu : 0x8000u));
+                lo = o > 2 ? o - 2 : 0;  // one step for the rounding of zlo, one for -0
+            }
+        }
+    }
+
+    const auto key_from_image = [&](uint32_t o, int idx) -> uint64_t {
+        uint16_t bits = (uint16_t)((o & 0x8000u) ? (o ^ 0x8000u) : (o ^ 0xFFFFu));
+        if (LOGSOFTMAX) {
+            const float z = (float)__builtin_bit_cast(f16, bits);
+            const f16 lp = (f16)((z - m) - lse);  // src/model/eagle.cuh:87
+            bits = __builtin_bit_cast(uint16_t, lp);
+        }
+        return make_key(bits, idx);
+    };
+    if (lo == 0) {
+        if (tid == 0) ncand = kRowCap + 1;  // no usable bound: every element is a candidate
+    } else if (lmax >= lo) {
+        // registers of this lane holding a candidate (saturating packed subtract: non-zero half <=> image >= lo)
+        const uint32_t below = (lo - 1) * 0x10001u;
+        uint32_t hits = 0;
+#pragma unroll
+        for (int r = 0; r < kRowElems / 2; ++r) {
+            const u16x2 d = __builtin_elementwise_sub_sat(__builtin_bit_cast(u16x2, img[r]), __builtin_bit_cast(u16x2, below));
+            hits |= (__builtin_bit_cast(uint32_t, d) != 0 ? 1u : 0u) << r;
+        }
+        while (hits) {
+            const int r = __builtin_ctz(hits);
+            hits &= hits - 1;
+            uint32_t o2 = img[0];
+#pragma unroll
+            for (int u = 1; u < kRowElems / 2; ++u) o2 = r == u ? img[u] : o2;
+            const int idx0 = ((r >> 2) * kRowThreads + tid) * 8 + (r & 3) * 2;
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const uint32_t o = (o2 >> (16 * h)) & 0xFFFFu;
+                if (o >= lo) {
+                    const int slot = atomicAdd(&ncand, 1);
+                    if (slot < kRowCap) cand[slot] = key_from_image(o, idx0 + h);
+                }
+            }
+        }
+    }
+    __syncthreads();
+    const int C = ncand;
+    if (C <= kRowCap) {
+        int shift = 6;
+        while ((1 << shift) < C) ++shift;
+        const int i = tid & ((1 << shift) - 1);
+        const int part = tid >> shift, nparts = kRowThreads >> shift;
+        // the mapped id of candidate tid is fetched now and used after the ranking
+        int32_t mapped = 0;
+        if (tid < C && p.ids) mapped = p.remap ? p.remap[key_index(cand[tid])] : key_index(cand[tid]);
+        if (i < C) {
+            const uint64_t my = cand[i];
+            const int chunk = (C + nparts - 1) / nparts;
+            const int j0 = part * chunk, j1 = min(C, j0 + chunk);
+            int r = 0;
+            int j = j0;
+            for (; j + 8 <= j1; j += 8) {
+                uint64_t o[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) o[u] = cand[j + u];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) r += o[u] > my ? 1 : 0;
+            }
+            for (; j < j1; ++j) r += cand[j] > my ? 1 : 0;
+            if (r) atomicAdd(&rank[i], r);
+        }
+        __syncthreads();
+        if (tid < C && rank[tid] < p.top) {
+            const uint64_t key = cand[tid];
+            const int idx = key_index(key);
+            const size_t o = (size_t)row * p.top + rank[tid];
+            p.val[o] = LOGSOFTMAX ? key_bits(key) : p.x[(size_t)row * p.dim + idx];
+            p.pos[o] = idx;
+            if (p.ids) p.ids[o] = mapped;
+        }
+        return;
+    }
+    uint64_t prev = ~0ull;
+    for (int round = 0; round < p.top; ++round) {
+        uint64_t mine = 0;
+#pragma unroll
+        for (int j = 0; j < kRowPieces; ++j) {
+            const bool pv = j * kRowThreads + tid < npieces;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const uint32_t o = (img[j * 4 + (e >> 1)] >> ((e & 1) * 16)) & 0xFFFFu;
+                const uint64_t key = pv ? key_from_image(o, (j * kRowThreads + tid) * 8 + e) : 0ull;
+                if (key < prev && key > mine) mine = key;
+            }
+        }
+        const uint64_t wbest = wave_max_u64(mine);
+        uint64_t* wb = wave_best[round & 1];
+        if (lane == 0) wb[wave] = wbest;
+        __syncthreads();
+        uint64_t best = wb[0];
+#pragma unroll
+        for (int w = 1; w < kRowWaves; ++w) best = wb[w] > best ? wb[w] : best;
+        if (tid == 0) emit_final<LOGSOFTMAX>(p, row, round, best);
+        prev = best;
+        if (best == 0) break;
+    }
+}
+
 // log_softmax in place (src/model/eagle.cuh:29-89): one workgroup per row.
 __global__ __launch_bounds__(1024) void log_softmax_kernel(uint16_t* x, int dim, float* row_stats) {
     __shared__ float red[16];
@@ -189,8 +406,6 @@ int launch_topk(const void* x, int n, int dim, int top, void* val, int32_t* pos,
     p.dim = dim;
     p.top = top;
     p.nchunks = ceil_div(dim, kChunk);
-    CPMCU_CHECK_ARG(p.nchunks * top <= kMaxCand, "topk: dim=%d with top=%d needs %d merge candidates, limit %d",
-                    dim, top, p.nchunks * top, kMaxCand);
     p.cand = (uint64_t*)workspace;
     p.val = (uint16_t*)val;
     p.pos = pos;
@@ -201,6 +416,15 @@ int launch_topk(const void* x, int n, int dim, int top, void* val, int32_t* pos,
     p.grid = stats ? stats->grid : 0;
     p.stride = stats ? stats->stride : 0;
     p.row_stats = stats ? stats->row_stats : nullptr;
+    // rows that fit one workgroup's registers: one launch, no candidate buffer
+    if (dim <= kRowMaxDim && dim % 8 == 0 && top <= kRowMaxTop && ((uintptr_t)x & 15) == 0) {
+        if (stats) hipLaunchKernelGGL(topk_row_kernel<true>, dim3(n), dim3(kRowThreads), 0, st, p);
+        else hipLaunchKernelGGL(topk_row_kernel<false>, dim3(n), dim3(kRowThreads), 0, st, p);
+        CPMCU_LAUNCH_CHECK();
+        return CPMCU_OK;
+    }
+    CPMCU_CHECK_ARG(p.nchunks * top <= kMaxCand, "topk: dim=%d with top=%d needs %d merge candidates, limit %d",
+                    dim, top, p.nchunks * top, kMaxCand);
     if (p.nchunks > 1) {
         const size_t need = (size_t)n * p.nchunks * top * sizeof(uint64_t);
         CPMCU_CHECK_ARG(workspace && workspace_bytes >= need, "topk: workspace of %zu bytes needed, %zu given", need, workspace_bytes);

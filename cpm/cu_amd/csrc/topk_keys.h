@@ -28,15 +28,55 @@ __device__ inline uint16_t key_bits(uint64_t key) {
 }
 __device__ inline int key_index(uint64_t key) { return (int)(0xFFFFFFFFu - (uint32_t)key); }
 
+// Wave-wide reductions on the DPP data path (no LDS round trip per step).  Each of the four steps
+// exchanges with the lane at xor 1, xor 2, then the mirror lane of its group of 8 and of its row of
+// 16 -- after the earlier steps the groups are uniform, so a mirror is as good as an xor -- and the
+// four row results are combined through scalar registers.  Every lane gets the result.
+template <int CTRL>
+__device__ inline uint32_t dpp_mov(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, true);
+}
+constexpr int kDppXor1 = 0xB1, kDppXor2 = 0x4E, kDppHalfMirror = 0x141, kDppMirror = 0x140;
+
+template <typename Op>
+__device__ inline uint32_t wave_reduce_b32(uint32_t v, Op op) {
+    v = op(v, dpp_mov<kDppXor1>(v));
+    v = op(v, dpp_mov<kDppXor2>(v));
+    v = op(v, dpp_mov<kDppHalfMirror>(v));
+    v = op(v, dpp_mov<kDppMirror>(v));
+    const uint32_t r0 = __builtin_amdgcn_readlane(v, 0), r1 = __builtin_amdgcn_readlane(v, 16);
+    const uint32_t r2 = __builtin_amdgcn_readlane(v, 32), r3 = __builtin_amdgcn_readlane(v, 48);
+    return op(op(r0, r1), op(r2, r3));
+}
+__device__ inline float wave_max_f32(float v) {
+    return __builtin_bit_cast(float, wave_reduce_b32(__builtin_bit_cast(uint32_t, v), [](uint32_t a, uint32_t b) {
+        return __builtin_bit_cast(uint32_t, fmaxf(__builtin_bit_cast(float, a), __builtin_bit_cast(float, b)));
+    }));
+}
+__device__ inline float wave_sum_f32(float v) {
+    return __builtin_bit_cast(float, wave_reduce_b32(__builtin_bit_cast(uint32_t, v), [](uint32_t a, uint32_t b) {
+        return __builtin_bit_cast(uint32_t, __builtin_bit_cast(float, a) + __builtin_bit_cast(float, b));
+    }));
+}
+
 __device__ inline uint64_t wave_max_u64(uint64_t v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        const uint32_t lo = __shfl_xor((uint32_t)v, off);
-        const uint32_t hi = __shfl_xor((uint32_t)(v >> 32), off);
+    const auto step = [](uint64_t a, uint32_t lo, uint32_t hi) {
         const uint64_t o = ((uint64_t)hi << 32) | lo;
-        v = o > v ? o : v;
+        return o > a ? o : a;
+    };
+    v = step(v, dpp_mov<kDppXor1>((uint32_t)v), dpp_mov<kDppXor1>((uint32_t)(v >> 32)));
+    v = step(v, dpp_mov<kDppXor2>((uint32_t)v), dpp_mov<kDppXor2>((uint32_t)(v >> 32)));
+    v = step(v, dpp_mov<kDppHalfMirror>((uint32_t)v), dpp_mov<kDppHalfMirror>((uint32_t)(v >> 32)));
+    v = step(v, dpp_mov<kDppMirror>((uint32_t)v), dpp_mov<kDppMirror>((uint32_t)(v >> 32)));
+    uint64_t best = 0;
+#pragma unroll
+    for (int r = 0; r < 64; r += 16) {
+        const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), r);
+        const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, r);
+        const uint64_t o = ((uint64_t)hi << 32) | lo;
+        best = o > best ? o : best;
     }
-    return v;
+    return best;
 }
 
 // k rounds of workgroup-wide max over the keys held in registers; round j's winner goes to
