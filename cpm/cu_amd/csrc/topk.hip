@@ -149,6 +149,9 @@ constexpr int kRowPieces = 4;                          // 16-byte pieces per thr
 constexpr int kRowElems = kRowPieces * 8;
 constexpr int kRowMaxDim = kRowThreads * kRowElems;    // 32768
 constexpr int kRowCap = kRowThreads;                   // candidate keys held in LDS
+constexpr int kRowBoundDrop = 4;                       // low bits of the bound that are not searched
+constexpr int kRowDenseWaves = 8;                      // waves that extract the candidates
+constexpr int kRowLaneCap = 512;                       // threads with candidates whose registers LDS can take
 constexpr int kRowMaxTop = 64;                         // the wave-level bound needs k <= 64 lanes
 
 typedef int16_t s16x2 __attribute__((ext_vector_type(2)));
@@ -156,12 +159,14 @@ typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
 
 template <bool LOGSOFTMAX>
 __global__ __launch_bounds__(kRowThreads) void topk_row_kernel(TopkParams p) {
-    __shared__ uint64_t cand[kRowCap];
+    __shared__ __attribute__((aligned(16))) uint64_t cand[kRowCap];
     __shared__ int rank[kRowCap];
     __shared__ uint64_t wave_best[2][kRowWaves];
     __shared__ float row_m_lse[2];
     __shared__ uint32_t wave_kth[kRowWaves];
-    __shared__ int ncand;
+    __shared__ int ncand, nlanes;
+    __shared__ uint4 lanebuf[kRowPieces][kRowLaneCap];  // piece-major: neighbouring slots are neighbouring 16 bytes
+    __shared__ int lane_owner[kRowLaneCap];
     const int row = blockIdx.x;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int npieces = p.dim >> 3;
@@ -173,28 +178,22 @@ __global__ __launch_bounds__(kRowThreads) void topk_row_kernel(TopkParams p) {
         const int pc = j * kRowThreads + tid;
         raw[j] = pc < npieces ? xr[pc] : make_uint4(~0u, ~0u, ~0u, ~0u);
     }
-    if (tid == 0) ncand = 0;
+    if (tid == 0) {
+        ncand = 0;
+        nlanes = 0;
+    }
     rank[tid] = 0;
+    cand[tid] = 0;
+    // row statistics from the GEMM's per-workgroup (max, sum exp(z - max)) partials, on wave 0: the
+    // first 256 partials are requested here and reduced after the bound search, whose instructions
+    // cover their latency
+    float pa[4], pb[4];
     if (LOGSOFTMAX && wave == 0) {
-        // row statistics from the GEMM's per-workgroup (max, sum exp(z - max)) partials, one wave
-        float a = -INFINITY, b = 0.f;
-        for (int c = lane; c < p.grid; c += 64) {
-            const float oa = p.part_max[(size_t)c * p.stride + row];
-            const float ob = p.part_sum[(size_t)c * p.stride + row];
-            const float mm = fmaxf(a, oa);
-            b = (mm == -INFINITY) ? 0.f : b * expf(a - mm) + ob * expf(oa - mm);
-            a = mm;
-        }
-        const float wm = wave_max_f32(a);
-        b = wave_sum_f32((a == -INFINITY) ? 0.f : b * expf(a - wm));
-        if (lane == 0) {
-            const float l = logf(b);
-            row_m_lse[0] = wm;
-            row_m_lse[1] = l;
-            if (p.row_stats) {
-                p.row_stats[row * 2 + 0] = wm;
-                p.row_stats[row * 2 + 1] = l;
-            }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int c = lane + u * 64;
+            pa[u] = c < p.grid ? p.part_max[(size_t)c * p.stride + row] : -INFINITY;
+            pb[u] = c < p.grid ? p.part_sum[(size_t)c * p.stride + row] : 0.f;
         }
     }
     // raw images, two per register
@@ -213,14 +212,48 @@ __global__ __launch_bounds__(kRowThreads) void topk_row_kernel(TopkParams p) {
         }
     }
     const uint32_t lmax = lmax2[0] > lmax2[1] ? lmax2[0] : lmax2[1];
-    // k-th largest of this wave's lane maxima (0 when fewer than k lanes hold anything), two bits a step
+    // k-th largest of this wave's lane maxima, rounded down to a multiple of 2^kRowBoundDrop (0 when
+    // fewer than k lanes hold anything): a slightly lower bound is as valid and costs fewer steps
+    // (with fused statistics wave 0 reduces those meanwhile and contributes no bound: any subset of
+    // the waves gives a valid one)
     uint32_t kth = 0;
-    for (int bit = 14; bit >= 0; bit -= 2) {
-        const uint32_t c1 = kth | (1u << bit), c2 = kth | (2u << bit), c3 = kth | (3u << bit);
-        const int n1 = __popcll(__ballot(lmax >= c1)), n2 = __popcll(__ballot(lmax >= c2)), n3 = __popcll(__ballot(lmax >= c3));
-        kth = n3 >= p.top ? c3 : n2 >= p.top ? c2 : n1 >= p.top ? c1 : kth;
+    if (!(LOGSOFTMAX && wave == 0)) {
+        for (int bit = 15; bit >= kRowBoundDrop; --bit) {
+            const uint32_t c = kth | (1u << bit);
+            if (__popcll(__ballot(lmax >= c)) >= p.top) kth = c;
+        }
     }
     if (lane == 0) wave_kth[wave] = kth;
+    if (LOGSOFTMAX && wave == 0) {
+        float a = -INFINITY, b = 0.f;
+        for (int c0 = lane;;) {
+            const float mm = fmaxf(fmaxf(a, fmaxf(pa[0], pa[1])), fmaxf(pa[2], pa[3]));
+            float acc = (a == -INFINITY) ? 0.f : b * __expf(a - mm);
+#pragma unroll
+            for (int u = 0; u < 4; ++u) acc += (pa[u] == -INFINITY) ? 0.f : pb[u] * __expf(pa[u] - mm);
+            a = mm;
+            b = acc;
+            c0 += 256;
+            if (c0 - lane >= p.grid) break;
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int c = c0 + u * 64;
+                pa[u] = c < p.grid ? p.part_max[(size_t)c * p.stride + row] : -INFINITY;
+                pb[u] = c < p.grid ? p.part_sum[(size_t)c * p.stride + row] : 0.f;
+            }
+        }
+        const float wm = wave_max_f32(a);
+        b = wave_sum_f32((a == -INFINITY) ? 0.f : b * __expf(a - wm));
+        if (lane == 0) {
+            const float l = __logf(b);
+            row_m_lse[0] = wm;
+            row_m_lse[1] = l;
+            if (p.row_stats) {
+                p.row_stats[row * 2 + 0] = wm;
+                p.row_stats[row * 2 + 1] = l;
+            }
+        }
+    }
     __syncthreads();
     uint32_t bound = wave_kth[0];
 #pragma unroll
@@ -254,37 +287,68 @@ __global__ __launch_bounds__(kRowThreads) void topk_row_kernel(TopkParams p) {
         }
         return make_key(bits, idx);
     };
-    if (lo == 0) {
-        if (tid == 0) ncand = kRowCap + 1;  // no usable bound: every element is a candidate
-    } else if (lmax >= lo) {
-        // registers of this lane holding a candidate (saturating packed subtract: non-zero half <=> image >= lo)
-        const uint32_t below = (lo - 1) * 0x10001u;
-        uint32_t hits = 0;
+    // threads holding anything at or above the bound hand their 16 registers to LDS ...
+    const bool bounded = lo != 0;
+    if (bounded && lmax >= lo) {
+        const int s = atomicAdd(&nlanes, 1);
+        if (s < kRowLaneCap) {
 #pragma unroll
-        for (int r = 0; r < kRowElems / 2; ++r) {
-            const u16x2 d = __builtin_elementwise_sub_sat(__builtin_bit_cast(u16x2, img[r]), __builtin_bit_cast(u16x2, below));
-            hits |= (__builtin_bit_cast(uint32_t, d) != 0 ? 1u : 0u) << r;
+            for (int j = 0; j < kRowPieces; ++j) lanebuf[j][s] = make_uint4(img[4 * j], img[4 * j + 1], img[4 * j + 2], img[4 * j + 3]);
+            lane_owner[s] = tid;
         }
-        while (hits) {
-            const int r = __builtin_ctz(hits);
-            hits &= hits - 1;
-            uint32_t o2 = img[0];
+    }
+    __syncthreads();
+    const int NT = nlanes;
+    const bool compact = bounded && NT <= kRowLaneCap;
+    // ... where a few waves take them over with most of their lanes busy: bit mask of the
+    // elements at or above the bound (saturating packed subtract: non-zero half <=> image >= lo),
+    // one exact 64-bit key per element
+    if (compact && wave < kRowDenseWaves) {
+        const u16x2 below = __builtin_bit_cast(u16x2, (lo - 1) * 0x10001u);
+        const u16x2 one2 = {1, 1};
+        const int per_wave = (NT + kRowDenseWaves - 1) / kRowDenseWaves;
+        for (int i = lane; i < per_wave; i += 64) {
+            const int s = wave * per_wave + i;
+            if (s >= NT) break;
+            // bit r: low half of register r is a candidate, bit 16 + r: its high half
+            uint32_t em = 0;
 #pragma unroll
-            for (int u = 1; u < kRowElems / 2; ++u) o2 = r == u ? img[u] : o2;
-            const int idx0 = ((r >> 2) * kRowThreads + tid) * 8 + (r & 3) * 2;
+            for (int j = 0; j < kRowPieces; ++j) {
+                const uint4 v = lanebuf[j][s];
+                const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                const uint32_t o = (o2 >> (16 * h)) & 0xFFFFu;
-                if (o >= lo) {
-                    const int slot = atomicAdd(&ncand, 1);
-                    if (slot < kRowCap) cand[slot] = key_from_image(o, idx0 + h);
+                for (int q = 0; q < 4; ++q) {
+                    const u16x2 d = __builtin_elementwise_sub_sat(__builtin_bit_cast(u16x2, w4[q]), below);
+                    em |= __builtin_bit_cast(uint32_t, __builtin_elementwise_min(d, one2)) << (4 * j + q);
                 }
+            }
+            const int owner = lane_owner[s];
+            // slots: prefix sum of the per-lane counts over the wave, one bit plane of the counts at a
+            // time, and one atomic by the first active lane
+            const int n = __popc(em);
+            const uint64_t lanes_below = (1ull << lane) - 1ull;
+            int before = 0, total = 0;
+            for (int bit = 0; __ballot((n >> bit) != 0) != 0; ++bit) {
+                const uint64_t plane = __ballot((n >> bit) & 1);
+                before += __popcll(plane & lanes_below) << bit;
+                total += __popcll(plane) << bit;
+            }
+            int base = 0;
+            if (lane == __builtin_ctzll(__ballot(true))) base = atomicAdd(&ncand, total);
+            int slot = __builtin_amdgcn_readfirstlane(base) + before;
+            while (em) {
+                const int t = __builtin_ctz(em);
+                em &= em - 1;
+                const int e = 2 * (t & 15) + (t >> 4);  // element of the owner thread
+                const uint32_t o = ((const uint16_t*)&lanebuf[e >> 3][s])[e & 7];
+                if (slot < kRowCap) cand[slot] = key_from_image(o, ((e >> 3) * kRowThreads + owner) * 8 + (e & 7));
+                ++slot;
             }
         }
     }
     __syncthreads();
     const int C = ncand;
-    if (C <= kRowCap) {
+    if (compact && C <= kRowCap) {
         int shift = 6;
         while ((1 << shift) < C) ++shift;
         const int i = tid & ((1 << shift) - 1);
@@ -293,19 +357,17 @@ __global__ __launch_bounds__(kRowThreads) void topk_row_kernel(TopkParams p) {
         int32_t mapped = 0;
         if (tid < C && p.ids) mapped = p.remap ? p.remap[key_index(cand[tid])] : key_index(cand[tid]);
         if (i < C) {
+            // slots from C on hold key 0, so whole groups of eight can be compared
             const uint64_t my = cand[i];
-            const int chunk = (C + nparts - 1) / nparts;
-            const int j0 = part * chunk, j1 = min(C, j0 + chunk);
+            const int chunk = ((C + nparts - 1) / nparts + 7) & ~7;
             int r = 0;
-            int j = j0;
-            for (; j + 8 <= j1; j += 8) {
+            for (int j = part * chunk; j < (part + 1) * chunk; j += 8) {
                 uint64_t o[8];
 #pragma unroll
                 for (int u = 0; u < 8; ++u) o[u] = cand[j + u];
 #pragma unroll
                 for (int u = 0; u < 8; ++u) r += o[u] > my ? 1 : 0;
             }
-            for (; j < j1; ++j) r += cand[j] > my ? 1 : 0;
             if (r) atomicAdd(&rank[i], r);
         }
         __syncthreads();
