@@ -22,6 +22,7 @@
 //     K-chunked and double-buffered for more rows).
 #include "common.h"
 #include "internal.h"
+#include "topk_keys.h"
 
 namespace cpmcu {
 namespace {
@@ -467,37 +468,30 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_chunked_kernel(HeadPar
     head_finish<NB>(p, ea, eb, red_a, red_b, tid, wave, lane, c);
 }
 
-// Final arg-max over the per-workgroup partials: one block per hidden row.
+// Final arg-max over the per-workgroup partials: one block per hidden row.  Largest value, lowest
+// index among equals: one 64-bit key (ordered image of the float, complemented index) per partial,
+// reduced per wave on the DPP path and across the four waves through LDS.
 __global__ __launch_bounds__(256) void head_argmax_finalize_kernel(const float* part_a, const float* part_b,
                                                                    int G, int stride, int32_t* gt) {
-    __shared__ float sa[256];
-    __shared__ int sb[256];
+    __shared__ uint64_t wave_key[4];
     const int row = blockIdx.x;
-    float a = -INFINITY;
-    int b = 0x7fffffff;
+    uint64_t best = 0;
     for (int c = threadIdx.x; c < G; c += 256) {
-        const float oa = part_a[(size_t)c * stride + row];
-        const int ob = __float_as_int(part_b[(size_t)c * stride + row]);
-        if (oa > a || (oa == a && ob < b)) {
-            a = oa;
-            b = ob;
-        }
+        const float oa = part_a[(size_t)c * stride + row] + 0.f;  // -0 -> +0: they compare equal
+        const uint32_t ob = (uint32_t)__float_as_int(part_b[(size_t)c * stride + row]);
+        const uint32_t bits = (uint32_t)__float_as_int(oa);
+        const uint32_t image = bits ^ ((bits >> 31) ? 0xFFFFFFFFu : 0x80000000u);
+        const uint64_t key = ((uint64_t)image << 32) | (0xFFFFFFFFu - ob);
+        best = key > best ? key : best;
     }
-    sa[threadIdx.x] = a;
-    sb[threadIdx.x] = b;
+    best = wave_max_u64(best);
+    if ((threadIdx.x & 63) == 0) wave_key[threadIdx.x >> 6] = best;
     __syncthreads();
-    for (int off = 128; off > 0; off >>= 1) {
-        if (threadIdx.x < off) {
-            const float oa = sa[threadIdx.x + off];
-            const int ob = sb[threadIdx.x + off];
-            if (oa > sa[threadIdx.x] || (oa == sa[threadIdx.x] && ob < sb[threadIdx.x])) {
-                sa[threadIdx.x] = oa;
-                sb[threadIdx.x] = ob;
-            }
-        }
-        __syncthreads();
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int w = 1; w < 4; ++w) best = wave_key[w] > best ? wave_key[w] : best;
+        gt[row] = (int32_t)(0xFFFFFFFFu - (uint32_t)best);
     }
-    if (threadIdx.x == 0) gt[row] = sb[0];
 }
 
 int g_num_cus = 0;

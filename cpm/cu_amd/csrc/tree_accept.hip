@@ -5,6 +5,7 @@
 // 2-byte moves for the transposed V pages.  The accept length never visits the host between the
 // three kernels: compaction reads it from device memory.
 #include "common.h"
+#include "topk_keys.h"
 
 namespace cpmcu {
 namespace {
@@ -15,9 +16,8 @@ __global__ __launch_bounds__(128) void tree_accept_kernel(int T, int W, int32_t*
                                                           const uint64_t* mask, const int32_t* parent,
                                                           int32_t* best) {
     __shared__ uint64_t s_correct[2];
-    __shared__ int32_t mx[128], mi[128];
+    __shared__ uint32_t s_best[2];
     const int i = threadIdx.x;
-    const int S = T > 64 ? 128 : 64;  // tournament slots: next_pow2(max(64, T))
     // :9-20  correct bit i <=> i == 0 or pred[i] == gt[parent[i]]
     const bool ok = (i == 0) || (i < T && pred[i] == gt[parent[i]]);
     const uint64_t ballot = __ballot(ok);
@@ -32,23 +32,22 @@ __global__ __launch_bounds__(128) void tree_accept_kernel(int T, int W, int32_t*
             if ((s_correct[w] & mw) != mw) full = false;
         }
     }
-    mx[i] = full ? pos[i] - P + 1 : 1;
-    mi[i] = full ? i : 0;
+    // :30-36  the tournament folds the slots in halves and the upper slot wins only when strictly
+    // greater, so two nodes of equal length meet in the round of their lowest differing index bit and
+    // the one with that bit clear wins: a maximum over (accepted length, bit-reversed node index
+    // ascending).  One key per node, reduced per wave on the DPP path and across the two waves through
+    // LDS.  A node that does not count enters as (1, node 0), the root's entry.
+    const uint32_t key = full ? ((uint32_t)(pos[i] - P + 1) << 8) | (255u - (__brev((uint32_t)i) >> 24)) : (1u << 8) | 255u;
+    const uint32_t wkey = wave_reduce_b32(key, [](uint32_t a, uint32_t b) { return a > b ? a : b; });
+    if ((i & 63) == 0) s_best[i >> 6] = wkey;
     __syncthreads();
-    // :30-36  tournament, upper slot wins only when strictly greater
-    for (int off = S >> 1; off > 0; off >>= 1) {
-        if (i < off && mx[i + off] > mx[i]) {
-            mx[i] = mx[i + off];
-            mi[i] = mi[i + off];
-        }
-        __syncthreads();
-    }
+    const uint32_t bkey = s_best[0] > s_best[1] ? s_best[0] : s_best[1];
+    const int p = (int)(__brev(255u - (bkey & 255u)) >> 24);
     if (i == 0) {
-        best[0] = mx[0];
-        best[1] = mi[0];
+        best[0] = (int32_t)(bkey >> 8);
+        best[1] = p;
     }
     // :42-45  scatter the accepted path (node indices by depth) into pred
-    const int p = mi[0];
     if (i < T && ((mask[(size_t)p * W + (i >> 6)] >> (i & 63)) & 1ull)) pred[pos[i] - P] = i;
 }
 
