@@ -234,7 +234,21 @@ def main():
             ops.tree_accept(vs.pred, vs.gt, wl.pos, vs.cache_length, wl.mask, wl.parent, best=vs.best)
             ops.kv_compact(wl.cache, vs.pred, vs.gt, vs.cache_length, vs.best, wl.T)
 
+    # the one-call tail of verify(): the same two launches also gather the accepted hidden rows, write
+    # next position ids and the packed (a, ids) result (length advance off here: the call is repeated)
+    prev_hidden = torch.zeros_like(wl.hidden)
+    next_pos = torch.zeros(wl.T, dtype=torch.int32, device="cuda")
+    packed = torch.zeros(1 + wl.T, dtype=torch.int32, device="cuda")
+
+    def accept_commit():
+        for _ in range(TAIL_REP):
+            vs.pred.copy_(wl.draft_ids)
+            ops.tree_accept(vs.pred, vs.gt, wl.pos, vs.cache_length, wl.mask, wl.parent, best=vs.best)
+            ops.accept_commit(wl.cache, vs.pred, vs.gt, vs.cache_length, vs.best, wl.T, hidden=wl.hidden, prev_hidden=prev_hidden,
+                              next_position_ids=next_pos, result=packed)
+
     ms_attn = timed_replays(torch, attn_all_layers, reps, 2, use_graph)[0] / wl.L
+    ms_commit = timed_replays(torch, accept_commit, reps, 2, use_graph)[0] / TAIL_REP
     ms_head = timed_replays(torch, head_only, reps, 2, use_graph)[0] / HEAD_REP
     ms_tail = timed_replays(torch, accept_compact, reps, 2, use_graph)[0] / TAIL_REP
 
@@ -337,6 +351,8 @@ def main():
         "roofline": roofline,
         "kernels": kernels,
         "frspec_head": frspec,
+        "commit_tail": {"kernel": "tree_accept_kernel+kv_compact_kernel(with hidden-row gather)+accepted_ids_kernel(ids, positions, packed result)",
+                        "us_per_call": round(ms_commit * 1e3, 2)},
         "contexts_us_per_step": contexts,
         "attention_by_context": ctx_attn,
         "cpu_baseline": cpu,

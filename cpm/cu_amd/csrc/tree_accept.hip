@@ -60,6 +60,11 @@ struct CompactParams {
     const int32_t* cache_length;
     const int32_t* best;
     int max_accept;
+    // accepted hidden rows (remap_hidden): extra workgroups behind the num_cache_blocks cache streams
+    int num_cache_blocks;
+    const f16x8* hidden;
+    f16x8* prev_hidden;
+    int hidden_pieces;  // 16-byte pieces per hidden row
 };
 
 // fix_kvcache_kernel_1/2, src/model/tree_drafter.cuh:48-77, on the paged layout.  One workgroup per
@@ -67,6 +72,18 @@ struct CompactParams {
 // is written; batches go in depth order, and because path[d] >= d a later batch never reads a row
 // an earlier batch wrote -- so the reference's staging buffer is not needed.
 __global__ __launch_bounds__(256) void kv_compact_kernel(CompactParams p) {
+    if ((int)blockIdx.x >= p.num_cache_blocks) {
+        // remap_hidden, src/model/eagle.cuh:108-115 (scale 1): prev_hidden[d] = hidden[path[d]], one row per
+        // workgroup; the path is still in pred because the ids replace it in a later launch
+        const int d = blockIdx.x - p.num_cache_blocks;
+        int a = p.best[0];
+        a = a < p.max_accept ? a : p.max_accept;
+        if (d >= a) return;
+        const f16x8* src = p.hidden + (size_t)p.pred[d] * p.hidden_pieces;
+        f16x8* dst = p.prev_hidden + (size_t)d * p.hidden_pieces;
+        for (int i = threadIdx.x; i < p.hidden_pieces; i += 256) dst[i] = src[i];
+        return;
+    }
     const int g = blockIdx.x % p.Hkv;
     const int kv = (blockIdx.x / p.Hkv) & 1;
     const int layer = blockIdx.x / (2 * p.Hkv);
@@ -118,15 +135,38 @@ __global__ __launch_bounds__(256) void kv_compact_kernel(CompactParams p) {
     }
 }
 
-// src/model/tree_drafter.cuh:74-76: pred[d] <- gt[pred[d]] once every cache has been moved.
-__global__ void accepted_ids_kernel(int32_t* pred, const int32_t* gt, const int32_t* best, int max_accept) {
+// src/model/tree_drafter.cuh:74-76: pred[d] <- gt[pred[d]] once every cache has been moved -- plus, for
+// the one-call form of verify(), what the reference does on the host or in one-line kernels after it
+// (src/model/minicpm4/minicpm4_eagle.cuh:411, cpmcu/speculative/tree_drafter.py:222,247-249):
+//   next_position_ids[d] = P + d (make_arange, src/model/eagle.cuh:125-127,184-186), result = (a, ids),
+//   cache_length += a (and the P + T scalar of the attention calls with it), pred[0] = last accepted id
+//   (the next tree's root).
+__global__ __launch_bounds__(128) void accepted_ids_kernel(int32_t* pred, const int32_t* gt, const int32_t* best, int max_accept,
+                                                           int32_t* cache_length, int32_t* kv_len, int32_t* next_position_ids,
+                                                           int32_t* result, int flags) {
     int a = best[0];
     a = a < max_accept ? a : max_accept;
     const int d = threadIdx.x;
+    const int P = cache_length ? cache_length[0] : 0;
     int id = 0;
     if (d < a) id = gt[pred[d]];
     __syncthreads();
-    if (d < a) pred[d] = id;
+    if (d < a) {
+        pred[d] = id;
+        if (next_position_ids) next_position_ids[d] = P + d;
+        if (result) result[1 + d] = id;
+    }
+    if (d == 0) {
+        if (result) result[0] = a;
+        if (flags & CPMCU_COMMIT_ADVANCE_LENGTH) {
+            cache_length[0] = P + a;
+            if (kv_len) kv_len[0] += a;
+        }
+    }
+    if (flags & CPMCU_COMMIT_NEXT_ROOT) {
+        __syncthreads();
+        if (d == a - 1) pred[0] = id;
+    }
 }
 
 // copy_to_kvcache, src/model/attn.cuh:14-21: token t of the T new rows goes to position *kv_len - T + t.
@@ -175,11 +215,35 @@ extern "C" int cpmcu_kv_compact(void* const* k_pools, void* const* v_pools, int 
                     "kv_compact: null pointer argument");
     CPMCU_CHECK_ARG(num_layers >= 1 && Hkv >= 1, "kv_compact: num_layers=%d Hkv=%d", num_layers, Hkv);
     CPMCU_CHECK_ARG(max_accept >= 1 && max_accept <= kMaxTree, "kv_compact: max_accept=%d outside [1, %d]", max_accept, kMaxTree);
-    CompactParams p{k_pools, v_pools, block_table, Hkv, pred, cache_length, best, max_accept};
+    CompactParams p{k_pools, v_pools, block_table, Hkv, pred, cache_length, best, max_accept, num_layers * 2 * Hkv, nullptr, nullptr, 0};
     hipStream_t st = resolve_stream(stream);
-    hipLaunchKernelGGL(kv_compact_kernel, dim3(num_layers * 2 * Hkv), dim3(256), 0, st, p);
+    hipLaunchKernelGGL(kv_compact_kernel, dim3(p.num_cache_blocks), dim3(256), 0, st, p);
     CPMCU_LAUNCH_CHECK();
-    hipLaunchKernelGGL(accepted_ids_kernel, dim3(1), dim3(128), 0, st, pred, gt, best, max_accept);
+    hipLaunchKernelGGL(accepted_ids_kernel, dim3(1), dim3(128), 0, st, pred, gt, best, max_accept, (int32_t*)nullptr,
+                       (int32_t*)nullptr, (int32_t*)nullptr, (int32_t*)nullptr, 0);
+    CPMCU_LAUNCH_CHECK();
+    return CPMCU_OK;
+}
+
+extern "C" int cpmcu_accept_commit(void* const* k_pools, void* const* v_pools, int num_layers,
+                                   const int32_t* block_table, int Hkv, int32_t* pred, const int32_t* gt,
+                                   int32_t* cache_length, int32_t* kv_len, const int32_t* best, int max_accept,
+                                   const void* hidden, int hidden_dim, void* prev_hidden, int32_t* next_position_ids,
+                                   int32_t* result, int flags, void* stream) {
+    CPMCU_CHECK_ARG(k_pools && v_pools && block_table && pred && gt && cache_length && best,
+                    "accept_commit: null pointer argument");
+    CPMCU_CHECK_ARG(num_layers >= 1 && Hkv >= 1, "accept_commit: num_layers=%d Hkv=%d", num_layers, Hkv);
+    CPMCU_CHECK_ARG(max_accept >= 1 && max_accept <= kMaxTree, "accept_commit: max_accept=%d outside [1, %d]", max_accept, kMaxTree);
+    CPMCU_CHECK_ARG((hidden == nullptr) == (prev_hidden == nullptr), "accept_commit: hidden and prev_hidden go together");
+    CPMCU_CHECK_ARG(!hidden || (hidden_dim >= 8 && hidden_dim % 8 == 0), "accept_commit: hidden_dim=%d must be a positive multiple of 8", hidden_dim);
+    CPMCU_CHECK_ARG((flags & ~(CPMCU_COMMIT_ADVANCE_LENGTH | CPMCU_COMMIT_NEXT_ROOT)) == 0, "accept_commit: unknown flags 0x%x", flags);
+    CompactParams p{k_pools, v_pools, block_table, Hkv, pred, cache_length, best, max_accept, num_layers * 2 * Hkv,
+                    (const f16x8*)hidden, (f16x8*)prev_hidden, hidden ? hidden_dim / 8 : 0};
+    hipStream_t st = resolve_stream(stream);
+    hipLaunchKernelGGL(kv_compact_kernel, dim3(p.num_cache_blocks + (hidden ? max_accept : 0)), dim3(256), 0, st, p);
+    CPMCU_LAUNCH_CHECK();
+    hipLaunchKernelGGL(accepted_ids_kernel, dim3(1), dim3(128), 0, st, pred, gt, best, max_accept, cache_length,
+                       kv_len, next_position_ids, result, flags);
     CPMCU_LAUNCH_CHECK();
     return CPMCU_OK;
 }

@@ -54,6 +54,7 @@ SIGNATURES = {
     "cpmcu_remap": (c_int, [_P, c_int, _P, _P, _P]),
     "cpmcu_tree_accept": (c_int, [c_int, _P, _P, _P, _P, _P, c_int, _P, _P, _P]),
     "cpmcu_kv_compact": (c_int, [_P, _P, c_int, _P, c_int, _P, _P, _P, _P, c_int, _P]),
+    "cpmcu_accept_commit": (c_int, [_P, _P, c_int, _P, c_int, _P, _P, _P, _P, _P, c_int, _P, c_int, _P, _P, _P, c_int, _P]),
     "cpmcu_draft_tree_state_bytes": (c_size_t, [c_int, c_int]),
     "cpmcu_draft_tree_begin": (c_int, [_P, c_int, c_int, _P, _P, _P, _P, _P, _P]),
     "cpmcu_draft_tree_extend": (c_int, [_P, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P]),

@@ -23,6 +23,14 @@ def _ptr(t):
     return ctypes.c_void_p(t.data_ptr())
 
 
+def _ptr_result(t):
+    """Like _ptr, but a pinned host tensor may stand in: the GPU writes it through the mapped address."""
+    if t is None:
+        return None
+    assert (t.is_cuda or t.is_pinned()) and t.is_contiguous(), "device-resident or pinned contiguous tensor required"
+    return ctypes.c_void_p(t.data_ptr())
+
+
 def _stream():
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
@@ -193,6 +201,22 @@ def kv_compact(cache, pred, gt, cache_length, best, max_accept):
     """fix_kv_cache (src/model/tree_drafter.cuh:48-77) on every layer of the paged cache."""
     _lib().kv_compact(_ptr(cache.k_ptrs), _ptr(cache.v_ptrs), cache.num_layers, _ptr(cache.block_table), cache.Hkv,
                       _ptr(pred), _ptr(gt), _ptr(cache_length), _ptr(best), int(max_accept), _stream())
+
+
+COMMIT_ADVANCE_LENGTH = 1
+COMMIT_NEXT_ROOT = 2
+
+
+def accept_commit(cache, pred, gt, cache_length, best, max_accept, hidden=None, prev_hidden=None,
+                  next_position_ids=None, result=None, advance_length=False, next_root=False, kv_len=None):
+    """The rest of verify() after the acceptance (src/model/minicpm4/minicpm4_eagle.cuh:398-418): compaction,
+    accepted ids, gather of the accepted hidden rows, next position ids, packed (a, ids) result and the
+    device-side advance of cache_length, in two launches with the accept length staying on the device."""
+    flags = (COMMIT_ADVANCE_LENGTH if advance_length else 0) | (COMMIT_NEXT_ROOT if next_root else 0)
+    hidden_dim = 0 if hidden is None else hidden.shape[-1]
+    _lib().accept_commit(_ptr(cache.k_ptrs), _ptr(cache.v_ptrs), cache.num_layers, _ptr(cache.block_table), cache.Hkv,
+                         _ptr(pred), _ptr(gt), _ptr(cache_length), _ptr(kv_len), _ptr(best), int(max_accept), _ptr(hidden), hidden_dim,
+                         _ptr(prev_hidden), _ptr(next_position_ids), _ptr_result(result), flags, _stream())
 
 
 class DraftTree:

@@ -282,6 +282,27 @@ int cpmcu_kv_compact(void* const* k_pools, void* const* v_pools, int num_layers,
                      int Hkv, int32_t* pred, const int32_t* gt, const int32_t* cache_length,
                      const int32_t* best, int max_accept, void* stream);
 
+/* The rest of verify() in the same two launches as cpmcu_kv_compact --
+ * MiniCPM4EagleImpl::verify, src/model/minicpm4/minicpm4_eagle.cuh:398-418, and the host side of the
+ * loop, cpmcu/speculative/tree_drafter.py:222,243-249.  On top of the compaction and the accepted ids:
+ *   prev_hidden[d][:] = hidden[path[d]][:] for d < a   (remap_hidden, src/model/eagle.cuh:108-115,169-172;
+ *       hidden [T][hidden_dim] fp16 = the target's final-norm output; both NULL: skipped);
+ *   next_position_ids[d] = P + d for d < a             (make_arange, src/model/eagle.cuh:125-127,184-186; NULL: skipped);
+ *   result[0] = a, result[1 + d] = accepted id d       (int32[1 + max_accept]; device memory or pinned,
+ *       device-visible host memory: one read after one synchronisation replaces the reference's
+ *       reads of the accept length and of tree_draft_ids[:a]; NULL: skipped);
+ *   CPMCU_COMMIT_ADVANCE_LENGTH: cache_length[0] = P + a on the device (the host's
+ *       cache_length[0] = prefix_length + i of the next iteration), and kv_len[0] += a when kv_len is
+ *       given: the device scalar P + T that the attention calls read (cpmcu/llm.py:272), so the next
+ *       step can be enqueued, or a captured graph of it replayed, without the host knowing a;
+ *   CPMCU_COMMIT_NEXT_ROOT: pred[0] = the last accepted id (tree_draft_ids[0] = tree_draft_ids[a - 1]). */
+#define CPMCU_COMMIT_ADVANCE_LENGTH 1
+#define CPMCU_COMMIT_NEXT_ROOT 2
+int cpmcu_accept_commit(void* const* k_pools, void* const* v_pools, int num_layers, const int32_t* block_table,
+                        int Hkv, int32_t* pred, const int32_t* gt, int32_t* cache_length, int32_t* kv_len,
+                        const int32_t* best, int max_accept, const void* hidden, int hidden_dim, void* prev_hidden,
+                        int32_t* next_position_ids, int32_t* result, int flags, void* stream);
+
 /* ---- Draft-tree construction around the FR-Spec head (the tree bookkeeping of draft()) ----
  * src/model/minicpm4/minicpm4_eagle.cuh:319-393 with src/model/eagle.cuh:91-106,121-127,188-214.
  * k = topk_per_iter (<= 32), num_iter iterations (k * num_iter <= 64: the draft mask is one

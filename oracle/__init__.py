@@ -44,6 +44,7 @@ def _load():
         "orc_argmax": (None, [c_p, i32, i32, c_p]),
         "orc_tree_accept": (i32, [i32, i32, c_p, c_p, c_p, i32, c_p, c_p, c_p, c_p]),
         "orc_kv_compact": (None, [c_p, i32, i32, i32, i32, c_p, c_p, c_p]),
+        "orc_accept_commit": (None, [c_p, i32, i32, i32, i32, c_p, c_p, c_p, i32, c_p, c_p, c_p, c_p, c_p]),
         "orc_draft_tree_begin": (None, [i32, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p]),
         "orc_draft_tree_extend": (None, [i32, i32, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p]),
         "orc_draft_tree_finish": (None, [i32, i32, i32, i32, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p]),
@@ -205,6 +206,31 @@ def kv_compact(caches, P, path, gt):
     ids = np.empty(a, np.int32)
     _lib.orc_kv_compact(ptrs, len(caches), row_halves, int(P), a, _p(path), _p(gt), _p(ids))
     return ids
+
+
+def accept_commit(caches, P, path, gt, hidden=None):
+    """verify() after the acceptance (src/model/minicpm4/minicpm4_eagle.cuh:403-411) on host arrays; caches are
+    modified in place.  Returns dict(prev_hidden [a,H] or None, next_pos [a], result [1+a] = (a, ids), new_length, next_root)."""
+    path = _c(path, np.int32)
+    gt = _c(gt, np.int32)
+    a = path.size
+    for c in caches:
+        assert c.dtype == np.float16 and c.flags.c_contiguous
+    row_halves = caches[0].shape[1]
+    ptrs = (ctypes.c_void_p * len(caches))(*[c.ctypes.data for c in caches])
+    H = 0
+    prev = None
+    if hidden is not None:
+        hidden = _c(hidden, np.float16)
+        H = hidden.shape[1]
+        prev = np.zeros((a, H), np.float16)
+    next_pos = np.empty(a, np.int32)
+    result = np.empty(1 + a, np.int32)
+    new_len = np.zeros(1, np.int32)
+    root = np.zeros(1, np.int32)
+    _lib.orc_accept_commit(ptrs, len(caches), row_halves, int(P), a, _p(path), _p(gt), _p(hidden), H, _p(prev),
+                           _p(next_pos), _p(result), _p(new_len), _p(root))
+    return dict(prev_hidden=prev, next_pos=next_pos, result=result, new_length=int(new_len[0]), next_root=int(root[0]))
 
 
 class DraftTree:

@@ -351,6 +351,27 @@ void orc_kv_compact(uint16_t* const* caches, int num_caches, int row_halves, int
         for (int d = 0; d < a; ++d) ids_out[d] = gt[path[d]];  // :74-76
 }
 
+// f2/f3 -- the rest of MiniCPM4EagleImpl::verify after the acceptance, src/model/minicpm4/minicpm4_eagle.cuh:403-411,
+// and the host side of the loop, cpmcu/speculative/tree_drafter.py:222,243-249.
+//   prev_hidden[d] = hidden[path[d] / scale]      remap_hidden_kernel, src/model/eagle.cuh:108-115 (scale 1 at :404)
+//   fix_kv_cache                                   orc_kv_compact
+//   next_pos[d] = d + P                            make_arange_kernel, src/model/eagle.cuh:125-127, called with num_prev = a
+//   result = (a, ids), *new_length = P + a, *next_root = ids[a - 1]
+void orc_accept_commit(uint16_t* const* caches, int num_caches, int row_halves, int P, int a, const int32_t* path,
+                       const int32_t* gt, const uint16_t* hidden, int hidden_dim, uint16_t* prev_hidden,
+                       int32_t* next_pos, int32_t* result, int32_t* new_length, int32_t* next_root) {
+    if (hidden)
+        for (int d = 0; d < a; ++d) {
+            const int real_row = path[d] / 1;
+            for (int i = 0; i < hidden_dim; ++i) prev_hidden[(size_t)d * hidden_dim + i] = hidden[(size_t)real_row * hidden_dim + i];
+        }
+    orc_kv_compact(caches, num_caches, row_halves, P, a, path, gt, result + 1);
+    result[0] = a;
+    for (int d = 0; d < a; ++d) next_pos[d] = d + P;
+    *new_length = P + a;
+    *next_root = result[a];
+}
+
 // f1 -- d = 0 of draft(): src/model/minicpm4/minicpm4_eagle.cuh:319-332, init_tree src/model/eagle.cuh:91-93
 void orc_draft_tree_begin(int k, const uint16_t* val, const int32_t* pos, const int32_t* token_id_remap,
                           uint16_t* tried_val, int32_t* tried_pos, uint16_t* cum, uint64_t* mask, int32_t* next_ids) {

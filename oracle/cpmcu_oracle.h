@@ -139,6 +139,9 @@ int orc_tree_accept(int T, int mask_words, const int32_t* pred, const int32_t* g
  * pinned by: numpy fancy-index copy; overlap case path=[0,2,3]. */
 void orc_kv_compact(uint16_t* const* caches, int num_caches, int row_halves, int P, int a,
                     const int32_t* path, const int32_t* gt, int32_t* ids_out);
+void orc_accept_commit(uint16_t* const* caches, int num_caches, int row_halves, int P, int a, const int32_t* path,
+                       const int32_t* gt, const uint16_t* hidden, int hidden_dim, uint16_t* prev_hidden,
+                       int32_t* next_pos, int32_t* result, int32_t* new_length, int32_t* next_root);
 
 /* ---- f1: draft-tree construction around the FR-Spec head ----
  * src/model/minicpm4/minicpm4_eagle.cuh:319-393 (the tree bookkeeping of draft()), with

@@ -110,6 +110,102 @@ def test_compaction_overlap_and_long_paths(gpu, orc):
     _compact_case(gpu, orc, synth.tree_from_parents(parents), 511, 49, layers=2, seed=3)
 
 
+def _commit_case(torch, orc, tree, P, leaf_depth, layers, seed, H=512, pinned_result=False):
+    """cpmcu_accept_commit against the oracle's restatement of verify()'s tail and against the separate operators."""
+    from cpm.cu_amd import ops
+    from cpm.cu_amd.kvcache import PagedKVCache
+    T = tree.T
+    S = P + T
+    npages = (S + 255) // 256 + 1
+    table = synth.rng(seed, 4).permutation(npages).astype(np.int32)
+    caches = [PagedKVCache(layers, HKV, npages, block_table=table) for _ in range(2)]
+    flat = []
+    for layer in range(layers):
+        k = synth.normal_f16((S, HKV, D), seed, 10 + layer)
+        v = synth.normal_f16((S, HKV, D), seed, 50 + layer)
+        for c in caches:
+            c.write_logical(layer, 0, to_dev(torch, k), to_dev(torch, v))
+        flat += [k.reshape(S, HKV * D).copy(), v.reshape(S, HKV * D).copy()]
+    gt = synth.rng(seed, 9).integers(0, VOCAB, T).astype(np.int32)
+    pred, leaf = synth.draft_ids_for_accept(tree, gt, leaf_depth, VOCAB, seed)
+    hidden = synth.normal_f16((T, H), seed, 90)
+    pos = tree.positions(P)
+    a, _, path = orc.tree_accept(pred, gt, pos, P, tree.mask, tree.parent)
+    want = orc.accept_commit(flat, P, path, gt, hidden)
+    assert np.array_equal(want["prev_hidden"].view(np.uint16), hidden[path].view(np.uint16))
+
+    d_gt, d_pos, d_mask, d_par = to_dev(torch, gt), to_dev(torch, pos), to_dev(torch, tree.mask), to_dev(torch, tree.parent)
+    # separate operators on the first copy
+    p1 = to_dev(torch, pred)
+    len1 = torch.tensor([P], dtype=torch.int32, device="cuda")
+    best1 = ops.tree_accept(p1, d_gt, d_pos, len1, d_mask, d_par)
+    ops.kv_compact(caches[0], p1, d_gt, len1, best1, T)
+    # the one-call form on the second
+    p2 = to_dev(torch, pred)
+    len2 = torch.tensor([P], dtype=torch.int32, device="cuda")
+    best2 = ops.tree_accept(p2, d_gt, d_pos, len2, d_mask, d_par)
+    d_hidden = to_dev(torch, hidden)
+    prev = torch.full((T, H), 7.0, dtype=torch.float16, device="cuda")
+    npos = torch.full((T,), -1, dtype=torch.int32, device="cuda")
+    if pinned_result:
+        result = torch.full((1 + T,), -1, dtype=torch.int32).pin_memory()
+    else:
+        result = torch.full((1 + T,), -1, dtype=torch.int32, device="cuda")
+    ops.accept_commit(caches[1], p2, d_gt, len2, best2, T, hidden=d_hidden, prev_hidden=prev, next_position_ids=npos,
+                      result=result, advance_length=True, next_root=True)
+    torch.cuda.synchronize()
+    res = result.numpy() if pinned_result else to_np(result)
+    assert int(to_np(best2)[0]) == a and res[0] == a
+    assert np.array_equal(res[: 1 + a], want["result"])
+    assert np.all(res[1 + a:] == -1)
+    assert int(to_np(len2)[0]) == want["new_length"] == P + a and int(to_np(len1)[0]) == P
+    assert np.array_equal(to_np(npos)[:a], want["next_pos"]) and np.all(to_np(npos)[a:] == -1)
+    assert np.array_equal(to_np(prev)[:a].view(np.uint16), want["prev_hidden"].view(np.uint16))
+    assert np.all(to_np(prev)[a:] == 7.0)  # rows beyond the accept length are not touched
+    ids1 = to_np(p1)[:a]
+    ids2 = to_np(p2)[:a].copy()
+    assert int(ids2[0]) == want["next_root"]  # the next tree's root
+    ids2[0] = res[1]
+    assert np.array_equal(ids1, ids2) and np.array_equal(ids1, want["result"][1:])
+    for layer in range(layers):
+        for c in caches:
+            k_dev, v_dev = c.read_logical(layer, 0, P + a)
+            assert np.array_equal(to_np(k_dev).reshape(P + a, -1).view(np.uint16), flat[2 * layer][: P + a].view(np.uint16))
+            assert np.array_equal(to_np(v_dev).reshape(P + a, -1).view(np.uint16), flat[2 * layer + 1][: P + a].view(np.uint16))
+    return a
+
+
+def test_accept_commit_every_depth(gpu, orc):
+    tree = synth.eagle_tree(6, 10, 60, seed=0)
+    for depth in range(int(tree.depth.max()) + 1):
+        assert _commit_case(gpu, orc, tree, 4096 - 7, depth, layers=3, seed=depth) == depth + 1
+    wide = synth.eagle_tree(8, 16, 128, seed=1)
+    _commit_case(gpu, orc, wide, 1000, int(wide.depth.max()), layers=2, seed=31, H=4096)
+    _commit_case(gpu, orc, synth.chain_tree(128), 250, 127, layers=2, seed=32, H=64)
+
+
+def test_accept_commit_result_in_pinned_host_memory(gpu, orc):
+    """The packed (a, ids) result written straight into pinned host memory: one synchronisation, no copy call."""
+    tree = synth.eagle_tree(6, 10, 60, seed=2)
+    _commit_case(gpu, orc, tree, 777, 3, layers=2, seed=40, pinned_result=True)
+
+
+def test_accept_commit_argument_checks(gpu):
+    from cpm.cu_amd import ops
+    from cpm.cu_amd.kvcache import PagedKVCache
+    torch = gpu
+    cache = PagedKVCache(1, HKV, 2)
+    i32 = lambda n: torch.zeros(n, dtype=torch.int32, device="cuda")
+    hidden = torch.zeros((4, 64), dtype=torch.float16, device="cuda")
+    with pytest.raises(ValueError):
+        ops.accept_commit(cache, i32(4), i32(4), i32(1), i32(2), 4, hidden=hidden)  # hidden without prev_hidden
+    with pytest.raises(ValueError):
+        ops.accept_commit(cache, i32(4), i32(4), i32(1), i32(2), 129)  # max_accept beyond the tree limit
+    odd = torch.zeros((4, 60), dtype=torch.float16, device="cuda")
+    with pytest.raises(ValueError):
+        ops.accept_commit(cache, i32(4), i32(4), i32(1), i32(2), 4, hidden=odd, prev_hidden=odd.clone())  # 60 % 8
+
+
 def test_model_level_entry_points(gpu, orc):
     """init_* -> init_storage -> load_model -> decode_attention / decode_lm_head / draft_head /
     verify_and_fix on the library-owned paged cache, against the oracle; and the error contract."""

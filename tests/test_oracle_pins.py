@@ -332,3 +332,26 @@ def test_attention_mask_range_wider_than_queries(orc):
     vt = torch.from_numpy(v.astype(np.float32)).permute(1, 0, 2).repeat_interleave(Hq // Hkv, 0)
     ref = torch.nn.functional.scaled_dot_product_attention(qt, kt, vt, attn_mask=torch.from_numpy(vis)).permute(1, 0, 2).numpy()
     assert np.abs(out - ref).max() < 5e-3
+
+
+def test_accept_commit_tail_against_numpy():
+    """The oracle's restatement of verify() after the acceptance, pinned on what fixes it independently:
+    the hidden gather is numpy fancy indexing, compaction is "rows P+path[d] land at P+d, nothing else
+    moves" (checked on rows tagged with their own index), positions are an arange, ids are gt[path]."""
+    import oracle as orc
+    rng = np.random.default_rng(5)
+    P, T, H, rows = 37, 20, 24, 80
+    path = np.array([0, 3, 4, 9, 17], np.int32)  # increasing, path[d] >= d
+    gt = rng.integers(0, 1000, T).astype(np.int32)
+    hidden = rng.standard_normal((T, H)).astype(np.float16)
+    caches = [np.repeat(np.arange(rows, dtype=np.float16)[:, None], 8, 1) + np.float16(c) * 0 for c in range(3)]
+    before = [c.copy() for c in caches]
+    out = orc.accept_commit(caches, P, path, gt, hidden)
+    a = len(path)
+    assert np.array_equal(out["prev_hidden"].view(np.uint16), hidden[path].view(np.uint16))
+    assert np.array_equal(out["next_pos"], P + np.arange(a))
+    assert np.array_equal(out["result"], np.concatenate([[a], gt[path]]))
+    assert out["new_length"] == P + a and out["next_root"] == gt[path[-1]]
+    for c, b in zip(caches, before):
+        assert np.array_equal(c[:P], b[:P]) and np.array_equal(c[P + a:], b[P + a:])
+        assert np.array_equal(c[P:P + a, 0], (P + path).astype(np.float16))  # the tag of the source row
