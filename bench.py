@@ -247,7 +247,29 @@ def main():
             ops.accept_commit(wl.cache, vs.pred, vs.gt, vs.cache_length, vs.best, wl.T, hidden=wl.hidden, prev_hidden=prev_hidden,
                               next_position_ids=next_pos, result=packed)
 
+    # rotary embedding of the tree rows: fused into the attention kernel (one table per step) against the
+    # reference's order (one in-place launch per layer in front of the attention)
+    inv_freq = torch.tensor((10000.0 ** (-np.arange(64, dtype=np.float64) / 64)).astype(np.float32), device="cuda")
+    q_scratch = [t.clone() for t in wl.q]
+    k_scratch = [t.clone() for t in wl.k_new]
+
+    def attn_rope_fused():
+        table = ops.rope_table(wl.pos, inv_freq)
+        for l in range(wl.L):
+            ops.tree_attention(wl.q[l], wl.cache, l, vs.kv_len, vs.max_kv_len, wl.mask, num_splits=args.splits, out=wl.attn_out[l],
+                               k_new=wl.k_new[l], v_new=wl.v_new[l], rope=table)
+
+    def attn_rope_separate():
+        table = ops.rope_table(wl.pos, inv_freq)
+        for l in range(wl.L):
+            ops.rope_apply_(table, q_scratch[l], k_scratch[l])
+            ops.tree_attention(q_scratch[l], wl.cache, l, vs.kv_len, vs.max_kv_len, wl.mask, num_splits=args.splits, out=wl.attn_out[l],
+                               k_new=k_scratch[l], v_new=wl.v_new[l])
+
     ms_attn = timed_replays(torch, attn_all_layers, reps, 2, use_graph)[0] / wl.L
+    ms_rope_fused = timed_replays(torch, attn_rope_fused, reps, 2, use_graph)[0] / wl.L
+    ms_rope_sep = timed_replays(torch, attn_rope_separate, reps, 2, use_graph)[0] / wl.L
+    del q_scratch, k_scratch
     ms_commit = timed_replays(torch, accept_commit, reps, 2, use_graph)[0] / TAIL_REP
     ms_head = timed_replays(torch, head_only, reps, 2, use_graph)[0] / HEAD_REP
     ms_tail = timed_replays(torch, accept_compact, reps, 2, use_graph)[0] / TAIL_REP
@@ -351,6 +373,8 @@ def main():
         "roofline": roofline,
         "kernels": kernels,
         "frspec_head": frspec,
+        "attention_with_rope": {"fused_us_per_layer": round(ms_rope_fused * 1e3, 2), "separate_launch_us_per_layer": round(ms_rope_sep * 1e3, 2),
+                                "note": "rotary embedding of q and the appended K rows; table computed once per step"},
         "commit_tail": {"kernel": "tree_accept_kernel+kv_compact_kernel(with hidden-row gather)+accepted_ids_kernel(ids, positions, packed result)",
                         "us_per_call": round(ms_commit * 1e3, 2)},
         "contexts_us_per_step": contexts,

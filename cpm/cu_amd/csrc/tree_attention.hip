@@ -69,6 +69,7 @@ struct AttnParams {
     const int32_t* kv_len;
     const f16* k_new;  // [T][Hkv][128] rows of the tree nodes to append, or null: already in the cache
     const f16* v_new;
+    const float2* rope;  // [T][64] (cos, sin) of the tree rows' positions, or null: q and k_new come rotated
     f16* k_pool_w;     // writable aliases of the pools (used only when k_new is set)
     f16* v_pool_w;
     const uint64_t* mask;
@@ -87,6 +88,16 @@ struct AttnParams {
     float* o_part;
     float* ml_part;
 };
+
+// One rotary pair: (a, b) -> (a cos - b sin, a sin + b cos), every product and sum rounded on its own
+// (no fused multiply-add), so the result does not depend on how a compiler contracts the expression.
+__device__ inline void rotate_pair(f16& a, f16& b, float2 cs) {
+#pragma clang fp contract(off)
+    const float fa = (float)a, fb = (float)b;
+    const float ac = fa * cs.x, bs = fb * cs.y, as = fa * cs.y, bc = fb * cs.x;
+    a = (f16)(ac - bs);
+    b = (f16)(as + bc);
+}
 
 __device__ inline f16x8 zero8() {
     f16x8 z;
@@ -228,8 +239,8 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
     // waiting for the device-side length; the length only clips the range.
     // With the fused append the last split also patches the appended rows into its tiles, which costs
     // about as much as an iteration: the partition counts two tiles' worth of extra work at the end
-    // of the stream, so that split gets fewer real tiles.
-    const int vtiles = p.ntiles_max + (p.k_new != nullptr && p.num_splits > 1 ? 2 : 0);
+    // of the stream (three when the appended K rows are also rotated there), so that split gets fewer real tiles.
+    const int vtiles = p.ntiles_max + (p.k_new != nullptr && p.num_splits > 1 ? (p.rope != nullptr ? 3 : 2) : 0);
     const int t0 = min((int)(((long long)split * vtiles) / p.num_splits), p.ntiles_max);
     const int t1_max = min((int)(((long long)(split + 1) * vtiles) / p.num_splits), p.ntiles_max);
     const int pg0 = (t0 * kTileN) / kPage;
@@ -292,6 +303,23 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
     for (int d = 0; d <= kDepth; ++d)
         if (d < niter) issue_iter(d);
 
+    // Fused rotary embedding of the query (rotary_embedding_kernel, src/model/rotary.cuh:11-22), placed behind
+    // the first tile requests so that its table reads and arithmetic run under their latency: the pair
+    // (d, d + 64) of a row sits in the same lane, registers ks and ks + 4, and rotates by the angle
+    // of (node position, d); products in fp32, results rounded to fp16 as the in-place kernel leaves them.
+    if (p.rope != nullptr && row_ok) {
+        const float2* cs = p.rope + (size_t)node * (kHeadDim / 2) + hf * 8;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                f16 a = qreg[ks][j], b = qreg[ks + 4][j];
+                rotate_pair(a, b, cs[ks * 16 + j]);
+                qreg[ks][j] = a;
+                qreg[ks + 4][j] = b;
+            }
+    }
+
     for (int it = 0; it < niter; ++it) {
         // Wait for this iteration's tiles.  The prologue issued iterations 0..kDepth and iteration
         // j >= 1 issues iteration j + kDepth right after its barrier, so the tiles issued so far are
@@ -333,7 +361,36 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
                 char* st = ring + (ie % kStages) * kStageBytes;
                 const bool append = p.k_new != nullptr && ce + kTileN > P;
                 const int pg = append ? s_pages[(ce + kTileN - 1) / kPage - pg0] : 0;  // a tile lies inside one page
-                if (append && mt == 0) {
+                if (append && p.rope != nullptr) {
+                    // Fused rotary embedding of the appended K rows (src/model/rotary.cuh:23-33): the tile holds
+                    // them as fetched from k_new; one thread per (key, 16-byte piece of the lower half) rotates
+                    // the piece with its partner 64 dims up, in LDS, and the M-tile-0 workgroup passes the
+                    // rotated pieces on to the pool.
+                    for (int x = tid; x < kTileN * 8; x += kThreads) {
+                        const int key = x >> 3, piece = x & 7;
+                        const int c = ce + key;
+                        if (c >= P && c < S) {
+                            f16x8* lo = reinterpret_cast<f16x8*>(st + k_lds_off(key, piece));
+                            f16x8* hi = reinterpret_cast<f16x8*>(st + k_lds_off(key, piece + 8));
+                            f16x8 a = *lo, b = *hi;
+                            const float2* cs = p.rope + (size_t)(c - P) * (kHeadDim / 2) + piece * 8;
+#pragma unroll
+                            for (int j = 0; j < 8; ++j) {
+                                f16 ra = a[j], rb = b[j];
+                                rotate_pair(ra, rb, cs[j]);
+                                a[j] = ra;
+                                b[j] = rb;
+                            }
+                            *lo = a;
+                            *hi = b;
+                            if (mt == 0) {
+                                f16* row = p.k_pool_w + (((size_t)pg * p.Hkv + g) * kPage + c % kPage) * kHeadDim;
+                                *reinterpret_cast<f16x8*>(row + piece * 8) = a;
+                                *reinterpret_cast<f16x8*>(row + (piece + 8) * 8) = b;
+                            }
+                        }
+                    }
+                } else if (append && mt == 0) {
                     // K is already in the tile (fetched from k_new): the M-tile-0 workgroup copies the new
                     // rows' 16-byte pieces on to the pool.
                     for (int x = tid; x < kTileN * 16; x += kThreads) {
@@ -672,12 +729,12 @@ extern "C" size_t cpmcu_tree_attention_workspace_bytes(int T, int Hq, int Hkv, i
     return align_up((size_t)Hkv * kMaxSplits * rows_pad * (kHeadDim + 2) * sizeof(float), 256);
 }
 
-extern "C" int cpmcu_tree_attention(const void* q, void* k_pool, void* v_pool,
-                                    const int32_t* block_table, const int32_t* kv_len, int max_kv_len,
-                                    const void* k_new, const void* v_new,
-                                    const uint64_t* mask, int mask_words, int mask_k_range, int T, int Hq, int Hkv,
-                                    float scale, void* out, void* workspace, size_t workspace_bytes,
-                                    int num_splits_override, void* stream) {
+static int tree_attention_impl(const void* q, void* k_pool, void* v_pool,
+                               const int32_t* block_table, const int32_t* kv_len, int max_kv_len,
+                               const void* k_new, const void* v_new, const float* rope_cos_sin,
+                               const uint64_t* mask, int mask_words, int mask_k_range, int T, int Hq, int Hkv,
+                               float scale, void* out, void* workspace, size_t workspace_bytes,
+                               int num_splits_override, void* stream) {
     CPMCU_CHECK_ARG(q && k_pool && v_pool && block_table && kv_len && out, "tree_attention: null pointer argument");
     CPMCU_CHECK_ARG(T >= 1 && T <= kMaxTree, "tree_attention: T=%d outside [1, %d]", T, kMaxTree);
     CPMCU_CHECK_ARG(Hkv >= 1 && Hq >= Hkv && Hq % Hkv == 0, "tree_attention: Hq=%d must be a multiple of Hkv=%d", Hq, Hkv);
@@ -699,6 +756,7 @@ extern "C" int cpmcu_tree_attention(const void* q, void* k_pool, void* v_pool,
     CPMCU_CHECK_ARG((k_new == nullptr) == (v_new == nullptr), "tree_attention: k_new and v_new must be given together");
     p.k_new = (const f16*)k_new;
     p.v_new = (const f16*)v_new;
+    p.rope = (const float2*)rope_cos_sin;
     p.k_pool_w = (f16*)k_pool;
     p.v_pool_w = (f16*)v_pool;
     p.mask = mask;
@@ -740,5 +798,75 @@ extern "C" int cpmcu_tree_attention(const void* q, void* k_pool, void* v_pool,
         hipLaunchKernelGGL(tree_attn_combine_kernel, dim3(ceil_div(threads_total, 256)), dim3(256), 0, st, p);
         CPMCU_LAUNCH_CHECK();
     }
+    return CPMCU_OK;
+}
+
+extern "C" int cpmcu_tree_attention(const void* q, void* k_pool, void* v_pool,
+                                    const int32_t* block_table, const int32_t* kv_len, int max_kv_len,
+                                    const void* k_new, const void* v_new,
+                                    const uint64_t* mask, int mask_words, int mask_k_range, int T, int Hq, int Hkv,
+                                    float scale, void* out, void* workspace, size_t workspace_bytes,
+                                    int num_splits_override, void* stream) {
+    return tree_attention_impl(q, k_pool, v_pool, block_table, kv_len, max_kv_len, k_new, v_new, nullptr, mask, mask_words,
+                               mask_k_range, T, Hq, Hkv, scale, out, workspace, workspace_bytes, num_splits_override, stream);
+}
+
+extern "C" int cpmcu_tree_attention_rope(const void* q, void* k_pool, void* v_pool,
+                                         const int32_t* block_table, const int32_t* kv_len, int max_kv_len,
+                                         const void* k_new, const void* v_new, const float* rope_cos_sin,
+                                         const uint64_t* mask, int mask_words, int mask_k_range, int T, int Hq, int Hkv,
+                                         float scale, void* out, void* workspace, size_t workspace_bytes,
+                                         int num_splits_override, void* stream) {
+    CPMCU_CHECK_ARG(rope_cos_sin, "tree_attention_rope: null rotary table");
+    return tree_attention_impl(q, k_pool, v_pool, block_table, kv_len, max_kv_len, k_new, v_new, rope_cos_sin, mask, mask_words,
+                               mask_k_range, T, Hq, Hkv, scale, out, workspace, workspace_bytes, num_splits_override, stream);
+}
+
+namespace cpmcu {
+namespace {
+
+// cos / sin of every (row position, frequency) pair, exactly the values rotary_embedding_kernel
+// (src/model/rotary.cuh:11-17) computes per element: freq = float(pos) * inv_freq[col].
+__global__ void rope_table_kernel(const int32_t* pos, const float* inv_freq, int half_dim, float2* out) {
+    const int t = blockIdx.x;
+    const float p = (float)pos[t];
+    for (int col = threadIdx.x; col < half_dim; col += blockDim.x) {
+        const float freq = p * inv_freq[col];
+        out[(size_t)t * half_dim + col] = make_float2(cosf(freq), sinf(freq));
+    }
+}
+
+// rotary_embedding_kernel, src/model/rotary.cuh:7-34, from a table: in place on q [T][Hq][128] and k [T][Hkv][128].
+__global__ __launch_bounds__(256) void rope_apply_kernel(const float2* table, int Hq, int Hkv, f16* q, f16* k) {
+    constexpr int half = kHeadDim / 2;
+    const int t = blockIdx.x;
+    const float2* cs = table + (size_t)t * half;
+    for (int i = threadIdx.x; i < (Hq + Hkv) * half; i += 256) {
+        const int row = i / half, col = i % half;
+        f16* x = row < Hq ? q + ((size_t)t * Hq + row) * kHeadDim : k + ((size_t)t * Hkv + (row - Hq)) * kHeadDim;
+        f16 a = x[col], b = x[col + half];
+        rotate_pair(a, b, cs[col]);
+        x[col] = a;
+        x[col + half] = b;
+    }
+}
+
+}  // namespace
+}  // namespace cpmcu
+
+extern "C" int cpmcu_rope_table(const int32_t* position_ids, const float* inv_freq, int T, float* cos_sin, void* stream) {
+    CPMCU_CHECK_ARG(position_ids && inv_freq && cos_sin, "rope_table: null pointer argument");
+    CPMCU_CHECK_ARG(T >= 1, "rope_table: T=%d", T);
+    hipLaunchKernelGGL(rope_table_kernel, dim3(T), dim3(64), 0, resolve_stream(stream), position_ids, inv_freq, kHeadDim / 2,
+                       (float2*)cos_sin);
+    CPMCU_LAUNCH_CHECK();
+    return CPMCU_OK;
+}
+
+extern "C" int cpmcu_rope_apply(const float* cos_sin, int T, int Hq, int Hkv, void* q, void* k, void* stream) {
+    CPMCU_CHECK_ARG(cos_sin && q && k, "rope_apply: null pointer argument");
+    CPMCU_CHECK_ARG(T >= 1 && Hq >= 1 && Hkv >= 1, "rope_apply: T=%d Hq=%d Hkv=%d", T, Hq, Hkv);
+    hipLaunchKernelGGL(rope_apply_kernel, dim3(T), dim3(256), 0, resolve_stream(stream), (const float2*)cos_sin, Hq, Hkv, (f16*)q, (f16*)k);
+    CPMCU_LAUNCH_CHECK();
     return CPMCU_OK;
 }

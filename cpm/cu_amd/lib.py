@@ -42,6 +42,9 @@ SIGNATURES = {
     "cpmcu_kv_append": (c_int, [_P, _P, _P, _P, _P, _P, c_int, c_int, _P]),
     "cpmcu_tree_attention_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "cpmcu_tree_attention": (c_int, [_P, _P, _P, _P, _P, c_int, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_float, _P, _P, c_size_t, c_int, _P]),
+    "cpmcu_tree_attention_rope": (c_int, [_P, _P, _P, _P, _P, c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_float, _P, _P, c_size_t, c_int, _P]),
+    "cpmcu_rope_table": (c_int, [_P, _P, c_int, _P, _P]),
+    "cpmcu_rope_apply": (c_int, [_P, c_int, c_int, c_int, _P, _P, _P]),
     "cpmcu_gather_rows": (c_int, [_P, _P, c_int, c_int, _P, _P]),
     "cpmcu_head_workspace_bytes": (c_size_t, [c_int, c_int]),
     "cpmcu_head_weight_tiled_bytes": (c_size_t, [c_int, c_int]),

@@ -60,14 +60,31 @@ def kv_append(cache, layer, k_new, v_new, kv_len):
                      _ptr(kv_len), T, cache.Hkv, _stream())
 
 
+def rope_table(position_ids, inv_freq):
+    """(cos, sin) of float(position) * inv_freq for every tree row: [T, 64, 2] fp32 (src/model/rotary.cuh:11-17)."""
+    T = position_ids.numel()
+    assert position_ids.dtype == torch.int32 and inv_freq.dtype == torch.float32 and inv_freq.numel() == HEAD_DIM // 2
+    out = torch.empty((T, HEAD_DIM // 2, 2), dtype=torch.float32, device=position_ids.device)
+    _lib().rope_table(_ptr(position_ids), _ptr(inv_freq), T, _ptr(out), _stream())
+    return out
+
+
+def rope_apply_(table, q, k):
+    """In-place rotary embedding of q [T,Hq,128] and k [T,Hkv,128] (rotary_embedding_kernel, src/model/rotary.cuh:7-34)."""
+    T, Hq, D = q.shape
+    assert D == HEAD_DIM and k.shape[0] == T and k.shape[2] == D and table.shape[0] == T
+    _lib().rope_apply(_ptr(table), T, Hq, k.shape[1], _ptr(q), _ptr(k), _stream())
+
+
 def tree_attention(q, cache, layer, kv_len, max_kv_len, mask=None, scale=None, num_splits=0, out=None,
-                   k_new=None, v_new=None, mask_k_range=0):
+                   k_new=None, v_new=None, mask_k_range=0, rope=None):
     """mha_fwd_kvcache with a tree mask (src/flash_attn/flash_api.hpp:292-392) on the paged cache.
 
     q [T, Hq, 128] fp16; kv_len int32[1] on the device = P + T; mask uint64 [T, W] or None (chain).
     k_new / v_new [T, Hkv, 128]: the tree rows' K/V; when given the kernel appends them to the cache
     itself (src/model/attn.cuh:200) instead of expecting them there.
     mask_k_range (0 = T): number of trailing keys the mask bits refer to; k*d for the drafter's layers.
+    rope [T, 64, 2] fp32 from rope_table: q and k_new are taken unrotated and rotated inside the kernel.
     """
     T, Hq, D = q.shape
     assert D == HEAD_DIM and q.dtype == torch.float16 and kv_len.dtype == torch.int32
@@ -85,6 +102,13 @@ def tree_attention(q, cache, layer, kv_len, max_kv_len, mask=None, scale=None, n
     if k_new is not None:
         assert k_new.dtype == torch.float16 and v_new.dtype == torch.float16
         assert k_new.numel() == T * cache.Hkv * HEAD_DIM and v_new.numel() == k_new.numel()
+    if rope is not None:
+        # rotary embedding of q and of the appended K rows fused into the kernel (table from rope_table)
+        assert rope.dtype == torch.float32 and rope.numel() == T * HEAD_DIM
+        _lib().tree_attention_rope(_ptr(q), _ptr(cache.k[layer]), _ptr(cache.v[layer]), _ptr(cache.block_table), _ptr(kv_len),
+                                   int(max_kv_len), _ptr(k_new), _ptr(v_new), _ptr(rope), _ptr(mask), W, int(mask_k_range), T, Hq,
+                                   cache.Hkv, ctypes.c_float(scale), _ptr(out), _ptr(ws), ws.numel(), int(num_splits), _stream())
+        return out
     _lib().tree_attention(_ptr(q), _ptr(cache.k[layer]), _ptr(cache.v[layer]), _ptr(cache.block_table), _ptr(kv_len),
                           int(max_kv_len), _ptr(k_new), _ptr(v_new), _ptr(mask), W, int(mask_k_range), T, Hq, cache.Hkv,
                           ctypes.c_float(scale), _ptr(out),

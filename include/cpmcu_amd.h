@@ -205,6 +205,24 @@ int cpmcu_tree_attention(const void* q, void* k_pool, void* v_pool, const int32_
                          void* out,
                          void* workspace, size_t workspace_bytes, int num_splits_override, void* stream);
 
+/* Rotary embedding of the T tree rows -- RotaryEmbedding::prefill / rotary_embedding_kernel,
+ * src/model/rotary.cuh:7-34,61-63, which Attention::decode runs on q and k before the append
+ * (src/model/attn.cuh:199-200).  The angles depend on (position, frequency) only, so they are computed
+ * once per step, not once per layer and element:
+ *   cos_sin [T][64][2] fp32 = (cos, sin)(float(position_ids[t]) * inv_freq[col])       cpmcu_rope_table
+ * and applied either inside the attention kernel (cpmcu_tree_attention_rope: the queries rotate in
+ * registers as they are loaded, the appended K rows rotate in the LDS tile on their way into the pool;
+ * q and k_new themselves are not modified; without k_new only q rotates) or in place by
+ * cpmcu_rope_apply (q [T][Hq][128], k [T][Hkv][128]), the reference's own form.  Pair (d, d + 64):
+ *   x'[d] = f16(x[d] * cos - x[d+64] * sin),  x'[d+64] = f16(x[d] * sin + x[d+64] * cos)   (fp32 arithmetic). */
+int cpmcu_rope_table(const int32_t* position_ids, const float* inv_freq, int T, float* cos_sin, void* stream);
+int cpmcu_rope_apply(const float* cos_sin, int T, int Hq, int Hkv, void* q, void* k, void* stream);
+int cpmcu_tree_attention_rope(const void* q, void* k_pool, void* v_pool, const int32_t* block_table,
+                              const int32_t* kv_len, int max_kv_len, const void* k_new, const void* v_new,
+                              const float* rope_cos_sin, const uint64_t* mask, int mask_words, int mask_k_range,
+                              int T, int Hq, int Hkv, float scale, void* out,
+                              void* workspace, size_t workspace_bytes, int num_splits_override, void* stream);
+
 /* remap_copy -- src/model/tree_drafter.cuh:79-86,103-107: dst[r][:] = src[remap[r]][:]. */
 int cpmcu_gather_rows(const void* src, const int32_t* remap, int rows, int dim, void* dst, void* stream);
 

@@ -44,6 +44,7 @@ def _load():
         "orc_argmax": (None, [c_p, i32, i32, c_p]),
         "orc_tree_accept": (i32, [i32, i32, c_p, c_p, c_p, i32, c_p, c_p, c_p, c_p]),
         "orc_kv_compact": (None, [c_p, i32, i32, i32, i32, c_p, c_p, c_p]),
+        "orc_rope": (None, [i32, i32, i32, i32, c_p, c_p, c_p, c_p, c_p]),
         "orc_accept_commit": (None, [c_p, i32, i32, i32, i32, c_p, c_p, c_p, i32, c_p, c_p, c_p, c_p, c_p]),
         "orc_draft_tree_begin": (None, [i32, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p]),
         "orc_draft_tree_extend": (None, [i32, i32, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p, c_p]),
@@ -206,6 +207,23 @@ def kv_compact(caches, P, path, gt):
     ids = np.empty(a, np.int32)
     _lib.orc_kv_compact(ptrs, len(caches), row_halves, int(P), a, _p(path), _p(gt), _p(ids))
     return ids
+
+
+def rope(q, k, pos=None, inv_freq=None, table=None):
+    """Rotary embedding (src/model/rotary.cuh:7-34) of q [T,Hq,D] and k [T,Hkv,D]; returns rotated copies.
+    Angles from (pos, inv_freq), or from a given table [T, D/2, 2] of (cos, sin)."""
+    q = np.array(q, dtype=np.float16, order="C", copy=True)
+    k = np.array(k, dtype=np.float16, order="C", copy=True)
+    T, Hq, Dh = q.shape
+    half = Dh // 2
+    if table is not None:
+        table = _c(table, np.float32).reshape(T, half, 2)
+    else:
+        pos = _c(pos, np.int32)
+        inv_freq = _c(inv_freq, np.float32)
+        assert inv_freq.size == half
+    _lib.orc_rope(T, Hq, k.shape[1], half, _p(inv_freq), _p(pos), _p(table), _p(q), _p(k))
+    return q, k
 
 
 def accept_commit(caches, P, path, gt, hidden=None):

@@ -351,6 +351,37 @@ void orc_kv_compact(uint16_t* const* caches, int num_caches, int row_halves, int
         for (int d = 0; d < a; ++d) ids_out[d] = gt[path[d]];  // :74-76
 }
 
+// f2 -- rotary_embedding_kernel, src/model/rotary.cuh:7-34: in place on q [T][Hq][2*half] and k [T][Hkv][2*half].
+// table (optional, [T][half][2]): use these (cos, sin) instead of computing them -- the staged form of
+// the check, which takes the device's table and leaves only the rotation itself to compare.
+void orc_rope(int T, int Hq, int Hkv, int half_dim, const float* inv_freq, const int32_t* pos, const float* table,
+              uint16_t* q, uint16_t* k) {
+    for (int t = 0; t < T; ++t) {
+        const int p = pos ? pos[t] : 0;                                    // :10
+        for (int pass = 0; pass < 2; ++pass) {
+            uint16_t* x = pass == 0 ? q : k;
+            const int heads = pass == 0 ? Hq : Hkv;
+            for (int i = 0; i < heads * half_dim; ++i) {                   // :12 / :23
+                const int row = i / half_dim, col = i % half_dim;
+                const size_t offset = (size_t)t * heads * half_dim * 2 + (size_t)row * half_dim * 2;
+                float cos_freq, sin_freq;
+                if (table) {
+                    cos_freq = table[((size_t)t * half_dim + col) * 2];
+                    sin_freq = table[((size_t)t * half_dim + col) * 2 + 1];
+                } else {
+                    const float freq = (float)p * inv_freq[col];           // :16
+                    cos_freq = cosf(freq);                                 // :17
+                    sin_freq = sinf(freq);
+                }
+                const float a = h2f(x[offset + col]);
+                const float b = h2f(x[offset + col + half_dim]);
+                x[offset + col] = f2h(a * cos_freq - b * sin_freq);            // :20
+                x[offset + col + half_dim] = f2h(a * sin_freq + b * cos_freq); // :21
+            }
+        }
+    }
+}
+
 // f2/f3 -- the rest of MiniCPM4EagleImpl::verify after the acceptance, src/model/minicpm4/minicpm4_eagle.cuh:403-411,
 // and the host side of the loop, cpmcu/speculative/tree_drafter.py:222,243-249.
 //   prev_hidden[d] = hidden[path[d] / scale]      remap_hidden_kernel, src/model/eagle.cuh:108-115 (scale 1 at :404)

@@ -139,6 +139,8 @@ int orc_tree_accept(int T, int mask_words, const int32_t* pred, const int32_t* g
  * pinned by: numpy fancy-index copy; overlap case path=[0,2,3]. */
 void orc_kv_compact(uint16_t* const* caches, int num_caches, int row_halves, int P, int a,
                     const int32_t* path, const int32_t* gt, int32_t* ids_out);
+void orc_rope(int T, int Hq, int Hkv, int half_dim, const float* inv_freq, const int32_t* pos, const float* table,
+              uint16_t* q, uint16_t* k);
 void orc_accept_commit(uint16_t* const* caches, int num_caches, int row_halves, int P, int a, const int32_t* path,
                        const int32_t* gt, const uint16_t* hidden, int hidden_dim, uint16_t* prev_hidden,
                        int32_t* next_pos, int32_t* result, int32_t* new_length, int32_t* next_root);

@@ -355,3 +355,32 @@ def test_accept_commit_tail_against_numpy():
     for c, b in zip(caches, before):
         assert np.array_equal(c[:P], b[:P]) and np.array_equal(c[P + a:], b[P + a:])
         assert np.array_equal(c[P:P + a, 0], (P + path).astype(np.float16))  # the tag of the source row
+
+
+def test_rope_against_complex_rotation():
+    """Rotary embedding pinned on what the mathematics fixes: the pair (x[d], x[d+64]) is the complex number
+    x[d] + i x[d+64] multiplied by exp(i * pos * inv_freq[d]) -- numpy complex128 here, so a swapped sign, a
+    transposed pair or a wrong frequency index fails; position 0 is the identity; the norm of every pair is kept."""
+    import oracle as orc
+    rng = np.random.default_rng(11)
+    T, Hq, Hkv, D = 7, 4, 2, 128
+    half = D // 2
+    q = rng.standard_normal((T, Hq, D)).astype(np.float16)
+    k = rng.standard_normal((T, Hkv, D)).astype(np.float16)
+    pos = np.array([0, 1, 2, 77, 4096, 40000, 131071], np.int32)
+    inv_freq = (10000.0 ** (-np.arange(half) / half)).astype(np.float32)
+    qr, kr = orc.rope(q, k, pos, inv_freq)
+    for x, xr in ((q, qr), (k, kr)):
+        z = x[..., :half].astype(np.float64) + 1j * x[..., half:].astype(np.float64)
+        ang = (pos.astype(np.float32)[:, None] * inv_freq[None, :]).astype(np.float32).astype(np.float64)  # float32 product, as the kernel forms it
+        w = z * np.exp(1j * ang)[:, None, :]
+        want = np.concatenate([w.real, w.imag], -1)
+        got = xr.astype(np.float64)
+        assert np.max(np.abs(got - want)) <= 2e-3 * max(1.0, np.max(np.abs(want)))  # one fp16 rounding + float32 cos/sin
+        assert np.array_equal(xr[0].view(np.uint16), x[0].view(np.uint16))          # position 0: identity
+    # a given table is used as is: the quarter turn maps (a, b) to (-b, a) exactly
+    table = np.zeros((T, half, 2), np.float32)
+    table[..., 1] = 1.0
+    qt, kt = orc.rope(q, k, table=table)
+    assert np.array_equal(qt[..., :half], -q[..., half:]) and np.array_equal(qt[..., half:], q[..., :half])
+    assert np.array_equal(kt[..., :half], -k[..., half:]) and np.array_equal(kt[..., half:], k[..., :half])
