@@ -174,7 +174,9 @@ __device__ inline void issue_tile_append(const AttnParams& p, int g, int tile, i
     }
 }
 
-template <int G>
+// ROPE: the instantiation that rotates q and the appended K rows (p.rope is set); the plain one carries
+// none of that code, so its registers and schedule are those of a kernel without the feature.
+template <int G, bool ROPE>
 __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams p) {
     constexpr int kRowWaves = kWaves / G;
     constexpr int kRowsPerWg = kRowWaves * kRowsPerWave;
@@ -240,7 +242,7 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
     // With the fused append the last split also patches the appended rows into its tiles, which costs
     // about as much as an iteration: the partition counts two tiles' worth of extra work at the end
     // of the stream (three when the appended K rows are also rotated there), so that split gets fewer real tiles.
-    const int vtiles = p.ntiles_max + (p.k_new != nullptr && p.num_splits > 1 ? (p.rope != nullptr ? 3 : 2) : 0);
+    const int vtiles = p.ntiles_max + (p.k_new != nullptr && p.num_splits > 1 ? (ROPE ? 3 : 2) : 0);
     const int t0 = min((int)(((long long)split * vtiles) / p.num_splits), p.ntiles_max);
     const int t1_max = min((int)(((long long)(split + 1) * vtiles) / p.num_splits), p.ntiles_max);
     const int pg0 = (t0 * kTileN) / kPage;
@@ -307,7 +309,7 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
     // the first tile requests so that its table reads and arithmetic run under their latency: the pair
     // (d, d + 64) of a row sits in the same lane, registers ks and ks + 4, and rotates by the angle
     // of (node position, d); products in fp32, results rounded to fp16 as the in-place kernel leaves them.
-    if (p.rope != nullptr && row_ok) {
+    if (ROPE && row_ok) {
         const float2* cs = p.rope + (size_t)node * (kHeadDim / 2) + hf * 8;
 #pragma unroll
         for (int ks = 0; ks < 4; ++ks)
@@ -361,7 +363,7 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
                 char* st = ring + (ie % kStages) * kStageBytes;
                 const bool append = p.k_new != nullptr && ce + kTileN > P;
                 const int pg = append ? s_pages[(ce + kTileN - 1) / kPage - pg0] : 0;  // a tile lies inside one page
-                if (append && p.rope != nullptr) {
+                if (ROPE && append) {
                     // Fused rotary embedding of the appended K rows (src/model/rotary.cuh:23-33): the tile holds
                     // them as fetched from k_new; one thread per (key, 16-byte piece of the lower half) rotates
                     // the piece with its partner 64 dims up, in LDS, and the M-tile-0 workgroup passes the
@@ -790,8 +792,13 @@ static int tree_attention_impl(const void* q, void* k_pool, void* v_pool,
     hipStream_t st = resolve_stream(stream);
     const int nsh = p.num_splits * Hkv;
     const int grid = kXcds * ceil_div(nsh, kXcds) * p.num_mtiles;
-    if (G == 1) hipLaunchKernelGGL(tree_attn_split_kernel<1>, dim3(grid), dim3(kThreads), 0, st, p);
-    else hipLaunchKernelGGL(tree_attn_split_kernel<2>, dim3(grid), dim3(kThreads), 0, st, p);
+    if (p.rope != nullptr) {
+        if (G == 1) hipLaunchKernelGGL((tree_attn_split_kernel<1, true>), dim3(grid), dim3(kThreads), 0, st, p);
+        else hipLaunchKernelGGL((tree_attn_split_kernel<2, true>), dim3(grid), dim3(kThreads), 0, st, p);
+    } else {
+        if (G == 1) hipLaunchKernelGGL((tree_attn_split_kernel<1, false>), dim3(grid), dim3(kThreads), 0, st, p);
+        else hipLaunchKernelGGL((tree_attn_split_kernel<2, false>), dim3(grid), dim3(kThreads), 0, st, p);
+    }
     CPMCU_LAUNCH_CHECK();
     if (p.num_splits > 1) {
         const int threads_total = Hkv * (p.rows_pad / kRowsPerWave) * 16 * 64;
