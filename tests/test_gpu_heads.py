@@ -71,6 +71,32 @@ def test_frspec_one_row_and_sixteen_rows(gpu, orc):
     _frspec_check(gpu, orc, n=16, V=5000, Vs=4100, H=512, k=7, seed=6)
 
 
+def test_frspec_clustered_logits_merge_in_fp16(gpu, orc):
+    """Nearly flat logits: z spreads over a few hundredths while log-probabilities sit near -ln(V), where an
+    fp16 ulp is 2^-7, so hundreds of distinct z collapse onto each rounded log-probability and the ranking is
+    decided by the lowest index among ties.  Both the candidate path of the row kernel (bound lowered by the
+    rounding slack) and its many-candidates fallback have to reproduce the oracle's order exactly."""
+    from cpm.cu_amd import ops
+    torch = gpu
+    for (n, Vs, H, k, std, seed) in [(4, 4096, 512, 10, 0.0005, 1), (10, 32768, 512, 10, 0.002, 2), (3, 2048, 1024, 32, 0.0002, 3),
+                                     (2, 4096, 512, 5, 0.0, 4)]:
+        hid = synth.normal_f16((n, H), seed, 1)
+        w = synth.normal_f16((Vs, H), seed, 2, std=std) if std > 0 else np.zeros((Vs, H), np.float16)
+        remap = synth.frspec_remap(Vs + 1000, Vs, seed)
+        r = ops.frspec_head_topk(to_dev(torch, hid), to_dev(torch, w), to_dev(torch, remap), k)
+        torch.cuda.synchronize()
+        z_dev = to_np(r["logits"])
+        stats = to_np(r["row_stats"])
+        lp_staged = orc.log_softmax_apply(z_dev, stats[:, 0], stats[:, 1])
+        distinct = len(np.unique(lp_staged[0]))
+        val_s, pos_s = orc.topk(lp_staged, k)
+        assert np.array_equal(to_np(r["pos"]), pos_s), "Vs=%d std=%g: %d distinct log-probs in row 0" % (Vs, std, distinct)
+        assert np.array_equal(to_np(r["val"]).view(np.uint16), val_s.view(np.uint16))
+        assert np.array_equal(to_np(r["ids"]), remap[pos_s])
+        if std == 0.0:
+            assert np.array_equal(pos_s, np.tile(np.arange(k, dtype=np.int32), (n, 1)))  # all equal: lowest indices
+
+
 def test_frspec_c3_full_size(gpu, orc):
     """Config 3: 10 frontier rows, 73448x4096 head, 32768-row subset, top-10 mapped to full-vocab ids."""
     exact = _frspec_check(gpu, orc, n=10, V=73448, Vs=32768, H=4096, k=10, seed=0)
@@ -193,6 +219,44 @@ def test_topk_heavy_ties_and_neg_inf(gpu, orc):
     assert np.array_equal(to_np(pos), p_ref)
     assert np.array_equal(to_np(val).view(np.uint16), v_ref.view(np.uint16))
     assert np.array_equal(p_ref[0], np.arange(32))
+
+
+@pytest.mark.parametrize("case", ["two_values", "mostly_neg_inf", "descending", "ascending", "wide_range", "k64", "tiny_rows"])
+def test_topk_row_kernel_shapes_of_data(gpu, orc, case):
+    """Inputs chosen against the one-launch row kernel's bound / candidate / fallback logic."""
+    from cpm.cu_amd import ops
+    torch = gpu
+    g = synth.rng(len(case), 5)
+    top = 10
+    if case == "two_values":
+        x = g.integers(0, 2, size=(4, 32768)).astype(np.float16)          # half the row ties for the top: fallback
+    elif case == "mostly_neg_inf":
+        x = np.full((3, 8192), -np.inf, np.float16)
+        x[0, 5] = 1.0                                                      # fewer finite values than k
+        x[1, ::700] = g.standard_normal(len(x[1, ::700])).astype(np.float16)
+        x[2, :12] = np.arange(12, dtype=np.float16)
+    elif case == "descending":
+        x = np.tile(np.linspace(8, -8, 32768, dtype=np.float32).astype(np.float16), (2, 1))   # all of the top in one wave
+    elif case == "ascending":
+        x = np.tile(np.linspace(-8, 8, 16384, dtype=np.float32).astype(np.float16), (2, 1))
+    elif case == "wide_range":
+        x = (g.standard_normal((5, 24576)) * np.exp(g.standard_normal((5, 24576)) * 3)).astype(np.float16)
+        x[0, 100] = np.float16(65504)
+        x[1, 200] = np.float16(-65504)
+        x[2, :64] = np.float16(6e-8)                                       # subnormals and signed zeros near the bound
+        x[3, ::2] = 0.0
+        x[3, 1::2] = -0.0
+    elif case == "k64":
+        x = g.standard_normal((3, 32768)).astype(np.float16)
+        top = 64
+    else:
+        x = g.standard_normal((6, 64)).astype(np.float16)                  # one wave holds everything
+        top = 8
+    val, pos = ops.topk(to_dev(torch, x), top)
+    torch.cuda.synchronize()
+    v_ref, p_ref = orc.topk(x, top)
+    assert np.array_equal(to_np(pos), p_ref)
+    assert np.array_equal(to_np(val).view(np.uint16), v_ref.view(np.uint16))
 
 
 def test_log_softmax_operator(gpu, orc):
