@@ -497,8 +497,14 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, sacc[kb][r]);
-            tmax = fmaxf(tmax, __shfl_xor(tmax, 32)) * p.scale_log2;  // scale > 0
-            if (__any(tmax > m_ref + kLazyLog2)) {  // some row's maximum moved far: re-reference all rows
+            {   // The row's other half of the keys lives 32 lanes away: one cross-half register swap instead of
+            // an LDS shuffle.  Written as assembly because the compiler builtin of this instruction hands
+            // back its first result twice.  The two wait states cover the vector write of tmax just before.
+            float mine = tmax, other = tmax;
+            asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1" : "+v"(mine), "+v"(other));
+            tmax = fmaxf(mine, other) * p.scale_log2;  // scale > 0
+        }
+        if (__any(tmax > m_ref + kLazyLog2)) {  // some row's maximum moved far: re-reference all rows
                 const float m_new = fmaxf(m_ref, tmax);
                 const float alpha = (m_new == -INFINITY) ? 1.f : __builtin_amdgcn_exp2f(m_ref - m_new);
                 m_ref = m_new;
