@@ -34,7 +34,7 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 # are carried here as constants and are reported only for the workload they were measured on.
 MEASURED_TRAFFIC_KIB = {
     "tree_attn_split_kernel+tree_attn_combine_kernel": 6358 + 8494 + 8710 + 480,
-    "head_gemm_chunked_kernel<4,4,256,4>+head_argmax_finalize_kernel": 594619 + 128 + 1052 + 2,
+    "head_gemm_chunked_kernel<4,4,256,2>+head_argmax_finalize_kernel": 594619 + 128 + 1052 + 2,
     "tree_accept_kernel+kv_compact_kernel+accepted_ids_kernel": 6 + 1137 + 335 + 4,
 }
 
@@ -281,7 +281,7 @@ def main():
         dict(kernel="tree_attn_split_kernel+tree_attn_combine_kernel", launches_per_step=wl.L, us_per_launch=round(ms_attn * 1e3, 2),
              bound="mfma", achieved=round(attn_tflops, 2), peak=MFMA_F16_PEAK_TFLOPS, unit="TFLOP/s",
              frac=round(attn_tflops / MFMA_F16_PEAK_TFLOPS, 4), hbm_gbs=round(attn_gbs, 1), traffic=None),
-        dict(kernel="head_gemm_chunked_kernel<4,4,256,4>+head_argmax_finalize_kernel", launches_per_step=1, us_per_launch=round(ms_head * 1e3, 2),
+        dict(kernel="head_gemm_chunked_kernel<4,4,256,2>+head_argmax_finalize_kernel", launches_per_step=1, us_per_launch=round(ms_head * 1e3, 2),
              bound="hbm", achieved=round(head_gbs, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(head_gbs / HBM_PEAK_GBS, 4),
              traffic=None),
         dict(kernel="tree_accept_kernel+kv_compact_kernel+accepted_ids_kernel", launches_per_step=1,

@@ -37,6 +37,12 @@ struct HeadParams {
     int kc;       // K chunk held in one LDS buffer
     int nch;      // H / kc
     int npasses;  // row-block passes per workgroup
+    // Shared last pass (chunked kernel, single sweep): when the row blocks do not fill the last pass, its
+    // blocks are dealt to the workgroups round-robin and each is worked on by several waves, every one
+    // taking a subset of the K chunks, so that all waves carry the same load.  full_passes = npasses - 1
+    // complete passes, rem_blocks = row blocks left for the last one; 0 = plain mapping.
+    int full_passes;
+    int rem_blocks;
     int apply_scale;
     float head_scale;
     int mode;
@@ -350,6 +356,23 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_chunked_kernel(HeadPar
     const int rotc = c % nch;  // workgroups start their K walk at different chunks (HBM channel spread)
     const f16 sc = (f16)p.head_scale;
 
+    // Shared last pass: this workgroup's r_c blocks of it, `share` waves on each (a power of two that
+    // divides the chunk count), wave w on block w / share with the chunks q % share == w % share.
+    const bool shared_last = p.rem_blocks > 0;
+    int r_c = 0, share = 1;
+    if (shared_last) {
+        r_c = c < p.rem_blocks ? (p.rem_blocks - c + G - 1) / G : 0;
+        if (r_c > kHeadWaves) r_c = kHeadWaves;  // cannot happen: rem_blocks <= kHeadWaves * G
+        while (r_c > 0 && share * 2 * r_c <= kHeadWaves && nch % (share * 2) == 0) share *= 2;
+    }
+    const int my_last = wave / share, my_sub = wave % share;
+    auto step_active = [&](int q, int pl) -> bool {
+        const int pass = (q / nch) * NP + pl;
+        if (!shared_last) return pass < p.npasses;
+        if (pass != p.full_passes) return pass < p.full_passes;
+        return my_last < r_c && (q % share) == my_sub;
+    };
+
     auto chunk_of = [&](int q) { return (q % nch + rotc) % nch; };
     // hidden chunk q -> LDS buffer q & 1 (asynchronous; completion is awaited with vmcnt below)
     auto issue_hidden = [&](int q) {
@@ -366,11 +389,14 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_chunked_kernel(HeadPar
             asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(dst) : "memory", "m0");
         }
     };
-    auto row_block = [&](int pass) { return (pass * kHeadWaves + wave) * G + c; };
+    auto row_block = [&](int pass) {
+        if (shared_last && pass == p.full_passes) return p.full_passes * kHeadWaves * G + c + my_last * G;
+        return (pass * kHeadWaves + wave) * G + c;
+    };
     int groups_since_dma = 0;  // W groups requested after the newest hidden chunk request
     auto load_w = [&](int q, int pl, f16x8* buf) {
         const int pass = (q / nch) * NP + pl;
-        if (pass >= p.npasses) return;
+        if (!step_active(q, pl)) return;
         ++groups_since_dma;
         if (p.w_tiled) {  // one contiguous KB per instruction, consecutive steps consecutive in memory
             int rb = row_block(pass);
@@ -445,7 +471,7 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_chunked_kernel(HeadPar
                 if (pn < NP) load_w(q, pn, bufs[pn % NBUF]);
                 else if (q + 1 < total_q) load_w(q + 1, pn - NP, bufs[(pn - NP) % NBUF]);
             }
-            if ((q / nch) * NP + pl < p.npasses) {
+            if (step_active(q, pl)) {
 #pragma unroll
                 for (int ks = 0; ks < PD; ++ks) {
                     const char* bk = base + ((ks ^ hi) << 6);
@@ -461,8 +487,37 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_chunked_kernel(HeadPar
 #pragma unroll
             for (int pl = 0; pl < NP; ++pl) {
                 const int pass = (q / nch) * NP + pl;
-                if (pass < p.npasses) head_epilogue<NB>(p, acc[pl], row_block(pass) * 16 + kgp * 4, l16, ea, eb);
+                if (pass < (shared_last ? p.full_passes : p.npasses))
+                    head_epilogue<NB>(p, acc[pl], row_block(pass) * 16 + kgp * 4, l16, ea, eb);
             }
+        }
+    }
+    if (shared_last) {
+        // The waves that shared a block of the last pass hold partial sums over their chunks: they meet in
+        // LDS (the hidden buffers are free now) and the first wave of each group adds them up in wave order.
+        __syncthreads();
+        f32x4* xch = reinterpret_cast<f32x4*>(lds);  // [wave][NB][64 lanes]
+        const int pl_last = p.full_passes % NP;
+        if (my_last < r_c) {
+#pragma unroll
+            for (int pl = 0; pl < NP; ++pl)
+                if (pl == pl_last)
+#pragma unroll
+                    for (int nb = 0; nb < NB; ++nb) xch[(wave * NB + nb) * 64 + lane] = acc[pl][nb];
+        }
+        __syncthreads();
+        if (my_last < r_c && my_sub == 0) {
+            f32x4 sum[NB];
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                sum[nb] = xch[(wave * NB + nb) * 64 + lane];
+                for (int o = 1; o < share; ++o) {
+                    const f32x4 x = xch[((wave + o) * NB + nb) * 64 + lane];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) sum[nb][r] += x[r];
+                }
+            }
+            head_epilogue<NB>(p, sum, row_block(p.full_passes) * 16 + kgp * 4, l16, ea, eb);
         }
     }
     head_finish<NB>(p, ea, eb, red_a, red_b, tid, wave, lane, c);
@@ -539,6 +594,8 @@ int launch_head_gemm(const void* hidden, const void* w, int w_layout, int n, int
     int G = num_cus();
     if (G * kHeadWaves > nrb) G = ceil_div(nrb, kHeadWaves);
     p.npasses = ceil_div(nrb, G * kHeadWaves);
+    p.full_passes = 0;
+    p.rem_blocks = 0;
     *grid_out = G;
     *stride_out = NB * 16;
     // Kernel shapes chosen by measurement on MI355X (73448 x 4096 and 32768 x 4096 heads).
@@ -552,10 +609,29 @@ int launch_head_gemm(const void* hidden, const void* w, int w_layout, int n, int
             default: hipLaunchKernelGGL(head_gemm_kernel<8>, dim3(G), dim3(kHeadThreads), 0, st, p); break;
         }
     } else if (p.w_tiled) {
+        // one sweep (all passes fit the accumulator sets) with a partly filled last pass: share it
+        const int rem = nrb - (p.npasses - 1) * G * kHeadWaves;
+        if (p.npasses <= (NB == 8 ? 2 : 4) && rem < G * kHeadWaves && getenv("CPMCU_HEAD_NO_SHARE") == nullptr) {  // <= NP below
+            p.full_passes = p.npasses - 1;
+            p.rem_blocks = rem;
+        }
+        // W register buffers: two when a wave works on several row blocks per chunk (the next block's
+        // group is the prefetch; 72 vs 65 % of HBM peak for 60 rows, 81 vs 79 % for 10), four when there
+        // is a single pass (FR-Spec head: 32768 rows = one block per wave; 49.7 vs 52.0 us)
+        const bool deep = p.npasses == 1;
         switch (NB) {
-            case 1: hipLaunchKernelGGL((head_gemm_chunked_kernel<1, 4, 256, 4>), dim3(G), dim3(kHeadThreads), 0, st, p); break;
-            case 2: hipLaunchKernelGGL((head_gemm_chunked_kernel<2, 4, 256, 4>), dim3(G), dim3(kHeadThreads), 0, st, p); break;
-            case 4: hipLaunchKernelGGL((head_gemm_chunked_kernel<4, 4, 256, 4>), dim3(G), dim3(kHeadThreads), 0, st, p); break;
+            case 1:
+                if (deep) hipLaunchKernelGGL((head_gemm_chunked_kernel<1, 4, 256, 4>), dim3(G), dim3(kHeadThreads), 0, st, p);
+                else hipLaunchKernelGGL((head_gemm_chunked_kernel<1, 4, 256, 2>), dim3(G), dim3(kHeadThreads), 0, st, p);
+                break;
+            case 2:
+                if (deep) hipLaunchKernelGGL((head_gemm_chunked_kernel<2, 4, 256, 4>), dim3(G), dim3(kHeadThreads), 0, st, p);
+                else hipLaunchKernelGGL((head_gemm_chunked_kernel<2, 4, 256, 2>), dim3(G), dim3(kHeadThreads), 0, st, p);
+                break;
+            case 4:
+                if (deep) hipLaunchKernelGGL((head_gemm_chunked_kernel<4, 4, 256, 4>), dim3(G), dim3(kHeadThreads), 0, st, p);
+                else hipLaunchKernelGGL((head_gemm_chunked_kernel<4, 4, 256, 2>), dim3(G), dim3(kHeadThreads), 0, st, p);
+                break;
             default: hipLaunchKernelGGL((head_gemm_chunked_kernel<8, 2, 128, 2>), dim3(G), dim3(kHeadThreads), 0, st, p); break;
         }
     } else {
