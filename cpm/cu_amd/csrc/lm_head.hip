@@ -610,6 +610,7 @@ int launch_head_gemm(const void* hidden, const void* w, int w_layout, int n, int
         }
     } else if (p.w_tiled) {
         // one sweep (all passes fit the accumulator sets) with a partly filled last pass: share it
+        // (CPMCU_HEAD_NO_SHARE in the environment keeps the plain mapping; tests compare the two)
         const int rem = nrb - (p.npasses - 1) * G * kHeadWaves;
         if (p.npasses <= (NB == 8 ? 2 : 4) && rem < G * kHeadWaves && getenv("CPMCU_HEAD_NO_SHARE") == nullptr) {  // <= NP below
             p.full_passes = p.npasses - 1;

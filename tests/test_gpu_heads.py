@@ -295,6 +295,29 @@ def test_tiled_weight_layout_gives_the_same_logits(gpu, orc, n, V, H):
     assert np.array_equal(to_np(gt_t)[clear], to_np(gt_r)[clear]) and np.array_equal(to_np(gt_t)[clear], orc.argmax(ref)[clear])
 
 
+@pytest.mark.parametrize("n,V,H", [(60, 73448, 4096), (10, 40000, 1024), (33, 36000, 512), (64, 34000, 512), (5, 32768 + 16 * 300, 512)])
+def test_shared_last_pass_equals_plain_mapping(gpu, orc, monkeypatch, n, V, H):
+    """Row-block counts that leave the last pass partly filled (1, 2 or more blocks per workgroup, with 2, 4 and 16
+    K chunks): the waves that share a block add their partial sums in LDS.  Same logits as the plain mapping up to
+    the fp32 summation order, same arg-max wherever the top two are apart, and both match the oracle."""
+    from cpm.cu_amd import ops
+    torch = gpu
+    hid = synth.normal_f16((n, H), V, 1)
+    w = synth.normal_f16((V, H), V, 2, std=0.02)
+    d_hid = to_dev(torch, hid)
+    wt = ops.tile_head_weight(to_dev(torch, w))
+    gt_s, z_s = ops.lm_head_argmax(d_hid, wt, want_logits=True)
+    torch.cuda.synchronize()
+    monkeypatch.setenv("CPMCU_HEAD_NO_SHARE", "1")
+    gt_p, z_p = ops.lm_head_argmax(d_hid, wt, want_logits=True)
+    torch.cuda.synchronize()
+    assert_close_f16(to_np(z_s), to_np(z_p), "shared vs plain last pass", atol=8e-3, rtol=2e-3)
+    z_ref = orc.lm_head(hid, w)
+    assert_close_f16(to_np(z_s), z_ref, "shared last pass vs oracle")
+    for z, gt in ((to_np(z_s), to_np(gt_s)), (to_np(z_p), to_np(gt_p))):
+        assert np.array_equal(gt, orc.argmax(z))  # staged: the kernel's own logits decide
+
+
 def test_tiled_frspec_head_with_fused_gather(gpu, orc):
     """tile_head_weight with a row map == gather_rows followed by tiling == the row-major sub-matrix."""
     from cpm.cu_amd import ops
