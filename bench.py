@@ -307,7 +307,7 @@ def main():
     ms_fr = timed_replays(torch, fr_head, reps, 2, use_graph)[0] / HEAD_REP
     fr_bytes = wl.shape["frspec_vocab"] * wl.shape["hidden"] * 2.0 + 10 * wl.shape["hidden"] * 2.0 + 10 * 10 * 6.0
     fr_gbs = fr_bytes / (ms_fr * 1e-3) / 1e9
-    frspec = dict(kernel="head_gemm_chunked_kernel<1,4,256,4>+topk_row_kernel", us_per_call=round(ms_fr * 1e3, 2), bound="hbm",
+    frspec = dict(kernel="head_gemm_chunked_kernel<1,2,512,2>+topk_row_kernel", us_per_call=round(ms_fr * 1e3, 2), bound="hbm",
                   achieved=round(fr_gbs, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(fr_gbs / HBM_PEAK_GBS, 4))
     del w_sub
 

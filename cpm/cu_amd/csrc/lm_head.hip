@@ -618,11 +618,12 @@ int launch_head_gemm(const void* hidden, const void* w, int w_layout, int n, int
         }
         // W register buffers: two when a wave works on several row blocks per chunk (the next block's
         // group is the prefetch; 72 vs 65 % of HBM peak for 60 rows, 81 vs 79 % for 10), four when there
-        // is a single pass (FR-Spec head: 32768 rows = one block per wave; 49.7 vs 52.0 us)
+        // is a single pass; the FR-Spec head (32768 rows = one block per wave, up to 16 hidden rows) does best
+        // with 512-column chunks in two buffers: 47.4 us with its top-k, against 50.0 (256 x 4) and 52.0 (256 x 2)
         const bool deep = p.npasses == 1;
         switch (NB) {
             case 1:
-                if (deep) hipLaunchKernelGGL((head_gemm_chunked_kernel<1, 4, 256, 4>), dim3(G), dim3(kHeadThreads), 0, st, p);
+                if (deep) hipLaunchKernelGGL((head_gemm_chunked_kernel<1, 2, 512, 2>), dim3(G), dim3(kHeadThreads), 0, st, p);
                 else hipLaunchKernelGGL((head_gemm_chunked_kernel<1, 4, 256, 2>), dim3(G), dim3(kHeadThreads), 0, st, p);
                 break;
             case 2:
