@@ -215,3 +215,63 @@ def test_draft_layer_mask_range(gpu, orc, k, d, P0, seed):
     torch.cuda.synchronize()
     ref = orc.tree_attention(q, kk, vv, mask, S - k, mask_k_range=k * d)
     assert_close_f16(to_np(out), ref, "draft-layer attention k=%d d=%d" % (k, d))
+
+
+def _sweep_configs():
+    """Seeded random (P, T, mode, splits, slack) tuples, biased to tile (64), page (256) and wave-row (2, 16 nodes)
+    boundaries; slack = how far the host-side bound on the KV length exceeds the true length."""
+    g = synth.rng(2024, 7)
+    edges_p = [0, 1, 2, 3, 62, 63, 64, 65, 127, 128, 129, 191, 192, 250, 255, 256, 257, 258, 319, 320, 511, 512, 513,
+               1023, 1024, 1025, 4095, 4096, 4097]
+    edges_t = [1, 2, 3, 8, 15, 16, 17, 31, 32, 33, 60, 63, 64, 65, 100, 127, 128]
+    out = []
+    for i in range(36):
+        P = int(edges_p[g.integers(len(edges_p))]) if g.random() < 0.7 else int(g.integers(0, 9000))
+        T = int(edges_t[g.integers(len(edges_t))]) if g.random() < 0.7 else int(g.integers(1, 129))
+        mode = ["in_cache", "append", "append_rope"][int(g.integers(3))]
+        splits = [0, 0, 1, 3][int(g.integers(4))]
+        slack = [0, 0, 1, 63, 64, 200, 1000][int(g.integers(7))]
+        out.append((P, T, mode, splits, slack, i))
+    return out
+
+
+@pytest.mark.parametrize("P,T,mode,splits,slack,seed", _sweep_configs())
+def test_randomised_shape_sweep(gpu, orc, P, T, mode, splits, slack, seed):
+    """Prefix lengths, tree sizes, split counts and bounds drawn around the kernel's tile, page and row-block
+    boundaries, in each of its three input modes, against the oracle; appended rows are checked bit for bit."""
+    from cpm.cu_amd import ops
+    from cpm.cu_amd.kvcache import PagedKVCache
+    torch = gpu
+    tree = synth.random_tree(T, 500 + seed, max_children=5, max_depth=10)
+    S = P + T
+    max_len = S + slack
+    npages = (max_len + 255) // 256 + 1
+    table = synth.rng(seed, 4).permutation(npages).astype(np.int32)
+    q = synth.normal_f16((T, HQ, D), seed, 1)
+    k = synth.normal_f16((S, HKV, D), seed, 2)
+    v = synth.normal_f16((S, HKV, D), seed, 3)
+    cache = PagedKVCache(1, HKV, npages, block_table=table, fill=float("nan"))
+    kv_len = torch.tensor([S], dtype=torch.int32, device="cuda")
+    mask = to_dev(torch, tree.mask)
+    q_ref, k_ref = q, k
+    if mode == "in_cache":
+        cache.write_logical(0, 0, to_dev(torch, k), to_dev(torch, v))
+        out = ops.tree_attention(to_dev(torch, q), cache, 0, kv_len, max_len, mask, num_splits=splits)
+    else:
+        if P:
+            cache.write_logical(0, 0, to_dev(torch, k[:P]), to_dev(torch, v[:P]))
+        rope = None
+        if mode == "append_rope":
+            inv_freq = (10000.0 ** (-np.arange(D // 2, dtype=np.float64) / (D // 2))).astype(np.float32)
+            rope = ops.rope_table(to_dev(torch, tree.positions(P)), to_dev(torch, inv_freq))
+            q_ref, k_rot = orc.rope(q, k[P:], table=to_np(rope))
+            k_ref = np.concatenate([k[:P], k_rot], 0)
+        out = ops.tree_attention(to_dev(torch, q), cache, 0, kv_len, max_len, mask, num_splits=splits,
+                                 k_new=to_dev(torch, k[P:]), v_new=to_dev(torch, v[P:]), rope=rope)
+    torch.cuda.synchronize()
+    ref = orc.tree_attention(q_ref, k_ref, v, tree.mask, P)
+    assert_close_f16(to_np(out), ref, "P=%d T=%d %s splits=%d slack=%d" % (P, T, mode, splits, slack))
+    if mode != "in_cache":
+        kc, vc = cache.read_logical(0, 0, S)
+        assert np.array_equal(to_np(kc).view(np.uint16), k_ref.view(np.uint16))
+        assert np.array_equal(to_np(vc).view(np.uint16), v.view(np.uint16))
