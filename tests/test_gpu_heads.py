@@ -137,14 +137,15 @@ def test_frspec_subset_vs_full_head(gpu, orc):
         assert clear <= set(int(t) for t in sub_ids[i])
 
 
-def _argmax_check(torch, orc, n, V, H, seed, scale=None, plant=None):
+def _argmax_check(torch, orc, n, V, H, seed, scale=None, plant=None, tiled=False):
     from cpm.cu_amd import ops
     hid = synth.normal_f16((n, H), seed, 1)
     w = synth.normal_f16((V, H), seed, 2, std=0.02)
     if plant is not None:
         plant(hid, w)
-    gt, logits = ops.lm_head_argmax(to_dev(torch, hid), to_dev(torch, w), head_scale=scale, want_logits=True)
-    gt2 = ops.lm_head_argmax(to_dev(torch, hid), to_dev(torch, w), head_scale=scale)  # logits not materialised
+    d_w = ops.tile_head_weight(to_dev(torch, w)) if tiled else to_dev(torch, w)
+    gt, logits = ops.lm_head_argmax(to_dev(torch, hid), d_w, head_scale=scale, want_logits=True)
+    gt2 = ops.lm_head_argmax(to_dev(torch, hid), d_w, head_scale=scale)  # logits not materialised
     torch.cuda.synchronize()
     z_dev = to_np(logits)
     z_ref = orc.lm_head(hid, w, head_scale=scale)
@@ -170,6 +171,28 @@ def test_target_head_row_counts(gpu, orc, n):
 def test_target_head_k_chunking(gpu, orc, n, H):
     """Hidden sizes that need several K chunks in LDS (double-buffered staging) for each row-block count."""
     _argmax_check(gpu, orc, n, V=1000, H=H, seed=100 + n)
+
+
+def _head_sweep_configs():
+    """Seeded random (rows, vocabulary, hidden, tiled, scale): row counts around the 16/32/64 thresholds of the
+    kernel shapes, vocabularies around multiples of 16 (row blocks) and of 2048 * 16 (full passes of 256 x 8 waves)."""
+    g = synth.rng(77, 3)
+    rows = [1, 2, 15, 16, 17, 31, 32, 33, 59, 60, 63, 64, 65, 128]
+    out = []
+    for i in range(24):
+        n = int(rows[g.integers(len(rows))])
+        base = int([16, 2048 * 16, 2 * 2048 * 16, 4096, 12000][g.integers(5)])
+        V = max(n, 1, base + int(g.integers(-20, 21))) if g.random() < 0.7 else int(g.integers(1, 40000))
+        H = int([512, 1024, 2048, 4096][g.integers(4)])
+        if V * H > 40000 * 2048:
+            H = 512
+        out.append((n, V, H, bool(g.integers(2)), [None, None, 0.3125, 2.0][int(g.integers(4))], i))
+    return out
+
+
+@pytest.mark.parametrize("n,V,H,tiled,scale,seed", _head_sweep_configs())
+def test_target_head_randomised_sweep(gpu, orc, n, V, H, tiled, scale, seed):
+    _argmax_check(gpu, orc, n, V=V, H=H, seed=900 + seed, scale=scale, tiled=tiled)
 
 
 def test_target_head_scale(gpu, orc):
