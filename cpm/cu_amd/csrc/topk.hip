@@ -3,13 +3,18 @@
 // Ordering contract of the reference's bitonic TopK (src/model/topk.cuh:17): value descending,
 // equal values -> lower index first.  Here every element becomes one 64-bit key
 //   (order-preserving 16-bit image of the fp16 value) << 32 | (0xFFFFFFFF - index)
-// so "largest key first" IS that ordering, keys are unique, and selection is k rounds of a
-// workgroup-wide max -- no sorting network, no padding to powers of two, any k.
+// so "largest key first" IS that ordering and keys are unique -- no sorting network, no padding to
+// powers of two, any k.  Two ways to the k largest keys:
+//   * topk_row_kernel, one launch: rows of up to 32768 values (the FR-Spec vocabulary) stay in the
+//     registers of one workgroup, which bounds the k-th value from its waves' lane maxima, compacts the
+//     few candidates above the bound and ranks them by counting;
+//   * topk_chunk_kernel + topk_merge_kernel: longer rows, k rounds of a workgroup-wide maximum per
+//     2048-element chunk and again over the chunks' winners.
 //
 // FR-Spec fusion: the draft head ranks log-probabilities that were rounded to fp16 BEFORE
-// ranking (src/model/eagle.cuh:87), so rounding ties must be reproduced exactly.  The chunk
-// kernel therefore recomputes f16((z - max) - ln sum) from the fp16 logits and the row
-// statistics reduced from the GEMM's per-workgroup partials, and ranks that.
+// ranking (src/model/eagle.cuh:87), so rounding ties must be reproduced exactly.  The kernels
+// therefore recompute f16((z - max) - ln sum) from the fp16 logits and the row statistics
+// reduced from the GEMM's per-workgroup partials, and rank that.
 #include "common.h"
 #include "internal.h"
 #include "topk_keys.h"
