@@ -108,6 +108,13 @@ PYBIND11_MODULE(C, m) {
               check(cpmcu_decode_attention(layer, input_length, padded_length, q, k_new, v_new, cache_length, mask_2d, out));
           },
           "KV append + tree attention of one layer on the model's paged cache");
+    m.def("draft_attention",
+          [](int draft_layer, int input_length, int padded_length, std::uintptr_t q, std::uintptr_t k_new, std::uintptr_t v_new,
+             std::uintptr_t cache_length, std::uintptr_t mask_2d, int mask_k_range, std::uintptr_t out) {
+              check(cpmcu_draft_attention(draft_layer, input_length, padded_length, q, k_new, v_new, cache_length, mask_2d,
+                                          mask_k_range, out));
+          },
+          "KV append + windowed attention of one of the drafter's own layers on its paged cache");
     m.def("decode_lm_head",
           [](int input_length, std::uintptr_t hidden, std::uintptr_t logits, std::uintptr_t gt) {
               check(cpmcu_decode_lm_head(input_length, hidden, logits, gt));

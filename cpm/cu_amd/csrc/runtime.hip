@@ -53,6 +53,8 @@ struct Model {
     // drafter (init_eagle_model / init_minicpm4_eagle_model)
     bool drafter = false;
     int num_iter = 0, topk_per_iter = 0, tree_size = 0, frspec_vocab = 0;
+    int draft_layers = 0;   // the drafter's own transformer layers: their KV pools follow the base model's
+    int eagle_window = 0;   // block sliding window of those layers, in tokens (0 = none)
     // storage
     bool storage = false;
     int num_pages = 0;
@@ -170,7 +172,7 @@ extern "C" int cpmcu_init_minicpm4_eagle_model(int num_layers, int num_iter, int
                                                int torch_dtype, int apply_eagle_quant, int group_size,
                                                int eagle_window_size, int frspec_vocab_size, float residual_scale,
                                                int use_input_norm, int use_attn_norm) {
-    (void)num_layers; (void)group_size; (void)eagle_window_size; (void)residual_scale; (void)use_input_norm; (void)use_attn_norm;
+    (void)group_size; (void)residual_scale; (void)use_input_norm; (void)use_attn_norm;
     int rc = require_model(false);
     if (rc) return rc;
     rc = check_dtype(torch_dtype);
@@ -186,7 +188,12 @@ extern "C" int cpmcu_init_minicpm4_eagle_model(int num_layers, int num_iter, int
     CPMCU_CHECK_ARG(num_iter >= 1 && topk_per_iter >= 1 && topk_per_iter <= tree_size - 1 && topk_per_iter <= 16,
                     "init_minicpm4_eagle_model: topk_per_iter=%d must be in [1, min(16, tree_size-1)]", topk_per_iter);
     CPMCU_CHECK_ARG(frspec_vocab_size >= 0 && frspec_vocab_size <= m.vocab, "init_minicpm4_eagle_model: frspec_vocab_size=%d", frspec_vocab_size);
+    CPMCU_CHECK_ARG(num_layers >= 0 && num_layers <= 64, "init_minicpm4_eagle_model: num_layers=%d outside [0, 64]", num_layers);
+    CPMCU_CHECK_ARG(eagle_window_size == 0 || eagle_window_size >= 128,
+                    "init_minicpm4_eagle_model: eagle_window_size=%d must be 0 or at least one block of 128", eagle_window_size);
     m.drafter = true;
+    m.draft_layers = num_layers;
+    m.eagle_window = eagle_window_size;
     m.num_iter = num_iter;
     m.topk_per_iter = topk_per_iter;
     m.tree_size = tree_size;
@@ -213,7 +220,7 @@ extern "C" int cpmcu_init_storage(int* max_context) {
         used += bytes;
         return CPMCU_OK;
     };
-    const int max_tree = m.drafter ? m.tree_size : 64;
+    const int max_tree = 64;  // decode_attention / draft_attention accept up to 64 rows whatever the tree size
     if ((rc = alloc((void**)&m.lm_head, cpmcu_head_weight_tiled_bytes(m.vocab, m.hidden)))) return rc;  // kept in tiled layout
     if (m.drafter && m.frspec_vocab != m.vocab) {
         if ((rc = alloc((void**)&m.fr_head, cpmcu_head_weight_tiled_bytes(m.frspec_vocab, m.hidden)))) return rc;
@@ -238,7 +245,8 @@ extern "C" int cpmcu_init_storage(int* max_context) {
     // KV pools take what is left of the budget, in whole pages (the reference gives the KV cache
     // all remaining pool memory, src/model/kvcache.cuh:50).
     const size_t page_bytes = (size_t)m.kv_heads * kPage * kHeadDim * 2;  // one of K/V, one layer
-    const size_t per_page_all = page_bytes * 2 * m.layers + 4;
+    const int all_layers = m.layers + m.draft_layers;  // the drafter's layers keep caches of the same length (src/model/minicpm4/minicpm4_eagle.cuh:76,183-184)
+    const size_t per_page_all = page_bytes * 2 * all_layers + 4;
     const size_t remaining = budget > used ? budget - used : 0;
     const size_t free_now = free_b > used ? free_b - used : 0;
     size_t pages = std::min(remaining, (size_t)(free_now * 0.95)) / per_page_all;
@@ -257,9 +265,9 @@ extern "C" int cpmcu_init_storage(int* max_context) {
     pages -= ws_pages;
     CPMCU_HIP(hipMalloc(&m.attn_ws, m.attn_ws_bytes));
     m.num_pages = (int)pages;
-    m.k_pools.assign(m.layers, nullptr);
-    m.v_pools.assign(m.layers, nullptr);
-    for (int l = 0; l < m.layers; ++l) {
+    m.k_pools.assign(all_layers, nullptr);
+    m.v_pools.assign(all_layers, nullptr);
+    for (int l = 0; l < all_layers; ++l) {
         CPMCU_HIP(hipMalloc(&m.k_pools[l], page_bytes * pages));
         CPMCU_HIP(hipMalloc(&m.v_pools[l], page_bytes * pages));
         CPMCU_HIP(hipMemset(m.k_pools[l], 0, page_bytes * pages));
@@ -377,6 +385,34 @@ extern "C" int cpmcu_decode_attention(int layer, int input_length, int padded_le
                                 m.attn_ws_bytes, 0, st);
 }
 
+extern "C" int cpmcu_draft_attention(int draft_layer, int input_length, int padded_length, uint64_t q, uint64_t k_new,
+                                     uint64_t v_new, uint64_t cache_length, uint64_t mask_2d, int mask_k_range, uint64_t out) {
+    int rc = require_model(true);
+    if (rc) return rc;
+    Model& m = *g_model;
+    if (!m.drafter) {
+        set_error("draft_attention: no drafter configured");
+        return CPMCU_ERR_RUNTIME;
+    }
+    CPMCU_CHECK_ARG(draft_layer >= 0 && draft_layer < m.draft_layers, "draft_attention: layer %d outside [0, %d)", draft_layer,
+                    m.draft_layers);
+    CPMCU_CHECK_ARG(input_length >= 1 && input_length <= 64, "draft_attention: input_length=%d outside [1, 64]", input_length);
+    CPMCU_CHECK_ARG(padded_length >= input_length && padded_length <= m.num_pages * kPage,
+                    "draft_attention: padded_length=%d outside [%d, %d]", padded_length, input_length, m.num_pages * kPage);
+    CPMCU_CHECK_ARG(q && k_new && v_new && cache_length && out, "draft_attention: null pointer argument");
+    CPMCU_CHECK_ARG(mask_2d ? (mask_k_range >= input_length && mask_k_range <= 64) : mask_k_range == 0,
+                    "draft_attention: mask_k_range=%d (one uint64 per row covers [input_length, 64] columns; 0 without a mask)",
+                    mask_k_range);
+    hipStream_t st = resolve_stream(nullptr);
+    PerfScope perf("DRAFT_ATTN_CORE", st);
+    const int l = m.layers + draft_layer;
+    const uint64_t* mask = mask_2d ? (const uint64_t*)mask_2d : m.chain_mask;
+    return cpmcu_tree_attention_window((const void*)q, m.k_pools[l], m.v_pools[l], m.block_table, (const int32_t*)cache_length,
+                                       padded_length, (const void*)k_new, (const void*)v_new, nullptr, m.eagle_window, mask, 1,
+                                       mask_k_range, input_length, m.q_heads, m.kv_heads, 1.f / sqrtf((float)kHeadDim), (void*)out,
+                                       m.attn_ws, m.attn_ws_bytes, 0, st);
+}
+
 extern "C" int cpmcu_decode_lm_head(int input_length, uint64_t hidden, uint64_t logits, uint64_t gt) {
     int rc = require_model(true);
     if (rc) return rc;
@@ -452,7 +488,8 @@ extern "C" int cpmcu_model_pointers(int layer, uint64_t* k_pool, uint64_t* v_poo
     int rc = require_model(true);
     if (rc) return rc;
     Model& m = *g_model;
-    CPMCU_CHECK_ARG(layer >= 0 && layer < m.layers, "model_pointers: layer %d outside [0, %d)", layer, m.layers);
+    CPMCU_CHECK_ARG(layer >= 0 && layer < m.layers + m.draft_layers, "model_pointers: layer %d outside [0, %d)", layer,
+                    m.layers + m.draft_layers);
     if (k_pool) *k_pool = (uint64_t)m.k_pools[layer];
     if (v_pool) *v_pool = (uint64_t)m.v_pools[layer];
     if (block_table) *block_table = (uint64_t)m.block_table;

@@ -77,7 +77,11 @@ struct AttnParams {
     int mask_k_range;  // trailing key columns the mask bits refer to (>= T; = T for the verify tree)
     int T, Hq, Hkv, group;
     int num_splits, num_mtiles, rows_pad;
-    int ntiles_max;  // ceil(max_kv_len / 64): the split partition is fixed by the host-side bound
+    int ntiles_max;  // tiles the split partition spans: ceil(max_kv_len / 64), fixed by the host-side bound
+                     // (with a window: the most tiles a window can hold, counted from its first tile)
+    int table_pages;    // entries of block_table the caller guarantees: ceil(max_kv_len / 256)
+    int window_blocks;  // block sliding window in blocks of 128 keys (0 = none): key blocks below
+                        // ceil(P / 128) - window_blocks are not visited (src/flash_attn/src/flash_blockmask.h:32,43-46)
     float scale_log2;
     f16* out;
     // Split partials in the accumulator's own layout, so that both the split kernel's stores and the
@@ -242,13 +246,20 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
     // With the fused append the last split also patches the appended rows into its tiles, which costs
     // about as much as an iteration: the partition counts two tiles' worth of extra work at the end
     // of the stream (three when the appended K rows are also rotated there), so that split gets fewer real tiles.
+    // A block sliding window moves the start of the stream to its first visible tile, which depends on
+    // the device-side length: such calls (the drafter's own layer, a few tiles in all) pay the extra
+    // round trip in front of the page ids.
+    int tile_lo = 0;
+    if (p.window_blocks > 0)
+        tile_lo = max((p.kv_len[0] - p.T + 127) / 128 - p.window_blocks, 0) * (128 / kTileN);
     const int vtiles = p.ntiles_max + (p.k_new != nullptr && p.num_splits > 1 ? (ROPE ? 3 : 2) : 0);
-    const int t0 = min((int)(((long long)split * vtiles) / p.num_splits), p.ntiles_max);
-    const int t1_max = min((int)(((long long)(split + 1) * vtiles) / p.num_splits), p.ntiles_max);
+    const int t0 = tile_lo + min((int)(((long long)split * vtiles) / p.num_splits), p.ntiles_max);
+    const int t1_max = tile_lo + min((int)(((long long)(split + 1) * vtiles) / p.num_splits), p.ntiles_max);
     const int pg0 = (t0 * kTileN) / kPage;
     if (t1_max > t0) {
         const int npg = ((t1_max * kTileN - 1) / kPage) - pg0 + 1;
-        for (int i = tid; i < npg; i += kThreads) s_pages[i] = p.block_table[pg0 + i];
+        // (a window's last tile slot can lie past the host bound; it is never consumed, and the table is not read there)
+        for (int i = tid; i < npg; i += kThreads) s_pages[i] = p.block_table[min(pg0 + i, p.table_pages - 1)];
     }
     const int S = p.kv_len[0];
     const int P = S - p.T;              // the T query tokens are the last T keys
@@ -469,6 +480,15 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
                         sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[ks * 2 + kb], qreg[ks], sacc[kb], 0, 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
             }
+            // The V^T operands of this tile are requested now, so that they arrive under the softmax
+            // arithmetic and the probability MFMAs start without waiting for LDS.
+            f16x8 vf[16];
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+#pragma unroll
+                for (int db = 0; db < 4; ++db)
+                    vf[j * 4 + db] = *reinterpret_cast<const f16x8*>(stage + v_lds_off(db * 32 + qcol, 2 * j + hf));
+            __builtin_amdgcn_sched_barrier(0);
             // sacc[kb][r] is the score of key  c0 + kb*32 + 8*(r/4) + 4*hf + r%4  for query qcol.
             if (c0 + kTileN > Pm) {  // tile touches masked columns or the end of the stream
                 // 64-bit visibility word of this tile for the lane's query: bit x <-> key c0 + x.  Prefix
@@ -540,12 +560,6 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
 
             // ---- O^T += V^T.P^T ----
             {
-                f16x8 vf[16];
-#pragma unroll
-                for (int j = 0; j < 4; ++j)
-#pragma unroll
-                    for (int db = 0; db < 4; ++db)
-                        vf[j * 4 + db] = *reinterpret_cast<const f16x8*>(stage + v_lds_off(db * 32 + qcol, 2 * j + hf));
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
@@ -739,7 +753,7 @@ extern "C" size_t cpmcu_tree_attention_workspace_bytes(int T, int Hq, int Hkv, i
 
 static int tree_attention_impl(const void* q, void* k_pool, void* v_pool,
                                const int32_t* block_table, const int32_t* kv_len, int max_kv_len,
-                               const void* k_new, const void* v_new, const float* rope_cos_sin,
+                               const void* k_new, const void* v_new, const float* rope_cos_sin, int block_window_size,
                                const uint64_t* mask, int mask_words, int mask_k_range, int T, int Hq, int Hkv,
                                float scale, void* out, void* workspace, size_t workspace_bytes,
                                int num_splits_override, void* stream) {
@@ -754,6 +768,8 @@ static int tree_attention_impl(const void* q, void* k_pool, void* v_pool,
                     "tree_attention: mask_words=%d does not match mask_k_range=%d", mask_words, mask_k_range);
     CPMCU_CHECK_ARG(num_splits_override >= 0 && num_splits_override <= kMaxSplits,
                     "tree_attention: num_splits_override=%d outside [0, %d]", num_splits_override, kMaxSplits);
+    CPMCU_CHECK_ARG(block_window_size == 0 || block_window_size >= 128,
+                    "tree_attention: block_window_size=%d must be 0 (no window) or at least one block of 128", block_window_size);
     const int group = Hq / Hkv;
     AttnParams p;
     p.q = (const f16*)q;
@@ -774,15 +790,21 @@ static int tree_attention_impl(const void* q, void* k_pool, void* v_pool,
     p.Hq = Hq;
     p.Hkv = Hkv;
     p.group = group;
-    const int G = choose_groups(max_kv_len);
+    // Keys the stream can hold: the whole context, or with a window its blocks plus the T new rows
+    // (the window starts on a block boundary at or above P - block_window_size).
+    p.window_blocks = block_window_size / 128;
+    int span = max_kv_len;
+    if (p.window_blocks > 0 && p.window_blocks * 128 + T < span) span = p.window_blocks * 128 + T;
+    const int G = choose_groups(span);
     p.num_mtiles = ceil_div(group * T, rows_per_wg(G));
     p.rows_pad = p.num_mtiles * rows_per_wg(G);
-    p.num_splits = num_splits_override > 0 ? num_splits_override : choose_splits(T, group, Hkv, max_kv_len, G);
+    p.num_splits = num_splits_override > 0 ? num_splits_override : choose_splits(T, group, Hkv, span, G);
     // a split keeps the physical page ids of its range in LDS
-    const int min_splits = ceil_div(ceil_div(max_kv_len, kPage) + 2, kMaxPagesPerSplit - 2);
+    const int min_splits = ceil_div(ceil_div(span, kPage) + 2, kMaxPagesPerSplit - 2);
     if (p.num_splits < min_splits) p.num_splits = min_splits;
     CPMCU_CHECK_ARG(p.num_splits <= kMaxSplits, "tree_attention: max_kv_len=%d is beyond the supported context", max_kv_len);
-    p.ntiles_max = ceil_div(max_kv_len, kTileN);
+    p.ntiles_max = ceil_div(span, kTileN);
+    p.table_pages = ceil_div(max_kv_len, kPage);
     p.scale_log2 = scale * 1.4426950408889634f;
     p.out = (f16*)out;
     p.o_part = nullptr;
@@ -820,7 +842,7 @@ extern "C" int cpmcu_tree_attention(const void* q, void* k_pool, void* v_pool,
                                     const uint64_t* mask, int mask_words, int mask_k_range, int T, int Hq, int Hkv,
                                     float scale, void* out, void* workspace, size_t workspace_bytes,
                                     int num_splits_override, void* stream) {
-    return tree_attention_impl(q, k_pool, v_pool, block_table, kv_len, max_kv_len, k_new, v_new, nullptr, mask, mask_words,
+    return tree_attention_impl(q, k_pool, v_pool, block_table, kv_len, max_kv_len, k_new, v_new, nullptr, 0, mask, mask_words,
                                mask_k_range, T, Hq, Hkv, scale, out, workspace, workspace_bytes, num_splits_override, stream);
 }
 
@@ -831,8 +853,21 @@ extern "C" int cpmcu_tree_attention_rope(const void* q, void* k_pool, void* v_po
                                          float scale, void* out, void* workspace, size_t workspace_bytes,
                                          int num_splits_override, void* stream) {
     CPMCU_CHECK_ARG(rope_cos_sin, "tree_attention_rope: null rotary table");
-    return tree_attention_impl(q, k_pool, v_pool, block_table, kv_len, max_kv_len, k_new, v_new, rope_cos_sin, mask, mask_words,
+    return tree_attention_impl(q, k_pool, v_pool, block_table, kv_len, max_kv_len, k_new, v_new, rope_cos_sin, 0, mask, mask_words,
                                mask_k_range, T, Hq, Hkv, scale, out, workspace, workspace_bytes, num_splits_override, stream);
+}
+
+extern "C" int cpmcu_tree_attention_window(const void* q, void* k_pool, void* v_pool,
+                                           const int32_t* block_table, const int32_t* kv_len, int max_kv_len,
+                                           const void* k_new, const void* v_new, const float* rope_cos_sin,
+                                           int block_window_size,
+                                           const uint64_t* mask, int mask_words, int mask_k_range, int T, int Hq, int Hkv,
+                                           float scale, void* out, void* workspace, size_t workspace_bytes,
+                                           int num_splits_override, void* stream) {
+    CPMCU_CHECK_ARG(block_window_size >= 0, "tree_attention_window: block_window_size=%d is negative", block_window_size);
+    return tree_attention_impl(q, k_pool, v_pool, block_table, kv_len, max_kv_len, k_new, v_new, rope_cos_sin, block_window_size,
+                               mask, mask_words, mask_k_range, T, Hq, Hkv, scale, out, workspace, workspace_bytes,
+                               num_splits_override, stream);
 }
 
 namespace cpmcu {

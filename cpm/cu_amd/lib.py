@@ -33,6 +33,7 @@ SIGNATURES = {
     "cpmcu_verify_and_fix": (c_int, [c_int, c_u64, c_u64, c_u64, c_u64, c_u64, c_u64, ctypes.POINTER(c_int)]),
     "cpmcu_print_perf_summary": (c_int, []),
     "cpmcu_decode_attention": (c_int, [c_int, c_int, c_int, c_u64, c_u64, c_u64, c_u64, c_u64, c_u64]),
+    "cpmcu_draft_attention": (c_int, [c_int, c_int, c_int, c_u64, c_u64, c_u64, c_u64, c_u64, c_int, c_u64]),
     "cpmcu_decode_lm_head": (c_int, [c_int, c_u64, c_u64, c_u64]),
     "cpmcu_draft_head": (c_int, [c_int, c_u64, c_u64, c_u64, c_u64]),
     "cpmcu_set_block_table": (c_int, [_P, c_int]),
@@ -43,6 +44,7 @@ SIGNATURES = {
     "cpmcu_tree_attention_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "cpmcu_tree_attention": (c_int, [_P, _P, _P, _P, _P, c_int, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_float, _P, _P, c_size_t, c_int, _P]),
     "cpmcu_tree_attention_rope": (c_int, [_P, _P, _P, _P, _P, c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_float, _P, _P, c_size_t, c_int, _P]),
+    "cpmcu_tree_attention_window": (c_int, [_P, _P, _P, _P, _P, c_int, _P, _P, _P, c_int, _P, c_int, c_int, c_int, c_int, c_int, c_float, _P, _P, c_size_t, c_int, _P]),
     "cpmcu_rope_table": (c_int, [_P, _P, c_int, _P, _P]),
     "cpmcu_rope_apply": (c_int, [_P, c_int, c_int, c_int, _P, _P, _P]),
     "cpmcu_gather_rows": (c_int, [_P, _P, c_int, c_int, _P, _P]),

@@ -77,7 +77,7 @@ def rope_apply_(table, q, k):
 
 
 def tree_attention(q, cache, layer, kv_len, max_kv_len, mask=None, scale=None, num_splits=0, out=None,
-                   k_new=None, v_new=None, mask_k_range=0, rope=None):
+                   k_new=None, v_new=None, mask_k_range=0, rope=None, block_window_size=0):
     """mha_fwd_kvcache with a tree mask (src/flash_attn/flash_api.hpp:292-392) on the paged cache.
 
     q [T, Hq, 128] fp16; kv_len int32[1] on the device = P + T; mask uint64 [T, W] or None (chain).
@@ -85,6 +85,8 @@ def tree_attention(q, cache, layer, kv_len, max_kv_len, mask=None, scale=None, n
     itself (src/model/attn.cuh:200) instead of expecting them there.
     mask_k_range (0 = T): number of trailing keys the mask bits refer to; k*d for the drafter's layers.
     rope [T, 64, 2] fp32 from rope_table: q and k_new are taken unrotated and rotated inside the kernel.
+    block_window_size (0 = none, else >= 128 tokens): the drafter layer's block sliding window
+    (src/flash_attn/src/flash_blockmask.h:32): key blocks of 128 below ceil(P/128) - window/128 are skipped.
     """
     T, Hq, D = q.shape
     assert D == HEAD_DIM and q.dtype == torch.float16 and kv_len.dtype == torch.int32
@@ -103,8 +105,15 @@ def tree_attention(q, cache, layer, kv_len, max_kv_len, mask=None, scale=None, n
         assert k_new.dtype == torch.float16 and v_new.dtype == torch.float16
         assert k_new.numel() == T * cache.Hkv * HEAD_DIM and v_new.numel() == k_new.numel()
     if rope is not None:
-        # rotary embedding of q and of the appended K rows fused into the kernel (table from rope_table)
         assert rope.dtype == torch.float32 and rope.numel() == T * HEAD_DIM
+    if block_window_size:
+        _lib().tree_attention_window(_ptr(q), _ptr(cache.k[layer]), _ptr(cache.v[layer]), _ptr(cache.block_table), _ptr(kv_len),
+                                     int(max_kv_len), _ptr(k_new), _ptr(v_new), _ptr(rope), int(block_window_size), _ptr(mask), W,
+                                     int(mask_k_range), T, Hq, cache.Hkv, ctypes.c_float(scale), _ptr(out), _ptr(ws), ws.numel(),
+                                     int(num_splits), _stream())
+        return out
+    if rope is not None:
+        # rotary embedding of q and of the appended K rows fused into the kernel (table from rope_table)
         _lib().tree_attention_rope(_ptr(q), _ptr(cache.k[layer]), _ptr(cache.v[layer]), _ptr(cache.block_table), _ptr(kv_len),
                                    int(max_kv_len), _ptr(k_new), _ptr(v_new), _ptr(rope), _ptr(mask), W, int(mask_k_range), T, Hq,
                                    cache.Hkv, ctypes.c_float(scale), _ptr(out), _ptr(ws), ws.numel(), int(num_splits), _stream())

@@ -130,6 +130,20 @@ int cpmcu_print_perf_summary(void);
 int cpmcu_decode_attention(int layer, int input_length, int padded_length, uint64_t q, uint64_t k_new,
                            uint64_t v_new, uint64_t cache_length, uint64_t mask_2d, uint64_t out);
 
+/* The same slice of Attention::decode for the drafter's own layer(s)
+ * (src/model/minicpm4/minicpm4_eagle.cuh:247,359; src/model/eagle.cuh:188-233): they keep KV caches of
+ * their own (minicpm4_eagle.cuh:76,183) and attend through the block sliding window
+ * eagle_window_size given to init_minicpm4_eagle_model (Attention::window_size,
+ * src/model/attn.cuh:228; see cpmcu_tree_attention_window).
+ *   draft_layer: index into the drafter's num_layers layers.
+ *   mask_2d / mask_k_range: Mask(eagle_mask_2d, k, k * d) of round d -- one uint64 per row whose bits
+ *           refer to the last mask_k_range <= 64 keys; 0 / 0 = causal chain (the drafter's prefill of
+ *           the accepted tokens, in chunks of <= 64 rows).
+ * The accepted-path compaction of cpmcu_verify_and_fix does not touch these caches, as in the
+ * reference (fix_kv_cache runs over the base model's caches only). */
+int cpmcu_draft_attention(int draft_layer, int input_length, int padded_length, uint64_t q, uint64_t k_new,
+                          uint64_t v_new, uint64_t cache_length, uint64_t mask_2d, int mask_k_range, uint64_t out);
+
 /* LMHead::prefill on the loaded lm_head (src/model/linear.cuh:82-101,
  * src/model/model.cuh:164) plus the arg-max the reference leaves to PyTorch
  * (cpmcu/speculative/tree_drafter.py:153,233).  logits ([>=n][vocab] fp16) and
@@ -148,7 +162,8 @@ int cpmcu_draft_head(int n, uint64_t hidden, uint64_t topk_val, uint64_t topk_po
 int cpmcu_set_block_table(const int32_t* host_table, int n);
 
 /* No reference counterpart: device addresses of the model's storage, for harnesses that fill the
- * paged cache directly (any of the outputs may be NULL). */
+ * paged cache directly (any of the outputs may be NULL).  Layers [num_hidden_layers,
+ * num_hidden_layers + drafter num_layers) are the drafter's own caches. */
 int cpmcu_model_pointers(int layer, uint64_t* k_pool, uint64_t* v_pool, uint64_t* block_table, int* num_pages);
 
 /* Synchronise the library's stream. */
@@ -222,6 +237,25 @@ int cpmcu_tree_attention_rope(const void* q, void* k_pool, void* v_pool, const i
                               const float* rope_cos_sin, const uint64_t* mask, int mask_words, int mask_k_range,
                               int T, int Hq, int Hkv, float scale, void* out,
                               void* workspace, size_t workspace_bytes, int num_splits_override, void* stream);
+
+/* The same attention with the block-granular sliding window of the drafter's own layer --
+ * fwdIterator without a block mask, src/flash_attn/src/flash_blockmask.h:9,16,32,43-46, reached through
+ * mha_fwd_kvcache's block_window_size (src/flash_attn/flash_api.hpp:316,368) = Attention::window_size
+ * (src/model/attn.cuh:228) = eagle_window_size of init_minicpm4_eagle_model.
+ *   block_window_size: in tokens; 0 = no window, otherwise >= 128.  With P = *kv_len - T, the key
+ *           blocks of 128 below  ceil(P / 128) - block_window_size / 128  are not visited (the
+ *           reference's split-KV kernel walks K in blocks of 128 for head dimension 128,
+ *           src/flash_attn/src/flash_fwd_launch_template.h:208): the queries see the keys from
+ *           128 * that block index on, under the same mask and causal rules as above.
+ *   rope_cos_sin: as for cpmcu_tree_attention_rope, or NULL for inputs that are already rotated.
+ * The kernel starts its KV stream at the window's first block, so the cost follows the window, not
+ * the context; max_kv_len still bounds *kv_len and the page table. */
+int cpmcu_tree_attention_window(const void* q, void* k_pool, void* v_pool, const int32_t* block_table,
+                                const int32_t* kv_len, int max_kv_len, const void* k_new, const void* v_new,
+                                const float* rope_cos_sin, int block_window_size,
+                                const uint64_t* mask, int mask_words, int mask_k_range,
+                                int T, int Hq, int Hkv, float scale, void* out,
+                                void* workspace, size_t workspace_bytes, int num_splits_override, void* stream);
 
 /* remap_copy -- src/model/tree_drafter.cuh:79-86,103-107: dst[r][:] = src[remap[r]][:]. */
 int cpmcu_gather_rows(const void* src, const int32_t* remap, int rows, int dim, void* dst, void* stream);

@@ -35,6 +35,7 @@ def _load():
         "orc_num_threads": (i32, []),
         "orc_set_num_threads": (None, [i32]),
         "orc_tree_attention": (None, [c_p, c_p, c_p, c_p, i32, i32, i32, i32, i32, i32, i32, f32, c_p, c_p]),
+        "orc_tree_attention_window": (None, [c_p, c_p, c_p, c_p, i32, i32, i32, i32, i32, i32, i32, i32, f32, c_p, c_p]),
         "orc_gather_rows": (None, [c_p, c_p, i32, i32, c_p]),
         "orc_lm_head": (None, [c_p, c_p, i32, i32, i32, i32, f32, c_p]),
         "orc_log_softmax": (None, [c_p, i32, i32, c_p, c_p]),
@@ -95,9 +96,10 @@ def mask_words(T):
     return (T + 63) // 64
 
 
-def tree_attention(q, k, v, mask, P, scale=None, return_lse=False, mask_k_range=None):
+def tree_attention(q, k, v, mask, P, scale=None, return_lse=False, mask_k_range=None, block_window_size=0):
     """q [T,Hq,D] f16; k,v [P+T,Hkv,D] f16; mask [T,W] uint64 -> out [T,Hq,D] f16.
-    mask_k_range (default T): number of trailing key columns the mask bits refer to."""
+    mask_k_range (default T): number of trailing key columns the mask bits refer to.
+    block_window_size (default 0 = none): the drafter layer's block sliding window, in tokens."""
     q = _c(q, np.float16)
     k = _c(k, np.float16)
     v = _c(v, np.float16)
@@ -112,8 +114,8 @@ def tree_attention(q, k, v, mask, P, scale=None, return_lse=False, mask_k_range=
     lse = np.empty((T, Hq), np.float32)
     R = T if mask_k_range is None else int(mask_k_range)
     assert T <= R <= S and W == (R + 63) // 64 or (W == 1 and R <= 64)
-    _lib.orc_tree_attention(_p(q), _p(k), _p(v), _p(mask), T, P, Hq, Hkv, D, W, R,
-                            ctypes.c_float(scale), _p(out), _p(lse))
+    _lib.orc_tree_attention_window(_p(q), _p(k), _p(v), _p(mask), T, P, Hq, Hkv, D, W, R, int(block_window_size),
+                                   ctypes.c_float(scale), _p(out), _p(lse))
     return (out, lse) if return_lse else out
 
 

@@ -146,10 +146,20 @@ void orc_set_num_threads(int n) { g_threads = n; }
 
 // A1 -- src/flash_attn/src/mask.h:139-229, softmax.h:66-91,239-256,
 // flash_fwd_kernel.h:1266,1610-1615, flash_api.hpp:103.
-void orc_tree_attention(const uint16_t* q, const uint16_t* k, const uint16_t* v,
-                        const uint64_t* mask, int T, int P, int Hq, int Hkv, int D,
-                        int mask_words, int mask_k_range, float scale, uint16_t* out, float* lse) {
+// block_window_size > 0 adds the block-granular sliding window of the drafter's own layer
+// (src/flash_attn/src/flash_blockmask.h:9,16,32,43-46 with kBlockN = 128,
+// src/flash_attn/src/flash_fwd_launch_template.h:208; passed as Attention::window_size,
+// src/model/attn.cuh:228): key blocks of 128 below
+// ceil(P / 128) - block_window_size / 128 are not visited at all.
+void orc_tree_attention_window(const uint16_t* q, const uint16_t* k, const uint16_t* v,
+                               const uint64_t* mask, int T, int P, int Hq, int Hkv, int D,
+                               int mask_words, int mask_k_range, int block_window_size, float scale,
+                               uint16_t* out, float* lse) {
     const int S = P + T;
+    const int kBlockN = 128;
+    // flash_blockmask.h:9,16: q_block_idx = loop_step_idx (0) + seqlen_k - seqlen_q = P;  :32 k_window_left
+    const int k_window_left = block_window_size > 0 ? (P + kBlockN - 1) / kBlockN - block_window_size / kBlockN : -1;
+    const int first_key = k_window_left > 0 ? k_window_left * kBlockN : 0;
     const int Pm = S - mask_k_range;  // mask.h: mask_k_begin = seqlen_k - mask_k_range
     const int group = Hq / Hkv;
     // flash_api.hpp:103  scale_softmax_log2 = softmax_scale * M_LOG2E
@@ -183,6 +193,7 @@ void orc_tree_attention(const uint16_t* q, const uint16_t* k, const uint16_t* v,
                         vis = (mrow[j >> 6] >> (j & 63)) & 1ull;
                     }
                     if (c > P + i) vis = false;  // mask.h:185-186,199-203 causal: col < row + 1 + seqlen_k - seqlen_q
+                    if (c < first_key) vis = false;  // flash_blockmask.h:43-46: blocks below k_window_left are skipped
                     if (vis) {
                         s[c] = dot_any(qf.data(), &kf[(size_t)c * D], D);
                         m = std::max(m, s[c]);
@@ -211,6 +222,12 @@ void orc_tree_attention(const uint16_t* q, const uint16_t* k, const uint16_t* v,
             }
         }
     }
+}
+
+void orc_tree_attention(const uint16_t* q, const uint16_t* k, const uint16_t* v,
+                        const uint64_t* mask, int T, int P, int Hq, int Hkv, int D,
+                        int mask_words, int mask_k_range, float scale, uint16_t* out, float* lse) {
+    orc_tree_attention_window(q, k, v, mask, T, P, Hq, Hkv, D, mask_words, mask_k_range, 0, scale, out, lse);
 }
 
 // a7 -- src/model/tree_drafter.cuh:79-86

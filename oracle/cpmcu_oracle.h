@@ -67,6 +67,21 @@ void orc_tree_attention(const uint16_t* q, const uint16_t* k, const uint16_t* v,
                         const uint64_t* mask, int T, int P, int Hq, int Hkv, int D,
                         int mask_words, int mask_k_range, float scale, uint16_t* out, float* lse);
 
+/* The same with the block-granular sliding window of the drafter's own layer
+ * (src/flash_attn/src/flash_blockmask.h:9,16,32,43-46; kBlockN = 128 for head
+ * dimension 128, src/flash_attn/src/flash_fwd_launch_template.h:208; the value is
+ * Attention::window_size, src/model/attn.cuh:228 = eagle_window_size):
+ * with block_window_size > 0 the key blocks of 128 below
+ *   k_window_left = ceil(P / 128) - block_window_size / 128
+ * are skipped whole; 0 = no window.
+ * pinned by: equality with orc_tree_attention on the cache cut to its visible
+ * keys [128 * k_window_left, P + T), identity for windows that cover the whole
+ * context, fp64 closed form with the explicit visible set. */
+void orc_tree_attention_window(const uint16_t* q, const uint16_t* k, const uint16_t* v,
+                               const uint64_t* mask, int T, int P, int Hq, int Hkv, int D,
+                               int mask_words, int mask_k_range, int block_window_size, float scale,
+                               uint16_t* out, float* lse);
+
 /* ---- a7: load-time gather of the frequency-ranked rows ----
  * src/model/tree_drafter.cuh:79-86,103-107:  dst[r][:] = src[remap[r]][:].
  * pinned by: numpy fancy indexing. */

@@ -275,6 +275,38 @@ def test_model_level_entry_points(gpu, orc):
         assert_close_f16(to_np(out), orc.tree_attention(q, k, v, tree.mask, P), "decode_attention layer %d" % layer)
         flat += [k.reshape(S, -1).copy(), v.reshape(S, -1).copy()]
 
+    # the drafter's own layer: separate cache, block sliding window of 1024 tokens (eagle_window_size above);
+    # prefix through causal chunks, then one draft round with Mask(eagle_mask_2d, k, k * d)
+    with pytest.raises(ValueError):
+        L.draft_attention(1, 1, 128, 1, 1, 1, 1, 0, 0, 1)  # only one drafter layer
+    kd, dd, Pd = 10, 3, 1500
+    Sd = Pd + kd * dd
+    kq = synth.normal_f16((kd, HQ, D), 9, 1)
+    kk = synth.normal_f16((Sd, HKV, D), 9, 2)
+    vv = synth.normal_f16((Sd, HKV, D), 9, 3)
+    g9 = synth.rng(9, 4)
+    bits = g9.integers(0, 2, size=(kd, kd * dd)).astype(np.uint64)
+    for i in range(kd):
+        bits[i, kd * dd - kd + i] = 1
+    dmask = np.array([sum(int(bits[i, j]) << j for j in range(kd * dd)) for i in range(kd)], np.uint64)
+    done = 0
+    while done < Sd - kd:
+        n = min(64, Sd - kd - done)
+        cl.fill_(done + n)
+        L.draft_attention(0, n, done + n, dev(kq[:1].repeat(n, 0)), dev(kk[done:done + n]), dev(vv[done:done + n]),
+                          cl.data_ptr(), 0, 0, dummy.data_ptr())
+        L.synchronize()
+        done += n
+    cl.fill_(Sd)
+    dout = torch.empty((kd, HQ, D), dtype=torch.float16, device="cuda")
+    L.draft_attention(0, kd, (Sd + 127) // 128 * 128, dev(kq), dev(kk[Sd - kd:]), dev(vv[Sd - kd:]), cl.data_ptr(), dev(dmask),
+                      kd * dd, dout.data_ptr())
+    L.synchronize()
+    ref_w = orc.tree_attention(kq, kk, vv, dmask.reshape(kd, 1), Sd - kd, mask_k_range=kd * dd, block_window_size=1024)
+    assert_close_f16(to_np(dout), ref_w, "draft_attention with the block window")
+    ref_full = orc.tree_attention(kq, kk, vv, dmask.reshape(kd, 1), Sd - kd, mask_k_range=kd * dd)
+    assert np.abs(ref_w.astype(np.float32) - ref_full.astype(np.float32)).max() > 1e-3  # the window cut keys off
+
     hid = synth.normal_f16((T, H), 7, 200)
     logits = torch.empty((64, V), dtype=torch.float16, device="cuda")
     gt = torch.empty(T, dtype=torch.int32, device="cuda")

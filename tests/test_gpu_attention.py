@@ -217,6 +217,84 @@ def test_draft_layer_mask_range(gpu, orc, k, d, P0, seed):
     assert_close_f16(to_np(out), ref, "draft-layer attention k=%d d=%d" % (k, d))
 
 
+@pytest.mark.parametrize("k,d,P0,window,splits,seed", [
+    (10, 1, 100, 128, 0, 1), (10, 3, 127, 128, 0, 2), (10, 3, 128, 128, 1, 3), (10, 3, 129, 128, 0, 4),
+    (10, 6, 1000, 128, 0, 5), (10, 6, 1000, 512, 3, 6), (10, 5, 1024, 1024, 0, 7), (10, 5, 1025, 1024, 0, 8),
+    (10, 6, 5000, 1024, 0, 9), (10, 6, 5000, 1024, 5, 10), (4, 5, 61, 256, 0, 11), (8, 8, 2049, 2048, 0, 12),
+    (10, 2, 9000, 8192, 0, 13), (10, 6, 300, 4096, 0, 14)])
+def test_draft_layer_block_window(gpu, orc, k, d, P0, window, splits, seed):
+    """The drafter's own layer with its block sliding window (eagle_window_size): only the key blocks of 128 from
+    ceil(P/128) - window/128 on are visited.  Queries are the newest k draft tokens, the mask covers k*d
+    columns, the new rows are appended by the kernel; the page table is a seeded permutation."""
+    from cpm.cu_amd import ops
+    from cpm.cu_amd.kvcache import PagedKVCache
+    torch = gpu
+    mask, q, kk, vv, S = _draft_layer_case(k, d, P0, seed)
+    max_len = S + [0, 1, 100, 300][seed % 4]
+    npages = (max_len + 255) // 256 + 1
+    table = synth.rng(seed, 4).permutation(npages).astype(np.int32)
+    cache = PagedKVCache(1, HKV, npages, block_table=table, fill=float("nan"))
+    cache.write_logical(0, 0, to_dev(torch, kk[:S - k]), to_dev(torch, vv[:S - k]))
+    kv_len = torch.tensor([S], dtype=torch.int32, device="cuda")
+    out = ops.tree_attention(to_dev(torch, q), cache, 0, kv_len, max_len, to_dev(torch, mask), mask_k_range=k * d,
+                             k_new=to_dev(torch, kk[S - k:]), v_new=to_dev(torch, vv[S - k:]), num_splits=splits,
+                             block_window_size=window)
+    torch.cuda.synchronize()
+    ref = orc.tree_attention(q, kk, vv, mask, S - k, mask_k_range=k * d, block_window_size=window)
+    assert_close_f16(to_np(out), ref, "windowed draft-layer attention k=%d d=%d P0=%d window=%d" % (k, d, P0, window))
+    kc, vc = cache.read_logical(0, 0, S)
+    assert np.array_equal(to_np(kc).view(np.uint16), kk.view(np.uint16))
+    assert np.array_equal(to_np(vc).view(np.uint16), vv.view(np.uint16))
+    # the window must matter whenever it cuts keys off: compare with the full-context result
+    P = S - k
+    if (P + 127) // 128 - window // 128 > 0:
+        full = orc.tree_attention(q, kk, vv, mask, P, mask_k_range=k * d)
+        assert np.abs(ref.astype(np.float32) - full.astype(np.float32)).max() > 1e-3
+
+
+@pytest.mark.parametrize("P,T,window,rope", [(4096, 60, 1024, False), (4097, 60, 1024, True), (700, 128, 256, True), (33000, 60, 2048, False)])
+def test_tree_block_window_with_rope(gpu, orc, P, T, window, rope):
+    """The window together with a verify-sized tree, the fused append and (optionally) the fused rotary
+    embedding: the cost-relevant part is that the stream starts at the window's first block."""
+    from cpm.cu_amd import ops
+    from cpm.cu_amd.kvcache import PagedKVCache
+    torch = gpu
+    tree = synth.random_tree(T, 900 + P, max_children=5, max_depth=10)
+    S = P + T
+    npages = (S + 255) // 256 + 1
+    q = synth.normal_f16((T, HQ, D), P, 1)
+    k = synth.normal_f16((S, HKV, D), P, 2)
+    v = synth.normal_f16((S, HKV, D), P, 3)
+    cache = PagedKVCache(1, HKV, npages, fill=float("nan"))
+    cache.write_logical(0, 0, to_dev(torch, k[:P]), to_dev(torch, v[:P]))
+    kv_len = torch.tensor([S], dtype=torch.int32, device="cuda")
+    table, q_ref, k_ref = None, q, k
+    if rope:
+        inv_freq = (10000.0 ** (-np.arange(D // 2, dtype=np.float64) / (D // 2))).astype(np.float32)
+        table = ops.rope_table(to_dev(torch, tree.positions(P)), to_dev(torch, inv_freq))
+        q_ref, k_rot = orc.rope(q, k[P:], table=to_np(table))
+        k_ref = np.concatenate([k[:P], k_rot], 0)
+    out = ops.tree_attention(to_dev(torch, q), cache, 0, kv_len, S, to_dev(torch, tree.mask), k_new=to_dev(torch, k[P:]),
+                             v_new=to_dev(torch, v[P:]), rope=table, block_window_size=window)
+    torch.cuda.synchronize()
+    ref = orc.tree_attention(q_ref, k_ref, v, tree.mask, P, block_window_size=window)
+    assert_close_f16(to_np(out), ref, "windowed tree attention P=%d T=%d window=%d rope=%s" % (P, T, window, rope))
+    kc, _ = cache.read_logical(0, P, T)
+    assert np.array_equal(to_np(kc).view(np.uint16), k_ref[P:].view(np.uint16))
+
+
+def test_block_window_argument_checks(gpu):
+    from cpm.cu_amd import ops
+    from cpm.cu_amd.kvcache import PagedKVCache
+    torch = gpu
+    cache = PagedKVCache(1, HKV, 2)
+    q = torch.zeros((4, HQ, D), dtype=torch.float16, device="cuda")
+    kv_len = torch.tensor([100], dtype=torch.int32, device="cuda")
+    for bad in (64, 127, -128):
+        with pytest.raises(Exception):
+            ops.tree_attention(q, cache, 0, kv_len, 100, None, block_window_size=bad)
+
+
 def _sweep_configs():
     """Seeded random (P, T, mode, splits, slack) tuples, biased to tile (64), page (256) and wave-row (2, 16 nodes)
     boundaries; slack = how far the host-side bound on the KV length exceeds the true length."""

@@ -334,6 +334,56 @@ def test_attention_mask_range_wider_than_queries(orc):
     assert np.abs(out - ref).max() < 5e-3
 
 
+def _window_first_key(P, window):
+    """First visible key of the block sliding window, written out from the reference's arithmetic
+    (src/flash_attn/src/flash_blockmask.h:16,32 with kBlockN = 128, loop_step_idx = 0): an independent
+    restatement in Python integers, used only to build the expected visible sets below."""
+    q_block_idx = P
+    k_window_left = (q_block_idx + 127) // 128 - window // 128
+    return max(k_window_left, 0) * 128
+
+
+@pytest.mark.parametrize("P,window", [(100, 128), (127, 128), (128, 128), (129, 128), (255, 128), (256, 256), (257, 256),
+                                      (1000, 128), (1000, 512), (1024, 1024), (1025, 1024), (3000, 1024), (900, 4096)])
+def test_attention_block_window(orc, P, window):
+    """The drafter layer's block sliding window (src/flash_attn/src/flash_blockmask.h:32,43-46) pinned three ways:
+    (1) torch's CPU scaled_dot_product_attention with the explicit visible set; (2) the windowed result equals
+    the plain oracle on a cache cut down to the visible keys, bit for bit (same keys, same order of
+    accumulation); (3) a window that covers the context changes nothing."""
+    import torch
+    g = synth.rng(77, P * 7 + window)
+    k_, d_ = 6, 3
+    T, R, Hq, Hkv, D = k_, k_ * d_, 4, 2, 32
+    S = P + T
+    q = g.standard_normal((T, Hq, D)).astype(np.float16)
+    k = g.standard_normal((S, Hkv, D)).astype(np.float16)
+    v = g.standard_normal((S, Hkv, D)).astype(np.float16)
+    bits = g.integers(0, 2, size=(T, R)).astype(np.uint64)
+    for i in range(T):
+        bits[i, R - T + i] = 1
+    mask = np.array([[sum(int(bits[i, j]) << j for j in range(R))] for i in range(T)], np.uint64)
+    out = orc.tree_attention(q, k, v, mask, P, mask_k_range=R, block_window_size=window)
+    first = _window_first_key(P, window)
+    assert first % 128 == 0 and first <= P and P - first <= window
+    vis = np.zeros((T, S), bool)
+    for i in range(T):
+        for c in range(S):
+            vis[i, c] = c >= first and c <= P + i and (c < S - R or bool(bits[i, c - (S - R)]))
+    qt = torch.from_numpy(q.astype(np.float32)).permute(1, 0, 2)
+    kt = torch.from_numpy(k.astype(np.float32)).permute(1, 0, 2).repeat_interleave(Hq // Hkv, 0)
+    vt = torch.from_numpy(v.astype(np.float32)).permute(1, 0, 2).repeat_interleave(Hq // Hkv, 0)
+    ref = torch.nn.functional.scaled_dot_product_attention(qt, kt, vt, attn_mask=torch.from_numpy(vis)).permute(1, 0, 2).numpy()
+    assert np.abs(out.astype(np.float32) - ref).max() < 5e-3
+    if S - first >= R:  # the cut cache still holds every column the mask bits refer to
+        cut = orc.tree_attention(q, k[first:], v[first:], mask, P - first, mask_k_range=R)
+        assert np.array_equal(out.view(np.uint16), cut.view(np.uint16))
+    if first == 0:
+        plain = orc.tree_attention(q, k, v, mask, P, mask_k_range=R)
+        assert np.array_equal(out.view(np.uint16), plain.view(np.uint16))
+    else:
+        assert not np.array_equal(out.view(np.uint16), orc.tree_attention(q, k, v, mask, P, mask_k_range=R).view(np.uint16))
+
+
 def test_accept_commit_tail_against_numpy():
     """The oracle's restatement of verify() after the acceptance, pinned on what fixes it independently:
     the hidden gather is numpy fancy indexing, compaction is "rows P+path[d] land at P+d, nothing else
