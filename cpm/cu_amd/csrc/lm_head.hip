@@ -14,12 +14,17 @@
 // loads of W in flight per CU, not about MFMA peak:
 //   * one persistent workgroup of 8 waves per CU; every wave owns whole 16-row blocks of W and
 //     the full K range, so nothing is reduced across waves inside the loop;
-//   * W goes HBM -> registers directly as the A operand of v_mfma_f32_16x16x32_f16 (lane =
-//     (row % 16, k-group): 4 lanes read 64 contiguous bytes of a row, the next k-step the other
-//     half of the 128-byte line), 16 loads in flight per wave, software-pipelined across row
-//     blocks;
-//   * the hidden rows are the B operand, staged once per workgroup in LDS (128 KB for n <= 16,
-//     K-chunked and double-buffered for more rows).
+//   * W goes HBM -> registers directly as the A operand of v_mfma_f32_16x16x32_f16.  In the tiled
+//     layout (cpmcu_head_weight_tile: [V/16][H/32][64 lanes][8 halves]) every wave instruction
+//     reads one contiguous KB and consecutive k-steps are consecutive in memory; the row-major
+//     layout is read as lane = (row % 16, k-group), 4 lanes per 64 contiguous bytes of a row;
+//   * the hidden rows are the B operand, staged in LDS: resident for the whole K range with up
+//     to 16 rows on the row-major path (head_gemm_kernel), otherwise walked in K chunks that are
+//     brought in by direct-to-LDS loads, double buffered, in the OUTER loop, with one accumulator
+//     set per row block of a sweep (head_gemm_chunked_kernel);
+//   * when the row blocks do not divide evenly over the wave slots, the blocks of the partly
+//     filled last pass are dealt round-robin to the workgroups and several waves share each of
+//     them, every one taking a subset of the K chunks; their partial sums meet in LDS.
 #include "common.h"
 #include "internal.h"
 #include "topk_keys.h"
