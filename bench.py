@@ -7,8 +7,11 @@ One "step" = one pass of the verify hot path over one batch of synthetic MiniCPM
 with every input already resident in HBM: for each of the 32 layers append the 60 tree rows' K/V and
 run tree-masked attention (one fused kernel + the split merge) over the paged cache (4096-token prefix + 60 tree rows), then the target
 lm_head (73448 x 4096) with fused arg-max, greedy tree acceptance and accepted-path KV compaction in
-all layers.  The step is captured once into a HIP graph (the reference replays a CUDA graph for
-decode as well) and replayed; exactly K replays are timed between synchronisations.
+all layers.  The step is captured into a HIP graph (the reference replays a CUDA graph for
+decode as well) and replayed; exactly K replays are timed between synchronisations.  At 4K context
+the K/V of all layers would fit the 256 MB last-level cache, so the timed steps rotate over four
+distinct copies of the K/V pools (one graph each): every pass over K/V comes from HBM.  The time of
+replays on a single copy is reported beside it (`us_per_step_one_kv_set`).
 
 Prints ONE JSON line.  `value` is microseconds per step (lower is better).  `roofline` is for the
 kernel that takes the largest share of the step; `kernels` lists all of them; `contexts` gives the
@@ -114,26 +117,31 @@ class Workload:
 
 
 def timed_replays(torch, fn, steps, warmup, use_graph):
-    """Capture fn() once (unless disabled), run `warmup` untimed and exactly `steps` timed calls."""
+    """Capture fn() once (unless disabled), run `warmup` untimed and exactly `steps` timed calls.
+    `fn` may be a list of callables: each is captured on its own and the calls cycle through them."""
+    fns = list(fn) if isinstance(fn, (list, tuple)) else [fn]
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
-        fn()  # eager once: allocates workspaces outside capture
-        stream.synchronize()
-        run = fn
-        if use_graph:
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, stream=stream):
-                fn()
-            run = graph.replay
-        for _ in range(warmup):
-            run()
+        runs = []
+        for f in fns:
+            f()  # eager once: allocates workspaces outside capture
+            stream.synchronize()
+            if use_graph:
+                graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(graph, stream=stream):
+                    f()
+                runs.append(graph.replay)
+            else:
+                runs.append(f)
+        for i in range(warmup):
+            runs[i % len(runs)]()
         stream.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         e0.record(stream)
-        for _ in range(steps):
-            run()
+        for i in range(steps):
+            runs[i % len(runs)]()
         e1.record(stream)
         stream.synchronize()
         torch.cuda.synchronize()
@@ -209,8 +217,32 @@ def main():
     def full_step():
         vs.enqueue(wl.q, wl.k_new, wl.v_new, wl.hidden, wl.draft_ids, attn_out=wl.attn_out, splits=args.splits)
 
-    ms_step, wall_ms = timed_replays(torch, full_step, args.steps, args.warmup, use_graph)
-    a_gpu, ids_gpu = vs.result()
+    # The 32 layers' K/V at 4K context (~150 MB) fit the 256 MB last-level cache, so replays of the step on
+    # one set of pools are partly served from it.  The headline therefore rotates the timed steps over
+    # KV_SETS distinct copies of the pools (step i works on copy i % KV_SETS): every pass over K/V comes
+    # from HBM, as it does in a decode loop that streams the dense layers' weights in between.  Longer
+    # contexts exceed the cache by themselves and use one set.
+    KV_SETS = 4 if wl.P <= 8192 else 1
+    caches = [wl.cache]
+    if KV_SETS > 1:
+        from cpm.cu_amd.kvcache import PagedKVCache
+        for _ in range(KV_SETS - 1):
+            c2 = PagedKVCache(wl.L, wl.cache.Hkv, wl.cache.num_pages, device="cuda", block_table=wl.cache.block_table)
+            for l in range(wl.L):
+                c2.k[l].copy_(wl.cache.k[l])
+                c2.v[l].copy_(wl.cache.v[l])
+            caches.append(c2)
+    rot_steps = [vs] + [VerifyStep(c, w_t, wl.mask, wl.parent, wl.pos, wl.P) for c in caches[1:]]
+
+    def step_on(st):
+        return lambda: st.enqueue(wl.q, wl.k_new, wl.v_new, wl.hidden, wl.draft_ids, attn_out=wl.attn_out, splits=args.splits)
+
+    ms_step, wall_ms = timed_replays(torch, [step_on(st) for st in rot_steps], args.steps, args.warmup, use_graph)
+    results = [st.result() for st in rot_steps]
+    a_gpu, ids_gpu = results[0]
+    sets_agree = all(r[0] == a_gpu and np.array_equal(r[1], ids_gpu) for r in results)
+    ms_step_warm = timed_replays(torch, full_step, max(5, args.steps // 2), 2, use_graph)[0] if KV_SETS > 1 else ms_step
+    del rot_steps
 
     # ---- per-operator timings (same inputs, each operator alone, graph-replayed) ----
     reps = max(5, args.steps // 5)
@@ -266,7 +298,15 @@ def main():
             ops.tree_attention(q_scratch[l], wl.cache, l, vs.kv_len, vs.max_kv_len, wl.mask, num_splits=args.splits, out=wl.attn_out[l],
                                k_new=k_scratch[l], v_new=wl.v_new[l])
 
-    ms_attn = timed_replays(torch, attn_all_layers, reps, 2, use_graph)[0] / wl.L
+    ms_attn_warm = timed_replays(torch, attn_all_layers, reps, 2, use_graph)[0] / wl.L
+    ms_attn = ms_attn_warm
+    if KV_SETS > 1:  # as the headline: every pass over K/V from HBM
+        def attn_cold():
+            for c in caches:
+                for l in range(wl.L):
+                    ops.tree_attention(wl.q[l], c, l, vs.kv_len, vs.max_kv_len, wl.mask, num_splits=args.splits, out=wl.attn_out[l],
+                                       k_new=wl.k_new[l], v_new=wl.v_new[l])
+        ms_attn = timed_replays(torch, attn_cold, reps, 2, use_graph)[0] / (wl.L * KV_SETS)
     ms_rope_fused = timed_replays(torch, attn_rope_fused, reps, 2, use_graph)[0] / wl.L
     ms_rope_sep = timed_replays(torch, attn_rope_separate, reps, 2, use_graph)[0] / wl.L
     del q_scratch, k_scratch
@@ -280,7 +320,8 @@ def main():
     kernels = [
         dict(kernel="tree_attn_split_kernel+tree_attn_combine_kernel", launches_per_step=wl.L, us_per_launch=round(ms_attn * 1e3, 2),
              bound="mfma", achieved=round(attn_tflops, 2), peak=MFMA_F16_PEAK_TFLOPS, unit="TFLOP/s",
-             frac=round(attn_tflops / MFMA_F16_PEAK_TFLOPS, 4), hbm_gbs=round(attn_gbs, 1), traffic=None),
+             frac=round(attn_tflops / MFMA_F16_PEAK_TFLOPS, 4), hbm_gbs=round(attn_gbs, 1), traffic=None,
+             us_per_launch_one_kv_set=round(ms_attn_warm * 1e3, 2)),
         dict(kernel="head_gemm_chunked_kernel<4,4,256,2>+head_argmax_finalize_kernel", launches_per_step=1, us_per_launch=round(ms_head * 1e3, 2),
              bound="hbm", achieved=round(head_gbs, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(head_gbs / HBM_PEAK_GBS, 4),
              traffic=None),
@@ -310,30 +351,12 @@ def main():
     frspec = dict(kernel="head_gemm_chunked_kernel<1,2,512,2>+topk_row_kernel", us_per_call=round(ms_fr * 1e3, 2), bound="hbm",
                   achieved=round(fr_gbs, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(fr_gbs / HBM_PEAK_GBS, 4))
 
-    # ---- cold-cache figures ----
-    # The 32 layers' K/V at 4K context (~150 MB) fit the 256 MB last-level cache and the FR-Spec matrix
-    # (268 MB) nearly does, so replays of ONE operator on the same buffers can be served from it.  (The
-    # full step is not affected: the 602 MB target head streams through the cache between two passes
-    # over the K/V.)  Here every replay walks several distinct copies, so each pass misses.
+    # ---- the FR-Spec head from a cold cache ----
+    # Its matrix (268 MB) nearly fits the last-level cache as well, so replays on one copy are partly served
+    # from it.  Here every replay walks several distinct copies, so each pass misses.
     cold = None
-    if wl.P <= 8192:
-        from cpm.cu_amd.kvcache import PagedKVCache
-        KV_SETS, FR_SETS = 4, 3
-        caches = [wl.cache]
-        for _ in range(KV_SETS - 1):
-            c2 = PagedKVCache(wl.L, wl.cache.Hkv, wl.cache.num_pages, device="cuda", block_table=wl.cache.block_table)
-            for l in range(wl.L):
-                c2.k[l].copy_(wl.cache.k[l])
-                c2.v[l].copy_(wl.cache.v[l])
-            caches.append(c2)
-
-        def attn_cold():
-            for c in caches:
-                for l in range(wl.L):
-                    ops.tree_attention(wl.q[l], c, l, vs.kv_len, vs.max_kv_len, wl.mask, num_splits=args.splits, out=wl.attn_out[l],
-                                       k_new=wl.k_new[l], v_new=wl.v_new[l])
-        ms_attn_cold = timed_replays(torch, attn_cold, reps, 2, use_graph)[0] / (wl.L * KV_SETS)
-        del caches
+    if KV_SETS > 1:
+        FR_SETS = 3
         w_subs = [w_sub] + [ops.tile_head_weight(wl.w, remap) for _ in range(FR_SETS - 1)]
 
         def fr_cold():
@@ -341,12 +364,11 @@ def main():
                 ops.frspec_head_topk(hid10, w, remap, 10)
         ms_fr_cold = timed_replays(torch, fr_cold, reps, 2, use_graph)[0] / FR_SETS
         del w_subs
-        cold = {"attention_us_per_layer": round(ms_attn_cold * 1e3, 2), "kv_sets_rotated": KV_SETS,
-                "frspec_head_us_per_call": round(ms_fr_cold * 1e3, 2), "frspec_weight_copies_rotated": FR_SETS,
+        cold = {"frspec_head_us_per_call": round(ms_fr_cold * 1e3, 2), "frspec_weight_copies_rotated": FR_SETS,
                 "frspec_frac_hbm": round(fr_bytes / (ms_fr_cold * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                "note": "each replay walks distinct copies of the K/V pools (4K context) / of the FR-Spec matrix, so no pass is "
-                        "served from the 256 MB last-level cache; the other figures replay one copy"}
-    del w_sub
+                "note": "the FR-Spec head with every replay walking distinct copies of its matrix, so that no pass is served "
+                        "from the 256 MB last-level cache; frspec_head above replays one copy"}
+    del w_sub, caches
     torch.cuda.empty_cache()
 
     # ---- CPU oracle on the host cores + parity of the step's integer results ----
@@ -360,6 +382,7 @@ def main():
         parity = dict(accept_length_gpu=a_gpu, accept_length_oracle=int(a_cpu),
                       ids_equal_oracle=bool(a_gpu == a_cpu and np.array_equal(ids_gpu, ids_cpu)),
                       staged_equal=bool(a_gpu == a_st and np.array_equal(ids_gpu, gt_gpu[path_st])),
+                      kv_sets_agree=bool(sets_agree),
                       argmax_rows_equal=int((gt_gpu == gt_cpu).sum()), rows=int(wl.T))
 
     # ---- the same step at longer contexts ----
@@ -406,8 +429,9 @@ def main():
         "data": "synthetic",
         "config": {"workload": args.workload + ": 32 layers x (KV append + tree attention, 32q/2kv heads, d128, 4096-token paged prefix + "
                                "60-node tree) + target head 73448x4096 with arg-max + tree acceptance + KV compaction",
-                   "batch": 1, "graph_replay": use_graph, "kv_splits": args.splits or "auto"},
+                   "batch": 1, "graph_replay": use_graph, "kv_splits": args.splits or "auto", "kv_sets_rotated": KV_SETS},
         "wall_ms_per_step": round(wall_ms, 5),
+        "us_per_step_one_kv_set": round(ms_step_warm * 1e3, 1),
         "roofline": roofline,
         "kernels": kernels,
         "frspec_head": frspec,
