@@ -355,6 +355,7 @@ def main():
     # Its matrix (268 MB) nearly fits the last-level cache as well, so replays on one copy are partly served
     # from it.  Here every replay walks several distinct copies, so each pass misses.
     cold = None
+    draft = None
     if KV_SETS > 1:
         FR_SETS = 3
         w_subs = [w_sub] + [ops.tile_head_weight(wl.w, remap) for _ in range(FR_SETS - 1)]
@@ -363,7 +364,41 @@ def main():
             for w in w_subs:
                 ops.frspec_head_topk(hid10, w, remap, 10)
         ms_fr_cold = timed_replays(torch, fr_cold, reps, 2, use_graph)[0] / FR_SETS
-        del w_subs
+
+        # ---- the draft side of the path: one whole draft of the FR-Spec drafter (6 rounds of 10) ----
+        # Per round: the drafter layer's own attention (10 queries, mask over 10*d columns, block sliding
+        # window of 1024 tokens, its own one-layer cache), the FR-Spec head with log-softmax + top-10 + id
+        # map-back, and the tree bookkeeping kernel; the final top-59 + tree build at the end.  The dense
+        # parts of the drafter layer (fc, projections, FFN) are not on the path and are not run; the head
+        # reads a different copy of its matrix every round, as it would after their weights.
+        from cpm.cu_amd.kvcache import PagedKVCache
+        k_it, n_it = 10, 6
+        dtree = ops.DraftTree(k_it, n_it, remap)
+        dcache = PagedKVCache(1, wl.cache.Hkv, wl.cache.num_pages, device="cuda", block_table=wl.cache.block_table)
+        dcache.k[0].copy_(wl.cache.k[0])
+        dcache.v[0].copy_(wl.cache.v[0])
+        hid1 = wl.hidden[:1].contiguous()
+        qd = wl.q[0][:k_it].contiguous()
+        kd = wl.k_new[0][:k_it].contiguous()
+        vd = wl.v_new[0][:k_it].contiguous()
+        d_len = [torch.tensor([wl.P + k_it * d], dtype=torch.int32, device="cuda") for d in range(n_it)]
+        d_out = torch.empty_like(qd)
+        tree_ids = torch.full((wl.T,), -1, dtype=torch.int32, device="cuda")
+
+        def draft_path():
+            r = ops.frspec_head_topk(hid1, w_subs[0], remap, k_it)
+            dtree.begin(r["val"][0], r["pos"][0])
+            for d in range(1, n_it):
+                ops.tree_attention(qd, dcache, 0, d_len[d], vs.max_kv_len, dtree.draft_mask, out=d_out, k_new=kd, v_new=vd,
+                                   mask_k_range=k_it * d, block_window_size=1024)
+                r = ops.frspec_head_topk(hid10, w_subs[d % FR_SETS], remap, k_it)
+                dtree.extend(d, r["val"], r["pos"])
+            dtree.finish(wl.T, vs.cache_length, tree_draft_ids=tree_ids)
+        ms_draft = timed_replays(torch, draft_path, reps, 2, use_graph)[0]
+        draft = {"us_per_draft": round(ms_draft * 1e3, 1), "rounds": n_it, "topk_per_round": k_it, "tree_size": wl.T,
+                 "operators": "6 x (FR-Spec head + log-softmax + top-10 + id map-back) + 5 x drafter-layer attention "
+                              "(window 1024) + tree bookkeeping (begin, 5 x extend, finish)"}
+        del w_subs, dcache, dtree
         cold = {"frspec_head_us_per_call": round(ms_fr_cold * 1e3, 2), "frspec_weight_copies_rotated": FR_SETS,
                 "frspec_frac_hbm": round(fr_bytes / (ms_fr_cold * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                 "note": "the FR-Spec head with every replay walking distinct copies of its matrix, so that no pass is served "
@@ -436,6 +471,7 @@ def main():
         "kernels": kernels,
         "frspec_head": frspec,
         "cold_cache": cold,
+        "draft_path": draft,
         "attention_with_rope": {"fused_us_per_layer": round(ms_rope_fused * 1e3, 2), "separate_launch_us_per_layer": round(ms_rope_sep * 1e3, 2),
                                 "note": "rotary embedding of q and the appended K rows; table computed once per step"},
         "commit_tail": {"kernel": "tree_accept_kernel+kv_compact_kernel(with hidden-row gather)+accepted_ids_kernel(ids, positions, packed result)",

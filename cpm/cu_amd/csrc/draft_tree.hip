@@ -9,7 +9,10 @@
 //             remap of the chosen nodes.
 // The reference spends about ten launches and a device-to-host copy per iteration on these; here
 // the prefix length is read from device memory, so building the tree needs no host round trip.
-// Selection uses the same 64-bit keys as the top-k kernels (value descending, lower index first).
+// Selection follows the ordering of the top-k kernels (value descending, lower index first).  The
+// histories are short (k*k = 100 and k + 5*k*k = 510 entries at the reference's settings), so it is
+// done by counting: every entry becomes a unique 32-bit key in LDS, every thread counts the keys above
+// its own, and that count is the entry's place in the sorted order -- no rounds, two barriers.
 #include "common.h"
 #include "topk_keys.h"
 
@@ -18,6 +21,26 @@ namespace {
 
 constexpr int kMaxK = 32;        // topk_per_iter
 constexpr int kMaxTried = kTopkThreads * kPerThread;  // history entries one workgroup can rank
+
+// (order-preserving 16-bit image of the fp16 value) << 16 | (0xFFFF - index): unique, never 0 for index < kMaxTried.
+__device__ inline uint32_t key32(uint16_t bits, int idx) { return (ord16(bits) << 16) | (uint32_t)(0xFFFF - idx); }
+static_assert(kMaxTried <= 0x10000, "the index must fit the low half of a 32-bit key");
+
+// Places of the `top` largest of s_keys[0, n): emit(place, index) is called by the thread that owns the
+// entry.  s_keys must be padded with zeros to a multiple of 4 and be visible (barrier) on entry.
+template <typename Emit>
+__device__ inline void rank_select(const uint32_t* s_keys, int n, int top, Emit emit) {
+    const int n4 = (n + 3) & ~3;
+    for (int x = threadIdx.x; x < n; x += kTopkThreads) {
+        const uint32_t mine = s_keys[x];
+        int above = 0;
+        for (int j = 0; j < n4; j += 4) {  // every lane reads the same 16 bytes: an LDS broadcast
+            const uint4 o = *reinterpret_cast<const uint4*>(s_keys + j);
+            above += (o.x > mine) + (o.y > mine) + (o.z > mine) + (o.w > mine);
+        }
+        if (above < top) emit(above, x);
+    }
+}
 
 struct DraftState {
     uint16_t* tried_val;    // [total] fp16 bits
@@ -65,18 +88,16 @@ __global__ void draft_begin_kernel(DraftState s, int k, const uint16_t* val, con
 __global__ __launch_bounds__(kTopkThreads) void draft_extend_kernel(DraftState s, int k, int d, uint16_t* val, const int32_t* pos,
                                                                     const int32_t* remap, int32_t* next_ids, int32_t* parent_rows,
                                                                     uint64_t* mask_out) {
+    __shared__ __attribute__((aligned(16))) uint32_t s_keys[kMaxK * kMaxK];
     __shared__ int32_t s_sel[kMaxK];
-    __shared__ uint16_t s_val[kMaxK];
+    __shared__ uint16_t s_val[kMaxK * kMaxK];
     __shared__ uint64_t s_oldmask[kMaxK];
     const int tid = threadIdx.x;
     const int kk = k * k;
     const int base = k + (d - 1) * kk;
     if (tid < k) s_oldmask[tid] = s.mask[tid];
-    uint64_t keys[kPerThread];
-#pragma unroll
-    for (int e = 0; e < kPerThread; ++e) {
-        const int x = tid * kPerThread + e;
-        uint64_t key = 0;
+    for (int x = tid; x < ((kk + 3) & ~3); x += kTopkThreads) {
+        uint32_t key = 0;
         if (x < kk) {
             const float c = (float)__builtin_bit_cast(f16, s.cum[x / k]);
             const f16 v = (f16)((float)__builtin_bit_cast(f16, val[x]) + c);  // half += half, rounded to half
@@ -84,15 +105,14 @@ __global__ __launch_bounds__(kTopkThreads) void draft_extend_kernel(DraftState s
             val[x] = bits;
             s.tried_val[base + x] = bits;
             s.tried_pos[base + x] = pos[x];
-            key = make_key(bits, x);
+            s_val[x] = bits;
+            key = key32(bits, x);
         }
-        keys[e] = key;
+        s_keys[x] = key;
     }
-    select_topk(keys, k, [&](int round, uint64_t key) {
-        s_sel[round] = key_index(key);
-        s_val[round] = key_bits(key);
-    });
-    // select_topk ends with a barrier: s_sel / s_val / s_oldmask are visible
+    __syncthreads();
+    rank_select(s_keys, kk, k, [&](int place, int x) { s_sel[place] = x; });
+    __syncthreads();
     if (tid < k) {
         const int p2 = s_sel[tid];
         s.tried_parent[(d - 1) * k + tid] = p2 + base;
@@ -102,27 +122,29 @@ __global__ __launch_bounds__(kTopkThreads) void draft_extend_kernel(DraftState s
         if (parent_rows) parent_rows[tid] = p2 / k;
         const int32_t fr = pos[p2];
         next_ids[tid] = remap ? remap[fr] : fr;
-        s.cum[tid] = s_val[tid];
+        s.cum[tid] = s_val[p2];
     }
 }
 
 __global__ __launch_bounds__(kTopkThreads) void draft_finish_kernel(DraftState s, int k, int num_iter, int T, const int32_t* cache_length,
                                                                     const int32_t* remap, int32_t* ids_out, int32_t* tree_pos,
                                                                     uint64_t* tree_mask, int32_t* tree_parent) {
-    __shared__ int32_t s_sel[kMaxTree];
-    __shared__ int32_t s_reverse[kMaxTried];
+    __shared__ __attribute__((aligned(16))) uint32_t s_keys[kMaxTried];
+    __shared__ int32_t s_sel[kMaxTree];      // history index of tree node i + 1
+    __shared__ int32_t s_reverse[kMaxTried]; // history index -> tree node (0: not selected, stands for the root)
+    __shared__ int32_t s_par[kMaxTree];
     const int tid = threadIdx.x;
     const int kk = k * k;
     const int total = k + (num_iter - 1) * kk;
     const int W = (T + 63) / 64;
-    uint64_t keys[kPerThread];
-#pragma unroll
-    for (int e = 0; e < kPerThread; ++e) {
-        const int x = tid * kPerThread + e;
-        keys[e] = x < total ? make_key(s.tried_val[x], x) : 0;
+    for (int x = tid; x < ((total + 3) & ~3); x += kTopkThreads) {
+        s_keys[x] = x < total ? key32(s.tried_val[x], x) : 0;
+        s_reverse[x < total ? x : total - 1] = 0;  // a parent that was not selected maps to the root
     }
-    for (int x = tid; x < total; x += kTopkThreads) s_reverse[x] = 0;  // a parent that was not selected maps to the root
-    select_topk(keys, T - 1, [&](int round, uint64_t key) { s_sel[round] = key_index(key); });
+    const int P = cache_length[0];
+    __syncthreads();
+    rank_select(s_keys, total, T - 1, [&](int place, int x) { s_sel[place] = x; });
+    __syncthreads();
     if (tid >= 1 && tid < T) {
         const int p = s_sel[tid - 1];
         s_reverse[p] = tid;
@@ -130,26 +152,38 @@ __global__ __launch_bounds__(kTopkThreads) void draft_finish_kernel(DraftState s
         ids_out[tid] = remap ? remap[fr] : fr;
     }
     __syncthreads();
-    if (tid == 0) {
-        const int P = cache_length[0];
-        for (int w = 0; w < W; ++w) tree_mask[w] = 0;
-        tree_mask[0] = 1;
-        tree_pos[0] = P;
-        tree_parent[0] = 0;
-        for (int i = 1; i < T; ++i) {  // parents come before children: cumulative log-probs fall along a path
-            int p = s_sel[i - 1];
-            tree_pos[i] = P + (p < k ? 1 : (p - k) / kk + 2);
-            if (p < k) {
-                p = -1;
-            } else {
+    // build_dynamic_tree (src/model/eagle.cuh:188-214), every node on its own thread: its parent is the
+    // tree node of its history parent; its mask row is its own bit plus those of its ancestors.
+    // Parents come before children (cumulative log-probs fall along a path, ties go to the older
+    // entry), which the sequential form of the reference relies on as well.
+    if (tid < T) {
+        int parent = 0;
+        if (tid == 0) {
+            tree_pos[0] = P;
+        } else {
+            int p = s_sel[tid - 1];
+            tree_pos[tid] = P + (p < k ? 1 : (p - k) / kk + 2);
+            if (p >= k) {
                 p -= k;
                 p = p < kk ? p / k : s.tried_parent[(p - kk) / k];
+                parent = s_reverse[p];
             }
-            const int parent = p == -1 ? 0 : s_reverse[p];
-            tree_parent[i] = parent;
-            for (int w = 0; w < W; ++w) tree_mask[(size_t)i * W + w] = tree_mask[(size_t)parent * W + w];
-            tree_mask[(size_t)i * W + (i >> 6)] |= 1ull << (i & 63);
         }
+        s_par[tid] = parent;
+        tree_parent[tid] = parent;
+    }
+    __syncthreads();
+    if (tid < T) {
+        uint64_t m0 = 1, m1 = 0;  // the root is everybody's ancestor
+        int node = tid;
+        for (int hop = 0; hop < T && node != 0; ++hop) {
+            if (node < 64) m0 |= 1ull << node;
+            else m1 |= 1ull << (node - 64);
+            const int up = s_par[node];
+            node = up < node ? up : 0;  // never walks downwards, so it ends
+        }
+        tree_mask[(size_t)tid * W] = m0;
+        if (W > 1) tree_mask[(size_t)tid * W + 1] = m1;
     }
 }
 
