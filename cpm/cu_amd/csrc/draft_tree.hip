@@ -31,9 +31,10 @@ static_assert(kMaxTried <= 0x10000, "the index must fit the low half of a 32-bit
 template <typename Emit>
 __device__ inline void rank_select(const uint32_t* s_keys, int n, int top, Emit emit) {
     const int n4 = (n + 3) & ~3;
-    for (int x = threadIdx.x; x < n; x += kTopkThreads) {
+    for (int x = threadIdx.x; x < n; x += blockDim.x) {
         const uint32_t mine = s_keys[x];
         int above = 0;
+#pragma unroll 8
         for (int j = 0; j < n4; j += 4) {  // every lane reads the same 16 bytes: an LDS broadcast
             const uint4 o = *reinterpret_cast<const uint4*>(s_keys + j);
             above += (o.x > mine) + (o.y > mine) + (o.z > mine) + (o.w > mine);
@@ -126,21 +127,33 @@ __global__ __launch_bounds__(kTopkThreads) void draft_extend_kernel(DraftState s
     }
 }
 
-__global__ __launch_bounds__(kTopkThreads) void draft_finish_kernel(DraftState s, int k, int num_iter, int T, const int32_t* cache_length,
-                                                                    const int32_t* remap, int32_t* ids_out, int32_t* tree_pos,
-                                                                    uint64_t* tree_mask, int32_t* tree_parent) {
+// One thread per history entry up to 1024 entries (two beyond): the counting loop is a chain of LDS
+// reads, and sixteen waves hide its latency where four would wait for it.
+constexpr int kFinishThreads = 1024;
+
+__global__ __launch_bounds__(kFinishThreads) void draft_finish_kernel(DraftState s, int k, int num_iter, int T, const int32_t* cache_length,
+                                                                      const int32_t* remap, int32_t* ids_out, int32_t* tree_pos,
+                                                                      uint64_t* tree_mask, int32_t* tree_parent) {
     __shared__ __attribute__((aligned(16))) uint32_t s_keys[kMaxTried];
-    __shared__ int32_t s_sel[kMaxTree];      // history index of tree node i + 1
+    __shared__ int32_t s_pos[kMaxTried];     // FR-Spec index of every history entry
     __shared__ int32_t s_reverse[kMaxTried]; // history index -> tree node (0: not selected, stands for the root)
+    __shared__ int32_t s_hpar[64];           // history parent of the entries chosen in rounds >= 1 (k * num_iter <= 64 of them)
+    __shared__ int32_t s_sel[kMaxTree];      // history index of tree node i + 1
     __shared__ int32_t s_par[kMaxTree];
     const int tid = threadIdx.x;
     const int kk = k * k;
     const int total = k + (num_iter - 1) * kk;
     const int W = (T + 63) / 64;
-    for (int x = tid; x < ((total + 3) & ~3); x += kTopkThreads) {
-        s_keys[x] = x < total ? key32(s.tried_val[x], x) : 0;
-        s_reverse[x < total ? x : total - 1] = 0;  // a parent that was not selected maps to the root
+    // everything the later phases need comes into LDS in one round trip to memory
+    for (int x = tid; x < ((total + 3) & ~3); x += kFinishThreads) {
+        const bool in = x < total;
+        s_keys[x] = in ? key32(s.tried_val[x], x) : 0;
+        if (in) {
+            s_pos[x] = s.tried_pos[x];
+            s_reverse[x] = 0;  // a parent that was not selected maps to the root
+        }
     }
+    if (tid < k * (num_iter - 1)) s_hpar[tid] = s.tried_parent[tid];
     const int P = cache_length[0];
     __syncthreads();
     rank_select(s_keys, total, T - 1, [&](int place, int x) { s_sel[place] = x; });
@@ -148,7 +161,7 @@ __global__ __launch_bounds__(kTopkThreads) void draft_finish_kernel(DraftState s
     if (tid >= 1 && tid < T) {
         const int p = s_sel[tid - 1];
         s_reverse[p] = tid;
-        const int32_t fr = s.tried_pos[p];
+        const int32_t fr = s_pos[p];
         ids_out[tid] = remap ? remap[fr] : fr;
     }
     __syncthreads();
@@ -165,7 +178,7 @@ __global__ __launch_bounds__(kTopkThreads) void draft_finish_kernel(DraftState s
             tree_pos[tid] = P + (p < k ? 1 : (p - k) / kk + 2);
             if (p >= k) {
                 p -= k;
-                p = p < kk ? p / k : s.tried_parent[(p - kk) / k];
+                p = p < kk ? p / k : s_hpar[(p - kk) / k];
                 parent = s_reverse[p];
             }
         }
@@ -237,7 +250,7 @@ extern "C" int cpmcu_draft_tree_finish(void* state, int k, int num_iter, int tre
     const int total = k + (num_iter - 1) * k * k;
     CPMCU_CHECK_ARG(tree_size >= 2 && tree_size <= kMaxTree && tree_size - 1 <= total,
                     "draft_tree_finish: tree_size=%d outside [2, min(%d, history %d + 1)]", tree_size, kMaxTree, total);
-    hipLaunchKernelGGL(draft_finish_kernel, dim3(1), dim3(kTopkThreads), 0, resolve_stream(stream), draft_state(state, k, num_iter), k,
+    hipLaunchKernelGGL(draft_finish_kernel, dim3(1), dim3(kFinishThreads), 0, resolve_stream(stream), draft_state(state, k, num_iter), k,
                        num_iter, tree_size, cache_length, token_id_remap, tree_draft_ids, tree_position_ids, tree_attn_mask, tree_parent);
     CPMCU_LAUNCH_CHECK();
     return CPMCU_OK;
