@@ -221,11 +221,12 @@ def test_draft_layer_mask_range(gpu, orc, k, d, P0, seed):
     (10, 1, 100, 128, 0, 1), (10, 3, 127, 128, 0, 2), (10, 3, 128, 128, 1, 3), (10, 3, 129, 128, 0, 4),
     (10, 6, 1000, 128, 0, 5), (10, 6, 1000, 512, 3, 6), (10, 5, 1024, 1024, 0, 7), (10, 5, 1025, 1024, 0, 8),
     (10, 6, 5000, 1024, 0, 9), (10, 6, 5000, 1024, 5, 10), (4, 5, 61, 256, 0, 11), (8, 8, 2049, 2048, 0, 12),
-    (10, 2, 9000, 8192, 0, 13), (10, 6, 300, 4096, 0, 14)])
+    (10, 2, 9000, 8192, 0, 13), (10, 6, 300, 4096, 0, 14), (10, 3, 115, 128, 0, 15), (10, 6, 140, 128, 2, 16)])
 def test_draft_layer_block_window(gpu, orc, k, d, P0, window, splits, seed):
     """The drafter's own layer with its block sliding window (eagle_window_size): only the key blocks of 128 from
     ceil(P/128) - window/128 on are visited.  Queries are the newest k draft tokens, the mask covers k*d
-    columns, the new rows are appended by the kernel; the page table is a seeded permutation."""
+    columns, the new rows are appended by the kernel; the page table is a seeded permutation.  The last two
+    cases put the first mask column below the window's first key: the window wins."""
     from cpm.cu_amd import ops
     from cpm.cu_amd.kvcache import PagedKVCache
     torch = gpu
