@@ -36,8 +36,8 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 # profiles/verify_step_hbm_traffic.md.  Counters cannot be read from inside this process, so the figures
 # are carried here as constants and are reported only for the workload they were measured on.
 MEASURED_TRAFFIC_KIB = {
-    "tree_attn_split_kernel+tree_attn_combine_kernel": 6360 + 8494 + 8710 + 480,
-    "head_gemm_chunked_kernel<4,4,256,2>+head_argmax_finalize_kernel": 592005 + 128 + 1049 + 2,
+    "tree_attn_split_kernel+tree_attn_combine_kernel": 6367 + 8494 + 8710 + 480,
+    "head_gemm_chunked_kernel<4,4,256,2>+head_argmax_finalize_kernel": 592012 + 128 + 1052 + 2,
     "tree_accept_kernel+kv_compact_kernel+accepted_ids_kernel": 6 + 1137 + 335 + 4,
 }
 
