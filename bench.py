@@ -317,6 +317,8 @@ def main():
     attn_tflops = wl.flops_attention_layer() / (ms_attn * 1e-3) / 1e12
     attn_gbs = wl.bytes_attention_layer() / (ms_attn * 1e-3) / 1e9
     head_gbs = wl.bytes_target_head() / (ms_head * 1e-3) / 1e9
+    tail_bytes = 2 * a_gpu * 2 * wl.L * wl.shape["kv_heads"] * wl.shape["head_dim"] * 2  # compaction: a rows, read + written
+    tail_gbs = tail_bytes / (ms_tail * 1e-3) / 1e9
     kernels = [
         dict(kernel="tree_attn_split_kernel+tree_attn_combine_kernel", launches_per_step=wl.L, us_per_launch=round(ms_attn * 1e3, 2),
              bound="mfma", achieved=round(attn_tflops, 2), peak=MFMA_F16_PEAK_TFLOPS, unit="TFLOP/s",
@@ -326,7 +328,10 @@ def main():
              bound="hbm", achieved=round(head_gbs, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(head_gbs / HBM_PEAK_GBS, 4),
              traffic=None),
         dict(kernel="tree_accept_kernel+kv_compact_kernel+accepted_ids_kernel", launches_per_step=1,
-             us_per_launch=round(ms_tail * 1e3, 2), bound="hbm", achieved=None, peak=HBM_PEAK_GBS, unit="GB/s", frac=None, traffic=None),
+             us_per_launch=round(ms_tail * 1e3, 2), bound="hbm", achieved=round(tail_gbs, 2), peak=HBM_PEAK_GBS, unit="GB/s",
+             frac=round(tail_gbs / HBM_PEAK_GBS, 5), traffic=None,
+             note="accepted rows read and written once in every layer's K and V: %d bytes at accept length %d; three launches of latency, "
+                  "not bandwidth" % (tail_bytes, a_gpu)),
     ]
     if args.workload == "c2_verify_4k" and args.splits == 0:
         for k in kernels:
