@@ -206,6 +206,12 @@ def main():
         del src, dst
 
     wl = Workload(torch, args.workload, args.accept_depth)
+    ctx_name = "%dK" % (wl.P // 1024) if wl.P % 1024 == 0 else str(wl.P)
+    metric_name = "verify us/step @8B shape, %d-node tree, %s ctx" % (wl.T, ctx_name)
+    wl_desc = ("%s: %d layers x (KV append + tree attention, %dq/%dkv heads, d%d, %d-token paged prefix + %d-node tree) + "
+               "target head %dx%d with arg-max + tree acceptance + KV compaction"
+               % (args.workload, wl.L, wl.shape["q_heads"], wl.shape["kv_heads"], wl.shape["head_dim"], wl.P, wl.T,
+                  wl.shape["vocab"], wl.shape["hidden"]))
     # the head weights are kept in the library's tiled layout, as its model-level loader keeps them
     w_t = ops.tile_head_weight(wl.w)
     vs = VerifyStep(wl.cache, w_t, wl.mask, wl.parent, wl.pos, wl.P)
@@ -455,7 +461,7 @@ def main():
             torch.cuda.empty_cache()
 
     out = {
-        "metric": "verify us/step @8B shape, 60-node tree, 4K ctx",
+        "metric": metric_name,
         "value": round(ms_step * 1e3, 1),
         "unit": "us/step",
         "n_gpus": 1,
@@ -467,9 +473,7 @@ def main():
         "vs_baseline": None,
         "dtype": "f16",
         "data": "synthetic",
-        "config": {"workload": args.workload + ": 32 layers x (KV append + tree attention, 32q/2kv heads, d128, 4096-token paged prefix + "
-                               "60-node tree) + target head 73448x4096 with arg-max + tree acceptance + KV compaction",
-                   "batch": 1, "graph_replay": use_graph, "kv_splits": args.splits or "auto", "kv_sets_rotated": KV_SETS},
+        "config": {"workload": wl_desc, "batch": 1, "graph_replay": use_graph, "kv_splits": args.splits or "auto", "kv_sets_rotated": KV_SETS},
         "wall_ms_per_step": round(wall_ms, 5),
         "us_per_step_one_kv_set": round(ms_step_warm * 1e3, 1),
         "roofline": roofline,
