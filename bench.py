@@ -52,6 +52,7 @@ def parse_args():
     ap.add_argument("--no-contexts", action="store_true", help="skip the 32K / 128K context step timings")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    ap.add_argument("--no-probes", action="store_true", help="skip the MFMA-rate probe of the machine")
     ap.add_argument("--accept-depth", type=int, default=3, help="draft tokens the rigged tree gets accepted")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also run a plain 256 MiB device copy three times: the known-size kernel that scales "
@@ -150,6 +151,32 @@ def timed_replays(torch, fn, steps, warmup, use_graph):
     return ev_ms / steps, wall_ms / steps
 
 
+def machine_probes(torch):
+    """What this GPU gives a kernel that does nothing but MFMAs from registers: with all-zero operands and
+    with random ones -- the sustained rate depends on the bits (clocks follow the power drawn).
+    Event-timed, eager."""
+    from cpm.cu_amd import lib, ops
+    out = {}
+    n = lib.get().raw.cpmcu_mfma_rate_probe_operand_bytes() // 2
+    g = torch.Generator(device="cuda")
+    g.manual_seed(7)
+    for name, data in (("zero_operands", torch.zeros(n, dtype=torch.float16, device="cuda")),
+                       ("random_operands", torch.randn(n, device="cuda", generator=g).to(torch.float16))):
+        ops.mfma_rate_probe(data, 200)
+        torch.cuda.synchronize()
+        best = 0.0
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            flops = ops.mfma_rate_probe(data, 40000)
+            e1.record()
+            torch.cuda.synchronize()
+            best = max(best, flops / (e0.elapsed_time(e1) * 1e-3) / 1e12)
+        out["mfma_tflops_" + name] = round(best, 1)
+    out["note"] = "v_mfma_f32_32x32x16_f16 from registers, 256 workgroups x 8 waves, nothing else in the loop"
+    return out
+
+
 def cpu_baseline(torch, wl, layers_sampled=2):
     """CPU oracle on a bounded sample: `layers_sampled` attention layers + the full target head +
     acceptance + compaction of those layers; the per-step figure scales the attention part to 32 layers."""
@@ -214,6 +241,7 @@ def main():
                   wl.shape["vocab"], wl.shape["hidden"]))
     # the head weights are kept in the library's tiled layout, as its model-level loader keeps them
     w_t = ops.tile_head_weight(wl.w)
+    probes = None if args.no_probes else machine_probes(torch)
     vs = VerifyStep(wl.cache, w_t, wl.mask, wl.parent, wl.pos, wl.P)
     # target arg-max once, to rig the draft ids for the chosen accept length
     gt = ops.lm_head_argmax(wl.hidden, w_t)
@@ -347,6 +375,10 @@ def main():
     roofline = {k: dominant[k] for k in ("bound", "achieved", "peak", "unit", "frac", "traffic")}
     roofline["kernel"] = dominant["kernel"]
     roofline["us_per_launch"] = dominant["us_per_launch"]
+    if probes is not None and dominant["bound"] == "mfma":
+        # the same achieved figure against what this GPU sustains for MFMAs alone on random operands
+        roofline["measured_ceiling"] = probes["mfma_tflops_random_operands"]
+        roofline["frac_of_measured_ceiling"] = round(dominant["achieved"] / probes["mfma_tflops_random_operands"], 4)
 
     # ---- FR-Spec draft head (config 3 shape), reported beside the verify step ----
     from cpm.cu_amd import synth
@@ -454,9 +486,11 @@ def main():
                                        k_new=w2.k_new[l], v_new=w2.v_new[l])
             ms_a2 = timed_replays(torch, attn2, n, 2, use_graph)[0] / w2.L
             contexts[str(w2.P)] = round(ms2 * 1e3, 1)
-            ctx_attn[str(w2.P)] = dict(us_per_layer=round(ms_a2 * 1e3, 2),
-                                       tflops=round(w2.flops_attention_layer() / (ms_a2 * 1e-3) / 1e12, 1),
-                                       frac_mfma=round(w2.flops_attention_layer() / (ms_a2 * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4))
+            tf2 = w2.flops_attention_layer() / (ms_a2 * 1e-3) / 1e12
+            ctx_attn[str(w2.P)] = dict(us_per_layer=round(ms_a2 * 1e3, 2), tflops=round(tf2, 1),
+                                       frac_mfma=round(tf2 / MFMA_F16_PEAK_TFLOPS, 4))
+            if probes is not None:  # against what MFMAs alone sustain on random operands on this GPU
+                ctx_attn[str(w2.P)]["frac_of_measured_ceiling"] = round(tf2 / probes["mfma_tflops_random_operands"], 4)
             del v2, w2
             torch.cuda.empty_cache()
 
@@ -477,6 +511,7 @@ def main():
         "wall_ms_per_step": round(wall_ms, 5),
         "us_per_step_one_kv_set": round(ms_step_warm * 1e3, 1),
         "roofline": roofline,
+        "machine_probes": probes,
         "kernels": kernels,
         "frspec_head": frspec,
         "cold_cache": cold,

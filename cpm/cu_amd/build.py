@@ -20,7 +20,7 @@ LIB_PATH = os.path.join(HERE, "libcpmcu_amd.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 ARCH = "gfx950"
 
-HIP_SOURCES = ["runtime.hip", "tree_attention.hip", "lm_head.hip", "topk.hip", "tree_accept.hip", "draft_tree.hip"]
+HIP_SOURCES = ["runtime.hip", "tree_attention.hip", "lm_head.hip", "topk.hip", "tree_accept.hip", "draft_tree.hip", "probe.hip"]
 HEADERS = sorted(f for f in os.listdir(CSRC) if f.endswith(".h"))
 
 # packed fp32 VALU ops stay off for every device translation unit

@@ -64,6 +64,8 @@ SIGNATURES = {
     "cpmcu_draft_tree_begin": (c_int, [_P, c_int, c_int, _P, _P, _P, _P, _P, _P]),
     "cpmcu_draft_tree_extend": (c_int, [_P, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P]),
     "cpmcu_draft_tree_finish": (c_int, [_P, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P]),
+    "cpmcu_mfma_rate_probe_operand_bytes": (c_size_t, []),
+    "cpmcu_mfma_rate_probe": (c_int, [_P, c_int, c_int, _P, _P, _P]),
 }
 
 

@@ -384,6 +384,20 @@ int cpmcu_draft_tree_finish(void* state, int k, int num_iter, int tree_size, con
                             const int32_t* token_id_remap, int32_t* tree_draft_ids, int32_t* tree_position_ids,
                             uint64_t* tree_attn_mask, int32_t* tree_parent, void* stream);
 
+/* ------------------------------------------------------------------------- */
+/* 3. Measurement helper (no counterpart in the reference)                    */
+/* ------------------------------------------------------------------------- */
+
+/* What the matrix pipes deliver to a kernel that does nothing else: `workgroups` workgroups of 8 waves,
+ * every lane holding 8 A and 8 B operands of v_mfma_f32_32x32x16_f16 in registers and issuing
+ * iters x 16 MFMAs on four accumulator chains.  operands: device fp16 data of
+ * cpmcu_mfma_rate_probe_operand_bytes() bytes -- the sustained rate depends on it (all-zero operands
+ * run at the published peak, random ones well below: clocks follow the power drawn), which is why
+ * the data is the caller's.  out: device float[workgroups * 512].  *flops (host, may be NULL)
+ * receives the floating-point operations one launch performs; time the launch with events. */
+size_t cpmcu_mfma_rate_probe_operand_bytes(void);
+int cpmcu_mfma_rate_probe(const void* operands, int iters, int workgroups, float* out, double* flops, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
