@@ -241,7 +241,6 @@ def main():
                   wl.shape["vocab"], wl.shape["hidden"]))
     # the head weights are kept in the library's tiled layout, as its model-level loader keeps them
     w_t = ops.tile_head_weight(wl.w)
-    probes = None if args.no_probes else machine_probes(torch)
     vs = VerifyStep(wl.cache, w_t, wl.mask, wl.parent, wl.pos, wl.P)
     # target arg-max once, to rig the draft ids for the chosen accept length
     gt = ops.lm_head_argmax(wl.hidden, w_t)
@@ -375,10 +374,6 @@ def main():
     roofline = {k: dominant[k] for k in ("bound", "achieved", "peak", "unit", "frac", "traffic")}
     roofline["kernel"] = dominant["kernel"]
     roofline["us_per_launch"] = dominant["us_per_launch"]
-    if probes is not None and dominant["bound"] == "mfma":
-        # the same achieved figure against what this GPU sustains for MFMAs alone on random operands
-        roofline["measured_ceiling"] = probes["mfma_tflops_random_operands"]
-        roofline["frac_of_measured_ceiling"] = round(dominant["achieved"] / probes["mfma_tflops_random_operands"], 4)
 
     # ---- FR-Spec draft head (config 3 shape), reported beside the verify step ----
     from cpm.cu_amd import synth
@@ -489,10 +484,19 @@ def main():
             tf2 = w2.flops_attention_layer() / (ms_a2 * 1e-3) / 1e12
             ctx_attn[str(w2.P)] = dict(us_per_layer=round(ms_a2 * 1e3, 2), tflops=round(tf2, 1),
                                        frac_mfma=round(tf2 / MFMA_F16_PEAK_TFLOPS, 4))
-            if probes is not None:  # against what MFMAs alone sustain on random operands on this GPU
-                ctx_attn[str(w2.P)]["frac_of_measured_ceiling"] = round(tf2 / probes["mfma_tflops_random_operands"], 4)
             del v2, w2
             torch.cuda.empty_cache()
+
+    # ---- what the matrix pipes sustain on this GPU (last, so that its heat does not touch the figures above) ----
+    probes = None if args.no_probes else machine_probes(torch)
+    if probes is not None:
+        ceiling = probes["mfma_tflops_random_operands"]
+        if roofline["bound"] == "mfma":  # the same achieved figure against MFMAs alone on random operands
+            roofline["measured_ceiling"] = ceiling
+            roofline["frac_of_measured_ceiling"] = round(roofline["achieved"] / ceiling, 4)
+        for v in ctx_attn.values():
+            if isinstance(v, dict):
+                v["frac_of_measured_ceiling"] = round(v["tflops"] / ceiling, 4)
 
     out = {
         "metric": metric_name,
