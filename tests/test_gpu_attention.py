@@ -296,6 +296,50 @@ def test_block_window_argument_checks(gpu):
             ops.tree_attention(q, cache, 0, kv_len, 100, None, block_window_size=bad)
 
 
+@pytest.mark.parametrize("T,num_iter,topk", [(60, 6, 10), (128, 8, 16)])
+def test_32k_context_one_layer_against_oracle(gpu, orc, T, num_iter, topk):
+    """Configs 4 and 5 at their real size for one layer: 32768-token prefix, 60- and 128-node trees."""
+    tree = synth.eagle_tree(num_iter, topk, T, seed=1)
+    out, ref = _case(gpu, orc, tree, 32768, seed=40 + T)
+    assert_close_f16(out, ref, "attention at 32K context, T=%d" % T)
+
+
+def test_128k_context_closed_form_and_split_invariance(gpu):
+    """Config 4 at 128K context, checked through properties that need no CPU pass over the keys:
+    (1) with identical K rows every visible key weighs the same, so row i is the mean of its visible
+    V rows -- prefix and ancestors -- which numpy computes in fp64 from running sums;
+    (2) on random K the result must not depend on the split count beyond fp16 rounding."""
+    from cpm.cu_amd import ops
+    from cpm.cu_amd.kvcache import PagedKVCache
+    torch = gpu
+    P, T = 131072, 60
+    S = P + T
+    tree = synth.eagle_tree(6, 10, T, seed=2)
+    npages = (S + 255) // 256 + 1
+    table = synth.rng(5, 4).permutation(npages).astype(np.int32)
+    q = synth.normal_f16((T, HQ, D), 70, 1)
+    v = synth.normal_f16((S, HKV, D), 70, 3)
+    k_same = np.broadcast_to(synth.normal_f16((1, HKV, D), 70, 2), (S, HKV, D)).copy()
+    cache = PagedKVCache(1, HKV, npages, block_table=table, fill=float("nan"))
+    cache.write_logical(0, 0, to_dev(torch, k_same), to_dev(torch, v))
+    kv_len = torch.tensor([S], dtype=torch.int32, device="cuda")
+    mask = to_dev(torch, tree.mask)
+    out = to_np(ops.tree_attention(to_dev(torch, q), cache, 0, kv_len, S, mask)).astype(np.float64)
+    v64 = v.astype(np.float64)
+    prefix_sum = v64[:P].sum(0)                                   # [Hkv, D]
+    for i in range(T):
+        anc = [j for j in range(T) if (int(tree.mask[i, j >> 6]) >> (j & 63)) & 1]
+        mean = (prefix_sum + v64[P + np.array(anc)].sum(0)) / (P + len(anc))
+        for h in range(HQ):
+            assert np.abs(out[i, h] - mean[h // (HQ // HKV)]).max() < 2e-3, (i, h)
+    # random keys: 32 (automatic), 16 and 64 splits agree
+    k = synth.normal_f16((S, HKV, D), 71, 2)
+    cache.write_logical(0, 0, to_dev(torch, k), to_dev(torch, v))
+    outs = [to_np(ops.tree_attention(to_dev(torch, q), cache, 0, kv_len, S, mask, num_splits=s)) for s in (0, 16, 64)]
+    for o in outs[1:]:
+        assert_close_f16(o, outs[0], "split invariance at 128K", atol=4e-3, rtol=4e-3)
+
+
 def _sweep_configs():
     """Seeded random (P, T, mode, splits, slack) tuples, biased to tile (64), page (256) and wave-row (2, 16 nodes)
     boundaries; slack = how far the host-side bound on the KV length exceeds the true length."""
