@@ -206,6 +206,7 @@ def cpu_baseline(torch, wl, layers_sampled=2):
     t_tail = time.perf_counter() - t0
     step_us = (t_attn * wl.L + t_head + t_tail) * 1e6
     return dict(value=round(step_us, 1), unit="us/step", cores=oracle.num_threads(), kind="port",
+                head_and_tail_us=round((t_head + t_tail) * 1e6, 1),
                 sample="%d of %d attention layers timed (x%d extrapolated) + full target head/arg-max + acceptance + compaction; "
                        "attention %.1f ms/layer, head %.1f ms" % (layers_sampled, wl.L, wl.L, t_attn * 1e3, t_head * 1e3)), (a, ids, gt)
 
@@ -484,6 +485,21 @@ def main():
             tf2 = w2.flops_attention_layer() / (ms_a2 * 1e-3) / 1e12
             ctx_attn[str(w2.P)] = dict(us_per_layer=round(ms_a2 * 1e3, 2), tflops=round(tf2, 1),
                                        frac_mfma=round(tf2 / MFMA_F16_PEAK_TFLOPS, 4))
+            if cpu is not None:
+                # the CPU oracle on ONE layer of this context (bounded sample), extrapolated to the step with the
+                # head and tail times of the 4K sample
+                import oracle
+                S2 = w2.P + w2.T
+                k2, v2k = w2.cache.read_logical(0, 0, S2)
+                k2, v2k, q2 = k2.cpu().numpy(), v2k.cpu().numpy(), w2.q[0].cpu().numpy()
+                t0 = time.perf_counter()
+                oracle.tree_attention(q2, k2, v2k, w2.tree.mask, w2.P)
+                t_layer = time.perf_counter() - t0
+                cpu.setdefault("contexts", {})[str(w2.P)] = dict(
+                    attention_ms_per_layer=round(t_layer * 1e3, 1),
+                    us_per_step_extrapolated=round(t_layer * 1e6 * w2.L + cpu["head_and_tail_us"], 1),
+                    sample="1 of %d attention layers timed once" % w2.L)
+                del k2, v2k, q2
             del v2, w2
             torch.cuda.empty_cache()
 
