@@ -727,8 +727,11 @@ int choose_splits(int T, int group, int Hkv, int max_kv_len, int G) {
 
 // KV groups per workgroup.  The 256-row shape pays off once every workgroup of a full-GPU launch has
 // a long enough run of tiles to amortise its larger split count (twice the partials to merge).
+// Measured with a 60-node tree: the two shapes meet at 32K context (50 us per layer either way); below,
+// the two-group shape is ahead (31.1 vs 32.8 us at 16K, 23.0 vs 26.8 at 8K), above, the 256-row shape
+// (67.7 vs 71.2 us at 48K, 156 vs 170 at 128K).
 // CPMCU_ATTN_KV_GROUPS=1|2 in the environment overrides the choice (tests exercise both shapes).
-constexpr int kLongContextTiles = 256;
+constexpr int kLongContextTiles = 512;
 int choose_groups(int max_kv_len) {
     if (const char* e = getenv("CPMCU_ATTN_KV_GROUPS")) {
         if (e[0] == '1' && e[1] == 0) return 1;
