@@ -726,18 +726,22 @@ int choose_splits(int T, int group, int Hkv, int max_kv_len, int G) {
 }
 
 // KV groups per workgroup.  The 256-row shape pays off once every workgroup of a full-GPU launch has
-// a long enough run of tiles to amortise its larger split count (twice the partials to merge).
-// Measured with a 60-node tree: the two shapes meet at 32K context (50 us per layer either way); below,
-// the two-group shape is ahead (31.1 vs 32.8 us at 16K, 23.0 vs 26.8 at 8K), above, the 256-row shape
-// (67.7 vs 71.2 us at 48K, 156 vs 170 at 128K).
+// a long enough run of tiles to amortise its larger split count (twice the partials to merge), and
+// only if its (KV head, M-tile) units times the split limit can fill the GPU at all: it is taken
+// when there are at least 4 such units and at least 16 tiles per workgroup.  Measured, us per layer,
+// 256-row shape vs two-group shape:  60-node tree (8 units): 32.8 / 31.1 at 16K, 50 / 50 at 32K,
+// 67.7 / 71.2 at 48K, 156 / 170 at 128K;  128-node tree (16 units): 30.3 / 29.5 at 4K, 56.1 / 59.3 at
+// 16K, 301 / 326 at 128K;  16 nodes or one (2 units): 74.8 / 62.4 and 73.2 / 55.0 at 128K.
 // CPMCU_ATTN_KV_GROUPS=1|2 in the environment overrides the choice (tests exercise both shapes).
-constexpr int kLongContextTiles = 512;
-int choose_groups(int max_kv_len) {
+constexpr int kLongRunTiles = 16;
+int choose_groups(int T, int group, int Hkv, int max_kv_len) {
     if (const char* e = getenv("CPMCU_ATTN_KV_GROUPS")) {
         if (e[0] == '1' && e[1] == 0) return 1;
         if (e[0] == '2' && e[1] == 0) return 2;
     }
-    return ceil_div(max_kv_len, kTileN) >= kLongContextTiles ? 1 : 2;
+    const int units = ceil_div(group * T, rows_per_wg(1)) * Hkv;
+    const int ntiles = ceil_div(max_kv_len, kTileN);
+    return units >= 4 && (long long)ntiles * units >= (long long)kLongRunTiles * 256 ? 1 : 2;
 }
 
 }  // namespace
@@ -798,7 +802,7 @@ static int tree_attention_impl(const void* q, void* k_pool, void* v_pool,
     p.window_blocks = block_window_size / 128;
     int span = max_kv_len;
     if (p.window_blocks > 0 && p.window_blocks * 128 + T < span) span = p.window_blocks * 128 + T;
-    const int G = choose_groups(span);
+    const int G = choose_groups(T, group, Hkv, span);
     p.num_mtiles = ceil_div(group * T, rows_per_wg(G));
     p.rows_pad = p.num_mtiles * rows_per_wg(G);
     p.num_splits = num_splits_override > 0 ? num_splits_override : choose_splits(T, group, Hkv, span, G);
