@@ -155,20 +155,20 @@ def machine_probes(torch):
     """What this GPU gives a kernel that does nothing but MFMAs from registers: with all-zero operands and
     with random ones -- the sustained rate depends on the bits (clocks follow the power drawn).
     Event-timed, eager."""
-    from cpm.cu_amd import lib, ops
+    import bench_probes
     out = {}
-    n = lib.get().raw.cpmcu_mfma_rate_probe_operand_bytes() // 2
+    n = bench_probes.load().bench_mfma_rate_probe_operand_bytes() // 2
     g = torch.Generator(device="cuda")
     g.manual_seed(7)
     for name, data in (("zero_operands", torch.zeros(n, dtype=torch.float16, device="cuda")),
                        ("random_operands", torch.randn(n, device="cuda", generator=g).to(torch.float16))):
-        ops.mfma_rate_probe(data, 200)
+        bench_probes.mfma_rate_probe(data, 200)
         torch.cuda.synchronize()
         best = 0.0
         for _ in range(3):
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
-            flops = ops.mfma_rate_probe(data, 40000)
+            flops, _ = bench_probes.mfma_rate_probe(data, 40000)
             e1.record()
             torch.cuda.synchronize()
             best = max(best, flops / (e0.elapsed_time(e1) * 1e-3) / 1e12)

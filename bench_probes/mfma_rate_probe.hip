@@ -2,11 +2,17 @@
 // else.  The roofline fraction of the attention kernel is quoted against the published peak
 // (2.5 PFLOP/s dense fp16 MFMA); this probe says how much of it a register-resident MFMA loop reaches on
 // the same GPU as a function of the operand DATA, because the rate the chip sustains depends on how
-// many bits toggle (clocks follow the power drawn).  No counterpart in the reference.
-#include "common.h"
+// many bits toggle (clocks follow the power drawn).  No counterpart in the reference, and not part of
+// libcpmcu_amd: bench.py loads this file's own small shared library (bench_probes/libbench_probes.so).
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
 
-namespace cpmcu {
 namespace {
+
+typedef _Float16 f16;
+typedef f16 f16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 constexpr int kProbeThreads = 512;  // 8 waves, two per SIMD
 constexpr int kProbeOperands = 16;  // 8 A and 8 B operand registers (of 8 halves) per lane
@@ -40,18 +46,20 @@ __global__ __launch_bounds__(kProbeThreads, 1) void mfma_rate_probe_kernel(const
 }
 
 }  // namespace
-}  // namespace cpmcu
 
-using namespace cpmcu;
+// Bytes of fp16 operand data one launch reads: 16 operand registers of 8 halves for each of 512 threads.
+extern "C" size_t bench_mfma_rate_probe_operand_bytes(void) { return (size_t)kProbeOperands * kProbeThreads * sizeof(f16x8); }
 
-extern "C" size_t cpmcu_mfma_rate_probe_operand_bytes(void) { return (size_t)kProbeOperands * kProbeThreads * sizeof(f16x8); }
-
-extern "C" int cpmcu_mfma_rate_probe(const void* operands, int iters, int workgroups, float* out, double* flops, void* stream) {
-    CPMCU_CHECK_ARG(operands && out, "mfma_rate_probe: null pointer argument");
-    CPMCU_CHECK_ARG(iters >= 1 && workgroups >= 1 && workgroups <= 4096, "mfma_rate_probe: iters=%d, workgroups=%d", iters, workgroups);
-    hipLaunchKernelGGL(mfma_rate_probe_kernel, dim3(workgroups), dim3(kProbeThreads), 0, resolve_stream(stream), (const f16x8*)operands, iters,
+// Enqueues `workgroups` workgroups of 8 waves on `stream` (NULL = the null stream), every lane issuing
+// iters x 16 v_mfma_f32_32x32x16_f16 on four accumulator chains from operands held in registers.
+// out: device float[workgroups * 512].  *flops (host, may be NULL) receives the floating-point
+// operations of the launch.  Returns 0, or a HIP error code / -1 for bad arguments.
+extern "C" int bench_mfma_rate_probe(const void* operands, int iters, int workgroups, float* out, double* flops, void* stream) {
+    if (!operands || !out || iters < 1 || workgroups < 1 || workgroups > 4096) return -1;
+    hipLaunchKernelGGL(mfma_rate_probe_kernel, dim3(workgroups), dim3(kProbeThreads), 0, (hipStream_t)stream, (const f16x8*)operands, iters,
                        out);
-    CPMCU_LAUNCH_CHECK();
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return (int)e;
     if (flops) *flops = (double)workgroups * (kProbeThreads / 64) * (double)iters * 16.0 * (2.0 * 32 * 32 * 16);
-    return CPMCU_OK;
+    return 0;
 }

@@ -20,7 +20,7 @@ LIB_PATH = os.path.join(HERE, "libcpmcu_amd.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 ARCH = "gfx950"
 
-HIP_SOURCES = ["runtime.hip", "tree_attention.hip", "lm_head.hip", "topk.hip", "tree_accept.hip", "draft_tree.hip", "probe.hip"]
+HIP_SOURCES = ["runtime.hip", "tree_attention.hip", "lm_head.hip", "topk.hip", "tree_accept.hip", "draft_tree.hip"]
 HEADERS = sorted(f for f in os.listdir(CSRC) if f.endswith(".h"))
 
 # packed fp32 VALU ops stay off for every device translation unit
@@ -75,6 +75,12 @@ def build_all(force=False, verbose=False):
         _run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden",
               f"-I{pybind11.get_include()}", f"-I{sysconfig.get_paths()['include']}", f"-I{INCLUDE}",
               entry, "-o", mod, f"-L{HERE}", "-lcpmcu_amd", "-Wl,-rpath,$ORIGIN"])
+    # bench.py's measurement helper: its own small library, outside the product
+    probe_src = os.path.join(ROOT, "bench_probes", "mfma_rate_probe.hip")
+    probe_lib = os.path.join(ROOT, "bench_probes", "libbench_probes.so")
+    if os.path.exists(probe_src) and (force or _stale(probe_lib, [probe_src])):
+        _run([HIPCC, f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-shared", "-Xclang", "-target-feature", "-Xclang",
+              "-packed-fp32-ops", probe_src, "-o", probe_lib])
     return LIB_PATH
 
 

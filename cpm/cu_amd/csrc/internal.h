@@ -4,6 +4,14 @@
 
 namespace cpmcu {
 
+// runtime.hip -- kernel-shape switches, read from the environment once when the library is first used
+// (CPMCU_ATTN_KV_GROUPS=1|2, CPMCU_HEAD_NO_SHARE) and changed afterwards through cpmcu_set_option.
+struct Options {
+    int attn_kv_groups = 0;        // 0 = chosen per call; 1 / 2 force that tree-attention kernel shape
+    int head_share_last_pass = 1;  // 0 keeps the plain row-block mapping of the head GEMM
+};
+Options& options();
+
 // lm_head.hip -- the streaming GEMM with its two epilogues.
 constexpr int kHeadModeStats = 0;
 constexpr int kHeadModeArgmax = 1;

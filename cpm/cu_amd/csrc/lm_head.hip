@@ -601,6 +601,7 @@ int launch_head_gemm(const void* hidden, const void* w, int w_layout, int n, int
     p.npasses = ceil_div(nrb, G * kHeadWaves);
     p.full_passes = 0;
     p.rem_blocks = 0;
+    CPMCU_CHECK_ARG(G <= head_max_grid(), "lm_head: %d workgroups exceed the %d rows of the partial planes", G, head_max_grid());
     *grid_out = G;
     *stride_out = NB * 16;
     // Kernel shapes chosen by measurement on MI355X (73448 x 4096 and 32768 x 4096 heads).
@@ -615,9 +616,9 @@ int launch_head_gemm(const void* hidden, const void* w, int w_layout, int n, int
         }
     } else if (p.w_tiled) {
         // one sweep (all passes fit the accumulator sets) with a partly filled last pass: share it
-        // (CPMCU_HEAD_NO_SHARE in the environment keeps the plain mapping; tests compare the two)
+        // (the option head_share_last_pass = 0 keeps the plain mapping; tests compare the two)
         const int rem = nrb - (p.npasses - 1) * G * kHeadWaves;
-        if (p.npasses <= 4 && rem < G * kHeadWaves && getenv("CPMCU_HEAD_NO_SHARE") == nullptr) {  // <= NP of every shape below
+        if (p.npasses <= 4 && rem < G * kHeadWaves && options().head_share_last_pass) {  // <= NP of every shape below
             p.full_passes = p.npasses - 1;
             p.rem_blocks = rem;
         }
@@ -643,6 +644,8 @@ int launch_head_gemm(const void* hidden, const void* w, int w_layout, int n, int
         }
     } else {
         switch (NB) {
+            // <= 16 rows whose K range exceeds two LDS buffers (H >= 6144): the row-walking kernel, chunked
+            case 1: hipLaunchKernelGGL(head_gemm_kernel<1>, dim3(G), dim3(kHeadThreads), 0, st, p); break;
             case 2: hipLaunchKernelGGL((head_gemm_chunked_kernel<2, 4, 512, 2>), dim3(G), dim3(kHeadThreads), 0, st, p); break;
             case 4: hipLaunchKernelGGL((head_gemm_chunked_kernel<4, 4, 128, 4>), dim3(G), dim3(kHeadThreads), 0, st, p); break;
             default: hipLaunchKernelGGL((head_gemm_chunked_kernel<8, 2, 128, 2>), dim3(G), dim3(kHeadThreads), 0, st, p); break;
@@ -699,17 +702,9 @@ extern "C" int cpmcu_head_weight_tile(const void* w, const int32_t* row_remap, i
     return CPMCU_OK;
 }
 
-extern "C" int cpmcu_lm_head_argmax(const void* hidden, const void* w, int w_layout, int n, int V, int H, int apply_scale,
-                                    float head_scale, void* logits, int32_t* gt, void* workspace,
-                                    size_t workspace_bytes, void* stream) {
-    CPMCU_CHECK_ARG(hidden && w, "lm_head_argmax: null pointer argument");
-    CPMCU_CHECK_ARG(n >= 1 && n <= 128, "lm_head_argmax: n=%d outside [1, 128]", n);
-    CPMCU_CHECK_ARG(V >= 1 && H >= 1, "lm_head_argmax: bad shape V=%d H=%d", V, H);
-    CPMCU_CHECK_ARG(logits || gt, "lm_head_argmax: both outputs are null");
-    CPMCU_CHECK_ARG(workspace && workspace_bytes >= cpmcu_head_workspace_bytes(n, V),
-                    "lm_head_argmax: workspace of %zu bytes needed, %zu given", cpmcu_head_workspace_bytes(n, V), workspace_bytes);
-    hipStream_t st = resolve_stream(stream);
-    float* part_a = (float*)workspace;
+// The target head on per-workgroup partials held at `part_a` (two float planes of head_max_grid() * 128).
+static int lm_head_argmax_on(const void* hidden, const void* w, int w_layout, int n, int V, int H, int apply_scale,
+                             float head_scale, void* logits, int32_t* gt, float* part_a, hipStream_t st) {
     float* part_b = part_a + (size_t)head_max_grid() * 128;
     int G = 0, stride = 0;
     int rc = launch_head_gemm(hidden, w, w_layout, n, V, H, apply_scale, head_scale, kHeadModeArgmax, logits, part_a, part_b, &G, &stride, st);
@@ -719,4 +714,16 @@ extern "C" int cpmcu_lm_head_argmax(const void* hidden, const void* w, int w_lay
         CPMCU_LAUNCH_CHECK();
     }
     return CPMCU_OK;
+}
+
+extern "C" int cpmcu_lm_head_argmax(const void* hidden, const void* w, int w_layout, int n, int V, int H, int apply_scale,
+                                    float head_scale, void* logits, int32_t* gt, void* workspace,
+                                    size_t workspace_bytes, void* stream) {
+    CPMCU_CHECK_ARG(hidden && w, "lm_head_argmax: null pointer argument");
+    CPMCU_CHECK_ARG(n >= 1 && n <= 128, "lm_head_argmax: n=%d outside [1, 128]", n);
+    CPMCU_CHECK_ARG(V >= 1 && H >= 1, "lm_head_argmax: bad shape V=%d H=%d", V, H);
+    CPMCU_CHECK_ARG(logits || gt, "lm_head_argmax: both outputs are null");
+    CPMCU_CHECK_ARG(workspace && workspace_bytes >= cpmcu_head_workspace_bytes(n, V),
+                    "lm_head_argmax: workspace of %zu bytes needed, %zu given", cpmcu_head_workspace_bytes(n, V), workspace_bytes);
+    return lm_head_argmax_on(hidden, w, w_layout, n, V, H, apply_scale, head_scale, logits, gt, (float*)workspace, resolve_stream(stream));
 }

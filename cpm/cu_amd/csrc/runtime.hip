@@ -37,6 +37,19 @@ hipStream_t resolve_stream(void* stream) {
     return g_stream;
 }
 
+Options& options() {
+    static Options opt = [] {
+        Options o;
+        if (const char* e = getenv("CPMCU_ATTN_KV_GROUPS")) {
+            if (e[0] == '1' && e[1] == 0) o.attn_kv_groups = 1;
+            if (e[0] == '2' && e[1] == 0) o.attn_kv_groups = 2;
+        }
+        if (getenv("CPMCU_HEAD_NO_SHARE") != nullptr) o.head_share_last_pass = 0;
+        return o;
+    }();
+    return opt;
+}
+
 namespace {
 
 struct PerfEntry {
@@ -134,6 +147,22 @@ using namespace cpmcu;
 
 extern "C" const char* cpmcu_last_error(void) { return g_error.c_str(); }
 extern "C" const char* cpmcu_version(void) { return "cpmcu_amd 0.1 (gfx950)"; }
+
+extern "C" int cpmcu_set_option(const char* name, int value) {
+    CPMCU_CHECK_ARG(name, "set_option: null name");
+    const std::string nm(name);
+    if (nm == "attn_kv_groups") {
+        CPMCU_CHECK_ARG(value >= 0 && value <= 2, "set_option: attn_kv_groups=%d outside [0, 2]", value);
+        options().attn_kv_groups = value;
+    } else if (nm == "head_share_last_pass") {
+        CPMCU_CHECK_ARG(value == 0 || value == 1, "set_option: head_share_last_pass=%d must be 0 or 1", value);
+        options().head_share_last_pass = value;
+    } else {
+        set_error("set_option: unknown option %s", name);
+        return CPMCU_ERR_INVALID_ARGUMENT;
+    }
+    return CPMCU_OK;
+}
 
 extern "C" int cpmcu_init_base_model(float memory_limit, int vocab_size, int num_hidden_layers, int hidden_size,
                                      int intermediate_size, int num_attention_heads, int num_key_value_heads,

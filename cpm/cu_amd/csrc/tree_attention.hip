@@ -33,6 +33,7 @@
 //  * Workgroups are mapped so that all M-tiles that stream the same KV range
 //    land on the same XCD (workgroup id modulo 8) and share its L2.
 #include "common.h"
+#include "internal.h"
 
 #include <type_traits>
 
@@ -737,13 +738,11 @@ int choose_splits(int T, int group, int Hkv, int max_kv_len, int G) {
 // 256-row shape vs two-group shape:  60-node tree (8 units): 32.8 / 31.1 at 16K, 50 / 50 at 32K,
 // 67.7 / 71.2 at 48K, 156 / 170 at 128K;  128-node tree (16 units): 30.3 / 29.5 at 4K, 56.1 / 59.3 at
 // 16K, 301 / 326 at 128K;  16 nodes or one (2 units): 74.8 / 62.4 and 73.2 / 55.0 at 128K.
-// CPMCU_ATTN_KV_GROUPS=1|2 in the environment overrides the choice (tests exercise both shapes).
+// The option attn_kv_groups (cpmcu_set_option; CPMCU_ATTN_KV_GROUPS=1|2 in the environment at load) overrides the
+// choice: tests exercise both shapes.
 constexpr int kLongRunTiles = 16;
 int choose_groups(int T, int group, int Hkv, int max_kv_len) {
-    if (const char* e = getenv("CPMCU_ATTN_KV_GROUPS")) {
-        if (e[0] == '1' && e[1] == 0) return 1;
-        if (e[0] == '2' && e[1] == 0) return 2;
-    }
+    if (options().attn_kv_groups != 0) return options().attn_kv_groups;
     const int units = ceil_div(group * T, rows_per_wg(1)) * Hkv;
     const int ntiles = ceil_div(max_kv_len, kTileN);
     return units >= 4 && (long long)ntiles * units >= (long long)kLongRunTiles * 256 ? 1 : 2;

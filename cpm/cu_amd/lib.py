@@ -22,6 +22,7 @@ _P = c_void_p
 SIGNATURES = {
     "cpmcu_last_error": (c_char_p, []),
     "cpmcu_version": (c_char_p, []),
+    "cpmcu_set_option": (c_int, [c_char_p, c_int]),
     "cpmcu_init_base_model": (c_int, [c_float, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_float, c_float, c_float]),
     "cpmcu_init_eagle_model": (c_int, [c_int] * 5),
     "cpmcu_init_minicpm4_eagle_model": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int]),
@@ -64,8 +65,6 @@ SIGNATURES = {
     "cpmcu_draft_tree_begin": (c_int, [_P, c_int, c_int, _P, _P, _P, _P, _P, _P]),
     "cpmcu_draft_tree_extend": (c_int, [_P, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P]),
     "cpmcu_draft_tree_finish": (c_int, [_P, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P]),
-    "cpmcu_mfma_rate_probe_operand_bytes": (c_size_t, []),
-    "cpmcu_mfma_rate_probe": (c_int, [_P, c_int, c_int, _P, _P, _P]),
 }
 
 

@@ -297,15 +297,3 @@ class DraftTree:
         _lib().draft_tree_finish(_ptr(self.state), self.k, self.num_iter, T, _ptr(cache_length), _ptr(self.remap),
                                  _ptr(tree_draft_ids), _ptr(pos), _ptr(mask), _ptr(parent), _stream())
         return tree_draft_ids, pos, mask, parent
-
-
-def mfma_rate_probe(operands, iters, workgroups=256):
-    """Enqueue the register-resident MFMA loop on `operands` (fp16, mfma_rate_probe_operand_bytes() bytes);
-    returns the floating-point operations of the launch.  Time it with events on the current stream."""
-    lib = _lib()
-    need = lib.raw.cpmcu_mfma_rate_probe_operand_bytes()
-    assert operands.dtype == torch.float16 and operands.numel() * 2 >= need and operands.is_contiguous()
-    out = _workspace("mfma_probe", workgroups * 512 * 4, operands.device)
-    flops = ctypes.c_double(0.0)
-    lib.mfma_rate_probe(_ptr(operands), int(iters), int(workgroups), _ptr(out), ctypes.byref(flops), _stream())
-    return flops.value

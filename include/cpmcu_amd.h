@@ -63,6 +63,15 @@ const char* cpmcu_last_error(void);
 /* Library version string and the GPU architecture the kernels were built for. */
 const char* cpmcu_version(void);
 
+/* No reference counterpart: kernel-shape switches for tests and tuning (process-wide, not thread-safe
+ * against concurrent calls).  Initial values come from the environment, read once when the library is
+ * first used.
+ *   "attn_kv_groups"        0 = chosen per call (default), 1 / 2 = force the 256-row / the two-KV-group
+ *                           shape of the tree-attention kernel (CPMCU_ATTN_KV_GROUPS=1|2);
+ *   "head_share_last_pass"  1 = the waves of a workgroup share the row blocks of a partly filled last pass
+ *                           of the head GEMM (default), 0 = plain mapping (CPMCU_HEAD_NO_SHARE set). */
+int cpmcu_set_option(const char* name, int value);
+
 /* ------------------------------------------------------------------------- */
 /* 1. Model-level mirror of src/entry.cu                                      */
 /* ------------------------------------------------------------------------- */
@@ -383,20 +392,6 @@ int cpmcu_draft_tree_extend(void* state, int k, int num_iter, int d, void* topk_
 int cpmcu_draft_tree_finish(void* state, int k, int num_iter, int tree_size, const int32_t* cache_length,
                             const int32_t* token_id_remap, int32_t* tree_draft_ids, int32_t* tree_position_ids,
                             uint64_t* tree_attn_mask, int32_t* tree_parent, void* stream);
-
-/* ------------------------------------------------------------------------- */
-/* 3. Measurement helper (no counterpart in the reference)                    */
-/* ------------------------------------------------------------------------- */
-
-/* What the matrix pipes deliver to a kernel that does nothing else: `workgroups` workgroups of 8 waves,
- * every lane holding 8 A and 8 B operands of v_mfma_f32_32x32x16_f16 in registers and issuing
- * iters x 16 MFMAs on four accumulator chains.  operands: device fp16 data of
- * cpmcu_mfma_rate_probe_operand_bytes() bytes -- the sustained rate depends on it (all-zero operands
- * run at the published peak, random ones well below: clocks follow the power drawn), which is why
- * the data is the caller's.  out: device float[workgroups * 512].  *flops (host, may be NULL)
- * receives the floating-point operations one launch performs; time the launch with events. */
-size_t cpmcu_mfma_rate_probe_operand_bytes(void);
-int cpmcu_mfma_rate_probe(const void* operands, int iters, int workgroups, float* out, double* flops, void* stream);
 
 #ifdef __cplusplus
 }

@@ -29,3 +29,18 @@ def gpu():
     lib.get()  # raises ImportError if libcpmcu_amd.so is missing: no fallback
     torch.cuda.set_device(0)
     return torch
+
+
+@pytest.fixture
+def set_option():
+    """Sets kernel-shape options of the library for one test and restores the defaults afterwards."""
+    from cpm.cu_amd import lib
+    defaults = {"attn_kv_groups": 0, "head_share_last_pass": 1}
+    touched = []
+
+    def setter(name, value):
+        lib.get().set_option(name.encode(), int(value))
+        touched.append(name)
+    yield setter
+    for name in touched:
+        lib.get().set_option(name.encode(), defaults[name])

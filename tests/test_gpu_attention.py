@@ -15,10 +15,10 @@ HQ, HKV, D = 32, 2, 128
 
 
 @pytest.fixture(autouse=True, params=["2", "1"], ids=["groups2", "groups1"])
-def kv_groups(request, monkeypatch):
+def kv_groups(request, set_option):
     """Every test of this module runs on both shapes of the split kernel (2 KV groups x 128 rows and
     1 x 256 rows per workgroup); without the override the library picks by context length."""
-    monkeypatch.setenv("CPMCU_ATTN_KV_GROUPS", request.param)
+    set_option("attn_kv_groups", int(request.param))
     return request.param
 
 

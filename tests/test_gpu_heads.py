@@ -16,17 +16,22 @@ from util import assert_close_f16, to_dev, to_np
 pytestmark = pytest.mark.gpu
 
 
-def _frspec_check(torch, orc, n, V, Vs, H, k, seed):
+def _frspec_check(torch, orc, n, V, Vs, H, k, seed, tiled=False):
+    """tiled: the sub-matrix is built by tile_head_weight(w, remap) -- gather fused with the re-tiling, the layout
+    the model-level loader and the benchmark keep -- instead of gather_rows into a row-major matrix."""
     from cpm.cu_amd import ops
     hid = synth.normal_f16((n, H), seed, 1)
     w = synth.normal_f16((V, H), seed, 2, std=0.02)
     remap = synth.frspec_remap(V, Vs, seed)
     d_w = to_dev(torch, w)
     d_remap = to_dev(torch, remap)
-    d_sub = ops.gather_rows(d_w, d_remap)  # remap_copy
     sub = orc.gather_rows(w, remap)
-    assert np.array_equal(to_np(d_sub).view(np.uint16), sub.view(np.uint16))
     assert np.array_equal(sub.view(np.uint16), w[remap].view(np.uint16))
+    if tiled:
+        d_sub = ops.tile_head_weight(d_w, d_remap)
+    else:
+        d_sub = ops.gather_rows(d_w, d_remap)  # remap_copy
+        assert np.array_equal(to_np(d_sub).view(np.uint16), sub.view(np.uint16))
 
     r = ops.frspec_head_topk(to_dev(torch, hid), d_sub, d_remap, k)
     torch.cuda.synchronize()
@@ -101,6 +106,22 @@ def test_frspec_c3_full_size(gpu, orc):
     """Config 3: 10 frontier rows, 73448x4096 head, 32768-row subset, top-10 mapped to full-vocab ids."""
     exact = _frspec_check(gpu, orc, n=10, V=73448, Vs=32768, H=4096, k=10, seed=0)
     print("c3 end-to-end ids bit-exact vs pure oracle:", exact)
+
+
+@pytest.mark.parametrize("n", [10, 1])
+def test_frspec_c3_full_size_tiled_layout(gpu, orc, n):
+    """Config 3 through the layout the benchmark and the model-level loader use: the 32768-row sub-matrix gathered
+    and tiled in one pass out of the 73448-row head, so the GEMM is the single-pass chunked shape (one 16-row block
+    per wave, 8 K chunks of 512 rotated over the workgroups, 256 workgroups).  n = 1 is the first draft round."""
+    exact = _frspec_check(gpu, orc, n=n, V=73448, Vs=32768, H=4096, k=10, seed=0, tiled=True)
+    print("c3 tiled, n=%d: end-to-end ids bit-exact vs pure oracle: %s" % (n, exact))
+
+
+def test_frspec_tiled_chunk_rotation_shapes(gpu, orc):
+    """The single-pass tiled shape away from config 3: several K chunks with fewer workgroups than chunks' rotation
+    period, a vocabulary that leaves the last row block partly filled, 16 rows."""
+    _frspec_check(gpu, orc, n=16, V=9000, Vs=4096 + 40, H=2048, k=10, seed=11, tiled=True)
+    _frspec_check(gpu, orc, n=7, V=40000, Vs=32768, H=1024, k=32, seed=12, tiled=True)
 
 
 def test_frspec_subset_vs_full_head(gpu, orc):
@@ -206,6 +227,22 @@ def test_target_head_planted_ties(gpu, orc):
         w[2999] = w[2998] = (hid[1].astype(np.float32) * 0.05).astype(np.float16)
     gt, z = _argmax_check(gpu, orc, 4, V=3000, H=512, seed=4, plant=plant)
     assert gt[0] == 700 and gt[1] == 2998
+
+
+@pytest.mark.parametrize("tiled", [False, True])
+def test_target_head_c1_full_size(gpu, orc, tiled):
+    """Config 1 head: 16 tree rows against the 73448x4096 head, in both weight layouts."""
+    _argmax_check(gpu, orc, 16, V=73448, H=4096, seed=1, tiled=tiled)
+
+
+@pytest.mark.parametrize("n", [1, 10, 16])
+@pytest.mark.parametrize("H", [6144, 8192])
+def test_row_major_head_with_many_k_chunks(gpu, orc, n, H):
+    """Up to 16 rows against a row-major matrix whose K range needs more than two LDS buffers: the row-walking
+    kernel in its chunked form.  Arg-max and the FR-Spec statistics come from per-workgroup partials, whose row
+    stride has to be the launched kernel's."""
+    _argmax_check(gpu, orc, n, V=2100, H=H, seed=40 + n)
+    _frspec_check(gpu, orc, n=n, V=2600, Vs=2048 + 24, H=H, k=10, seed=50 + n)
 
 
 def test_target_head_c2_full_size(gpu, orc):
@@ -319,7 +356,7 @@ def test_tiled_weight_layout_gives_the_same_logits(gpu, orc, n, V, H):
 
 
 @pytest.mark.parametrize("n,V,H", [(60, 73448, 4096), (10, 40000, 1024), (33, 36000, 512), (64, 34000, 512), (5, 32768 + 16 * 300, 512)])
-def test_shared_last_pass_equals_plain_mapping(gpu, orc, monkeypatch, n, V, H):
+def test_shared_last_pass_equals_plain_mapping(gpu, orc, set_option, n, V, H):
     """Row-block counts that leave the last pass partly filled (1, 2 or more blocks per workgroup, with 2, 4 and 16
     K chunks): the waves that share a block add their partial sums in LDS.  Same logits as the plain mapping up to
     the fp32 summation order, same arg-max wherever the top two are apart, and both match the oracle."""
@@ -331,7 +368,7 @@ def test_shared_last_pass_equals_plain_mapping(gpu, orc, monkeypatch, n, V, H):
     wt = ops.tile_head_weight(to_dev(torch, w))
     gt_s, z_s = ops.lm_head_argmax(d_hid, wt, want_logits=True)
     torch.cuda.synchronize()
-    monkeypatch.setenv("CPMCU_HEAD_NO_SHARE", "1")
+    set_option("head_share_last_pass", 0)
     gt_p, z_p = ops.lm_head_argmax(d_hid, wt, want_logits=True)
     torch.cuda.synchronize()
     assert_close_f16(to_np(z_s), to_np(z_p), "shared vs plain last pass", atol=8e-3, rtol=2e-3)

@@ -50,11 +50,11 @@ def test_rope_table_and_in_place_operator(gpu, orc):
 
 
 @pytest.mark.parametrize("P,T,groups", [(1000, 60, "2"), (4096 - 30, 60, "2"), (300, 17, "1"), (70000, 64, "1"), (0, 9, "2")])
-def test_attention_with_fused_rope(gpu, orc, monkeypatch, P, T, groups):
+def test_attention_with_fused_rope(gpu, orc, set_option, P, T, groups):
     from cpm.cu_amd import ops
     from cpm.cu_amd.kvcache import PagedKVCache
     torch = gpu
-    monkeypatch.setenv("CPMCU_ATTN_KV_GROUPS", groups)
+    set_option("attn_kv_groups", int(groups))
     seed = P + T
     tree = synth.random_tree(T, seed, max_children=4, max_depth=8)
     mask = to_dev(torch, tree.mask)

@@ -1,0 +1,181 @@
+"""Whole verify steps at the benchmark configurations' real sizes, and the same path driven through the pybind
+module `C` (the names of the reference's src/entry.cu:510-534), against the CPU oracle.
+
+  * config 5 as ONE step: 32 layers, 32768-token prefix, 128-node tree, target arg-max rigged so that the seeded
+    paths accept 0..8 draft tokens; accept length, accepted ids and the compacted rows of all 64 caches bit-exact,
+    attention of a sampled layer within the fp16 tolerance;
+  * `C.init_base_model -> C.init_minicpm4_eagle_model -> C.init_storage -> C.load_model -> C.decode_attention ->
+    C.decode_lm_head -> C.verify_and_fix`, the call sequence of cpmcu/llm.py and cpmcu/speculative/tree_drafter.py
+    restricted to the path.
+"""
+import numpy as np
+import pytest
+
+from cpm.cu_amd import synth
+from util import assert_close_f16, to_dev, to_np
+
+pytestmark = pytest.mark.gpu
+
+HQ, HKV, D = 32, 2, 128
+
+
+def test_c5_wide_tree_step_32_layers_every_depth(gpu, orc):
+    from cpm.cu_amd import ops
+    from cpm.cu_amd.driver import VerifyStep
+    from cpm.cu_amd.kvcache import PagedKVCache
+    torch = gpu
+    cfg = synth.CONFIGS["c5_wide_32k"]
+    L, P, T = cfg["layers"], cfg["prefix"], cfg["T"]
+    V, H = 20000, 1024  # the head at full size has its own tests; the step needs a target arg-max, not 602 MB of weights
+    S = P + T
+    tree = synth.eagle_tree(cfg["num_iter"], cfg["topk"], T, seed=3)  # a seed whose tree reaches all 8 draft levels
+    assert int(tree.depth.max()) == 8
+    npages = (S + 255) // 256 + 1
+    table = synth.rng(5, 4).permutation(npages).astype(np.int32)
+    cache = PagedKVCache(L, HKV, npages, block_table=table)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(5)
+    for l in range(L):  # ~N(0,1) prefix, generated on the device in the pools' own layout
+        cache.k[l].normal_(generator=g)
+        cache.v[l].normal_(generator=g)
+    rn = lambda *s, std=1.0: (torch.randn(*s, device="cuda", generator=g) * std).to(torch.float16)
+    q = [rn(T, HQ, D) for _ in range(L)]
+    k_new = [rn(T, HKV, D) for _ in range(L)]
+    v_new = [rn(T, HKV, D) for _ in range(L)]
+    hidden = rn(T, H)
+    w = rn(V, H, std=0.02)
+    w_t = ops.tile_head_weight(w)
+    mask, parent, pos = to_dev(torch, tree.mask), to_dev(torch, tree.parent), to_dev(torch, tree.positions(P))
+    attn_out = [torch.empty(T, HQ, D, dtype=torch.float16, device="cuda") for _ in range(L)]
+    # what the step must leave alone: the prefix rows of every cache (checked through logical reads of a few
+    # layers in full and of every layer's last prefix page)
+    sampled = (0, 17, 31)
+    before = {l: cache.read_logical(l, 0, P) for l in sampled}
+    tail0 = P - 256
+    before_tail = [cache.read_logical(l, tail0, 256) for l in range(L)]
+
+    vs = VerifyStep(cache, w_t, mask, parent, pos, P)
+    gt = to_np(ops.lm_head_argmax(hidden, w_t))
+    assert np.array_equal(gt, orc.argmax(to_np(ops.lm_head_argmax(hidden, w_t, want_logits=True)[1])))
+    k_new_np = [to_np(t).reshape(T, -1) for t in k_new]
+    v_new_np = [to_np(t).reshape(T, -1) for t in v_new]
+    for depth in range(9):
+        pred, leaf = synth.draft_ids_for_accept(tree, gt, depth, V, 100 + depth)
+        vs.enqueue(q, k_new, v_new, hidden, to_dev(torch, pred), attn_out=attn_out)
+        a, ids = vs.result()
+        a_ref, node_ref, path = orc.tree_accept(pred, gt, tree.positions(P), P, tree.mask, tree.parent)
+        assert a == a_ref == depth + 1 and list(path) == tree.path_to(leaf)
+        assert int(vs.best[1].item()) == node_ref
+        assert np.array_equal(to_np(vs.gt), gt)
+        # the oracle's compaction of the tree rows (prefix length 0 on the T appended rows of each cache)
+        flat = []
+        for l in range(L):
+            flat += [k_new_np[l].copy(), v_new_np[l].copy()]
+        ids_ref = orc.kv_compact(flat, 0, path, gt)
+        assert np.array_equal(ids, ids_ref) and np.array_equal(ids, gt[path])
+        for l in range(L):
+            kd, vd = cache.read_logical(l, P, a)
+            assert np.array_equal(to_np(kd).reshape(a, -1).view(np.uint16), flat[2 * l][:a].view(np.uint16)), (depth, l)
+            assert np.array_equal(to_np(vd).reshape(a, -1).view(np.uint16), flat[2 * l + 1][:a].view(np.uint16)), (depth, l)
+        if depth == 0:
+            # attention of one sampled layer against the oracle (prefix read back from the pool + the tree rows)
+            l = 17
+            kp, vp = before[l]
+            k_all = np.concatenate([to_np(kp), to_np(k_new[l])])
+            v_all = np.concatenate([to_np(vp), to_np(v_new[l])])
+            ref = orc.tree_attention(to_np(q[l]), k_all, v_all, tree.mask, P)
+            assert_close_f16(to_np(attn_out[l]), ref, "config 5 step, attention of layer %d" % l)
+    for l in sampled:
+        kd, vd = cache.read_logical(l, 0, P)
+        assert torch.equal(kd, before[l][0]) and torch.equal(vd, before[l][1]), "prefix of layer %d changed" % l
+    for l in range(L):
+        kd, vd = cache.read_logical(l, tail0, 256)
+        assert torch.equal(kd, before_tail[l][0]) and torch.equal(vd, before_tail[l][1]), "last prefix page of layer %d changed" % l
+
+
+def test_pybind_module_drives_the_path_end_to_end(gpu, orc):
+    """The reference's own entry-point names, positional signatures and raw-address conventions
+    (tensor.data_ptr(); host pointer for load_model), nothing else: what cpmcu/llm.py would call."""
+    from cpm.cu_amd import C
+    torch = gpu
+    V, Vs, H, layers, T, P = 5000, 2048, 512, 2, 60, 333
+    keep = []
+
+    def dev(a):
+        t = to_dev(torch, a)
+        keep.append(t)
+        return t.data_ptr()
+    C.init_base_model(0.02, V, layers, H, 1024, HQ, HKV, D, 1e-5, 0, 2048, 1.0, 0.25, 1.0)
+    C.init_minicpm4_eagle_model(1, 6, 10, T, 0, False, 128, 1024, Vs, 1.0, True, True)
+    ctx = C.init_storage()
+    assert isinstance(ctx, int) and ctx >= 4096
+    w = synth.normal_f16((V, H), 21, 2, std=0.02)
+    remap = synth.frspec_remap(V, Vs, 21)
+    with pytest.raises(ValueError):
+        C.load_model("model.embed_tokens.weight", w.ctypes.data)
+    C.load_model("eagle.token_id_remap", remap.ctypes.data)
+    C.load_model("lm_head.weight", w.ctypes.data)
+    tree = synth.eagle_tree(6, 10, T, seed=4)
+    S = P + T
+    cl = torch.tensor([0], dtype=torch.int32, device="cuda")
+    dummy = torch.empty((64, HQ, D), dtype=torch.float16, device="cuda")
+    flat = []
+    for layer in range(layers):
+        k = synth.normal_f16((S, HKV, D), 22, 10 + layer)
+        v = synth.normal_f16((S, HKV, D), 22, 50 + layer)
+        q = synth.normal_f16((T, HQ, D), 22, 90 + layer)
+        done = 0
+        while done < P:  # the prefix goes in as causal chunks of <= 64 rows
+            n = min(64, P - done)
+            cl.fill_(done + n)
+            C.decode_attention(layer, n, done + n, dev(np.repeat(q[:1], n, 0)), dev(k[done:done + n]), dev(v[done:done + n]),
+                               cl.data_ptr(), 0, dummy.data_ptr())
+            C.synchronize()
+            done += n
+        cl.fill_(S)
+        out = torch.empty((T, HQ, D), dtype=torch.float16, device="cuda")
+        C.decode_attention(layer, T, (S + 127) // 128 * 128, dev(q), dev(k[P:]), dev(v[P:]), cl.data_ptr(), dev(tree.mask), out.data_ptr())
+        C.synchronize()
+        assert_close_f16(to_np(out), orc.tree_attention(q, k, v, tree.mask, P), "C.decode_attention layer %d" % layer)
+        flat += [k.reshape(S, -1).copy(), v.reshape(S, -1).copy()]
+    hid = synth.normal_f16((T, H), 22, 200)
+    logits = torch.empty((64, V), dtype=torch.float16, device="cuda")
+    gt = torch.empty(T, dtype=torch.int32, device="cuda")
+    C.decode_lm_head(T, dev(hid), logits.data_ptr(), gt.data_ptr())
+    C.synchronize()
+    assert_close_f16(to_np(logits[:T]), orc.lm_head(hid, w, head_scale=0.25), "C.decode_lm_head")
+    gt_np = to_np(gt)
+    assert np.array_equal(gt_np, orc.argmax(to_np(logits[:T])))
+    # the draft head on the loaded FR-Spec sub-matrix
+    val = torch.empty((10, 10), dtype=torch.float16, device="cuda")
+    pos = torch.empty((10, 10), dtype=torch.int32, device="cuda")
+    ids = torch.empty((10, 10), dtype=torch.int32, device="cuda")
+    C.draft_head(10, dev(hid[:10]), val.data_ptr(), pos.data_ptr(), ids.data_ptr())
+    C.synchronize()
+    assert np.array_equal(to_np(ids), remap[to_np(pos)])
+    # verify_and_fix returns the accept length; pred[:a] becomes the accepted ids; every cache is compacted
+    pred, leaf = synth.draft_ids_for_accept(tree, gt_np, 4, V, 6)
+    d_pred = to_dev(torch, pred)
+    cl.fill_(P)
+    a = C.verify_and_fix(T, d_pred.data_ptr(), gt.data_ptr(), dev(tree.positions(P)), cl.data_ptr(), dev(tree.mask), dev(tree.parent))
+    a_ref, _, path = orc.tree_accept(pred, gt_np, tree.positions(P), P, tree.mask, tree.parent)
+    ids_ref = orc.kv_compact(flat, P, path, gt_np)
+    assert a == a_ref == 5
+    assert np.array_equal(to_np(d_pred)[:a], ids_ref)
+    # the compacted caches as the next decode step sees them
+    S2 = P + a + 1
+    one = synth.chain_tree(1)
+    for layer in range(layers):
+        kn = synth.normal_f16((1, HKV, D), 23, 10 + layer)
+        vn = synth.normal_f16((1, HKV, D), 23, 50 + layer)
+        qn = synth.normal_f16((1, HQ, D), 23, 90 + layer)
+        cl.fill_(S2)
+        out = torch.empty((1, HQ, D), dtype=torch.float16, device="cuda")
+        C.decode_attention(layer, 1, (S2 + 127) // 128 * 128, dev(qn), dev(kn), dev(vn), cl.data_ptr(), 0, out.data_ptr())
+        C.synchronize()
+        k_flat = np.concatenate([flat[2 * layer][: P + a].reshape(-1, HKV, D), kn])
+        v_flat = np.concatenate([flat[2 * layer + 1][: P + a].reshape(-1, HKV, D), vn])
+        assert_close_f16(to_np(out), orc.tree_attention(qn, k_flat, v_flat, one.mask, P + a), "C: decode after compaction, layer %d" % layer)
+    with pytest.raises(RuntimeError, match="outside the verify/draft path"):
+        C.decode(T, 128, 0, 0, 0, 0, 0, False)
+    C.shutdown()
