@@ -25,6 +25,8 @@
 //   * when the row blocks do not divide evenly over the wave slots, the blocks of the partly
 //     filled last pass are dealt round-robin to the workgroups and several waves share each of
 //     them, every one taking a subset of the K chunks; their partial sums meet in LDS.
+#include <mutex>
+
 #include "common.h"
 #include "internal.h"
 #include "topk_keys.h"
@@ -726,4 +728,53 @@ extern "C" int cpmcu_lm_head_argmax(const void* hidden, const void* w, int w_lay
     CPMCU_CHECK_ARG(workspace && workspace_bytes >= cpmcu_head_workspace_bytes(n, V),
                     "lm_head_argmax: workspace of %zu bytes needed, %zu given", cpmcu_head_workspace_bytes(n, V), workspace_bytes);
     return lm_head_argmax_on(hidden, w, w_layout, n, V, H, apply_scale, head_scale, logits, gt, (float*)workspace, resolve_stream(stream));
+}
+
+// ---- the same operator for callers that cannot allocate ----
+// The per-workgroup partials live in a file-scope device array instead of a caller-provided workspace.
+// Every GPU holds its own copy of the array at its own address; the address is looked up once per
+// device (with that device current) and kept.  On the host the array's name is only a handle for that
+// lookup -- kernels are always given the looked-up pointer.
+namespace {
+constexpr int kStaticHeadMaxRows = 128;
+constexpr size_t kStaticHeadScratchBytes = (size_t)2 * 1024 * kStaticHeadMaxRows * sizeof(float);  // both partial planes: 1 MiB
+static __device__ __align__(256) unsigned char scratch[kStaticHeadScratchBytes];
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices] = {};
+std::mutex g_scratch_mutex;
+
+int static_head_scratch(float** out) {
+    int dev = -1;
+    CPMCU_HIP(hipGetDevice(&dev));
+    CPMCU_CHECK_ARG(dev >= 0 && dev < kMaxDevices, "lm_head_argmax_static: device index %d outside [0, %d)", dev, kMaxDevices);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* ptr = nullptr;
+        CPMCU_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        g_scratch_ptr[dev] = ptr;
+    }
+    *out = (float*)g_scratch_ptr[dev];
+    return CPMCU_OK;
+}
+}  // namespace
+
+extern "C" size_t cpmcu_lm_head_argmax_static_scratch_bytes(void) { return kStaticHeadScratchBytes; }
+
+extern "C" int cpmcu_lm_head_argmax_static(const void* hidden, const void* w, int w_layout, int n, int V, int H, int apply_scale,
+                                           float head_scale, void* logits, int32_t* gt, void* stream) {
+    CPMCU_CHECK_ARG(hidden && w, "lm_head_argmax_static: null pointer argument");
+    CPMCU_CHECK_ARG(n >= 1 && n <= kStaticHeadMaxRows, "lm_head_argmax_static: n=%d outside [1, %d], the rows the built-in scratch holds",
+                    n, kStaticHeadMaxRows);
+    CPMCU_CHECK_ARG(V >= 1 && H >= 1, "lm_head_argmax_static: bad shape V=%d H=%d", V, H);
+    CPMCU_CHECK_ARG(logits || gt, "lm_head_argmax_static: both outputs are null");
+    static_assert(kStaticHeadScratchBytes >= (size_t)2 * 1024 * 128 * sizeof(float), "two planes of head_max_grid() x 128 floats");
+    CPMCU_CHECK_ARG(head_max_grid() * 128 * 2 * sizeof(float) <= kStaticHeadScratchBytes,
+                    "lm_head_argmax_static: the built-in scratch of %zu bytes is too small for %d workgroups", kStaticHeadScratchBytes,
+                    head_max_grid());
+    float* part = nullptr;
+    int rc = static_head_scratch(&part);
+    if (rc != CPMCU_OK) return rc;
+    // NULL selects HIP's null stream here: the library's own stream is created on first use, and this entry
+    // point creates nothing
+    return lm_head_argmax_on(hidden, w, w_layout, n, V, H, apply_scale, head_scale, logits, gt, part, (hipStream_t)stream);
 }

@@ -54,6 +54,8 @@ SIGNATURES = {
     "cpmcu_head_weight_tile": (c_int, [_P, _P, c_int, c_int, _P, _P]),
     "cpmcu_frspec_head_topk": (c_int, [_P, _P, c_int, _P, c_int, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, c_size_t, _P]),
     "cpmcu_lm_head_argmax": (c_int, [_P, _P, c_int, c_int, c_int, c_int, c_int, c_float, _P, _P, _P, c_size_t, _P]),
+    "cpmcu_lm_head_argmax_static_scratch_bytes": (c_size_t, []),
+    "cpmcu_lm_head_argmax_static": (c_int, [_P, _P, c_int, c_int, c_int, c_int, c_int, c_float, _P, _P, _P]),
     "cpmcu_log_softmax": (c_int, [_P, c_int, c_int, _P, _P]),
     "cpmcu_topk_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "cpmcu_topk": (c_int, [_P, c_int, c_int, c_int, _P, _P, _P, c_size_t, _P]),

@@ -310,6 +310,22 @@ int cpmcu_lm_head_argmax(const void* hidden, const void* w, int w_layout, int n,
                          float head_scale, void* logits, int32_t* gt, void* workspace,
                          size_t workspace_bytes, void* stream);
 
+/* cpmcu_lm_head_argmax for callers that cannot allocate device memory or bring a workspace: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference.  Same arguments and results as cpmcu_lm_head_argmax without the workspace: the per-workgroup
+ * arg-max partials live in a device array built into the library
+ * (cpmcu_lm_head_argmax_static_scratch_bytes() = 1 MiB, held by every GPU the library runs on until the
+ * process ends), which bounds the call to n <= 128 rows; more rows are rejected with
+ * CPMCU_ERR_INVALID_ARGUMENT.  The call allocates nothing and synchronises nothing; the first call on a
+ * device looks up that device's copy of the array (make it outside a capture).  stream = NULL is HIP's
+ * null stream here, not the library's own stream (which is created on first use).
+ * All calls on one GPU share the array, so calls that overlap on one GPU (different streams) race;
+ * calls on one stream are ordered and need no clearing in between: every launch rewrites the partials
+ * it reads. */
+size_t cpmcu_lm_head_argmax_static_scratch_bytes(void);
+int cpmcu_lm_head_argmax_static(const void* hidden, const void* w, int w_layout, int n, int V, int H, int apply_scale,
+                                float head_scale, void* logits, int32_t* gt, void* stream);
+
 /* log_softmax in place -- src/model/eagle.cuh:29-89.  x [n][dim] fp16;
  * row_stats [n][2] fp32 (max, ln sum) output, may be NULL. */
 int cpmcu_log_softmax(void* x, int n, int dim, float* row_stats, void* stream);
