@@ -9,10 +9,11 @@ interface for that path:
 * ``cpm.cu_amd.kvcache`` -- the paged KV-cache layout (K row-major pages, V transposed pages)
 * ``cpm.cu_amd.synth``   -- seeded synthetic trees / workloads of the benchmark configurations
 * ``cpm.cu_amd.driver``  -- the per-step loop of cpmcu/speculative/tree_drafter.py:222-250
+* ``cpm.cu_amd.model``   -- the library's process-global model (its own paged cache, heads and HIP graphs) from Python
 * ``cpm.cu_amd.C``       -- pybind11 module with the function names of the reference's src/entry.cu
 
 There is no CPU fallback: importing ``lib`` without the built shared library raises.
 """
 import torch  # noqa: F401,E402  -- first, so the shared library binds to the HIP runtime torch loads
 
-__all__ = ["lib", "ops", "kvcache", "synth", "driver"]
+__all__ = ["lib", "ops", "kvcache", "synth", "driver", "model"]

@@ -730,6 +730,21 @@ extern "C" int cpmcu_lm_head_argmax(const void* hidden, const void* w, int w_lay
     return lm_head_argmax_on(hidden, w, w_layout, n, V, H, apply_scale, head_scale, logits, gt, (float*)workspace, resolve_stream(stream));
 }
 
+// The GEMM alone: the arg-max stays in per-workgroup partials for cpmcu_verify_tail to finish.
+extern "C" int cpmcu_lm_head_partials(const void* hidden, const void* w, int w_layout, int n, int V, int H, int apply_scale,
+                                      float head_scale, void* logits, void* workspace, size_t workspace_bytes, int* num_partials,
+                                      int* partial_stride, void* stream) {
+    CPMCU_CHECK_ARG(hidden && w && num_partials && partial_stride, "lm_head_partials: null pointer argument");
+    CPMCU_CHECK_ARG(n >= 1 && n <= 128, "lm_head_partials: n=%d outside [1, 128]", n);
+    CPMCU_CHECK_ARG(V >= 1 && H >= 1, "lm_head_partials: bad shape V=%d H=%d", V, H);
+    CPMCU_CHECK_ARG(workspace && workspace_bytes >= cpmcu_head_workspace_bytes(n, V),
+                    "lm_head_partials: workspace of %zu bytes needed, %zu given", cpmcu_head_workspace_bytes(n, V), workspace_bytes);
+    float* part_a = (float*)workspace;
+    float* part_b = part_a + (size_t)head_max_grid() * 128;
+    return launch_head_gemm(hidden, w, w_layout, n, V, H, apply_scale, head_scale, kHeadModeArgmax, logits, part_a, part_b, num_partials,
+                            partial_stride, resolve_stream(stream));
+}
+
 // ---- the same operator for callers that cannot allocate ----
 // The per-workgroup partials live in a file-scope device array instead of a caller-provided workspace.
 // Every GPU holds its own copy of the array at its own address; the address is looked up once per

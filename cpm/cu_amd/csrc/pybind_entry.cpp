@@ -2,10 +2,12 @@
 // module (src/entry.cu:510-534) over the C-ABI of libcpmcu_amd.  Pointers are raw addresses
 // (tensor.data_ptr()) exactly as there.  No torch types, no HIP calls: this file is plain C++.
 #include <pybind11/pybind11.h>
+#include <pybind11/stl.h>
 
 #include <cstdint>
 #include <stdexcept>
 #include <string>
+#include <vector>
 
 #include "cpmcu_amd.h"
 
@@ -125,6 +127,21 @@ PYBIND11_MODULE(C, m) {
               check(cpmcu_draft_head(n, hidden, topk_val, topk_pos, topk_ids));
           },
           "FR-Spec draft head + log-softmax + top-k + id map-back");
+    m.def("verify_step",
+          [](int num_tokens, int padded_length, std::vector<std::uintptr_t> q, std::vector<std::uintptr_t> k_new,
+             std::vector<std::uintptr_t> v_new, std::vector<std::uintptr_t> attn_out, std::uintptr_t hidden, std::uintptr_t draft_ids,
+             std::uintptr_t position_ids, std::uintptr_t cache_length, std::uintptr_t kv_length, std::uintptr_t attn_mask,
+             std::uintptr_t tree_parent, std::uintptr_t block_table, std::uintptr_t gt_out, std::uintptr_t accepted_ids,
+             std::uintptr_t prev_hidden, std::uintptr_t next_position_ids, std::uintptr_t result, int flags, bool cuda_graph) {
+              if (q.size() != k_new.size() || q.size() != v_new.size() || q.size() != attn_out.size())
+                  throw py::value_error("verify_step: the per-layer address lists differ in length");
+              std::vector<uint64_t> a(q.begin(), q.end()), b(k_new.begin(), k_new.end()), c(v_new.begin(), v_new.end()),
+                  d(attn_out.begin(), attn_out.end());
+              check(cpmcu_verify_step((int)a.size(), num_tokens, padded_length, a.data(), b.data(), c.data(), d.data(), hidden, draft_ids,
+                                              position_ids, cache_length, kv_length, attn_mask, tree_parent, block_table, gt_out,
+                                              accepted_ids, prev_hidden, next_position_ids, result, flags, cuda_graph));
+          },
+          "One verify step of the path (attention of every layer, target head, acceptance, compaction), optionally as a replayed graph");
     m.def("synchronize", []() { check(cpmcu_synchronize()); });
     m.def("shutdown", []() { check(cpmcu_shutdown()); });
 }

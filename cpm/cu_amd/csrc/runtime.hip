@@ -2,9 +2,12 @@
 // the reference's pybind module (src/entry.cu:98-534) for the verify/draft path: one process-global
 // model that owns the lm_head, the FR-Spec sub-matrix, the paged KV pools of every layer, one page
 // table and scratch.
+#include <cmath>
 #include <cstdlib>
 #include <cstring>
+#include <initializer_list>
 #include <map>
+#include <utility>
 #include <string>
 #include <vector>
 
@@ -86,10 +89,19 @@ struct Model {
     f16* draft_logits = nullptr;  // [16][frspec_vocab]
     float* row_stats = nullptr;   // [16][2]
     int32_t* d_best = nullptr;
-    int32_t* h_best = nullptr;  // pinned
+    int32_t* d_ids = nullptr;     // [64] accepted ids of the last verify
+    int32_t* h_result = nullptr;  // pinned, device-visible: (a, ids) of the last verify
     uint64_t* chain_mask = nullptr;
     bool perf = false;
     std::map<std::string, PerfEntry> perf_log;
+    // captured verify steps, keyed like the reference's decode graph (src/entry.cu:475-492) on
+    // (padded_length, num_tokens); the signature covers every address baked into the graph
+    struct StepGraph {
+        hipGraph_t graph = nullptr;
+        hipGraphExec_t exec = nullptr;
+        uint64_t signature = 0;
+    };
+    std::map<std::pair<int, int>, std::vector<StepGraph>> step_graphs;
 };
 
 Model* g_model = nullptr;
@@ -264,7 +276,8 @@ extern "C" int cpmcu_init_storage(int* max_context) {
         if ((rc = alloc((void**)&m.row_stats, 16 * 2 * sizeof(float)))) return rc;
     }
     if ((rc = alloc((void**)&m.d_best, 2 * sizeof(int32_t)))) return rc;
-    CPMCU_HIP(hipHostMalloc((void**)&m.h_best, 2 * sizeof(int32_t), hipHostMallocDefault));
+    if ((rc = alloc((void**)&m.d_ids, 64 * sizeof(int32_t)))) return rc;
+    CPMCU_HIP(hipHostMalloc((void**)&m.h_result, (1 + 64) * sizeof(int32_t), hipHostMallocDefault));
     if ((rc = alloc((void**)&m.chain_mask, 64 * sizeof(uint64_t)))) return rc;
     {
         uint64_t rows[64];
@@ -483,18 +496,147 @@ extern "C" int cpmcu_verify_and_fix(int num_tokens, uint64_t pred, uint64_t gt, 
     CPMCU_CHECK_ARG(pred && gt && position_ids && cache_length && attn_mask && tree_parent, "verify_and_fix: null pointer argument");
     hipStream_t st = resolve_stream(nullptr);
     PerfScope perf("VERIFY_AND_FIX", st);
-    rc = cpmcu_tree_accept(num_tokens, (int32_t*)pred, (const int32_t*)gt, (const int32_t*)position_ids,
-                           (const int32_t*)cache_length, (const uint64_t*)attn_mask, 1, (const int32_t*)tree_parent,
-                           m.d_best, st);
+    // One launch accepts and compacts every cache (each workgroup redoes the acceptance, so nothing waits for
+    // the accept length); it writes (a, node) straight into pinned host memory, so the single synchronisation
+    // of the step (src/model/minicpm4/minicpm4_eagle.cuh:400-401) moves to the end and needs no copy.  The
+    // accepted ids replace the draft ids in pred behind it (pred is read by every workgroup of the first launch).
+    rc = cpmcu_verify_tail(m.d_k_pools, m.d_v_pools, m.layers, m.block_table, m.kv_heads, num_tokens, (const int32_t*)pred,
+                           (const int32_t*)gt, nullptr, 0, 0, (const int32_t*)position_ids, (const int32_t*)cache_length,
+                           (const uint64_t*)attn_mask, 1, (const int32_t*)tree_parent, nullptr, 0, nullptr, nullptr, m.d_best, nullptr,
+                           m.d_ids, nullptr, m.h_result, st);
     if (rc) return rc;
-    // compaction reads the accept length on the device, so the single D2H copy + sync of the step
-    // (src/model/minicpm4/minicpm4_eagle.cuh:400-401) moves to the end
-    rc = cpmcu_kv_compact(m.d_k_pools, m.d_v_pools, m.layers, m.block_table, m.kv_heads, (int32_t*)pred,
-                          (const int32_t*)gt, (const int32_t*)cache_length, m.d_best, num_tokens, st);
+    rc = cpmcu_verify_tail_inplace(m.d_best, m.d_ids, num_tokens, (int32_t*)pred, nullptr, nullptr, nullptr, 0, st);
     if (rc) return rc;
-    CPMCU_HIP(hipMemcpyAsync(m.h_best, m.d_best, 2 * sizeof(int32_t), hipMemcpyDeviceToHost, st));
     CPMCU_HIP(hipStreamSynchronize(st));
-    if (accept_length) *accept_length = m.h_best[0];
+    if (accept_length) *accept_length = m.h_result[0];
+    return CPMCU_OK;
+}
+
+namespace {
+
+struct StepArgs {
+    int T, padded_length;
+    const uint64_t *q, *k_new, *v_new, *attn_out;  // host arrays [layers] of device addresses
+    uint64_t hidden, draft_ids, position_ids, cache_length, kv_length, attn_mask, tree_parent, block_table;
+    uint64_t gt_out, accepted_ids, prev_hidden, next_position_ids, result;
+    int flags;
+};
+
+// Every launch of one verify step, in order, on `st`: per layer the KV append + tree attention on the model's
+// paged cache, the target head (arg-max left as partials), the one-launch tail, and with
+// CPMCU_COMMIT_ADVANCE_LENGTH the single-workgroup launch that advances the lengths and positions.
+int enqueue_verify_step(Model& m, const StepArgs& a, hipStream_t st) {
+    const int32_t* table = a.block_table ? (const int32_t*)a.block_table : m.block_table;
+    const float scale = 1.f / sqrtf((float)kHeadDim);
+    for (int l = 0; l < m.layers; ++l) {
+        int rc = cpmcu_tree_attention((const void*)a.q[l], m.k_pools[l], m.v_pools[l], table, (const int32_t*)a.kv_length, a.padded_length,
+                                      (const void*)a.k_new[l], (const void*)a.v_new[l], (const uint64_t*)a.attn_mask, 1, 0, a.T, m.q_heads,
+                                      m.kv_heads, scale, (void*)a.attn_out[l], m.attn_ws, m.attn_ws_bytes, 0, st);
+        if (rc) return rc;
+    }
+    int num_partials = 0, stride = 0;
+    int rc = cpmcu_lm_head_partials((const void*)a.hidden, m.lm_head, CPMCU_W_TILED, a.T, m.vocab, m.hidden, 1, m.scale_lmhead, nullptr,
+                                    m.head_ws, m.head_ws_bytes, &num_partials, &stride, st);
+    if (rc) return rc;
+    rc = cpmcu_verify_tail(m.d_k_pools, m.d_v_pools, m.layers, table, m.kv_heads, a.T, (const int32_t*)a.draft_ids, nullptr, m.head_ws,
+                           num_partials, stride, (const int32_t*)a.position_ids, (const int32_t*)a.cache_length,
+                           (const uint64_t*)a.attn_mask, 1, (const int32_t*)a.tree_parent, a.prev_hidden ? (const void*)a.hidden : nullptr,
+                           m.hidden, (void*)a.prev_hidden, (int32_t*)a.gt_out, m.d_best, nullptr, (int32_t*)a.accepted_ids,
+                           (int32_t*)a.next_position_ids, (int32_t*)a.result, st);
+    if (rc) return rc;
+    if (a.flags & CPMCU_COMMIT_ADVANCE_LENGTH)
+        rc = cpmcu_verify_tail_inplace(m.d_best, (const int32_t*)a.accepted_ids, a.T, nullptr, (int32_t*)a.cache_length,
+                                       (int32_t*)a.kv_length, (int32_t*)a.position_ids, CPMCU_COMMIT_ADVANCE_LENGTH, st);
+    return rc;
+}
+
+uint64_t step_signature(const Model& m, const StepArgs& a) {
+    uint64_t h = 1469598103934665603ull;
+    auto mix = [&](uint64_t v) {
+        for (int b = 0; b < 8; ++b) {
+            h ^= (v >> (8 * b)) & 0xff;
+            h *= 1099511628211ull;
+        }
+    };
+    for (int l = 0; l < m.layers; ++l) {
+        mix(a.q[l]);
+        mix(a.k_new[l]);
+        mix(a.v_new[l]);
+        mix(a.attn_out[l]);
+    }
+    for (uint64_t v : {a.hidden, a.draft_ids, a.position_ids, a.cache_length, a.kv_length, a.attn_mask, a.tree_parent, a.block_table,
+                       a.gt_out, a.accepted_ids, a.prev_hidden, a.next_position_ids, a.result, (uint64_t)a.flags})
+        mix(v);
+    return h;
+}
+
+void destroy_step_graphs(Model& m) {
+    for (auto& kv : m.step_graphs)
+        for (auto& g : kv.second) {
+            if (g.exec) (void)hipGraphExecDestroy(g.exec);
+            if (g.graph) (void)hipGraphDestroy(g.graph);
+        }
+    m.step_graphs.clear();
+}
+
+}  // namespace
+
+extern "C" int cpmcu_verify_step(int num_layers, int num_tokens, int padded_length, const uint64_t* q, const uint64_t* k_new, const uint64_t* v_new,
+                                 const uint64_t* attn_out, uint64_t hidden, uint64_t draft_ids, uint64_t position_ids,
+                                 uint64_t cache_length, uint64_t kv_length, uint64_t attn_mask, uint64_t tree_parent,
+                                 uint64_t block_table, uint64_t gt_out, uint64_t accepted_ids, uint64_t prev_hidden,
+                                 uint64_t next_position_ids, uint64_t result, int flags, int cuda_graph) {
+    int rc = require_model(true);
+    if (rc) return rc;
+    Model& m = *g_model;
+    if (!m.drafter) {
+        set_error("verify is not supported: no drafter configured");  // src/model/model.cuh:172-173
+        return CPMCU_ERR_RUNTIME;
+    }
+    CPMCU_CHECK_ARG(m.lm_head_loaded, "verify_step: lm_head.weight has not been loaded");
+    CPMCU_CHECK_ARG(num_layers == m.layers, "verify_step: %d per-layer addresses given, the model has %d layers", num_layers, m.layers);
+    CPMCU_CHECK_ARG(num_tokens >= 1 && num_tokens <= 64, "verify_step: num_tokens=%d outside [1, 64]", num_tokens);
+    CPMCU_CHECK_ARG(padded_length >= num_tokens && padded_length <= m.num_pages * kPage, "verify_step: padded_length=%d outside [%d, %d]",
+                    padded_length, num_tokens, m.num_pages * kPage);
+    CPMCU_CHECK_ARG(q && k_new && v_new && attn_out, "verify_step: null per-layer address array");
+    for (int l = 0; l < m.layers; ++l)
+        CPMCU_CHECK_ARG(q[l] && k_new[l] && v_new[l] && attn_out[l], "verify_step: null address for layer %d", l);
+    CPMCU_CHECK_ARG(hidden && draft_ids && position_ids && cache_length && kv_length && attn_mask && tree_parent && accepted_ids,
+                    "verify_step: null pointer argument");
+    CPMCU_CHECK_ARG((flags & ~CPMCU_COMMIT_ADVANCE_LENGTH) == 0, "verify_step: unknown flags 0x%x", flags);
+    const StepArgs a{num_tokens, padded_length, q, k_new, v_new, attn_out, hidden, draft_ids, position_ids, cache_length, kv_length,
+                     attn_mask, tree_parent, block_table, gt_out, accepted_ids, prev_hidden, next_position_ids, result, flags};
+    hipStream_t st = resolve_stream(nullptr);
+    if (!cuda_graph) {
+        PerfScope perf("VERIFY_STEP", st);
+        return enqueue_verify_step(m, a, st);
+    }
+    // Graph path, as decode(..., cuda_graph = true) of the reference: captured once per (padded_length, num_tokens)
+    // -- and per set of addresses, which a graph bakes in -- and replayed afterwards.  Every length the kernels
+    // need is read from device memory, so the same graph serves every step of that padded length.
+    const uint64_t sig = step_signature(m, a);
+    auto& bucket = m.step_graphs[{padded_length, num_tokens}];
+    for (auto& g : bucket)
+        if (g.signature == sig) {
+            CPMCU_HIP(hipGraphLaunch(g.exec, st));
+            return CPMCU_OK;
+        }
+    Model::StepGraph g;
+    g.signature = sig;
+    CPMCU_HIP(hipStreamBeginCapture(st, hipStreamCaptureModeRelaxed));
+    rc = enqueue_verify_step(m, a, st);
+    const hipError_t e = hipStreamEndCapture(st, &g.graph);
+    if (rc) {
+        if (g.graph) (void)hipGraphDestroy(g.graph);
+        return rc;
+    }
+    if (e != hipSuccess) {
+        set_error("verify_step: stream capture failed: %s", hipGetErrorString(e));
+        return CPMCU_ERR_HIP;
+    }
+    CPMCU_HIP(hipGraphInstantiate(&g.exec, g.graph, nullptr, nullptr, 0));
+    bucket.push_back(g);
+    CPMCU_HIP(hipGraphLaunch(g.exec, st));
     return CPMCU_OK;
 }
 
@@ -535,6 +677,7 @@ extern "C" int cpmcu_shutdown(void) {
     if (!g_model) return CPMCU_OK;
     Model& m = *g_model;
     if (g_stream) (void)hipStreamSynchronize(g_stream);
+    destroy_step_graphs(m);
     if (m.fr_head && m.fr_head != m.lm_head) (void)hipFree(m.fr_head);
     (void)hipFree(m.lm_head);
     (void)hipFree(m.token_id_remap);
@@ -548,8 +691,9 @@ extern "C" int cpmcu_shutdown(void) {
     (void)hipFree(m.draft_logits);
     (void)hipFree(m.row_stats);
     (void)hipFree(m.d_best);
+    (void)hipFree(m.d_ids);
     (void)hipFree(m.chain_mask);
-    if (m.h_best) (void)hipHostFree(m.h_best);
+    if (m.h_result) (void)hipHostFree(m.h_result);
     delete g_model;
     g_model = nullptr;
     return CPMCU_OK;

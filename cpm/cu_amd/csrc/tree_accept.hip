@@ -5,6 +5,7 @@
 // 2-byte moves for the transposed V pages.  The accept length never visits the host between the
 // three kernels: compaction reads it from device memory.
 #include "common.h"
+#include "internal.h"
 #include "topk_keys.h"
 
 namespace cpmcu {
@@ -48,7 +49,9 @@ __global__ __launch_bounds__(128) void tree_accept_kernel(int T, int W, int32_t*
         best[1] = p;
     }
     // :42-45  scatter the accepted path (node indices by depth) into pred
-    if (i < T && ((mask[(size_t)p * W + (i >> 6)] >> (i & 63)) & 1ull)) pred[pos[i] - P] = i;
+    // (a node whose position does not lie in [P, P + T) -- positions that were not advanced with the prefix
+    // length -- scatters nothing instead of writing outside pred)
+    if (i < T && ((mask[(size_t)p * W + (i >> 6)] >> (i & 63)) & 1ull) && (unsigned)(pos[i] - P) < (unsigned)T) pred[pos[i] - P] = i;
 }
 
 struct CompactParams {
@@ -169,6 +172,219 @@ __global__ __launch_bounds__(128) void accepted_ids_kernel(int32_t* pred, const 
     }
 }
 
+// ---- the whole tail of verify() in one launch ----
+// Arg-max finish (when the target head hands over its per-workgroup partials instead of gt), greedy
+// acceptance (verify_kernel, src/model/tree_drafter.cuh:5-46), compaction of every cache
+// (fix_kvcache_kernel_1/2, :48-77), the gather of the accepted hidden rows (remap_hidden,
+// src/model/eagle.cuh:108-115) and the accepted ids (:74-76) with the host-side bookkeeping of
+// cpmcu/speculative/tree_drafter.py:222,243-249.  The acceptance is a few hundred bytes of integer work,
+// so EVERY workgroup redoes it (and the arg-max finish in front of it) from the same inputs and then does
+// its own share: one cache stream, one hidden row, or -- the last workgroup -- the outputs.  Nothing is
+// read that another workgroup of the launch writes: the draft ids come in through `draft` and the path /
+// accepted ids go out through separate arrays, and no workgroup writes the lengths.
+struct TailParams {
+    int T, W;
+    const int32_t* draft;         // draft token ids (pred on entry of verify)
+    const int32_t* gt;            // target arg-max per node, or null: taken from the head's partials
+    const float* part_a;          // [num_partials][partial_stride] best value
+    const float* part_b;          // [num_partials][partial_stride] best index (int bits)
+    int num_partials, partial_stride;
+    const int32_t* pos;
+    const int32_t* cache_length;  // P (read only)
+    const uint64_t* mask;
+    const int32_t* parent;
+    // compaction
+    void* const* k_pools;
+    void* const* v_pools;
+    const int32_t* block_table;
+    int Hkv;
+    int num_cache_blocks;         // num_layers * 2 * Hkv workgroups
+    // accepted hidden rows: num_hidden_blocks workgroups behind the cache streams
+    const f16x8* hidden;
+    f16x8* prev_hidden;
+    int hidden_pieces, num_hidden_blocks;
+    // outputs, written by the last workgroup (any may be null)
+    int32_t* gt_out;              // [T]
+    int32_t* best;                // (a, winning node)
+    int32_t* path;                // [T]: node indices of the accepted path by depth (first a entries)
+    int32_t* ids;                 // [T]: accepted token ids (first a entries)
+    int32_t* next_position_ids;   // [T]: P + d
+    int32_t* result;              // [1 + T]: (a, ids)
+};
+
+__device__ inline uint64_t argmax_key(float value, uint32_t index) {
+    const uint32_t bits = (uint32_t)__float_as_int(value + 0.f);  // -0 -> +0: they compare equal
+    const uint32_t image = bits ^ ((bits >> 31) ? 0xFFFFFFFFu : 0x80000000u);
+    return ((uint64_t)image << 32) | (0xFFFFFFFFu - index);
+}
+
+constexpr int kTailThreads = 256;
+
+__global__ __launch_bounds__(kTailThreads) void verify_tail_kernel(TailParams p) {
+    __shared__ int32_t s_gt[kMaxTree];
+    __shared__ int32_t s_path[kMaxTree];
+    __shared__ uint64_t s_key[kTailThreads];
+    __shared__ uint64_t s_correct[2];
+    __shared__ uint32_t s_best[2];
+    const int tid = threadIdx.x;
+    const int T = p.T, W = p.W;
+
+    // ---- target arg-max per node: given, or the finish of the head's per-workgroup partials (largest value,
+    // lowest index among equals: the same 64-bit keys as the head's own finish kernel) ----
+    if (p.gt != nullptr) {
+        if (tid < T) s_gt[tid] = p.gt[tid];
+    } else {
+        const int rows = p.partial_stride;        // 16 .. 128, a power of two
+        const int row = tid & (rows - 1);
+        const int clanes = kTailThreads / rows;   // partial lanes per row
+        uint64_t bestk = 0;
+        if (row < T) {
+            for (int c = tid / rows; c < p.num_partials; c += clanes) {
+                const float a = p.part_a[(size_t)c * rows + row];
+                const uint32_t b = (uint32_t)__float_as_int(p.part_b[(size_t)c * rows + row]);
+                const uint64_t k = argmax_key(a, b);
+                bestk = k > bestk ? k : bestk;
+            }
+        }
+        s_key[tid] = bestk;
+        __syncthreads();
+        if (tid < rows && tid < T) {
+            uint64_t k = s_key[tid];
+            for (int l = 1; l < clanes; ++l) {
+                const uint64_t o = s_key[l * rows + tid];
+                k = o > k ? o : k;
+            }
+            s_gt[tid] = (int32_t)(0xFFFFFFFFu - (uint32_t)k);
+        }
+    }
+    __syncthreads();
+
+    // ---- acceptance (as tree_accept_kernel above, on 128 of the threads) ----
+    const int i = tid;
+    const bool ok = (i == 0) || (i < T && p.draft[i] == s_gt[p.parent[i]]);
+    const uint64_t ballot = __ballot(ok);
+    if (i < 128 && (i & 63) == 0) s_correct[i >> 6] = ballot;
+    __syncthreads();
+    const int P = p.cache_length[0];
+    bool full = i < T;
+    if (full) {
+        for (int w = 0; w < W; ++w) {
+            const uint64_t mw = p.mask[(size_t)i * W + w];
+            if ((s_correct[w] & mw) != mw) full = false;
+        }
+    }
+    const uint32_t key = full ? ((uint32_t)(p.pos[i] - P + 1) << 8) | (255u - (__brev((uint32_t)i) >> 24)) : (1u << 8) | 255u;
+    const uint32_t wkey = wave_reduce_b32(key, [](uint32_t a, uint32_t b) { return a > b ? a : b; });
+    if (i < 128 && (i & 63) == 0) s_best[i >> 6] = wkey;
+    __syncthreads();
+    const uint32_t bkey = s_best[0] > s_best[1] ? s_best[0] : s_best[1];
+    const int win = (int)(__brev(255u - (bkey & 255u)) >> 24);
+    int a = (int)(bkey >> 8);
+    a = a < T ? a : T;
+    if (tid < kMaxTree) s_path[tid] = tid < T ? tid : 0;  // (defined even where stale positions scatter nothing)
+    __syncthreads();
+    if (i < T && ((p.mask[(size_t)win * W + (i >> 6)] >> (i & 63)) & 1ull) && (unsigned)(p.pos[i] - P) < (unsigned)T) s_path[p.pos[i] - P] = i;
+    __syncthreads();
+
+    const int blk = blockIdx.x;
+    if (blk < p.num_cache_blocks) {
+        // ---- compaction of one (layer, K|V, kv head) stream: sources of a batch are read before any of its
+        // destinations is written, batches go in depth order and path[d] >= d, so no staging buffer ----
+        const int g = blk % p.Hkv;
+        const int kv = (blk / p.Hkv) & 1;
+        const int layer = blk / (2 * p.Hkv);
+        if (kv == 0) {
+            f16* pool = (f16*)p.k_pools[layer];
+            const int rr = tid >> 4, ch = tid & 15;  // 16 rows x 16 pieces of 16 bytes
+            for (int d0 = 0; d0 < a; d0 += 16) {
+                const int d = d0 + rr;
+                f16x8 x;
+                const bool act = d < a && s_path[d] != d;  // a row that stays where it is moves nothing
+                if (act) {
+                    const int ts = P + s_path[d];
+                    const int pg = p.block_table[ts / kPage];
+                    x = *reinterpret_cast<const f16x8*>(pool + (((size_t)pg * p.Hkv + g) * kPage + ts % kPage) * kHeadDim + ch * 8);
+                }
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();
+                if (act) {
+                    const int td = P + d;
+                    const int pg = p.block_table[td / kPage];
+                    *reinterpret_cast<f16x8*>(pool + (((size_t)pg * p.Hkv + g) * kPage + td % kPage) * kHeadDim + ch * 8) = x;
+                }
+            }
+        } else {
+            f16* pool = (f16*)p.v_pools[layer];
+            const int rr = tid >> 7, dd = tid & 127;  // 2 tokens x 128 dims
+            for (int d0 = 0; d0 < a; d0 += 2) {
+                const int d = d0 + rr;
+                f16 x = (f16)0.f;
+                const bool act = d < a && s_path[d] != d;
+                if (act) {
+                    const int ts = P + s_path[d];
+                    const int pg = p.block_table[ts / kPage];
+                    x = pool[(((size_t)pg * p.Hkv + g) * kHeadDim + dd) * kPage + v_slot16(ts % kPage)];
+                }
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();
+                if (act) {
+                    const int td = P + d;
+                    const int pg = p.block_table[td / kPage];
+                    pool[(((size_t)pg * p.Hkv + g) * kHeadDim + dd) * kPage + v_slot16(td % kPage)] = x;
+                }
+            }
+        }
+        return;
+    }
+    if (blk < p.num_cache_blocks + p.num_hidden_blocks) {
+        // remap_hidden (src/model/eagle.cuh:108-115, scale 1): prev_hidden[d] = hidden[path[d]]
+        const int d = blk - p.num_cache_blocks;
+        if (d >= a) return;
+        const f16x8* src = p.hidden + (size_t)s_path[d] * p.hidden_pieces;
+        f16x8* dst = p.prev_hidden + (size_t)d * p.hidden_pieces;
+        for (int x = tid; x < p.hidden_pieces; x += kTailThreads) dst[x] = src[x];
+        return;
+    }
+    // ---- the last workgroup: every integer result of the step ----
+    if (tid < T) {
+        if (p.gt_out) p.gt_out[tid] = s_gt[tid];
+        if (tid < a) {
+            const int node = s_path[tid];
+            const int id = s_gt[node];
+            if (p.path) p.path[tid] = node;
+            if (p.ids) p.ids[tid] = id;
+            if (p.next_position_ids) p.next_position_ids[tid] = P + tid;
+            if (p.result) p.result[1 + tid] = id;
+        }
+    }
+    if (tid == 0) {
+        if (p.best) {
+            p.best[0] = a;
+            p.best[1] = win;
+        }
+        if (p.result) p.result[0] = a;
+    }
+}
+
+// What must not happen inside the launch above because other workgroups still read the old values: the
+// in-place updates.  pred[0..a) <- accepted ids (the reference's verify leaves them there,
+// src/model/tree_drafter.cuh:74-76), cache_length / kv_len += a, pred[0] <- last accepted id.
+__global__ __launch_bounds__(128) void verify_tail_inplace_kernel(const int32_t* best, const int32_t* ids, int T, int32_t* pred,
+                                                                  int32_t* cache_length, int32_t* kv_len, int32_t* position_ids, int flags) {
+    int a = best[0];
+    a = a < T ? a : T;
+    const int d = threadIdx.x;
+    if (pred && d < a && !(flags & CPMCU_COMMIT_NEXT_ROOT)) pred[d] = ids[d];
+    if (position_ids && (flags & CPMCU_COMMIT_ADVANCE_LENGTH) && d < T) position_ids[d] += a;  // same tree shape, prefix a longer
+    if (d == 0) {
+        if (flags & CPMCU_COMMIT_ADVANCE_LENGTH) {
+            cache_length[0] += a;
+            if (kv_len) kv_len[0] += a;
+        }
+        if (pred && (flags & CPMCU_COMMIT_NEXT_ROOT)) pred[0] = ids[a - 1];
+    }
+}
+
 // copy_to_kvcache, src/model/attn.cuh:14-21: token t of the T new rows goes to position *kv_len - T + t.
 __global__ __launch_bounds__(256) void kv_append_kernel(f16* k_pool, f16* v_pool, const int32_t* block_table,
                                                         const f16* k_new, const f16* v_new,
@@ -244,6 +460,71 @@ extern "C" int cpmcu_accept_commit(void* const* k_pools, void* const* v_pools, i
     CPMCU_LAUNCH_CHECK();
     hipLaunchKernelGGL(accepted_ids_kernel, dim3(1), dim3(128), 0, st, pred, gt, best, max_accept, cache_length,
                        kv_len, next_position_ids, result, flags);
+    CPMCU_LAUNCH_CHECK();
+    return CPMCU_OK;
+}
+
+extern "C" int cpmcu_verify_tail(void* const* k_pools, void* const* v_pools, int num_layers, const int32_t* block_table, int Hkv,
+                                 int T, const int32_t* draft_ids, const int32_t* gt, const void* head_partials, int num_partials,
+                                 int partial_stride, const int32_t* position_ids, const int32_t* cache_length,
+                                 const uint64_t* attn_mask, int mask_words, const int32_t* tree_parent, const void* hidden,
+                                 int hidden_dim, void* prev_hidden, int32_t* gt_out, int32_t* best, int32_t* path,
+                                 int32_t* accepted_ids, int32_t* next_position_ids, int32_t* result, void* stream) {
+    CPMCU_CHECK_ARG(k_pools && v_pools && block_table && draft_ids && position_ids && cache_length && attn_mask && tree_parent,
+                    "verify_tail: null pointer argument");
+    CPMCU_CHECK_ARG(num_layers >= 1 && Hkv >= 1, "verify_tail: num_layers=%d Hkv=%d", num_layers, Hkv);
+    CPMCU_CHECK_ARG(T >= 1 && T <= kMaxTree, "verify_tail: tree size %d outside [1, %d]", T, kMaxTree);
+    CPMCU_CHECK_ARG(mask_words >= 1 && mask_words <= 2 && mask_words * 64 >= T, "verify_tail: mask_words=%d does not cover T=%d", mask_words, T);
+    CPMCU_CHECK_ARG((gt != nullptr) != (head_partials != nullptr), "verify_tail: give either gt or the head's partials");
+    if (head_partials) {
+        const bool pow2 = partial_stride >= 16 && partial_stride <= 128 && (partial_stride & (partial_stride - 1)) == 0;
+        CPMCU_CHECK_ARG(pow2 && partial_stride >= T && num_partials >= 1 && num_partials <= head_max_grid(),
+                        "verify_tail: %d partials of stride %d do not describe a head launch on %d rows", num_partials, partial_stride, T);
+    }
+    CPMCU_CHECK_ARG((hidden == nullptr) == (prev_hidden == nullptr), "verify_tail: hidden and prev_hidden go together");
+    CPMCU_CHECK_ARG(!hidden || (hidden_dim >= 8 && hidden_dim % 8 == 0), "verify_tail: hidden_dim=%d must be a positive multiple of 8", hidden_dim);
+    TailParams p;
+    p.T = T;
+    p.W = mask_words;
+    p.draft = draft_ids;
+    p.gt = gt;
+    p.part_a = (const float*)head_partials;
+    p.part_b = head_partials ? (const float*)head_partials + (size_t)head_max_grid() * 128 : nullptr;
+    p.num_partials = num_partials;
+    p.partial_stride = partial_stride;
+    p.pos = position_ids;
+    p.cache_length = cache_length;
+    p.mask = attn_mask;
+    p.parent = tree_parent;
+    p.k_pools = k_pools;
+    p.v_pools = v_pools;
+    p.block_table = block_table;
+    p.Hkv = Hkv;
+    p.num_cache_blocks = num_layers * 2 * Hkv;
+    p.hidden = (const f16x8*)hidden;
+    p.prev_hidden = (f16x8*)prev_hidden;
+    p.hidden_pieces = hidden ? hidden_dim / 8 : 0;
+    p.num_hidden_blocks = hidden ? T : 0;
+    p.gt_out = gt_out;
+    p.best = best;
+    p.path = path;
+    p.ids = accepted_ids;
+    p.next_position_ids = next_position_ids;
+    p.result = result;
+    hipLaunchKernelGGL(verify_tail_kernel, dim3(p.num_cache_blocks + p.num_hidden_blocks + 1), dim3(kTailThreads), 0, resolve_stream(stream), p);
+    CPMCU_LAUNCH_CHECK();
+    return CPMCU_OK;
+}
+
+extern "C" int cpmcu_verify_tail_inplace(const int32_t* best, const int32_t* accepted_ids, int T, int32_t* pred, int32_t* cache_length,
+                                         int32_t* kv_len, int32_t* position_ids, int flags, void* stream) {
+    CPMCU_CHECK_ARG(best && accepted_ids, "verify_tail_inplace: null pointer argument");
+    CPMCU_CHECK_ARG(T >= 1 && T <= kMaxTree, "verify_tail_inplace: tree size %d outside [1, %d]", T, kMaxTree);
+    CPMCU_CHECK_ARG((flags & ~(CPMCU_COMMIT_ADVANCE_LENGTH | CPMCU_COMMIT_NEXT_ROOT)) == 0, "verify_tail_inplace: unknown flags 0x%x", flags);
+    CPMCU_CHECK_ARG(!(flags & CPMCU_COMMIT_ADVANCE_LENGTH) || cache_length, "verify_tail_inplace: the length advance needs cache_length");
+    CPMCU_CHECK_ARG(!(flags & CPMCU_COMMIT_NEXT_ROOT) || pred, "verify_tail_inplace: the next root goes into pred");
+    hipLaunchKernelGGL(verify_tail_inplace_kernel, dim3(1), dim3(128), 0, resolve_stream(stream), best, accepted_ids, T, pred, cache_length,
+                       kv_len, position_ids, flags);
     CPMCU_LAUNCH_CHECK();
     return CPMCU_OK;
 }

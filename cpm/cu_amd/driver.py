@@ -25,7 +25,12 @@ from . import ops
 
 
 class VerifyStep:
-    def __init__(self, cache, lm_head, tree_mask, tree_parent, tree_positions, prefix_len, head_scale=None, commit=False):
+    """fused=True (default): the head leaves its arg-max as per-workgroup partials and ONE launch finishes it,
+    accepts, compacts every cache and writes the ids (``ops.verify_tail``); the draft ids are read where the
+    caller keeps them.  fused=False keeps the operator-by-operator tail (arg-max finish, ``tree_accept``,
+    ``kv_compact`` / ``accept_commit``), which needs the draft ids copied into ``pred`` first."""
+
+    def __init__(self, cache, lm_head, tree_mask, tree_parent, tree_positions, prefix_len, head_scale=None, commit=False, fused=True):
         dev = cache.device
         self.cache = cache
         self.w = lm_head
@@ -43,6 +48,8 @@ class VerifyStep:
         self.pred = torch.empty(self.T, dtype=torch.int32, device=dev)
         self.attn_out = None
         self.commit = bool(commit)
+        self.fused = bool(fused)
+        self.path = torch.zeros(self.T, dtype=torch.int32, device=dev)
         if self.commit:
             self.prev_hidden = None  # allocated at the first step, when the hidden size is known
             self.next_positions = torch.zeros(self.T, dtype=torch.int32, device=dev)
@@ -59,6 +66,20 @@ class VerifyStep:
                                    k_new=k_new_layers[l], v_new=v_new_layers[l])
             if attn_out is None:
                 self.attn_out = o
+        if self.fused:
+            parts = ops.lm_head_partials(hidden, self.w, head_scale=self.head_scale)
+            if self.commit and self.prev_hidden is None:
+                self.prev_hidden = torch.zeros((self.T, hidden.shape[1]), dtype=torch.float16, device=hidden.device)
+            ops.verify_tail(c, draft_ids, parts, self.pos, self.cache_length, self.mask, self.parent,
+                            hidden=hidden if self.commit else None, prev_hidden=self.prev_hidden if self.commit else None,
+                            gt_out=self.gt, best=self.best, path=self.path, accepted_ids=self.pred,
+                            next_position_ids=self.next_positions if self.commit else None,
+                            result=self.packed if self.commit else None)
+            if self.commit:
+                # lengths and tree positions advance on the device: the next step of the same tree shape needs no host write
+                ops.verify_tail_inplace(self.best, self.pred, cache_length=self.cache_length, kv_len=self.kv_len,
+                                        position_ids=self.pos, advance_length=True)
+            return
         ops.lm_head_argmax(hidden, self.w, head_scale=self.head_scale, gt=self.gt)
         self.pred.copy_(draft_ids)
         ops.tree_accept(self.pred, self.gt, self.pos, self.cache_length, self.mask, self.parent, best=self.best)

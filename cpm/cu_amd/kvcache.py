@@ -40,6 +40,20 @@ class PagedKVCache:
         self.k_ptrs = torch.tensor([t.data_ptr() for t in self.k], dtype=torch.int64, device=self.device)
         self.v_ptrs = torch.tensor([t.data_ptr() for t in self.v], dtype=torch.int64, device=self.device)
 
+    @classmethod
+    def from_pools(cls, k_pools, v_pools, block_table):
+        """A cache over pools that already exist (tensor views [pages, Hkv, 256, 128] / [pages, Hkv, 128, 256])."""
+        self = cls.__new__(cls)
+        self.num_layers = len(k_pools)
+        self.Hkv = k_pools[0].shape[1]
+        self.num_pages = k_pools[0].shape[0]
+        self.device = k_pools[0].device
+        self.k, self.v = list(k_pools), list(v_pools)
+        self.block_table = block_table
+        self.k_ptrs = torch.tensor([t.data_ptr() for t in self.k], dtype=torch.int64, device=self.device)
+        self.v_ptrs = torch.tensor([t.data_ptr() for t in self.v], dtype=torch.int64, device=self.device)
+        return self
+
     @property
     def capacity(self):
         return self.block_table.numel() * PAGE

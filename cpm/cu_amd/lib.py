@@ -32,6 +32,7 @@ SIGNATURES = {
     "cpmcu_decode": (c_int, [c_int, c_int, c_u64, c_u64, c_u64, c_u64, c_u64, c_int]),
     "cpmcu_draft": (c_int, [c_u64] * 5),
     "cpmcu_verify_and_fix": (c_int, [c_int, c_u64, c_u64, c_u64, c_u64, c_u64, c_u64, ctypes.POINTER(c_int)]),
+    "cpmcu_verify_step": (c_int, [c_int, c_int, c_int, _P, _P, _P, _P] + [c_u64] * 13 + [c_int, c_int]),
     "cpmcu_print_perf_summary": (c_int, []),
     "cpmcu_decode_attention": (c_int, [c_int, c_int, c_int, c_u64, c_u64, c_u64, c_u64, c_u64, c_u64]),
     "cpmcu_draft_attention": (c_int, [c_int, c_int, c_int, c_u64, c_u64, c_u64, c_u64, c_u64, c_int, c_u64]),
@@ -54,6 +55,7 @@ SIGNATURES = {
     "cpmcu_head_weight_tile": (c_int, [_P, _P, c_int, c_int, _P, _P]),
     "cpmcu_frspec_head_topk": (c_int, [_P, _P, c_int, _P, c_int, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, c_size_t, _P]),
     "cpmcu_lm_head_argmax": (c_int, [_P, _P, c_int, c_int, c_int, c_int, c_int, c_float, _P, _P, _P, c_size_t, _P]),
+    "cpmcu_lm_head_partials": (c_int, [_P, _P, c_int, c_int, c_int, c_int, c_int, c_float, _P, _P, c_size_t, ctypes.POINTER(c_int), ctypes.POINTER(c_int), _P]),
     "cpmcu_lm_head_argmax_static_scratch_bytes": (c_size_t, []),
     "cpmcu_lm_head_argmax_static": (c_int, [_P, _P, c_int, c_int, c_int, c_int, c_int, c_float, _P, _P, _P]),
     "cpmcu_log_softmax": (c_int, [_P, c_int, c_int, _P, _P]),
@@ -63,6 +65,8 @@ SIGNATURES = {
     "cpmcu_tree_accept": (c_int, [c_int, _P, _P, _P, _P, _P, c_int, _P, _P, _P]),
     "cpmcu_kv_compact": (c_int, [_P, _P, c_int, _P, c_int, _P, _P, _P, _P, c_int, _P]),
     "cpmcu_accept_commit": (c_int, [_P, _P, c_int, _P, c_int, _P, _P, _P, _P, _P, c_int, _P, c_int, _P, _P, _P, c_int, _P]),
+    "cpmcu_verify_tail": (c_int, [_P, _P, c_int, _P, c_int, c_int, _P, _P, _P, c_int, c_int, _P, _P, _P, c_int, _P, _P, c_int, _P, _P, _P, _P, _P, _P, _P, _P]),
+    "cpmcu_verify_tail_inplace": (c_int, [_P, _P, c_int, _P, _P, _P, _P, c_int, _P]),
     "cpmcu_draft_tree_state_bytes": (c_size_t, [c_int, c_int]),
     "cpmcu_draft_tree_begin": (c_int, [_P, c_int, c_int, _P, _P, _P, _P, _P, _P]),
     "cpmcu_draft_tree_extend": (c_int, [_P, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P]),

@@ -134,6 +134,8 @@ def gather_rows(src, remap):
 
 
 W_ROW_MAJOR, W_TILED = 0, 1
+COMMIT_ADVANCE_LENGTH = 1
+COMMIT_NEXT_ROOT = 2
 
 
 class TiledWeight:
@@ -195,6 +197,49 @@ def lm_head_argmax(hidden, w, head_scale=None, want_logits=False, gt=None):
     return (gt, logits) if want_logits else gt
 
 
+class HeadPartials:
+    """The target head's arg-max left as per-workgroup partials (cpmcu_lm_head_partials): finished by verify_tail."""
+
+    def __init__(self, workspace, num_partials, stride, n):
+        self.workspace, self.num_partials, self.stride, self.n = workspace, int(num_partials), int(stride), int(n)
+
+
+def lm_head_partials(hidden, w, head_scale=None, logits=None):
+    """The target head's GEMM without the launch that finishes its arg-max; see verify_tail."""
+    n, H = hidden.shape
+    w, layout, V = _weight(w)
+    ws = _workspace("head", _lib().raw.cpmcu_head_workspace_bytes(n, V), hidden.device)
+    num, stride = ctypes.c_int(0), ctypes.c_int(0)
+    _lib().lm_head_partials(_ptr(hidden), _ptr(w), layout, n, V, H, 0 if head_scale is None else 1,
+                            ctypes.c_float(1.0 if head_scale is None else head_scale), _ptr(logits), _ptr(ws), ws.numel(),
+                            ctypes.byref(num), ctypes.byref(stride), _stream())
+    return HeadPartials(ws, num.value, stride.value, n)
+
+
+def verify_tail(cache, draft_ids, gt, position_ids, cache_length, attn_mask, tree_parent, hidden=None, prev_hidden=None,
+                gt_out=None, best=None, path=None, accepted_ids=None, next_position_ids=None, result=None):
+    """The whole tail of verify() in one launch (src/model/minicpm4/minicpm4_eagle.cuh:398-418): arg-max finish
+    when `gt` is a HeadPartials, acceptance, compaction of every layer, accepted ids, hidden-row gather.
+    draft_ids is read only; results go to best (a, node), path [T], accepted_ids [T], gt_out [T], ..."""
+    T = draft_ids.numel()
+    W = attn_mask.numel() // T
+    parts = gt if isinstance(gt, HeadPartials) else None
+    hidden_dim = 0 if hidden is None else hidden.shape[-1]
+    _lib().verify_tail(_ptr(cache.k_ptrs), _ptr(cache.v_ptrs), cache.num_layers, _ptr(cache.block_table), cache.Hkv, T,
+                       _ptr(draft_ids), None if parts else _ptr(gt), _ptr(parts.workspace) if parts else None,
+                       parts.num_partials if parts else 0, parts.stride if parts else 0, _ptr(position_ids), _ptr(cache_length),
+                       _ptr(attn_mask), W, _ptr(tree_parent), _ptr(hidden), hidden_dim, _ptr(prev_hidden), _ptr(gt_out), _ptr(best),
+                       _ptr(path), _ptr(accepted_ids), _ptr(next_position_ids), _ptr_result(result), _stream())
+
+
+def verify_tail_inplace(best, accepted_ids, pred=None, cache_length=None, kv_len=None, position_ids=None, advance_length=False,
+                        next_root=False):
+    """The in-place updates behind verify_tail: pred[:a] <- ids (or pred[0] <- last id), lengths and positions += a."""
+    flags = (COMMIT_ADVANCE_LENGTH if advance_length else 0) | (COMMIT_NEXT_ROOT if next_root else 0)
+    _lib().verify_tail_inplace(_ptr(best), _ptr(accepted_ids), accepted_ids.numel(), _ptr(pred), _ptr(cache_length), _ptr(kv_len),
+                               _ptr(position_ids), flags, _stream())
+
+
 def log_softmax_(x):
     """In place (src/model/eagle.cuh:29-89); returns row_stats [n,2] (max, ln sum)."""
     n, dim = x.shape
@@ -234,10 +279,6 @@ def kv_compact(cache, pred, gt, cache_length, best, max_accept):
     """fix_kv_cache (src/model/tree_drafter.cuh:48-77) on every layer of the paged cache."""
     _lib().kv_compact(_ptr(cache.k_ptrs), _ptr(cache.v_ptrs), cache.num_layers, _ptr(cache.block_table), cache.Hkv,
                       _ptr(pred), _ptr(gt), _ptr(cache_length), _ptr(best), int(max_accept), _stream())
-
-
-COMMIT_ADVANCE_LENGTH = 1
-COMMIT_NEXT_ROOT = 2
 
 
 def accept_commit(cache, pred, gt, cache_length, best, max_accept, hidden=None, prev_hidden=None,

@@ -55,6 +55,10 @@ extern "C" {
 #define CPMCU_ERR_UNSUPPORTED 3      /* -> RuntimeError: entry point outside the verify/draft path */
 #define CPMCU_ERR_HIP 4              /* -> RuntimeError: a HIP call failed */
 
+/* flags of cpmcu_accept_commit, cpmcu_verify_tail_inplace and cpmcu_verify_step */
+#define CPMCU_COMMIT_ADVANCE_LENGTH 1
+#define CPMCU_COMMIT_NEXT_ROOT 2
+
 #define CPMCU_PAGE_SIZE 256
 #define CPMCU_HEAD_DIM 128
 #define CPMCU_MAX_TREE 128
@@ -124,6 +128,34 @@ int cpmcu_draft(uint64_t tree_draft_ids, uint64_t tree_position_ids, uint64_t ca
 int cpmcu_verify_and_fix(int num_tokens, uint64_t pred, uint64_t gt, uint64_t position_ids,
                          uint64_t cache_length, uint64_t attn_mask, uint64_t tree_parent,
                          int* accept_length);
+
+/* One whole verify step on the model's storage, with the library's own HIP graph -- the part of
+ * decode(..., cuda_graph = true) + verify_and_fix (src/entry.cu:474-496,502-504) that lies on the path: for
+ * every layer the KV append of the num_tokens tree rows and the tree attention on the paged cache
+ * (cpmcu_decode_attention), the target head with its arg-max (cpmcu_decode_lm_head without the logits), greedy
+ * acceptance, compaction of every cache and the accepted ids (cpmcu_verify_and_fix) -- 34 launches for 32
+ * layers.  The dense layers that produce q / k_new / v_new / hidden between those calls are outside the path,
+ * so their outputs are inputs here.
+ *   q, k_new, v_new, attn_out: HOST arrays [num_layers] (= num_hidden_layers) of device addresses: q[l] [T][Hq][128],
+ *       k_new[l] / v_new[l] [T][Hkv*128], attn_out[l] like q[l];
+ *   hidden [T][hidden_size]; draft_ids int32[T] (read only); position_ids int32[T]; cache_length int32[1] = P;
+ *   kv_length int32[1] = P + T (the pre-incremented length of cpmcu/llm.py:272, kept as a scalar of its own so
+ *       that neither is rewritten between the calls of a step); attn_mask uint64[T]; tree_parent int32[T];
+ *   block_table: device int32[] logical -> physical pages to use for this step, or 0 = the model's table;
+ *   outputs: gt_out int32[T] (0 = skip), accepted_ids int32[T] (first a entries), prev_hidden [T][hidden_size]
+ *       (0 = skip: rows hidden[path[d]], src/model/eagle.cuh:108-115), next_position_ids int32[T] (0 = skip),
+ *       result int32[1 + T] = (a, ids) in device or pinned host memory (0 = skip);
+ *   flags: CPMCU_COMMIT_ADVANCE_LENGTH advances cache_length, kv_length and position_ids by a on the device
+ *       (one more single-workgroup launch), so the next step of the same tree shape needs no host write.
+ *   cuda_graph != 0: the step is captured once per (padded_length, num_tokens) -- the reference's key,
+ *       src/entry.cu:476 -- and per set of addresses, and replayed afterwards (hipGraphLaunch); keep the buffers
+ *       static, as cpmcu/llm.py does.  The call only enqueues on the library's stream: synchronise
+ *       (cpmcu_synchronize) before reading results. */
+int cpmcu_verify_step(int num_layers, int num_tokens, int padded_length, const uint64_t* q, const uint64_t* k_new, const uint64_t* v_new,
+                      const uint64_t* attn_out, uint64_t hidden, uint64_t draft_ids, uint64_t position_ids,
+                      uint64_t cache_length, uint64_t kv_length, uint64_t attn_mask, uint64_t tree_parent, uint64_t block_table,
+                      uint64_t gt_out, uint64_t accepted_ids, uint64_t prev_hidden, uint64_t next_position_ids,
+                      uint64_t result, int flags, int cuda_graph);
 
 /* src/entry.cu:506-508 print_perf_summary: prints the per-operator event timings
  * collected when CPMCU_PERF=1 is set in the environment. */
@@ -310,6 +342,14 @@ int cpmcu_lm_head_argmax(const void* hidden, const void* w, int w_layout, int n,
                          float head_scale, void* logits, int32_t* gt, void* workspace,
                          size_t workspace_bytes, void* stream);
 
+/* The target head's GEMM without its finishing launch: the per-workgroup arg-max partials stay in
+ * `workspace` (same size as for cpmcu_lm_head_argmax) and are finished by cpmcu_verify_tail, which is their
+ * only consumer in a verify step.  *num_partials / *partial_stride (host) describe them for that call.
+ * logits as above, or NULL. */
+int cpmcu_lm_head_partials(const void* hidden, const void* w, int w_layout, int n, int V, int H, int apply_scale,
+                           float head_scale, void* logits, void* workspace, size_t workspace_bytes, int* num_partials,
+                           int* partial_stride, void* stream);
+
 /* cpmcu_lm_head_argmax for callers that cannot allocate device memory or bring a workspace: code under
  * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the
  * reference.  Same arguments and results as cpmcu_lm_head_argmax without the workspace: the per-workgroup
@@ -373,12 +413,38 @@ int cpmcu_kv_compact(void* const* k_pools, void* const* v_pools, int num_layers,
  *       given: the device scalar P + T that the attention calls read (cpmcu/llm.py:272), so the next
  *       step can be enqueued, or a captured graph of it replayed, without the host knowing a;
  *   CPMCU_COMMIT_NEXT_ROOT: pred[0] = the last accepted id (tree_draft_ids[0] = tree_draft_ids[a - 1]). */
-#define CPMCU_COMMIT_ADVANCE_LENGTH 1
-#define CPMCU_COMMIT_NEXT_ROOT 2
 int cpmcu_accept_commit(void* const* k_pools, void* const* v_pools, int num_layers, const int32_t* block_table,
                         int Hkv, int32_t* pred, const int32_t* gt, int32_t* cache_length, int32_t* kv_len,
                         const int32_t* best, int max_accept, const void* hidden, int hidden_dim, void* prev_hidden,
                         int32_t* next_position_ids, int32_t* result, int flags, void* stream);
+
+/* The whole tail of a verify step in ONE launch -- MiniCPM4EagleImpl::verify,
+ * src/model/minicpm4/minicpm4_eagle.cuh:398-418: greedy acceptance
+ * (src/model/tree_drafter.cuh:5-46), compaction of the accepted rows in every cache (:48-77), the accepted
+ * ids (:74-76), the gather of the accepted hidden rows (src/model/eagle.cuh:108-115) and, in front of all
+ * that, the finish of the target arg-max when the head leaves it as partials (cpmcu_lm_head_partials).
+ * Every workgroup of the launch recomputes the acceptance from the same few hundred bytes and then moves
+ * its own cache stream, so nothing waits for a second launch.  Unlike cpmcu_tree_accept / cpmcu_kv_compact
+ * the draft ids are read-only and every result has its own array:
+ *   draft_ids int32[T] in; gt int32[T] in, or NULL with head_partials = the workspace of
+ *   cpmcu_lm_head_partials (+ its num_partials, partial_stride); cache_length int32[1] = P, read only;
+ *   hidden [T][hidden_dim] / prev_hidden [T][hidden_dim]: prev_hidden[d] = hidden[path[d]], both NULL to skip;
+ *   outputs (each may be NULL): gt_out int32[T]; best int32[2] = (a, winning node); path int32[T] (first a
+ *   entries: node indices by depth); accepted_ids int32[T] (first a entries: gt[path[d]]);
+ *   next_position_ids int32[T] (P + d); result int32[1 + T] = (a, ids), device or pinned host memory.
+ * The in-place updates that other workgroups of that launch must not see are a second, single-workgroup
+ * launch, cpmcu_verify_tail_inplace: pred[0..a) <- accepted ids (what the reference's verify leaves in
+ * tree_draft_ids; pred may be NULL), and with flags as for cpmcu_accept_commit cache_length[0] += a,
+ * kv_len[0] += a (kv_len may be NULL), position_ids[0..T) += a (may be NULL: the positions a tree of the same
+ * shape has in the next step), pred[0] <- the last accepted id instead of the id copy. */
+int cpmcu_verify_tail(void* const* k_pools, void* const* v_pools, int num_layers, const int32_t* block_table, int Hkv,
+                      int T, const int32_t* draft_ids, const int32_t* gt, const void* head_partials, int num_partials,
+                      int partial_stride, const int32_t* position_ids, const int32_t* cache_length,
+                      const uint64_t* attn_mask, int mask_words, const int32_t* tree_parent, const void* hidden,
+                      int hidden_dim, void* prev_hidden, int32_t* gt_out, int32_t* best, int32_t* path,
+                      int32_t* accepted_ids, int32_t* next_position_ids, int32_t* result, void* stream);
+int cpmcu_verify_tail_inplace(const int32_t* best, const int32_t* accepted_ids, int T, int32_t* pred, int32_t* cache_length,
+                              int32_t* kv_len, int32_t* position_ids, int flags, void* stream);
 
 /* ---- Draft-tree construction around the FR-Spec head (the tree bookkeeping of draft()) ----
  * src/model/minicpm4/minicpm4_eagle.cuh:319-393 with src/model/eagle.cuh:91-106,121-127,188-214.

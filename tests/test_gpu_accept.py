@@ -206,6 +206,116 @@ def test_accept_commit_argument_checks(gpu):
         ops.accept_commit(cache, i32(4), i32(4), i32(1), i32(2), 4, hidden=odd, prev_hidden=odd.clone())  # 60 % 8
 
 
+def _tail_case(torch, orc, tree, P, leaf_depth, layers, seed, H=512, V=3000, from_partials=False):
+    """cpmcu_verify_tail (+ cpmcu_verify_tail_inplace) against the oracle's acceptance, compaction and tail bookkeeping,
+    with gt given or left as the head's per-workgroup partials."""
+    from cpm.cu_amd import ops
+    from cpm.cu_amd.kvcache import PagedKVCache
+    T = tree.T
+    S = P + T
+    npages = (S + 255) // 256 + 1
+    table = synth.rng(seed, 4).permutation(npages).astype(np.int32)
+    cache = PagedKVCache(layers, HKV, npages, block_table=table)
+    flat = []
+    for layer in range(layers):
+        k = synth.normal_f16((S, HKV, D), seed, 10 + layer)
+        v = synth.normal_f16((S, HKV, D), seed, 50 + layer)
+        cache.write_logical(layer, 0, to_dev(torch, k), to_dev(torch, v))
+        flat += [k.reshape(S, HKV * D).copy(), v.reshape(S, HKV * D).copy()]
+    hidden = synth.normal_f16((T, H), seed, 90)
+    d_hidden = to_dev(torch, hidden)
+    if from_partials:
+        w = to_dev(torch, synth.normal_f16((V, H), seed, 91, std=0.02))
+        wt = ops.tile_head_weight(w)
+        gt = to_np(ops.lm_head_argmax(d_hidden, wt))  # the two-launch head: what the partials must finish to
+    else:
+        gt = synth.rng(seed, 9).integers(0, VOCAB, T).astype(np.int32)
+    pred, leaf = synth.draft_ids_for_accept(tree, gt, leaf_depth, V if from_partials else VOCAB, seed)
+    pos = tree.positions(P)
+    a, node, path = orc.tree_accept(pred, gt, pos, P, tree.mask, tree.parent)
+    want = orc.accept_commit(flat, P, path, gt, hidden)
+    d_pred, d_pos, d_mask, d_par = to_dev(torch, pred), to_dev(torch, pos), to_dev(torch, tree.mask), to_dev(torch, tree.parent)
+    d_len = torch.tensor([P], dtype=torch.int32, device="cuda")
+    d_kvlen = torch.tensor([P + T], dtype=torch.int32, device="cuda")
+    i32 = lambda n, fill=-1: torch.full((n,), fill, dtype=torch.int32, device="cuda")
+    gt_out, best, pth, ids, npos, result = i32(T), i32(2), i32(T), i32(T), i32(T), i32(1 + T)
+    prev = torch.full((T, H), 7.0, dtype=torch.float16, device="cuda")
+    src = ops.lm_head_partials(d_hidden, wt) if from_partials else to_dev(torch, gt)
+    ops.verify_tail(cache, d_pred, src, d_pos, d_len, d_mask, d_par, hidden=d_hidden, prev_hidden=prev, gt_out=gt_out, best=best,
+                    path=pth, accepted_ids=ids, next_position_ids=npos, result=result)
+    torch.cuda.synchronize()
+    assert np.array_equal(to_np(d_pred), pred), "the draft ids are read only"
+    assert np.array_equal(to_np(gt_out), gt)
+    assert to_np(best).tolist() == [a, node]
+    assert np.array_equal(to_np(pth)[:a], path) and np.all(to_np(pth)[a:] == -1)
+    assert np.array_equal(to_np(ids)[:a], want["result"][1:]) and np.all(to_np(ids)[a:] == -1)
+    assert np.array_equal(to_np(result)[: 1 + a], want["result"]) and np.all(to_np(result)[1 + a:] == -1)
+    assert np.array_equal(to_np(npos)[:a], want["next_pos"]) and np.all(to_np(npos)[a:] == -1)
+    assert np.array_equal(to_np(prev)[:a].view(np.uint16), want["prev_hidden"].view(np.uint16)) and np.all(to_np(prev)[a:] == 7.0)
+    assert int(to_np(d_len)[0]) == P
+    for layer in range(layers):
+        k_dev, v_dev = cache.read_logical(layer, 0, P + a)
+        assert np.array_equal(to_np(k_dev).reshape(P + a, -1).view(np.uint16), flat[2 * layer][: P + a].view(np.uint16))
+        assert np.array_equal(to_np(v_dev).reshape(P + a, -1).view(np.uint16), flat[2 * layer + 1][: P + a].view(np.uint16))
+    # the in-place part: ids into pred, lengths and positions advanced; then the next-root form
+    p2 = to_dev(torch, pred)
+    ops.verify_tail_inplace(best, ids, pred=p2, cache_length=d_len, kv_len=d_kvlen, position_ids=d_pos, advance_length=True)
+    torch.cuda.synchronize()
+    assert np.array_equal(to_np(p2)[:a], want["result"][1:]) and np.array_equal(to_np(p2)[a:], pred[a:])
+    assert int(to_np(d_len)[0]) == want["new_length"] and int(to_np(d_kvlen)[0]) == P + T + a
+    assert np.array_equal(to_np(d_pos), tree.positions(P + a))
+    p3 = to_dev(torch, pred)
+    ops.verify_tail_inplace(best, ids, pred=p3, next_root=True)
+    torch.cuda.synchronize()
+    assert int(to_np(p3)[0]) == want["next_root"] and np.array_equal(to_np(p3)[1:], pred[1:])
+    return a
+
+
+def test_verify_tail_every_depth(gpu, orc):
+    tree = synth.eagle_tree(6, 10, 60, seed=0)
+    for depth in range(int(tree.depth.max()) + 1):
+        assert _tail_case(gpu, orc, tree, 4096 - 7, depth, layers=3, seed=depth) == depth + 1
+    wide = synth.eagle_tree(8, 16, 128, seed=3)
+    for depth in (0, 5, 8):
+        _tail_case(gpu, orc, wide, 1000, depth, layers=2, seed=31 + depth, H=1024)
+    _tail_case(gpu, orc, synth.chain_tree(128), 250, 127, layers=2, seed=32, H=64)   # several read/write batches
+    _tail_case(gpu, orc, synth.tree_from_parents([0, 0, 0, 2]), 300, 2, layers=2, seed=33)  # path [0, 2, 3]: overlap
+    _tail_case(gpu, orc, synth.chain_tree(1), 77, 0, layers=1, seed=34)
+
+
+@pytest.mark.parametrize("T,num_iter,topk", [(16, 4, 4), (17, 4, 4), (60, 6, 10), (64, 6, 10), (100, 8, 16), (128, 8, 16)])
+def test_verify_tail_finishes_the_head_partials(gpu, orc, T, num_iter, topk):
+    """gt left as the head GEMM's per-workgroup partials (one row-block count per kernel shape): the tail's own
+    finish must give the arg-max of the two-launch head, and everything behind it follows."""
+    tree = synth.eagle_tree(num_iter, topk, T, seed=T)
+    _tail_case(gpu, orc, tree, 513, min(2, int(tree.depth.max())), layers=2, seed=T, H=512, V=40000, from_partials=True)
+
+
+def test_verify_tail_random_trees_duplicate_siblings(gpu, orc):
+    """Tiny vocabulary: accidental matches and duplicate sibling tokens, so the tournament's tie rule decides."""
+    from cpm.cu_amd import ops
+    from cpm.cu_amd.kvcache import PagedKVCache
+    torch = gpu
+    cache = PagedKVCache(1, HKV, 3)
+    for seed in range(30):
+        T = int(synth.rng(seed, 1).integers(1, 129))
+        tree = synth.random_tree(T, seed, max_children=6, max_depth=12)
+        g = synth.rng(seed, 2)
+        pred = g.integers(0, 3, T).astype(np.int32)
+        gt = g.integers(0, 3, T).astype(np.int32)
+        P = int(g.integers(0, 300))
+        pos = tree.positions(P)
+        a, node, path = orc.tree_accept(pred, gt, pos, P, tree.mask, tree.parent)
+        best = torch.zeros(2, dtype=torch.int32, device="cuda")
+        pth = torch.zeros(T, dtype=torch.int32, device="cuda")
+        ids = torch.zeros(T, dtype=torch.int32, device="cuda")
+        ops.verify_tail(cache, to_dev(torch, pred), to_dev(torch, gt), to_dev(torch, pos), torch.tensor([P], dtype=torch.int32, device="cuda"),
+                        to_dev(torch, tree.mask), to_dev(torch, tree.parent), best=best, path=pth, accepted_ids=ids)
+        torch.cuda.synchronize()
+        assert to_np(best).tolist() == [a, node], seed
+        assert np.array_equal(to_np(pth)[:a], path) and np.array_equal(to_np(ids)[:a], gt[path])
+
+
 def test_model_level_entry_points(gpu, orc):
     """init_* -> init_storage -> load_model -> decode_attention / decode_lm_head / draft_head /
     verify_and_fix on the library-owned paged cache, against the oracle; and the error contract."""

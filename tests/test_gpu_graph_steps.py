@@ -85,7 +85,8 @@ def test_graph_replayed_steps_equal_host_driven_steps(gpu, orc):
             bv[l].copy_(x["v"][l])
         bh.copy_(x["hidden"])
         bd.copy_(x["pred"])
-        step.pos.copy_(depth + step.cache_length)  # positions follow the device-side prefix length
+        # (the tree positions follow the device-side prefix length by themselves: the step's tail advances them)
+        assert np.array_equal(to_np(step.pos), tree.positions(Pb))
         a, ids = gs.run()
         assert (a, ids.tolist()) == hist_a[s], "step %d: graph replay (%d, %s) vs host-driven %s" % (s, a, ids.tolist(), hist_a[s])
         assert np.array_equal(to_np(step.prev_hidden)[:a].view(np.uint16), to_np(x["hidden"])[x["path"]].view(np.uint16))

@@ -179,3 +179,88 @@ def test_pybind_module_drives_the_path_end_to_end(gpu, orc):
     with pytest.raises(RuntimeError, match="outside the verify/draft path"):
         C.decode(T, 128, 0, 0, 0, 0, 0, False)
     C.shutdown()
+
+
+def test_library_graph_replays_equal_eager_steps(gpu, orc):
+    """cpmcu_verify_step on the library's own storage: the same sequence of steps enqueued eagerly and as replays of
+    the library's HIP graphs (one per padded length, lengths and positions advancing on the device) must give the same
+    accept lengths, ids, gathered hidden rows and caches, and both must match the oracle's acceptance on the device's
+    own arg-max.  The second model instance reuses the process-global model after a shutdown."""
+    from cpm.cu_amd import ops
+    from cpm.cu_amd.model import PathModel
+    torch = gpu
+    V, H, LAYERS, T, P0, STEPS = 3000, 512, 3, 24, 1000, 10
+    tree = synth.random_tree(T, 3, max_children=3, max_depth=6)
+    mask, parent = to_dev(torch, tree.mask), to_dev(torch, tree.parent)
+    w = synth.normal_f16((V, H), 3, 2, std=0.02)
+    w_dev = ops.tile_head_weight(to_dev(torch, w))
+    rg = synth.rng(3, 8)
+    inputs = []
+    for s in range(STEPS):
+        x = dict(q=[to_dev(torch, synth.normal_f16((T, HQ, D), 3, 1000 + 10 * s + l)) for l in range(LAYERS)],
+                 k=[to_dev(torch, synth.normal_f16((T, HKV, D), 3, 2000 + 10 * s + l)) for l in range(LAYERS)],
+                 v=[to_dev(torch, synth.normal_f16((T, HKV, D), 3, 3000 + 10 * s + l)) for l in range(LAYERS)],
+                 hidden=to_dev(torch, synth.normal_f16((T, H), 3, 4000 + s)))
+        x["gt"] = to_np(ops.lm_head_argmax(x["hidden"], w_dev, head_scale=0.5))
+        x["depth"] = int(rg.integers(0, int(tree.depth.max()) + 1))
+        pred, leaf = synth.draft_ids_for_accept(tree, x["gt"], x["depth"], V, 300 + s)
+        x["pred"], x["path"] = to_dev(torch, pred), tree.path_to(leaf)
+        x["pred_np"] = pred
+        inputs.append(x)
+    del w_dev
+
+    def run(graph):
+        m = PathModel(V, LAYERS, H, HQ, HKV, memory_limit=0.01, scale_lmhead=0.5, tree_size=T, num_iter=6, topk=4)
+        try:
+            m.load_head(w)
+            cache = m.cache()
+            for layer in range(LAYERS):
+                cache.write_logical(layer, 0, to_dev(torch, synth.normal_f16((P0, HKV, D), 3, 10 + layer)),
+                                    to_dev(torch, synth.normal_f16((P0, HKV, D), 3, 50 + layer)))
+            f16 = dict(dtype=torch.float16, device="cuda")
+            bq = [torch.zeros((T, HQ, D), **f16) for _ in range(LAYERS)]
+            bk = [torch.zeros((T, HKV, D), **f16) for _ in range(LAYERS)]
+            bv = [torch.zeros((T, HKV, D), **f16) for _ in range(LAYERS)]
+            bo = [torch.zeros((T, HQ, D), **f16) for _ in range(LAYERS)]
+            bh, prev = torch.zeros((T, H), **f16), torch.zeros((T, H), **f16)
+            bd = torch.zeros(T, dtype=torch.int32, device="cuda")
+            pos = to_dev(torch, tree.positions(P0))
+            clen = torch.tensor([P0], dtype=torch.int32, device="cuda")
+            kvlen = torch.tensor([P0 + T], dtype=torch.int32, device="cuda")
+            ids = torch.zeros(T, dtype=torch.int32, device="cuda")
+            gt_out = torch.zeros(T, dtype=torch.int32, device="cuda")
+            result = torch.zeros(1 + T, dtype=torch.int32).pin_memory()
+            P, hist, paddings = P0, [], set()
+            for x in inputs:
+                for l in range(LAYERS):
+                    bq[l].copy_(x["q"][l]); bk[l].copy_(x["k"][l]); bv[l].copy_(x["v"][l])
+                bh.copy_(x["hidden"]); bd.copy_(x["pred"])
+                torch.cuda.synchronize()  # the library's stream is not torch's
+                padded = (P + T + 31) // 32 * 32
+                paddings.add(padded)
+                m.verify_step(T, padded, bq, bk, bv, bo, bh, bd, pos, clen, kvlen, mask, parent, ids, gt_out=gt_out, prev_hidden=prev,
+                              result=result, advance_length=True, cuda_graph=graph)
+                m.synchronize()
+                a = int(result[0])
+                a_ref, _, path = orc.tree_accept(x["pred_np"], x["gt"], tree.positions(P), P, tree.mask, tree.parent)
+                assert a == a_ref == x["depth"] + 1 and list(path) == x["path"]
+                assert np.array_equal(to_np(gt_out), x["gt"]) and np.array_equal(result[1:1 + a].numpy(), x["gt"][path])
+                assert np.array_equal(to_np(ids)[:a], x["gt"][path])
+                assert np.array_equal(to_np(prev)[:a].view(np.uint16), to_np(x["hidden"])[path].view(np.uint16))
+                assert np.array_equal(to_np(bd), x["pred_np"]), "the draft ids are read only"
+                P += a
+                assert int(to_np(clen)[0]) == P and int(to_np(kvlen)[0]) == P + T and np.array_equal(to_np(pos), tree.positions(P))
+                hist.append((a, result[1:1 + a].numpy().tolist(), to_np(bo[LAYERS - 1]).copy()))
+            kv = [tuple(to_np(t) for t in cache.read_logical(layer, 0, P)) for layer in range(LAYERS)]
+            return hist, kv, P, len(paddings)
+        finally:
+            m.close()
+
+    hist_e, kv_e, P_e, _ = run(False)
+    hist_g, kv_g, P_g, npad = run(True)
+    assert P_e == P_g and npad >= 2, "the run should cross a padded length (%d seen)" % npad
+    for (a1, i1, o1), (a2, i2, o2) in zip(hist_e, hist_g):
+        assert (a1, i1) == (a2, i2)
+        assert np.array_equal(o1.view(np.uint16), o2.view(np.uint16))  # same launches, same split geometry: same bits
+    for (k1, v1), (k2, v2) in zip(kv_e, kv_g):
+        assert np.array_equal(k1.view(np.uint16), k2.view(np.uint16)) and np.array_equal(v1.view(np.uint16), v2.view(np.uint16))
