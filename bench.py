@@ -3,24 +3,27 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c2_verify_4k]
 
-One "step" = one pass of the verify hot path over one batch of synthetic MiniCPM4-8B-shaped input,
-with every input already resident in HBM: for each of the 32 layers append the 60 tree rows' K/V and
-run tree-masked attention (one fused kernel + the split merge) over the paged cache (4096-token prefix + 60 tree rows), then the target
-lm_head (73448 x 4096) with fused arg-max, greedy tree acceptance and accepted-path KV compaction in
-all layers.  The step is captured into a HIP graph (the reference replays a CUDA graph for
-decode as well) and replayed; exactly K replays are timed between synchronisations.  At 4K context
-the K/V of all layers would fit the 256 MB last-level cache, so the timed steps rotate over four
-distinct copies of the K/V pools (one graph each): every pass over K/V comes from HBM.  The time of
-replays on a single copy is reported beside it (`us_per_step_one_kv_set`).
+One "step" = one pass of the verify hot path over one batch of synthetic MiniCPM4-8B-shaped input, with every
+input already resident in HBM: for each of the 32 layers append the 60 tree rows' K/V and run tree-masked attention
+over the paged cache (4096-token prefix + 60 tree rows), then the target lm_head (73448 x 4096) with its arg-max,
+greedy tree acceptance and accepted-path KV compaction in all layers.
 
-Prints ONE JSON line.  `value` is microseconds per step (lower is better).  `roofline` is for the
-kernel that takes the largest share of the step; `kernels` lists all of them; `contexts` gives the
-step time at 4K / 32K / 128K context; `cpu_baseline` is the CPU oracle timed on this host on a
-bounded sample of the same workload (a reported baseline only).
+The step runs where a user of the library runs it: on the library's own storage (`cpmcu_init_storage` pools, the
+loaded lm_head) through `cpmcu_verify_step` with the library's own HIP graph (captured once per padded length, as
+the reference captures decode, src/entry.cu:475-492) on the library's stream.  Exactly K graph launches are timed
+with events on that stream.  At 4K context the K/V of all layers would fit the 256 MB last-level cache, so the timed
+steps rotate over four distinct sets of K/V pages of the same pools (four page tables, one graph each): every pass
+over K/V comes from HBM.  The time of replays on a single set is reported beside it (`us_per_step_one_kv_set`).
+
+Prints ONE JSON line.  `value` is microseconds per step (lower is better).  `roofline` is for the kernel that takes
+the largest share of the step; `kernels` lists all of them (names as reported by the library for the dispatch
+actually taken); `contexts_us_per_step` gives the step at 4K / 32K / 128K context; `cpu_baseline` is the CPU oracle
+timed on this host on a bounded sample of the same workload (a reported baseline only).
 """
 import argparse
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -30,15 +33,17 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 
-# HBM bytes per launch on c2_verify_4k with the automatic split count, from rocprofv3's FETCH_SIZE and
-# WRITE_SIZE counters (KiB per dispatch, one counter per run, eager launches), each scaled by what the
-# same counter read for a plain 256 MiB copy (x2.000 and x1.000): the table and the two commands are in
-# profiles/verify_step_hbm_traffic.md.  Counters cannot be read from inside this process, so the figures
-# are carried here as constants and are reported only for the workload they were measured on.
-MEASURED_TRAFFIC_KIB = {
-    "tree_attn_split_kernel+tree_attn_combine_kernel": 6367 + 8494 + 8710 + 480,
-    "head_gemm_chunked_kernel<4,4,256,2>+head_argmax_finalize_kernel": 592012 + 128 + 1052 + 2,
-    "tree_accept_kernel+kv_compact_kernel+accepted_ids_kernel": 6 + 1137 + 335 + 4,
+# HBM bytes per launch on c2_verify_4k with the automatic split count, from rocprofv3's FETCH_SIZE and WRITE_SIZE
+# counters (KiB per dispatch, one counter per run, eager launches), each scaled by what the same counter read for a
+# plain 256 MiB copy (x2.000 and x1.000): the table and the two commands are in profiles/verify_step_hbm_traffic.md.
+# Counters cannot be read from inside this process, so the figures are carried here as constants, keyed by the kernel
+# names the library reports for the dispatch taken: a different instantiation finds no entry and reports null.
+MEASURED_TRAFFIC = {
+    "source": "profiles/verify_step_hbm_traffic.md",
+    "kib_per_launch": {
+        "tree_attn_split_kernel<2,false>+tree_attn_combine_kernel": 6367 + 8494 + 8710 + 480,
+        "head_gemm_chunked_kernel<4,4,256,2>": 592012 + 128,
+    },
 }
 
 
@@ -48,11 +53,11 @@ def parse_args():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="c2_verify_4k")
-    ap.add_argument("--splits", type=int, default=0, help="force the KV split count of tree attention (0 = auto)")
     ap.add_argument("--no-contexts", action="store_true", help="skip the 32K / 128K context step timings")
     ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    ap.add_argument("--no-graph", action="store_true", help="enqueue the step's launches eagerly instead of replaying the library's HIP graph")
     ap.add_argument("--no-probes", action="store_true", help="skip the MFMA-rate probe of the machine")
+    ap.add_argument("--no-operators", action="store_true", help="skip the per-operator timings (heads, tail, draft path)")
     ap.add_argument("--accept-depth", type=int, default=3, help="draft tokens the rigged tree gets accepted")
     ap.add_argument("--traffic-probe", action="store_true",
                     help="also run a plain 256 MiB device copy three times: the known-size kernel that scales "
@@ -60,66 +65,9 @@ def parse_args():
     return ap.parse_args()
 
 
-class Workload:
-    """Synthetic tensors of one configuration, resident on the GPU."""
-
-    def __init__(self, torch, name, accept_depth, seed=0):
-        import numpy as np
-        from cpm.cu_amd import synth
-        from cpm.cu_amd.kvcache import PagedKVCache
-        cfg = dict(synth.CONFIGS[name])
-        shp = synth.MINICPM4_8B
-        self.name, self.cfg, self.shape = name, cfg, shp
-        L, P, T = cfg["layers"], cfg["prefix"], cfg["T"]
-        Hq, Hkv, D, H, V = shp["q_heads"], shp["kv_heads"], shp["head_dim"], shp["hidden"], shp["vocab"]
-        self.L, self.P, self.T = L, P, T
-        dev = torch.device("cuda:0")
-        g = torch.Generator(device=dev)
-        g.manual_seed(seed)
-        S = P + T
-        npages = (S + 255) // 256 + 1
-        table = synth.rng(seed, 4).permutation(npages).astype(np.int32)  # seeded page-table permutation
-        self.cache = PagedKVCache(L, Hkv, npages, device=dev, block_table=table)
-        for l in range(L):  # ~N(0,1) prefix K/V, written page by page in the kernels' layout
-            self.cache.k[l].normal_(generator=g)
-            self.cache.v[l].normal_(generator=g)
-        rn = lambda *s, std=1.0: (torch.randn(*s, device=dev, dtype=torch.float32, generator=g) * std).to(torch.float16)
-        self.q = [rn(T, Hq, D) for _ in range(L)]
-        self.k_new = [rn(T, Hkv, D) for _ in range(L)]
-        self.v_new = [rn(T, Hkv, D) for _ in range(L)]
-        self.hidden = rn(T, H)
-        self.w = rn(V, H, std=0.02)
-        self.tree = synth.eagle_tree(cfg["num_iter"], cfg["topk"], T, seed)
-        tm = torch.from_numpy(self.tree.mask.view(np.int64)).to(dev)
-        self.mask = tm
-        self.parent = torch.from_numpy(self.tree.parent).to(dev)
-        self.pos = torch.from_numpy(self.tree.positions(P)).to(dev)
-        self.accept_depth = min(accept_depth, int(self.tree.depth.max()))
-        self.draft_ids = None  # rigged from the target arg-max once it is known
-        self.attn_out = [torch.empty(T, Hq, D, dtype=torch.float16, device=dev) for _ in range(L)]
-
-    def rig_draft(self, torch, gt_np):
-        from cpm.cu_amd import synth
-        pred, self.leaf = synth.draft_ids_for_accept(self.tree, gt_np, self.accept_depth, self.shape["vocab"], 1)
-        self.draft_np = pred
-        self.draft_ids = torch.from_numpy(pred).cuda()
-
-    def flops_attention_layer(self):
-        s = self.shape
-        return 4.0 * s["q_heads"] * self.T * s["head_dim"] * (self.P + self.T)
-
-    def bytes_attention_layer(self):
-        s = self.shape
-        return 2.0 * (self.P + self.T) * s["kv_heads"] * s["head_dim"] * 2 + 2.0 * self.T * s["q_heads"] * s["head_dim"] * 2
-
-    def bytes_target_head(self):
-        s = self.shape
-        return s["vocab"] * s["hidden"] * 2.0 + self.T * s["hidden"] * 2.0 + self.T * 4.0
-
-
-def timed_replays(torch, fn, steps, warmup, use_graph):
-    """Capture fn() once (unless disabled), run `warmup` untimed and exactly `steps` timed calls.
-    `fn` may be a list of callables: each is captured on its own and the calls cycle through them."""
+def timed_torch(torch, fn, steps, warmup, use_graph=True):
+    """Operator timings on a torch side stream: fn() captured once into a graph (unless disabled), `warmup` untimed and
+    exactly `steps` timed calls between two events on that stream.  fn may be a list: the calls cycle through it."""
     fns = list(fn) if isinstance(fn, (list, tuple)) else [fn]
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
@@ -139,16 +87,138 @@ def timed_replays(torch, fn, steps, warmup, use_graph):
         stream.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
-        t0 = time.perf_counter()
         e0.record(stream)
         for i in range(steps):
             runs[i % len(runs)]()
         e1.record(stream)
         stream.synchronize()
         torch.cuda.synchronize()
-        wall_ms = (time.perf_counter() - t0) * 1e3
-        ev_ms = e0.elapsed_time(e1)
-    return ev_ms / steps, wall_ms / steps
+    return e0.elapsed_time(e1) / steps
+
+
+class StepBuffers:
+    """The static input / output buffers of the verify step, as cpmcu/llm.py keeps them for the reference."""
+
+    def __init__(self, torch, L, T, Hq, Hkv, D, H, gen):
+        dev = "cuda"
+        rn = lambda *s: torch.randn(*s, device=dev, dtype=torch.float32, generator=gen).to(torch.float16)
+        self.q = [rn(T, Hq, D) for _ in range(L)]
+        self.k_new = [rn(T, Hkv, D) for _ in range(L)]
+        self.v_new = [rn(T, Hkv, D) for _ in range(L)]
+        self.attn_out = [torch.empty(T, Hq, D, dtype=torch.float16, device=dev) for _ in range(L)]
+        self.hidden = rn(T, H)
+        self.draft_ids = torch.zeros(T, dtype=torch.int32, device=dev)
+        self.accepted = torch.zeros(T, dtype=torch.int32, device=dev)
+        self.gt = torch.zeros(T, dtype=torch.int32, device=dev)
+        self.result = torch.zeros(1 + T, dtype=torch.int32).pin_memory()  # (a, ids): written by the GPU
+
+
+def run_context(torch, np, model, synth, oracle_mod, args, name, bufs, tree, use_graph, kv_sets, gen, want_cpu):
+    """The verify step of one configuration on the library's storage: fills the pools, captures / replays the
+    library's graph(s), times K launches on the library's stream, checks the integer results against the oracle."""
+    from cpm.cu_amd import ops
+    cfg = dict(synth.CONFIGS[name])
+    shp = synth.MINICPM4_8B
+    L, P, T = cfg["layers"], cfg["prefix"], cfg["T"]
+    Hq, Hkv = shp["q_heads"], shp["kv_heads"]
+    S = P + T
+    npages = (S + 255) // 256 + 1
+    assert kv_sets * npages <= model.num_pages, "the library's pools are too small for %s" % name
+    # page tables: set i lives in physical pages [i * npages, (i + 1) * npages), permuted by a seeded permutation
+    tables = []
+    for i in range(kv_sets):
+        perm = synth.rng(cfg["seed"], 4 + i).permutation(npages).astype(np.int32) + i * npages
+        tables.append(torch.from_numpy(perm).cuda())
+    for l in range(L):  # ~N(0,1) K/V, written in the pools' own layout
+        model._k[l][: kv_sets * npages].normal_(generator=gen)
+        model._v[l][: kv_sets * npages].normal_(generator=gen)
+    mask = torch.from_numpy(tree.mask.view(np.int64)).cuda()
+    parent = torch.from_numpy(tree.parent).cuda()
+    pos = torch.from_numpy(tree.positions(P)).cuda()
+    clen = torch.tensor([P], dtype=torch.int32, device="cuda")
+    kvlen = torch.tensor([S], dtype=torch.int32, device="cuda")
+    padded = (S + 127) // 128 * 128  # padded_length, cpmcu/llm.py:273
+    torch.cuda.synchronize()
+
+    def step(i):
+        model.verify_step(T, padded, bufs.q, bufs.k_new, bufs.v_new, bufs.attn_out, bufs.hidden, bufs.draft_ids, pos, clen, kvlen,
+                          mask, parent, bufs.accepted, gt_out=bufs.gt, result=bufs.result, block_table=tables[i % kv_sets],
+                          cuda_graph=use_graph)
+
+    # target arg-max once (through the step itself), to rig the draft ids for the chosen accept length
+    step(0)
+    model.synchronize()
+    gt_np = bufs.gt.cpu().numpy()
+    depth = min(args.accept_depth, int(tree.depth.max()))
+    draft_np, leaf = synth.draft_ids_for_accept(tree, gt_np, depth, shp["vocab"], 1)
+    bufs.draft_ids.copy_(torch.from_numpy(draft_np).cuda())
+    torch.cuda.synchronize()
+
+    stream = model.stream()
+
+    def timed(steps, warmup, sets):
+        for i in range(max(warmup, sets)):  # every graph is captured (and launched once) before the timed region
+            step(i % sets)
+        model.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record(stream)
+        for i in range(steps):
+            step(i % sets)
+        e1.record(stream)
+        model.synchronize()
+        wall = (time.perf_counter() - t0) * 1e3
+        return e0.elapsed_time(e1) / steps, wall / steps
+
+    results = []
+    for i in range(kv_sets):
+        step(i)
+        model.synchronize()
+        a = int(bufs.result[0])
+        results.append((a, bufs.result[1:1 + a].numpy().copy()))
+    steps = args.steps if name == args.workload else max(3, args.steps // 5)
+    ms_step, wall_ms = timed(steps, args.warmup, kv_sets)
+    ms_one = timed(max(5, steps // 2), 2, 1)[0] if kv_sets > 1 else ms_step
+
+    out = dict(name=name, P=P, T=T, L=L, ms_step=ms_step, wall_ms=wall_ms, ms_one_set=ms_one, steps=steps, results=results,
+               draft_np=draft_np, gt_np=gt_np, tables=tables, padded=padded, mask=mask, parent=parent, pos=pos, clen=clen,
+               kvlen=kvlen, npages=npages)
+    caches = [model.cache(block_table=t) for t in tables]
+    # what the last step left at rows [P, P + a) of layer 0 and of the last layer (the attention-alone timing below
+    # appends the tree rows again)
+    a0 = results[0][0]
+    out["compacted"] = {l: tuple(t.cpu().numpy().reshape(a0, -1) for t in caches[0].read_logical(l, P, a0)) for l in (0, L - 1)}
+
+    # attention alone: 32 layers on the same pools (operator level, torch side stream), every K/V pass from HBM
+
+    def attn_all():
+        for c in caches:
+            for l in range(L):
+                ops.tree_attention(bufs.q[l], c, l, kvlen, padded, mask, out=bufs.attn_out[l], k_new=bufs.k_new[l], v_new=bufs.v_new[l])
+    reps = max(3, steps // 5)
+    out["ms_attn"] = timed_torch(torch, attn_all, reps, 2) / (L * kv_sets)
+    if kv_sets > 1:
+        def attn_one():
+            for l in range(L):
+                ops.tree_attention(bufs.q[l], caches[0], l, kvlen, padded, mask, out=bufs.attn_out[l], k_new=bufs.k_new[l], v_new=bufs.v_new[l])
+        out["ms_attn_one_set"] = timed_torch(torch, attn_one, reps, 2) / L
+    else:
+        out["ms_attn_one_set"] = out["ms_attn"]
+    out["attn_plan"] = ops.attention_plan(T, Hq, Hkv, padded)
+    out["caches"] = caches
+
+    # the CPU oracle on a bounded sample of this context: one attention layer, 1 warm-up + median of 3
+    if want_cpu:
+        k_all, v_all = caches[0].read_logical(0, 0, S)
+        k_np, v_np, q_np = k_all.cpu().numpy(), v_all.cpu().numpy(), bufs.q[0].cpu().numpy()
+        del k_all, v_all
+        times = []
+        for rep in range(4):
+            t0 = time.perf_counter()
+            oracle_mod.tree_attention(q_np, k_np, v_np, tree.mask, P)
+            times.append(time.perf_counter() - t0)
+        out["cpu_attn_s"] = statistics.median(times[1:])
+    return out
 
 
 def machine_probes(torch):
@@ -177,40 +247,6 @@ def machine_probes(torch):
     return out
 
 
-def cpu_baseline(torch, wl, layers_sampled=2):
-    """CPU oracle on a bounded sample: `layers_sampled` attention layers + the full target head +
-    acceptance + compaction of those layers; the per-step figure scales the attention part to 32 layers."""
-    import numpy as np
-    import oracle
-    P, T = wl.P, wl.T
-    S = P + T
-    ks, vs, qs = [], [], []
-    for l in range(layers_sampled):
-        k, v = wl.cache.read_logical(l, 0, S)
-        ks.append(k.cpu().numpy())
-        vs.append(v.cpu().numpy())
-        qs.append(wl.q[l].cpu().numpy())
-    hid = wl.hidden.cpu().numpy()
-    w = wl.w.cpu().numpy()
-    t0 = time.perf_counter()
-    for l in range(layers_sampled):
-        oracle.tree_attention(qs[l], ks[l], vs[l], wl.tree.mask, P)
-    t_attn = (time.perf_counter() - t0) / layers_sampled
-    t0 = time.perf_counter()
-    gt = oracle.argmax(oracle.lm_head(hid, w))
-    t_head = time.perf_counter() - t0
-    t0 = time.perf_counter()
-    a, node, path = oracle.tree_accept(wl.draft_np, gt, wl.tree.positions(P), P, wl.tree.mask, wl.tree.parent)
-    flat = [x.reshape(S, -1).copy() for l in range(layers_sampled) for x in (ks[l], vs[l])]
-    ids = oracle.kv_compact(flat, P, path, gt)
-    t_tail = time.perf_counter() - t0
-    step_us = (t_attn * wl.L + t_head + t_tail) * 1e6
-    return dict(value=round(step_us, 1), unit="us/step", cores=oracle.num_threads(), kind="port",
-                head_and_tail_us=round((t_head + t_tail) * 1e6, 1),
-                sample="%d of %d attention layers timed (x%d extrapolated) + full target head/arg-max + acceptance + compaction; "
-                       "attention %.1f ms/layer, head %.1f ms" % (layers_sampled, wl.L, wl.L, t_attn * 1e3, t_head * 1e3)), (a, ids, gt)
-
-
 def main():
     args = parse_args()
     if args.gpus != 1:
@@ -219,11 +255,15 @@ def main():
         sys.exit(2)
     import numpy as np
     import torch
-    from cpm.cu_amd import lib, ops
-    from cpm.cu_amd.driver import VerifyStep
+    from cpm.cu_amd import lib, ops, synth
+    from cpm.cu_amd.model import PathModel
     lib.get()  # fails loudly without the HIP library
     torch.cuda.set_device(0)
     use_graph = not args.no_graph
+    want_cpu = not args.no_cpu_baseline
+    oracle_mod = None
+    if want_cpu:
+        import oracle as oracle_mod
 
     if args.traffic_probe:
         src = torch.full((256 << 20,), 7, dtype=torch.uint8, device="cuda")
@@ -233,275 +273,255 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    wl = Workload(torch, args.workload, args.accept_depth)
-    ctx_name = "%dK" % (wl.P // 1024) if wl.P % 1024 == 0 else str(wl.P)
-    metric_name = "verify us/step @8B shape, %d-node tree, %s ctx" % (wl.T, ctx_name)
+    shp = synth.MINICPM4_8B
+    cfg = dict(synth.CONFIGS[args.workload])
+    L, T = cfg["layers"], cfg["T"]
+    Hq, Hkv, D, H, V = shp["q_heads"], shp["kv_heads"], shp["head_dim"], shp["hidden"], shp["vocab"]
+    names = [args.workload]
+    if not args.no_contexts and args.workload == "c2_verify_4k":
+        names += ["c4_verify_32k", "c4_verify_128k"]
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(cfg["seed"])
+
+    # ---- the library's model: heads + paged pools sized for the longest context of this run ----
+    kv_sets_of = lambda n: 4 if synth.CONFIGS[n]["prefix"] <= 8192 else 1
+    pages_needed = max(kv_sets_of(n) * ((synth.CONFIGS[n]["prefix"] + synth.CONFIGS[n]["T"] + 255) // 256 + 1) for n in names)
+    page_bytes_all_layers = (L + 1) * 2 * Hkv * 256 * D * 2  # target layers + the drafter's one layer, K and V
+    total_mem = torch.cuda.mem_get_info()[1]
+    want_bytes = pages_needed * page_bytes_all_layers * 1.15 + 3 * V * H * 2 + (1 << 30)
+    memory_limit = min(0.9, want_bytes / total_mem)
+    w_dev = (torch.randn(V, H, device="cuda", dtype=torch.float32, generator=gen) * 0.02).to(torch.float16)
+    w_host = w_dev.cpu().numpy()
+    remap_np = synth.frspec_remap(V, shp["frspec_vocab"], 0)
+    model = PathModel(V, L, H, Hq, Hkv, memory_limit=memory_limit, scale_lmhead=1.0, frspec_vocab=shp["frspec_vocab"], tree_size=T,
+                      num_iter=cfg["num_iter"], topk=cfg["topk"], draft_layers=1, eagle_window=1024)
+    assert model.num_pages >= pages_needed, (model.num_pages, pages_needed)
+    model.load_head(w_host, remap_np)
+    bufs = StepBuffers(torch, L, T, Hq, Hkv, D, H, gen)
+    tree = synth.eagle_tree(cfg["num_iter"], cfg["topk"], T, cfg["seed"])
+
+    main_run = run_context(torch, np, model, synth, oracle_mod, args, args.workload, bufs, tree, use_graph,
+                           kv_sets_of(args.workload), gen, want_cpu)
+    P = main_run["P"]
+    ms_step, ms_attn = main_run["ms_step"], main_run["ms_attn"]
+    a_gpu, ids_gpu = main_run["results"][0]
+    sets_agree = all(r[0] == a_gpu and np.array_equal(r[1], ids_gpu) for r in main_run["results"])
+    ctx_name = "%dK" % (P // 1024) if P % 1024 == 0 else str(P)
+    metric_name = "verify us/step @8B shape, %d-node tree, %s ctx" % (T, ctx_name)
     wl_desc = ("%s: %d layers x (KV append + tree attention, %dq/%dkv heads, d%d, %d-token paged prefix + %d-node tree) + "
-               "target head %dx%d with arg-max + tree acceptance + KV compaction"
-               % (args.workload, wl.L, wl.shape["q_heads"], wl.shape["kv_heads"], wl.shape["head_dim"], wl.P, wl.T,
-                  wl.shape["vocab"], wl.shape["hidden"]))
-    # the head weights are kept in the library's tiled layout, as its model-level loader keeps them
-    w_t = ops.tile_head_weight(wl.w)
-    vs = VerifyStep(wl.cache, w_t, wl.mask, wl.parent, wl.pos, wl.P)
-    # target arg-max once, to rig the draft ids for the chosen accept length
-    gt = ops.lm_head_argmax(wl.hidden, w_t)
-    torch.cuda.synchronize()
-    wl.rig_draft(torch, gt.cpu().numpy())
+               "target head %dx%d with arg-max + tree acceptance + KV compaction, on the library's storage through "
+               "cpmcu_verify_step" % (args.workload, L, Hq, Hkv, D, P, T, V, H))
 
-    def full_step():
-        vs.enqueue(wl.q, wl.k_new, wl.v_new, wl.hidden, wl.draft_ids, attn_out=wl.attn_out, splits=args.splits)
+    flops_attn = lambda Pc: 4.0 * Hq * T * D * (Pc + T)
+    bytes_attn = lambda Pc: 2.0 * (Pc + T) * Hkv * D * 2 + 2.0 * T * Hq * D * 2
+    bytes_head = V * H * 2.0 + T * H * 2.0 + T * 4.0
 
-    # The 32 layers' K/V at 4K context (~150 MB) fit the 256 MB last-level cache, so replays of the step on
-    # one set of pools are partly served from it.  The headline therefore rotates the timed steps over
-    # KV_SETS distinct copies of the pools (step i works on copy i % KV_SETS): every pass over K/V comes
-    # from HBM, as it does in a decode loop that streams the dense layers' weights in between.  Longer
-    # contexts exceed the cache by themselves and use one set.
-    KV_SETS = 4 if wl.P <= 8192 else 1
-    caches = [wl.cache]
-    if KV_SETS > 1:
-        from cpm.cu_amd.kvcache import PagedKVCache
-        for _ in range(KV_SETS - 1):
-            c2 = PagedKVCache(wl.L, wl.cache.Hkv, wl.cache.num_pages, device="cuda", block_table=wl.cache.block_table)
-            for l in range(wl.L):
-                c2.k[l].copy_(wl.cache.k[l])
-                c2.v[l].copy_(wl.cache.v[l])
-            caches.append(c2)
-    rot_steps = [vs] + [VerifyStep(c, w_t, wl.mask, wl.parent, wl.pos, wl.P) for c in caches[1:]]
+    # ---- per-operator timings on the main workload (operator level, same pools and buffers, graph-replayed) ----
+    kernels, frspec, cold, draft, rope_cmp = [], None, None, None, None
+    attn_tflops = flops_attn(P) / (ms_attn * 1e-3) / 1e12
+    attn_name = main_run["attn_plan"][0]
+    kernels.append(dict(kernel=attn_name, launches_per_step=L, us_per_launch=round(ms_attn * 1e3, 2), bound="mfma",
+                        achieved=round(attn_tflops, 2), peak=MFMA_F16_PEAK_TFLOPS, unit="TFLOP/s",
+                        frac=round(attn_tflops / MFMA_F16_PEAK_TFLOPS, 4),
+                        hbm_gbs=round(bytes_attn(P) / (ms_attn * 1e-3) / 1e9, 1), traffic=None,
+                        kv_splits=main_run["attn_plan"][1], workgroups=main_run["attn_plan"][3],
+                        us_per_launch_one_kv_set=round(main_run["ms_attn_one_set"] * 1e3, 2)))
+    if not args.no_operators:
+        reps = max(5, args.steps // 5)
+        w_t = ops.tile_head_weight(w_dev)  # the layout the library's loader keeps
+        cache0 = main_run["caches"][0]
+        mask, parent, pos, clen, kvlen, padded = (main_run[k] for k in ("mask", "parent", "pos", "clen", "kvlen", "padded"))
+        HEAD_REP, TAIL_REP = 4, 8  # several repetitions per graph, so that the graph launch itself does not dominate
+        head_name = ops.head_plan(T, w_t)[0]
 
-    def step_on(st):
-        return lambda: st.enqueue(wl.q, wl.k_new, wl.v_new, wl.hidden, wl.draft_ids, attn_out=wl.attn_out, splits=args.splits)
+        def head_only():
+            for _ in range(HEAD_REP):
+                ops.lm_head_partials(bufs.hidden, w_t)
+        ms_head = timed_torch(torch, head_only, reps, 5) / HEAD_REP  # (the first replays run at ramping clocks)
+        parts = ops.lm_head_partials(bufs.hidden, w_t)
+        best = torch.zeros(2, dtype=torch.int32, device="cuda")
+        path = torch.zeros(T, dtype=torch.int32, device="cuda")
 
-    ms_step, wall_ms = timed_replays(torch, [step_on(st) for st in rot_steps], args.steps, args.warmup, use_graph)
-    results = [st.result() for st in rot_steps]
-    a_gpu, ids_gpu = results[0]
-    sets_agree = all(r[0] == a_gpu and np.array_equal(r[1], ids_gpu) for r in results)
-    ms_step_warm = timed_replays(torch, full_step, max(5, args.steps // 2), 2, use_graph)[0] if KV_SETS > 1 else ms_step
-    del rot_steps
+        def tail_only():  # arg-max finish + acceptance + compaction + ids in one launch
+            for _ in range(TAIL_REP):
+                ops.verify_tail(cache0, bufs.draft_ids, parts, pos, clen, mask, parent, gt_out=bufs.gt, best=best, path=path,
+                                accepted_ids=bufs.accepted)
+        ms_tail = timed_torch(torch, tail_only, reps, 2) / TAIL_REP
+        head_gbs = bytes_head / (ms_head * 1e-3) / 1e9
+        head_tail_gbs = bytes_head / ((ms_head + ms_tail) * 1e-3) / 1e9
+        tail_bytes = 2 * a_gpu * 2 * L * Hkv * D * 2  # compaction: a rows, read + written, in every K and V cache
+        kernels.append(dict(kernel=head_name, launches_per_step=1, us_per_launch=round(ms_head * 1e3, 2), bound="hbm",
+                            achieved=round(head_gbs, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(head_gbs / HBM_PEAK_GBS, 4), traffic=None,
+                            frac_with_tail_launch=round(head_tail_gbs / HBM_PEAK_GBS, 4),
+                            note="the target head's GEMM; its arg-max is finished inside the tail launch (frac_with_tail_launch "
+                                 "charges that whole launch -- acceptance and compaction included -- to the head)"))
+        kernels.append(dict(kernel="verify_tail_kernel", launches_per_step=1, us_per_launch=round(ms_tail * 1e3, 2), bound="hbm",
+                            achieved=round(tail_bytes / (ms_tail * 1e-3) / 1e9, 2), peak=HBM_PEAK_GBS, unit="GB/s",
+                            frac=round(tail_bytes / (ms_tail * 1e-3) / 1e9 / HBM_PEAK_GBS, 5), traffic=None,
+                            note="arg-max finish + acceptance + compaction of %d bytes at accept length %d + ids: one launch of latency, "
+                                 "not bandwidth" % (tail_bytes, a_gpu)))
 
-    # ---- per-operator timings (same inputs, each operator alone, graph-replayed) ----
-    reps = max(5, args.steps // 5)
+        # rotary embedding of the tree rows: fused into the attention kernel (one table per step) against the reference's
+        # order (one in-place launch per layer in front of the attention)
+        inv_freq = torch.tensor((10000.0 ** (-np.arange(64, dtype=np.float64) / 64)).astype(np.float32), device="cuda")
+        q_scratch = [t.clone() for t in bufs.q]
+        k_scratch = [t.clone() for t in bufs.k_new]
 
-    def attn_all_layers():  # with the KV append of the tree rows fused in, as in the step
-        for l in range(wl.L):
-            ops.tree_attention(wl.q[l], wl.cache, l, vs.kv_len, vs.max_kv_len, wl.mask, num_splits=args.splits, out=wl.attn_out[l],
-                               k_new=wl.k_new[l], v_new=wl.v_new[l])
+        def attn_rope_fused():
+            table = ops.rope_table(pos, inv_freq)
+            for l in range(L):
+                ops.tree_attention(bufs.q[l], cache0, l, kvlen, padded, mask, out=bufs.attn_out[l], k_new=bufs.k_new[l],
+                                   v_new=bufs.v_new[l], rope=table)
 
-    HEAD_REP = 4  # several repetitions per graph, so that the graph launch itself does not dominate
+        def attn_rope_separate():
+            table = ops.rope_table(pos, inv_freq)
+            for l in range(L):
+                ops.rope_apply_(table, q_scratch[l], k_scratch[l])
+                ops.tree_attention(q_scratch[l], cache0, l, kvlen, padded, mask, out=bufs.attn_out[l], k_new=k_scratch[l],
+                                   v_new=bufs.v_new[l])
+        rope_cmp = {"fused_us_per_layer": round(timed_torch(torch, attn_rope_fused, reps, 2) / L * 1e3, 2),
+                    "separate_launch_us_per_layer": round(timed_torch(torch, attn_rope_separate, reps, 2) / L * 1e3, 2),
+                    "note": "rotary embedding of q and the appended K rows; table computed once per step; one K/V set"}
+        del q_scratch, k_scratch
 
-    def head_only():
-        for _ in range(HEAD_REP):
-            ops.lm_head_argmax(wl.hidden, w_t, gt=vs.gt)
-
-    TAIL_REP = 8  # several repetitions per graph, so that the graph launch itself does not dominate
-
-    def accept_compact():
-        for _ in range(TAIL_REP):
-            vs.pred.copy_(wl.draft_ids)
-            ops.tree_accept(vs.pred, vs.gt, wl.pos, vs.cache_length, wl.mask, wl.parent, best=vs.best)
-            ops.kv_compact(wl.cache, vs.pred, vs.gt, vs.cache_length, vs.best, wl.T)
-
-    # the one-call tail of verify(): the same two launches also gather the accepted hidden rows, write
-    # next position ids and the packed (a, ids) result (length advance off here: the call is repeated)
-    prev_hidden = torch.zeros_like(wl.hidden)
-    next_pos = torch.zeros(wl.T, dtype=torch.int32, device="cuda")
-    packed = torch.zeros(1 + wl.T, dtype=torch.int32, device="cuda")
-
-    def accept_commit():
-        for _ in range(TAIL_REP):
-            vs.pred.copy_(wl.draft_ids)
-            ops.tree_accept(vs.pred, vs.gt, wl.pos, vs.cache_length, wl.mask, wl.parent, best=vs.best)
-            ops.accept_commit(wl.cache, vs.pred, vs.gt, vs.cache_length, vs.best, wl.T, hidden=wl.hidden, prev_hidden=prev_hidden,
-                              next_position_ids=next_pos, result=packed)
-
-    # rotary embedding of the tree rows: fused into the attention kernel (one table per step) against the
-    # reference's order (one in-place launch per layer in front of the attention)
-    inv_freq = torch.tensor((10000.0 ** (-np.arange(64, dtype=np.float64) / 64)).astype(np.float32), device="cuda")
-    q_scratch = [t.clone() for t in wl.q]
-    k_scratch = [t.clone() for t in wl.k_new]
-
-    def attn_rope_fused():
-        table = ops.rope_table(wl.pos, inv_freq)
-        for l in range(wl.L):
-            ops.tree_attention(wl.q[l], wl.cache, l, vs.kv_len, vs.max_kv_len, wl.mask, num_splits=args.splits, out=wl.attn_out[l],
-                               k_new=wl.k_new[l], v_new=wl.v_new[l], rope=table)
-
-    def attn_rope_separate():
-        table = ops.rope_table(wl.pos, inv_freq)
-        for l in range(wl.L):
-            ops.rope_apply_(table, q_scratch[l], k_scratch[l])
-            ops.tree_attention(q_scratch[l], wl.cache, l, vs.kv_len, vs.max_kv_len, wl.mask, num_splits=args.splits, out=wl.attn_out[l],
-                               k_new=k_scratch[l], v_new=wl.v_new[l])
-
-    ms_attn_warm = timed_replays(torch, attn_all_layers, reps, 2, use_graph)[0] / wl.L
-    ms_attn = ms_attn_warm
-    if KV_SETS > 1:  # as the headline: every pass over K/V from HBM
-        def attn_cold():
-            for c in caches:
-                for l in range(wl.L):
-                    ops.tree_attention(wl.q[l], c, l, vs.kv_len, vs.max_kv_len, wl.mask, num_splits=args.splits, out=wl.attn_out[l],
-                                       k_new=wl.k_new[l], v_new=wl.v_new[l])
-        ms_attn = timed_replays(torch, attn_cold, reps, 2, use_graph)[0] / (wl.L * KV_SETS)
-    ms_rope_fused = timed_replays(torch, attn_rope_fused, reps, 2, use_graph)[0] / wl.L
-    ms_rope_sep = timed_replays(torch, attn_rope_separate, reps, 2, use_graph)[0] / wl.L
-    del q_scratch, k_scratch
-    ms_commit = timed_replays(torch, accept_commit, reps, 2, use_graph)[0] / TAIL_REP
-    ms_head = timed_replays(torch, head_only, reps, 2, use_graph)[0] / HEAD_REP
-    ms_tail = timed_replays(torch, accept_compact, reps, 2, use_graph)[0] / TAIL_REP
-
-    attn_tflops = wl.flops_attention_layer() / (ms_attn * 1e-3) / 1e12
-    attn_gbs = wl.bytes_attention_layer() / (ms_attn * 1e-3) / 1e9
-    head_gbs = wl.bytes_target_head() / (ms_head * 1e-3) / 1e9
-    tail_bytes = 2 * a_gpu * 2 * wl.L * wl.shape["kv_heads"] * wl.shape["head_dim"] * 2  # compaction: a rows, read + written
-    tail_gbs = tail_bytes / (ms_tail * 1e-3) / 1e9
-    kernels = [
-        dict(kernel="tree_attn_split_kernel+tree_attn_combine_kernel", launches_per_step=wl.L, us_per_launch=round(ms_attn * 1e3, 2),
-             bound="mfma", achieved=round(attn_tflops, 2), peak=MFMA_F16_PEAK_TFLOPS, unit="TFLOP/s",
-             frac=round(attn_tflops / MFMA_F16_PEAK_TFLOPS, 4), hbm_gbs=round(attn_gbs, 1), traffic=None,
-             us_per_launch_one_kv_set=round(ms_attn_warm * 1e3, 2)),
-        dict(kernel="head_gemm_chunked_kernel<4,4,256,2>+head_argmax_finalize_kernel", launches_per_step=1, us_per_launch=round(ms_head * 1e3, 2),
-             bound="hbm", achieved=round(head_gbs, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(head_gbs / HBM_PEAK_GBS, 4),
-             traffic=None),
-        dict(kernel="tree_accept_kernel+kv_compact_kernel+accepted_ids_kernel", launches_per_step=1,
-             us_per_launch=round(ms_tail * 1e3, 2), bound="hbm", achieved=round(tail_gbs, 2), peak=HBM_PEAK_GBS, unit="GB/s",
-             frac=round(tail_gbs / HBM_PEAK_GBS, 5), traffic=None,
-             note="accepted rows read and written once in every layer's K and V: %d bytes at accept length %d; three launches of latency, "
-                  "not bandwidth" % (tail_bytes, a_gpu)),
-    ]
-    if args.workload == "c2_verify_4k" and args.splits == 0:
-        for k in kernels:
-            k["traffic"] = MEASURED_TRAFFIC_KIB[k["kernel"]] * 1024
-            k["traffic_unit"] = "bytes/launch"
-    dominant = max(kernels, key=lambda k: k["us_per_launch"] * k["launches_per_step"])
-    roofline = {k: dominant[k] for k in ("bound", "achieved", "peak", "unit", "frac", "traffic")}
-    roofline["kernel"] = dominant["kernel"]
-    roofline["us_per_launch"] = dominant["us_per_launch"]
-
-    # ---- FR-Spec draft head (config 3 shape), reported beside the verify step ----
-    from cpm.cu_amd import synth
-    remap = torch.from_numpy(synth.frspec_remap(wl.shape["vocab"], wl.shape["frspec_vocab"], 0)).cuda()
-    w_sub = ops.tile_head_weight(wl.w, remap)  # remap_copy fused with the re-tiling
-    hid10 = wl.hidden[:10].contiguous()
-    def fr_head():
-        for _ in range(HEAD_REP):
-            ops.frspec_head_topk(hid10, w_sub, remap, 10)
-    ms_fr = timed_replays(torch, fr_head, reps, 2, use_graph)[0] / HEAD_REP
-    fr_bytes = wl.shape["frspec_vocab"] * wl.shape["hidden"] * 2.0 + 10 * wl.shape["hidden"] * 2.0 + 10 * 10 * 6.0
-    fr_gbs = fr_bytes / (ms_fr * 1e-3) / 1e9
-    frspec = dict(kernel="head_gemm_chunked_kernel<1,2,512,2>+topk_row_kernel", us_per_call=round(ms_fr * 1e3, 2), bound="hbm",
-                  achieved=round(fr_gbs, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(fr_gbs / HBM_PEAK_GBS, 4))
-
-    # ---- the FR-Spec head from a cold cache ----
-    # Its matrix (268 MB) nearly fits the last-level cache as well, so replays on one copy are partly served
-    # from it.  Here every replay walks several distinct copies, so each pass misses.
-    cold = None
-    draft = None
-    if KV_SETS > 1:
+        # ---- FR-Spec draft head (config 3 shape) ----
+        remap = torch.from_numpy(remap_np).cuda()
         FR_SETS = 3
-        w_subs = [w_sub] + [ops.tile_head_weight(wl.w, remap) for _ in range(FR_SETS - 1)]
+        w_subs = [ops.tile_head_weight(w_dev, remap) for _ in range(FR_SETS)]  # remap_copy fused with the re-tiling
+        hid10 = bufs.hidden[:10].contiguous()
+        fr_name = ops.head_plan(10, w_subs[0])[0] + "+topk_row_kernel<true>"
 
+        def fr_head():
+            for _ in range(HEAD_REP):
+                ops.frspec_head_topk(hid10, w_subs[0], remap, 10)
+        ms_fr = timed_torch(torch, fr_head, reps, 5) / HEAD_REP
+        fr_bytes = shp["frspec_vocab"] * H * 2.0 + 10 * H * 2.0 + 10 * 10 * 6.0
+        fr_gbs = fr_bytes / (ms_fr * 1e-3) / 1e9
+        frspec = dict(kernel=fr_name, us_per_call=round(ms_fr * 1e3, 2), bound="hbm", achieved=round(fr_gbs, 1), peak=HBM_PEAK_GBS,
+                      unit="GB/s", frac=round(fr_gbs / HBM_PEAK_GBS, 4))
+
+        # the same head from a cold cache: its matrix (268 MB) nearly fits the last-level cache, so replays on one copy are
+        # partly served from it; here every replay walks several distinct copies, so each pass misses
         def fr_cold():
             for w in w_subs:
                 ops.frspec_head_topk(hid10, w, remap, 10)
-        ms_fr_cold = timed_replays(torch, fr_cold, reps, 2, use_graph)[0] / FR_SETS
+        ms_fr_cold = timed_torch(torch, fr_cold, reps, 5) / FR_SETS
+        cold = {"frspec_head_us_per_call": round(ms_fr_cold * 1e3, 2), "frspec_weight_copies_rotated": FR_SETS,
+                "frspec_frac_hbm": round(fr_bytes / (ms_fr_cold * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                "note": "the FR-Spec head with every replay walking distinct copies of its matrix, so that no pass is served "
+                        "from the 256 MB last-level cache; frspec_head above replays one copy"}
 
         # ---- the draft side of the path: one whole draft of the FR-Spec drafter (6 rounds of 10) ----
-        # Per round: the drafter layer's own attention (10 queries, mask over 10*d columns, block sliding
-        # window of 1024 tokens, its own one-layer cache), the FR-Spec head with log-softmax + top-10 + id
-        # map-back, and the tree bookkeeping kernel; the final top-59 + tree build at the end.  The dense
-        # parts of the drafter layer (fc, projections, FFN) are not on the path and are not run; the head
-        # reads a different copy of its matrix every round, as it would after their weights.
-        from cpm.cu_amd.kvcache import PagedKVCache
-        k_it, n_it = 10, 6
+        # Per round: the drafter layer's own attention (10 queries, mask over 10*d columns, block sliding window of 1024
+        # tokens, its own one-layer cache), the FR-Spec head with log-softmax + top-10 + id map-back, and the tree
+        # bookkeeping kernel; the final top-59 + tree build at the end.  The dense parts of the drafter layer (fc,
+        # projections, FFN) are not on the path and are not run; the head reads a different copy of its matrix every
+        # round, as it would after their weights.
+        k_it, n_it = cfg["topk"], cfg["num_iter"]
         dtree = ops.DraftTree(k_it, n_it, remap)
-        dcache = PagedKVCache(1, wl.cache.Hkv, wl.cache.num_pages, device="cuda", block_table=wl.cache.block_table)
-        dcache.k[0].copy_(wl.cache.k[0])
-        dcache.v[0].copy_(wl.cache.v[0])
-        hid1 = wl.hidden[:1].contiguous()
-        qd = wl.q[0][:k_it].contiguous()
-        kd = wl.k_new[0][:k_it].contiguous()
-        vd = wl.v_new[0][:k_it].contiguous()
-        d_len = [torch.tensor([wl.P + k_it * d], dtype=torch.int32, device="cuda") for d in range(n_it)]
+        dcache = model.cache(block_table=main_run["tables"][0], num_layers=L + 1)  # layer L: the drafter's own cache
+        dcache.k[L][: main_run["npages"]].copy_(dcache.k[0][: main_run["npages"]])
+        dcache.v[L][: main_run["npages"]].copy_(dcache.v[0][: main_run["npages"]])
+        hid1 = bufs.hidden[:1].contiguous()
+        qd, kd, vd = bufs.q[0][:k_it].contiguous(), bufs.k_new[0][:k_it].contiguous(), bufs.v_new[0][:k_it].contiguous()
+        d_len = [torch.tensor([P + k_it * d], dtype=torch.int32, device="cuda") for d in range(n_it)]
         d_out = torch.empty_like(qd)
-        tree_ids = torch.full((wl.T,), -1, dtype=torch.int32, device="cuda")
+        tree_ids = torch.full((T,), -1, dtype=torch.int32, device="cuda")
 
         def draft_path():
             r = ops.frspec_head_topk(hid1, w_subs[0], remap, k_it)
             dtree.begin(r["val"][0], r["pos"][0])
             for d in range(1, n_it):
-                ops.tree_attention(qd, dcache, 0, d_len[d], vs.max_kv_len, dtree.draft_mask, out=d_out, k_new=kd, v_new=vd,
+                ops.tree_attention(qd, dcache, L, d_len[d], padded, dtree.draft_mask, out=d_out, k_new=kd, v_new=vd,
                                    mask_k_range=k_it * d, block_window_size=1024)
                 r = ops.frspec_head_topk(hid10, w_subs[d % FR_SETS], remap, k_it)
                 dtree.extend(d, r["val"], r["pos"])
-            dtree.finish(wl.T, vs.cache_length, tree_draft_ids=tree_ids)
-        ms_draft = timed_replays(torch, draft_path, reps, 2, use_graph)[0]
-        draft = {"us_per_draft": round(ms_draft * 1e3, 1), "rounds": n_it, "topk_per_round": k_it, "tree_size": wl.T,
+            dtree.finish(T, clen, tree_draft_ids=tree_ids)
+        ms_draft = timed_torch(torch, draft_path, reps, 2)
+        draft = {"us_per_draft": round(ms_draft * 1e3, 1), "rounds": n_it, "topk_per_round": k_it, "tree_size": T,
                  "operators": "6 x (FR-Spec head + log-softmax + top-10 + id map-back) + 5 x drafter-layer attention "
                               "(window 1024) + tree bookkeeping (begin, 5 x extend, finish)"}
-        del w_subs, dcache, dtree
-        cold = {"frspec_head_us_per_call": round(ms_fr_cold * 1e3, 2), "frspec_weight_copies_rotated": FR_SETS,
-                "frspec_frac_hbm": round(fr_bytes / (ms_fr_cold * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
-                "note": "the FR-Spec head with every replay walking distinct copies of its matrix, so that no pass is served "
-                        "from the 256 MB last-level cache; frspec_head above replays one copy"}
-    del w_sub, caches
-    torch.cuda.empty_cache()
+        del w_subs, dtree, dcache, w_t
+        torch.cuda.empty_cache()
+
+    if args.workload == "c2_verify_4k":
+        for k in kernels:
+            kib = MEASURED_TRAFFIC["kib_per_launch"].get(k["kernel"])
+            if kib is not None:
+                k["traffic"] = kib * 1024
+                k["traffic_unit"] = "bytes/launch"
+    dominant = max(kernels, key=lambda k: k["us_per_launch"] * k["launches_per_step"])
+    roofline = {k: dominant[k] for k in ("bound", "achieved", "peak", "unit", "frac", "traffic")}
+    roofline["kernel"] = dominant["kernel"]
+    roofline["us_per_launch"] = dominant["us_per_launch"]
 
     # ---- CPU oracle on the host cores + parity of the step's integer results ----
     cpu = None
     parity = None
-    if not args.no_cpu_baseline:
-        import oracle
-        cpu, (a_cpu, ids_cpu, gt_cpu) = cpu_baseline(torch, wl)
-        gt_gpu = vs.gt.cpu().numpy()
-        a_st, _, path_st = oracle.tree_accept(wl.draft_np, gt_gpu, wl.tree.positions(wl.P), wl.P, wl.tree.mask, wl.tree.parent)
+    if want_cpu:
+        hid = bufs.hidden.cpu().numpy()
+        head_times, gt_cpu = [], None
+        for rep in range(4):  # 1 warm-up + 3 timed
+            t0 = time.perf_counter()
+            gt_cpu = oracle_mod.argmax(oracle_mod.lm_head(hid, w_host))
+            head_times.append(time.perf_counter() - t0)
+        t_head = statistics.median(head_times[1:])
+        tail_times = []
+        S = P + T
+        # one layer's two caches as they were before the compaction: the prefix from the pool, the tree rows from the inputs
+        kp_, vp_ = main_run["caches"][0].read_logical(0, 0, P)
+        k_new0, v_new0 = bufs.k_new[0].cpu().numpy().reshape(T, -1), bufs.v_new[0].cpu().numpy().reshape(T, -1)
+        flat0 = [np.concatenate([kp_.cpu().numpy().reshape(P, -1), k_new0]), np.concatenate([vp_.cpu().numpy().reshape(P, -1), v_new0])]
+        for rep in range(4):
+            flat = [x.copy() for x in flat0]
+            t0 = time.perf_counter()
+            a_cpu, node_cpu, path_cpu = oracle_mod.tree_accept(main_run["draft_np"], gt_cpu, tree.positions(P), P, tree.mask, tree.parent)
+            ids_cpu = oracle_mod.kv_compact(flat, P, path_cpu, gt_cpu)
+            tail_times.append(time.perf_counter() - t0)
+        t_tail = statistics.median(tail_times[1:]) * L  # one layer's two caches timed, all layers' extrapolated
+        t_attn = main_run["cpu_attn_s"]
+        step_us = (t_attn * L + t_head + t_tail) * 1e6
+        cpu = dict(value=round(step_us, 1), unit="us/step", cores=oracle_mod.num_threads(), kind="port",
+                   head_and_tail_us=round((t_head + t_tail) * 1e6, 1),
+                   sample="1 of %d attention layers (x%d extrapolated) + the full target head/arg-max + acceptance + compaction of one "
+                          "layer's caches (x%d); each timed 4 times, first discarded, median of 3; attention %.1f ms/layer, head %.1f ms"
+                          % (L, L, L, t_attn * 1e3, t_head * 1e3))
+        gt_gpu = main_run["gt_np"]
+        a_st, _, path_st = oracle_mod.tree_accept(main_run["draft_np"], gt_gpu, tree.positions(P), P, tree.mask, tree.parent)
+        # the compacted rows of the first and the last layer (first K/V set) against the oracle's compaction of the same rows
+        rows_ok = a_gpu == len(path_st) and np.array_equal(flat[0][P:P + a_gpu], k_new0[path_cpu])
+        for l, (kd_, vd_) in main_run["compacted"].items():
+            kn, vn = bufs.k_new[l].cpu().numpy().reshape(T, -1), bufs.v_new[l].cpu().numpy().reshape(T, -1)
+            rows_ok = bool(rows_ok and np.array_equal(kd_, kn[path_st]) and np.array_equal(vd_, vn[path_st]))
         parity = dict(accept_length_gpu=a_gpu, accept_length_oracle=int(a_cpu),
                       ids_equal_oracle=bool(a_gpu == a_cpu and np.array_equal(ids_gpu, ids_cpu)),
                       staged_equal=bool(a_gpu == a_st and np.array_equal(ids_gpu, gt_gpu[path_st])),
-                      kv_sets_agree=bool(sets_agree),
-                      argmax_rows_equal=int((gt_gpu == gt_cpu).sum()), rows=int(wl.T))
+                      compacted_rows_equal=rows_ok, kv_sets_agree=bool(sets_agree),
+                      argmax_rows_equal=int((gt_gpu == gt_cpu).sum()), rows=int(T))
 
-    # ---- the same step at longer contexts ----
-    contexts = {str(wl.P): round(ms_step * 1e3, 1)}
-    ctx_attn = {str(wl.P): round(ms_attn * 1e3, 2)}
-    if not args.no_contexts and args.workload == "c2_verify_4k":
-        w_keep, hid_keep = wl.w, wl.hidden
-        del vs, wl
+    # ---- the same step at longer contexts (same model, pools refilled) ----
+    contexts = {str(P): round(ms_step * 1e3, 1)}
+    ctx_attn = {str(P): dict(us_per_layer=round(ms_attn * 1e3, 2), tflops=round(attn_tflops, 1),
+                             frac_mfma=round(attn_tflops / MFMA_F16_PEAK_TFLOPS, 4), kernel=attn_name,
+                             step_minus_attention_us=round((ms_step - L * ms_attn) * 1e3, 1))}
+    main_run.pop("caches", None)
+    for name in names[1:]:
+        r = run_context(torch, np, model, synth, oracle_mod, args, name, bufs, tree, use_graph, kv_sets_of(name), gen, want_cpu)
+        Pc = r["P"]
+        contexts[str(Pc)] = round(r["ms_step"] * 1e3, 1)
+        tf = flops_attn(Pc) / (r["ms_attn"] * 1e-3) / 1e12
+        ctx_attn[str(Pc)] = dict(us_per_layer=round(r["ms_attn"] * 1e3, 2), tflops=round(tf, 1), frac_mfma=round(tf / MFMA_F16_PEAK_TFLOPS, 4),
+                                 kernel=r["attn_plan"][0], step_minus_attention_us=round((r["ms_step"] - L * r["ms_attn"]) * 1e3, 1))
+        if cpu is not None:
+            cpu.setdefault("contexts", {})[str(Pc)] = dict(
+                attention_ms_per_layer=round(r["cpu_attn_s"] * 1e3, 1),
+                us_per_step_extrapolated=round(r["cpu_attn_s"] * 1e6 * L + cpu["head_and_tail_us"], 1),
+                sample="1 of %d attention layers timed 4 times, first discarded, median of 3" % L)
+        r.pop("caches", None)
+        del r
         torch.cuda.empty_cache()
-        for name in ("c4_verify_32k", "c4_verify_128k"):
-            w2 = Workload.__new__(Workload)
-            Workload.__init__(w2, torch, name, args.accept_depth)
-            w2.w, w2.hidden = w_keep, hid_keep  # same head
-            v2 = VerifyStep(w2.cache, w_t, w2.mask, w2.parent, w2.pos, w2.P)
-            w2.rig_draft(torch, gt.cpu().numpy())
-            n = max(3, args.steps // 5)
-            ms2 = timed_replays(torch, lambda: v2.enqueue(w2.q, w2.k_new, w2.v_new, w2.hidden, w2.draft_ids, attn_out=w2.attn_out,
-                                                          splits=args.splits), n, 2, use_graph)[0]
 
-            def attn2():
-                for l in range(w2.L):
-                    ops.tree_attention(w2.q[l], w2.cache, l, v2.kv_len, v2.max_kv_len, w2.mask, num_splits=args.splits, out=w2.attn_out[l],
-                                       k_new=w2.k_new[l], v_new=w2.v_new[l])
-            ms_a2 = timed_replays(torch, attn2, n, 2, use_graph)[0] / w2.L
-            contexts[str(w2.P)] = round(ms2 * 1e3, 1)
-            tf2 = w2.flops_attention_layer() / (ms_a2 * 1e-3) / 1e12
-            ctx_attn[str(w2.P)] = dict(us_per_layer=round(ms_a2 * 1e3, 2), tflops=round(tf2, 1),
-                                       frac_mfma=round(tf2 / MFMA_F16_PEAK_TFLOPS, 4))
-            if cpu is not None:
-                # the CPU oracle on ONE layer of this context (bounded sample), extrapolated to the step with the
-                # head and tail times of the 4K sample
-                import oracle
-                S2 = w2.P + w2.T
-                k2, v2k = w2.cache.read_logical(0, 0, S2)
-                k2, v2k, q2 = k2.cpu().numpy(), v2k.cpu().numpy(), w2.q[0].cpu().numpy()
-                t0 = time.perf_counter()
-                oracle.tree_attention(q2, k2, v2k, w2.tree.mask, w2.P)
-                t_layer = time.perf_counter() - t0
-                cpu.setdefault("contexts", {})[str(w2.P)] = dict(
-                    attention_ms_per_layer=round(t_layer * 1e3, 1),
-                    us_per_step_extrapolated=round(t_layer * 1e6 * w2.L + cpu["head_and_tail_us"], 1),
-                    sample="1 of %d attention layers timed once" % w2.L)
-                del k2, v2k, q2
-            del v2, w2
-            torch.cuda.empty_cache()
+    model.close()
 
     # ---- what the matrix pipes sustain on this GPU (last, so that its heat does not touch the figures above) ----
     probes = None if args.no_probes else machine_probes(torch)
@@ -511,8 +531,7 @@ def main():
             roofline["measured_ceiling"] = ceiling
             roofline["frac_of_measured_ceiling"] = round(roofline["achieved"] / ceiling, 4)
         for v in ctx_attn.values():
-            if isinstance(v, dict):
-                v["frac_of_measured_ceiling"] = round(v["tflops"] / ceiling, 4)
+            v["frac_of_measured_ceiling"] = round(v["tflops"] / ceiling, 4)
 
     out = {
         "metric": metric_name,
@@ -527,19 +546,19 @@ def main():
         "vs_baseline": None,
         "dtype": "f16",
         "data": "synthetic",
-        "config": {"workload": wl_desc, "batch": 1, "graph_replay": use_graph, "kv_splits": args.splits or "auto", "kv_sets_rotated": KV_SETS},
-        "wall_ms_per_step": round(wall_ms, 5),
-        "us_per_step_one_kv_set": round(ms_step_warm * 1e3, 1),
+        "config": {"workload": wl_desc, "batch": 1, "library_graph": use_graph, "kv_splits": main_run["attn_plan"][1],
+                   "kv_sets_rotated": kv_sets_of(args.workload),
+                   "launches_per_step": L * (2 if main_run["attn_plan"][1] > 1 else 1) + 2},
+        "wall_ms_per_step": round(main_run["wall_ms"], 5),
+        "us_per_step_one_kv_set": round(main_run["ms_one_set"] * 1e3, 1),
         "roofline": roofline,
         "machine_probes": probes,
         "kernels": kernels,
+        "traffic_source": MEASURED_TRAFFIC["source"],
         "frspec_head": frspec,
         "cold_cache": cold,
         "draft_path": draft,
-        "attention_with_rope": {"fused_us_per_layer": round(ms_rope_fused * 1e3, 2), "separate_launch_us_per_layer": round(ms_rope_sep * 1e3, 2),
-                                "note": "rotary embedding of q and the appended K rows; table computed once per step"},
-        "commit_tail": {"kernel": "tree_accept_kernel+kv_compact_kernel(with hidden-row gather)+accepted_ids_kernel(ids, positions, packed result)",
-                        "us_per_call": round(ms_commit * 1e3, 2)},
+        "attention_with_rope": rope_cmp,
         "contexts_us_per_step": contexts,
         "attention_by_context": ctx_attn,
         "cpu_baseline": cpu,

@@ -15,9 +15,14 @@ Options& options();
 // lm_head.hip -- the streaming GEMM with its two epilogues.
 constexpr int kHeadModeStats = 0;
 constexpr int kHeadModeArgmax = 1;
+// (row-walking kernel by row blocks of hidden, or the K-chunked kernel <NB, NP, KC, NBUF>)
+enum class HeadShape { Row1, Row2, Row4, Row8, C_1_2_512_2, C_1_4_256_2, C_2_4_256_4, C_2_4_256_2, C_4_4_256_4, C_4_4_256_2, C_8_4_128_2,
+                       C_2_4_512_2, C_4_4_128_4, C_8_2_128_2 };
+const char* head_shape_name(HeadShape s);
+// dry_run: only choose the kernel shape and grid (reported through shape_out / grid_out), launch nothing.
 int launch_head_gemm(const void* hidden, const void* w, int w_layout, int n, int V, int H, int apply_scale, float head_scale,
                      int mode, void* logits, float* part_a, float* part_b, int* grid_out, int* stride_out,
-                     hipStream_t st);
+                     hipStream_t st, HeadShape* shape_out = nullptr, bool dry_run = false);
 int head_max_grid();
 
 // topk.hip -- exact top-k (value descending, ties -> lower index) with an optional fused

@@ -572,10 +572,70 @@ int pick_nb(int n) { return n <= 16 ? 1 : n <= 32 ? 2 : n <= 64 ? 4 : 8; }
 
 }  // namespace
 
+const char* head_shape_name(HeadShape s) {
+    switch (s) {
+        case HeadShape::Row1: return "head_gemm_kernel<1>";
+        case HeadShape::Row2: return "head_gemm_kernel<2>";
+        case HeadShape::Row4: return "head_gemm_kernel<4>";
+        case HeadShape::Row8: return "head_gemm_kernel<8>";
+        case HeadShape::C_1_2_512_2: return "head_gemm_chunked_kernel<1,2,512,2>";
+        case HeadShape::C_1_4_256_2: return "head_gemm_chunked_kernel<1,4,256,2>";
+        case HeadShape::C_2_4_256_4: return "head_gemm_chunked_kernel<2,4,256,4>";
+        case HeadShape::C_2_4_256_2: return "head_gemm_chunked_kernel<2,4,256,2>";
+        case HeadShape::C_4_4_256_4: return "head_gemm_chunked_kernel<4,4,256,4>";
+        case HeadShape::C_4_4_256_2: return "head_gemm_chunked_kernel<4,4,256,2>";
+        case HeadShape::C_8_4_128_2: return "head_gemm_chunked_kernel<8,4,128,2>";
+        case HeadShape::C_2_4_512_2: return "head_gemm_chunked_kernel<2,4,512,2>";
+        case HeadShape::C_4_4_128_4: return "head_gemm_chunked_kernel<4,4,128,4>";
+        case HeadShape::C_8_2_128_2: return "head_gemm_chunked_kernel<8,2,128,2>";
+    }
+    return "?";
+}
+
+namespace {
+
+// Kernel shapes chosen by measurement on MI355X (73448 x 4096 and 32768 x 4096 heads).
+HeadShape pick_head_shape(int NB, int H, bool w_tiled, int nch, int npasses, int nrb, int G, int* full_passes, int* rem_blocks) {
+    if (H % 256 != 0 || (!w_tiled && nch <= 2)) {
+        // every wave walks whole rows; hidden rows LDS-resident (<= 16 rows) or chunked per row block.
+        // Best for row-major weights with <= 16 rows (1 KB runs per row), and the fallback for odd H.
+        return NB == 1 ? HeadShape::Row1 : NB == 2 ? HeadShape::Row2 : NB == 4 ? HeadShape::Row4 : HeadShape::Row8;
+    }
+    if (w_tiled) {
+        // one sweep (all passes fit the accumulator sets) with a partly filled last pass: share it
+        // (the option head_share_last_pass = 0 keeps the plain mapping; tests compare the two)
+        const int rem = nrb - (npasses - 1) * G * kHeadWaves;
+        if (npasses <= 4 && rem < G * kHeadWaves && options().head_share_last_pass) {  // <= NP of every shape below
+            *full_passes = npasses - 1;
+            *rem_blocks = rem;
+        }
+        // W register buffers: two when a wave works on several row blocks per chunk (the next block's
+        // group is the prefetch; 72 vs 65 % of HBM peak for 60 rows, 81 vs 79 % for 10), four when there
+        // is a single pass; the FR-Spec head (32768 rows = one block per wave, up to 16 hidden rows) does best
+        // with 512-column chunks in two buffers: 47.4 us with its top-k, against 50.0 (256 x 4) and 52.0 (256 x 2)
+        const bool deep = npasses == 1;
+        switch (NB) {
+            case 1: return deep ? HeadShape::C_1_2_512_2 : HeadShape::C_1_4_256_2;
+            case 2: return deep ? HeadShape::C_2_4_256_4 : HeadShape::C_2_4_256_2;
+            case 4: return deep ? HeadShape::C_4_4_256_4 : HeadShape::C_4_4_256_2;
+            default: return HeadShape::C_8_4_128_2;  // 165 vs 190 us with <8,2,128,2> at 128 rows
+        }
+    }
+    switch (NB) {
+        // <= 16 rows whose K range exceeds two LDS buffers (H >= 6144): the row-walking kernel, chunked
+        case 1: return HeadShape::Row1;
+        case 2: return HeadShape::C_2_4_512_2;
+        case 4: return HeadShape::C_4_4_128_4;
+        default: return HeadShape::C_8_2_128_2;
+    }
+}
+
+}  // namespace
+
 // Shared launcher of the GEMM; returns the grid size used (= number of partial rows) in *grid_out.
 int launch_head_gemm(const void* hidden, const void* w, int w_layout, int n, int V, int H, int apply_scale, float head_scale,
                      int mode, void* logits, float* part_a, float* part_b, int* grid_out, int* stride_out,
-                     hipStream_t st) {
+                     hipStream_t st, HeadShape* shape_out, bool dry_run) {
     CPMCU_CHECK_ARG(w_layout == CPMCU_W_ROW_MAJOR || w_layout == CPMCU_W_TILED, "lm_head: unknown weight layout %d", w_layout);
     const int NB = pick_nb(n);
     const int kc_max = 2048 / NB;
@@ -606,53 +666,29 @@ int launch_head_gemm(const void* hidden, const void* w, int w_layout, int n, int
     CPMCU_CHECK_ARG(G <= head_max_grid(), "lm_head: %d workgroups exceed the %d rows of the partial planes", G, head_max_grid());
     *grid_out = G;
     *stride_out = NB * 16;
-    // Kernel shapes chosen by measurement on MI355X (73448 x 4096 and 32768 x 4096 heads).
-    if (H % 256 != 0 || (!p.w_tiled && p.nch <= 2)) {
-        // every wave walks whole rows; hidden rows LDS-resident (<= 16 rows) or chunked per row block.
-        // Best for row-major weights with <= 16 rows (1 KB runs per row), and the fallback for odd H.
-        switch (NB) {
-            case 1: hipLaunchKernelGGL(head_gemm_kernel<1>, dim3(G), dim3(kHeadThreads), 0, st, p); break;
-            case 2: hipLaunchKernelGGL(head_gemm_kernel<2>, dim3(G), dim3(kHeadThreads), 0, st, p); break;
-            case 4: hipLaunchKernelGGL(head_gemm_kernel<4>, dim3(G), dim3(kHeadThreads), 0, st, p); break;
-            default: hipLaunchKernelGGL(head_gemm_kernel<8>, dim3(G), dim3(kHeadThreads), 0, st, p); break;
-        }
-    } else if (p.w_tiled) {
-        // one sweep (all passes fit the accumulator sets) with a partly filled last pass: share it
-        // (the option head_share_last_pass = 0 keeps the plain mapping; tests compare the two)
-        const int rem = nrb - (p.npasses - 1) * G * kHeadWaves;
-        if (p.npasses <= 4 && rem < G * kHeadWaves && options().head_share_last_pass) {  // <= NP of every shape below
-            p.full_passes = p.npasses - 1;
-            p.rem_blocks = rem;
-        }
-        // W register buffers: two when a wave works on several row blocks per chunk (the next block's
-        // group is the prefetch; 72 vs 65 % of HBM peak for 60 rows, 81 vs 79 % for 10), four when there
-        // is a single pass; the FR-Spec head (32768 rows = one block per wave, up to 16 hidden rows) does best
-        // with 512-column chunks in two buffers: 47.4 us with its top-k, against 50.0 (256 x 4) and 52.0 (256 x 2)
-        const bool deep = p.npasses == 1;
-        switch (NB) {
-            case 1:
-                if (deep) hipLaunchKernelGGL((head_gemm_chunked_kernel<1, 2, 512, 2>), dim3(G), dim3(kHeadThreads), 0, st, p);
-                else hipLaunchKernelGGL((head_gemm_chunked_kernel<1, 4, 256, 2>), dim3(G), dim3(kHeadThreads), 0, st, p);
-                break;
-            case 2:
-                if (deep) hipLaunchKernelGGL((head_gemm_chunked_kernel<2, 4, 256, 4>), dim3(G), dim3(kHeadThreads), 0, st, p);
-                else hipLaunchKernelGGL((head_gemm_chunked_kernel<2, 4, 256, 2>), dim3(G), dim3(kHeadThreads), 0, st, p);
-                break;
-            case 4:
-                if (deep) hipLaunchKernelGGL((head_gemm_chunked_kernel<4, 4, 256, 4>), dim3(G), dim3(kHeadThreads), 0, st, p);
-                else hipLaunchKernelGGL((head_gemm_chunked_kernel<4, 4, 256, 2>), dim3(G), dim3(kHeadThreads), 0, st, p);
-                break;
-            default: hipLaunchKernelGGL((head_gemm_chunked_kernel<8, 4, 128, 2>), dim3(G), dim3(kHeadThreads), 0, st, p); break;  // 165 vs 190 us with <8,2,128,2> at 128 rows
-        }
-    } else {
-        switch (NB) {
-            // <= 16 rows whose K range exceeds two LDS buffers (H >= 6144): the row-walking kernel, chunked
-            case 1: hipLaunchKernelGGL(head_gemm_kernel<1>, dim3(G), dim3(kHeadThreads), 0, st, p); break;
-            case 2: hipLaunchKernelGGL((head_gemm_chunked_kernel<2, 4, 512, 2>), dim3(G), dim3(kHeadThreads), 0, st, p); break;
-            case 4: hipLaunchKernelGGL((head_gemm_chunked_kernel<4, 4, 128, 4>), dim3(G), dim3(kHeadThreads), 0, st, p); break;
-            default: hipLaunchKernelGGL((head_gemm_chunked_kernel<8, 2, 128, 2>), dim3(G), dim3(kHeadThreads), 0, st, p); break;
-        }
+    const HeadShape shape = pick_head_shape(NB, H, p.w_tiled, p.nch, p.npasses, nrb, G, &p.full_passes, &p.rem_blocks);
+    if (shape_out) *shape_out = shape;
+    if (dry_run) return CPMCU_OK;
+#define CPMCU_HEAD_ROW(nb) hipLaunchKernelGGL(head_gemm_kernel<nb>, dim3(G), dim3(kHeadThreads), 0, st, p)
+#define CPMCU_HEAD_CHUNKED(nb, np, kc, nbuf) hipLaunchKernelGGL((head_gemm_chunked_kernel<nb, np, kc, nbuf>), dim3(G), dim3(kHeadThreads), 0, st, p)
+    switch (shape) {
+        case HeadShape::Row1: CPMCU_HEAD_ROW(1); break;
+        case HeadShape::Row2: CPMCU_HEAD_ROW(2); break;
+        case HeadShape::Row4: CPMCU_HEAD_ROW(4); break;
+        case HeadShape::Row8: CPMCU_HEAD_ROW(8); break;
+        case HeadShape::C_1_2_512_2: CPMCU_HEAD_CHUNKED(1, 2, 512, 2); break;
+        case HeadShape::C_1_4_256_2: CPMCU_HEAD_CHUNKED(1, 4, 256, 2); break;
+        case HeadShape::C_2_4_256_4: CPMCU_HEAD_CHUNKED(2, 4, 256, 4); break;
+        case HeadShape::C_2_4_256_2: CPMCU_HEAD_CHUNKED(2, 4, 256, 2); break;
+        case HeadShape::C_4_4_256_4: CPMCU_HEAD_CHUNKED(4, 4, 256, 4); break;
+        case HeadShape::C_4_4_256_2: CPMCU_HEAD_CHUNKED(4, 4, 256, 2); break;
+        case HeadShape::C_8_4_128_2: CPMCU_HEAD_CHUNKED(8, 4, 128, 2); break;
+        case HeadShape::C_2_4_512_2: CPMCU_HEAD_CHUNKED(2, 4, 512, 2); break;
+        case HeadShape::C_4_4_128_4: CPMCU_HEAD_CHUNKED(4, 4, 128, 4); break;
+        case HeadShape::C_8_2_128_2: CPMCU_HEAD_CHUNKED(8, 2, 128, 2); break;
     }
+#undef CPMCU_HEAD_ROW
+#undef CPMCU_HEAD_CHUNKED
     CPMCU_LAUNCH_CHECK();
     return CPMCU_OK;
 }
@@ -709,7 +745,7 @@ static int lm_head_argmax_on(const void* hidden, const void* w, int w_layout, in
                              float head_scale, void* logits, int32_t* gt, float* part_a, hipStream_t st) {
     float* part_b = part_a + (size_t)head_max_grid() * 128;
     int G = 0, stride = 0;
-    int rc = launch_head_gemm(hidden, w, w_layout, n, V, H, apply_scale, head_scale, kHeadModeArgmax, logits, part_a, part_b, &G, &stride, st);
+    int rc = launch_head_gemm(hidden, w, w_layout, n, V, H, apply_scale, head_scale, kHeadModeArgmax, logits, part_a, part_b, &G, &stride, st, nullptr, false);
     if (rc != CPMCU_OK) return rc;
     if (gt) {
         hipLaunchKernelGGL(head_argmax_finalize_kernel, dim3(n), dim3(256), 0, st, part_a, part_b, G, stride, gt);
@@ -730,6 +766,19 @@ extern "C" int cpmcu_lm_head_argmax(const void* hidden, const void* w, int w_lay
     return lm_head_argmax_on(hidden, w, w_layout, n, V, H, apply_scale, head_scale, logits, gt, (float*)workspace, resolve_stream(stream));
 }
 
+// Which kernel a head call of this shape launches (no launch): the name for reports.
+extern "C" int cpmcu_head_plan(int n, int V, int H, int w_layout, char* kernel_name, size_t kernel_name_bytes, int* num_workgroups) {
+    CPMCU_CHECK_ARG(n >= 1 && n <= 128 && V >= 1 && H >= 1, "head_plan: bad shape n=%d V=%d H=%d", n, V, H);
+    HeadShape shape;
+    int G = 0, stride = 0;
+    int rc = launch_head_gemm(nullptr, nullptr, w_layout, n, V, H, 0, 1.f, kHeadModeArgmax, nullptr, nullptr, nullptr, &G, &stride, nullptr,
+                              &shape, true);
+    if (rc != CPMCU_OK) return rc;
+    if (kernel_name && kernel_name_bytes > 0) snprintf(kernel_name, kernel_name_bytes, "%s", head_shape_name(shape));
+    if (num_workgroups) *num_workgroups = G;
+    return CPMCU_OK;
+}
+
 // The GEMM alone: the arg-max stays in per-workgroup partials for cpmcu_verify_tail to finish.
 extern "C" int cpmcu_lm_head_partials(const void* hidden, const void* w, int w_layout, int n, int V, int H, int apply_scale,
                                       float head_scale, void* logits, void* workspace, size_t workspace_bytes, int* num_partials,
@@ -742,7 +791,7 @@ extern "C" int cpmcu_lm_head_partials(const void* hidden, const void* w, int w_l
     float* part_a = (float*)workspace;
     float* part_b = part_a + (size_t)head_max_grid() * 128;
     return launch_head_gemm(hidden, w, w_layout, n, V, H, apply_scale, head_scale, kHeadModeArgmax, logits, part_a, part_b, num_partials,
-                            partial_stride, resolve_stream(stream));
+                            partial_stride, resolve_stream(stream), nullptr, false);
 }
 
 // ---- the same operator for callers that cannot allocate ----

@@ -668,6 +668,8 @@ extern "C" int cpmcu_model_pointers(int layer, uint64_t* k_pool, uint64_t* v_poo
     return CPMCU_OK;
 }
 
+extern "C" uint64_t cpmcu_stream(void) { return (uint64_t)(uintptr_t)resolve_stream(nullptr); }
+
 extern "C" int cpmcu_synchronize(void) {
     CPMCU_HIP(hipStreamSynchronize(resolve_stream(nullptr)));
     return CPMCU_OK;

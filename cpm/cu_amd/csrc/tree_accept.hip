@@ -223,11 +223,29 @@ constexpr int kTailThreads = 256;
 __global__ __launch_bounds__(kTailThreads) void verify_tail_kernel(TailParams p) {
     __shared__ int32_t s_gt[kMaxTree];
     __shared__ int32_t s_path[kMaxTree];
+    __shared__ uint64_t s_mask[kMaxTree][2];
     __shared__ uint64_t s_key[kTailThreads];
     __shared__ uint64_t s_correct[2];
     __shared__ uint32_t s_best[2];
+    __shared__ int32_t s_pages[2];
     const int tid = threadIdx.x;
     const int T = p.T, W = p.W;
+    const int i = tid;
+
+    // Everything the acceptance reads from memory is requested first, so that it arrives under the arg-max
+    // finish: the launch is a chain of memory round trips, and these need not be links of it.
+    const int P = p.cache_length[0];
+    int my_draft = 0, my_parent = 0, my_pos = 0;
+    uint64_t mw[2] = {0, 0};
+    if (i < T) {
+        my_draft = p.draft[i];
+        my_parent = p.parent[i];
+        my_pos = p.pos[i];
+        mw[0] = p.mask[(size_t)i * W];
+        if (W > 1) mw[1] = p.mask[(size_t)i * W + 1];
+    }
+    // the tree rows [P, P + T) lie in at most two logical pages
+    if (tid < 2) s_pages[tid] = p.block_table[P / kPage + tid * ((P + T - 1) / kPage > P / kPage ? 1 : 0)];
 
     // ---- target arg-max per node: given, or the finish of the head's per-workgroup partials (largest value,
     // lowest index among equals: the same 64-bit keys as the head's own finish kernel) ----
@@ -239,11 +257,21 @@ __global__ __launch_bounds__(kTailThreads) void verify_tail_kernel(TailParams p)
         const int clanes = kTailThreads / rows;   // partial lanes per row
         uint64_t bestk = 0;
         if (row < T) {
-            for (int c = tid / rows; c < p.num_partials; c += clanes) {
-                const float a = p.part_a[(size_t)c * rows + row];
-                const uint32_t b = (uint32_t)__float_as_int(p.part_b[(size_t)c * rows + row]);
-                const uint64_t k = argmax_key(a, b);
-                bestk = k > bestk ? k : bestk;
+            constexpr int kBatch = 32;  // partials of one row requested together: one round trip per batch
+            for (int c0 = tid / rows; c0 < p.num_partials; c0 += clanes * kBatch) {
+                float av[kBatch];
+                uint32_t bv[kBatch];
+#pragma unroll
+                for (int u = 0; u < kBatch; ++u) {
+                    const int c = min(c0 + u * clanes, p.num_partials - 1);  // clamp: a repeat changes nothing in a maximum
+                    av[u] = p.part_a[(size_t)c * rows + row];
+                    bv[u] = (uint32_t)__float_as_int(p.part_b[(size_t)c * rows + row]);
+                }
+#pragma unroll
+                for (int u = 0; u < kBatch; ++u) {
+                    const uint64_t k = argmax_key(av[u], bv[u]);
+                    bestk = k > bestk ? k : bestk;
+                }
             }
         }
         s_key[tid] = bestk;
@@ -257,23 +285,24 @@ __global__ __launch_bounds__(kTailThreads) void verify_tail_kernel(TailParams p)
             s_gt[tid] = (int32_t)(0xFFFFFFFFu - (uint32_t)k);
         }
     }
+    if (i < kMaxTree) {
+        s_mask[i][0] = mw[0];
+        s_mask[i][1] = mw[1];
+        s_path[i] = i < T ? i : 0;  // (defined even where stale positions scatter nothing)
+    }
     __syncthreads();
 
     // ---- acceptance (as tree_accept_kernel above, on 128 of the threads) ----
-    const int i = tid;
-    const bool ok = (i == 0) || (i < T && p.draft[i] == s_gt[p.parent[i]]);
+    const bool ok = (i == 0) || (i < T && my_draft == s_gt[my_parent]);
     const uint64_t ballot = __ballot(ok);
     if (i < 128 && (i & 63) == 0) s_correct[i >> 6] = ballot;
     __syncthreads();
-    const int P = p.cache_length[0];
     bool full = i < T;
     if (full) {
-        for (int w = 0; w < W; ++w) {
-            const uint64_t mw = p.mask[(size_t)i * W + w];
-            if ((s_correct[w] & mw) != mw) full = false;
-        }
+        for (int w = 0; w < W; ++w)
+            if ((s_correct[w] & mw[w]) != mw[w]) full = false;
     }
-    const uint32_t key = full ? ((uint32_t)(p.pos[i] - P + 1) << 8) | (255u - (__brev((uint32_t)i) >> 24)) : (1u << 8) | 255u;
+    const uint32_t key = full ? ((uint32_t)(my_pos - P + 1) << 8) | (255u - (__brev((uint32_t)i) >> 24)) : (1u << 8) | 255u;
     const uint32_t wkey = wave_reduce_b32(key, [](uint32_t a, uint32_t b) { return a > b ? a : b; });
     if (i < 128 && (i & 63) == 0) s_best[i >> 6] = wkey;
     __syncthreads();
@@ -281,10 +310,10 @@ __global__ __launch_bounds__(kTailThreads) void verify_tail_kernel(TailParams p)
     const int win = (int)(__brev(255u - (bkey & 255u)) >> 24);
     int a = (int)(bkey >> 8);
     a = a < T ? a : T;
-    if (tid < kMaxTree) s_path[tid] = tid < T ? tid : 0;  // (defined even where stale positions scatter nothing)
+    if (i < T && ((s_mask[win][i >> 6] >> (i & 63)) & 1ull) && (unsigned)(my_pos - P) < (unsigned)T) s_path[my_pos - P] = i;
     __syncthreads();
-    if (i < T && ((p.mask[(size_t)win * W + (i >> 6)] >> (i & 63)) & 1ull) && (unsigned)(p.pos[i] - P) < (unsigned)T) s_path[p.pos[i] - P] = i;
-    __syncthreads();
+    const int page_lo = P / kPage;
+    auto page_of = [&](int token) { return s_pages[token / kPage - page_lo]; };
 
     const int blk = blockIdx.x;
     if (blk < p.num_cache_blocks) {
@@ -302,14 +331,14 @@ __global__ __launch_bounds__(kTailThreads) void verify_tail_kernel(TailParams p)
                 const bool act = d < a && s_path[d] != d;  // a row that stays where it is moves nothing
                 if (act) {
                     const int ts = P + s_path[d];
-                    const int pg = p.block_table[ts / kPage];
+                    const int pg = page_of(ts);
                     x = *reinterpret_cast<const f16x8*>(pool + (((size_t)pg * p.Hkv + g) * kPage + ts % kPage) * kHeadDim + ch * 8);
                 }
                 asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                 __syncthreads();
                 if (act) {
                     const int td = P + d;
-                    const int pg = p.block_table[td / kPage];
+                    const int pg = page_of(td);
                     *reinterpret_cast<f16x8*>(pool + (((size_t)pg * p.Hkv + g) * kPage + td % kPage) * kHeadDim + ch * 8) = x;
                 }
             }
@@ -322,14 +351,14 @@ __global__ __launch_bounds__(kTailThreads) void verify_tail_kernel(TailParams p)
                 const bool act = d < a && s_path[d] != d;
                 if (act) {
                     const int ts = P + s_path[d];
-                    const int pg = p.block_table[ts / kPage];
+                    const int pg = page_of(ts);
                     x = pool[(((size_t)pg * p.Hkv + g) * kHeadDim + dd) * kPage + v_slot16(ts % kPage)];
                 }
                 asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
                 __syncthreads();
                 if (act) {
                     const int td = P + d;
-                    const int pg = p.block_table[td / kPage];
+                    const int pg = page_of(td);
                     pool[(((size_t)pg * p.Hkv + g) * kHeadDim + dd) * kPage + v_slot16(td % kPage)] = x;
                 }
             }

@@ -748,10 +748,45 @@ int choose_groups(int T, int group, int Hkv, int max_kv_len) {
     return units >= 4 && (long long)ntiles * units >= (long long)kLongRunTiles * 256 ? 1 : 2;
 }
 
+// Shape of one attention launch: which kernel shape, how many KV splits and M-tiles.
+struct LaunchPlan {
+    int span;        // keys the stream can hold: the whole context, or with a window its blocks plus the T new rows
+                     // (the window starts on a block boundary at or above P - block_window_size)
+    int kv_groups, num_mtiles, num_splits;
+};
+LaunchPlan plan_launch(int T, int group, int Hkv, int max_kv_len, int block_window_size, int num_splits_override) {
+    LaunchPlan pl;
+    const int window_blocks = block_window_size / 128;
+    pl.span = max_kv_len;
+    if (window_blocks > 0 && window_blocks * 128 + T < pl.span) pl.span = window_blocks * 128 + T;
+    pl.kv_groups = choose_groups(T, group, Hkv, pl.span);
+    pl.num_mtiles = ceil_div(group * T, rows_per_wg(pl.kv_groups));
+    pl.num_splits = num_splits_override > 0 ? num_splits_override : choose_splits(T, group, Hkv, pl.span, pl.kv_groups);
+    // a split keeps the physical page ids of its range in LDS
+    const int min_splits = ceil_div(ceil_div(pl.span, kPage) + 2, kMaxPagesPerSplit - 2);
+    if (pl.num_splits < min_splits) pl.num_splits = min_splits;
+    return pl;
+}
+
 }  // namespace
 }  // namespace cpmcu
 
 using namespace cpmcu;
+
+// Which kernels an attention call of this shape launches (no launch): names and geometry for reports.
+extern "C" int cpmcu_tree_attention_plan(int T, int Hq, int Hkv, int max_kv_len, int with_rope, int block_window_size,
+                                         int num_splits_override, char* kernel_names, size_t kernel_names_bytes, int* num_splits,
+                                         int* kv_groups, int* num_workgroups) {
+    CPMCU_CHECK_ARG(T >= 1 && T <= kMaxTree && Hkv >= 1 && Hq >= Hkv && Hq % Hkv == 0 && max_kv_len >= T, "tree_attention_plan: bad shape");
+    const LaunchPlan pl = plan_launch(T, Hq / Hkv, Hkv, max_kv_len, block_window_size, num_splits_override);
+    if (kernel_names && kernel_names_bytes > 0)
+        snprintf(kernel_names, kernel_names_bytes, "tree_attn_split_kernel<%d,%s>%s", pl.kv_groups, with_rope ? "true" : "false",
+                 pl.num_splits > 1 ? "+tree_attn_combine_kernel" : "");
+    if (num_splits) *num_splits = pl.num_splits;
+    if (kv_groups) *kv_groups = pl.kv_groups;
+    if (num_workgroups) *num_workgroups = kXcds * ceil_div(pl.num_splits * Hkv, kXcds) * pl.num_mtiles;
+    return CPMCU_OK;
+}
 
 extern "C" size_t cpmcu_tree_attention_workspace_bytes(int T, int Hq, int Hkv, int max_kv_len) {
     (void)max_kv_len;
@@ -802,18 +837,13 @@ static int tree_attention_impl(const void* q, void* k_pool, void* v_pool,
     p.Hq = Hq;
     p.Hkv = Hkv;
     p.group = group;
-    // Keys the stream can hold: the whole context, or with a window its blocks plus the T new rows
-    // (the window starts on a block boundary at or above P - block_window_size).
     p.window_blocks = block_window_size / 128;
-    int span = max_kv_len;
-    if (p.window_blocks > 0 && p.window_blocks * 128 + T < span) span = p.window_blocks * 128 + T;
-    const int G = choose_groups(T, group, Hkv, span);
-    p.num_mtiles = ceil_div(group * T, rows_per_wg(G));
+    const LaunchPlan plan = plan_launch(T, group, Hkv, max_kv_len, block_window_size, num_splits_override);
+    const int span = plan.span;
+    const int G = plan.kv_groups;
+    p.num_mtiles = plan.num_mtiles;
     p.rows_pad = p.num_mtiles * rows_per_wg(G);
-    p.num_splits = num_splits_override > 0 ? num_splits_override : choose_splits(T, group, Hkv, span, G);
-    // a split keeps the physical page ids of its range in LDS
-    const int min_splits = ceil_div(ceil_div(span, kPage) + 2, kMaxPagesPerSplit - 2);
-    if (p.num_splits < min_splits) p.num_splits = min_splits;
+    p.num_splits = plan.num_splits;
     CPMCU_CHECK_ARG(p.num_splits <= kMaxSplits, "tree_attention: max_kv_len=%d is beyond the supported context", max_kv_len);
     p.ntiles_max = ceil_div(span, kTileN);
     p.table_pages = ceil_div(max_kv_len, kPage);

@@ -40,6 +40,7 @@ SIGNATURES = {
     "cpmcu_draft_head": (c_int, [c_int, c_u64, c_u64, c_u64, c_u64]),
     "cpmcu_set_block_table": (c_int, [_P, c_int]),
     "cpmcu_model_pointers": (c_int, [c_int, ctypes.POINTER(c_u64), ctypes.POINTER(c_u64), ctypes.POINTER(c_u64), ctypes.POINTER(c_int)]),
+    "cpmcu_stream": (c_u64, []),
     "cpmcu_synchronize": (c_int, []),
     "cpmcu_shutdown": (c_int, []),
     "cpmcu_kv_append": (c_int, [_P, _P, _P, _P, _P, _P, c_int, c_int, _P]),
@@ -47,6 +48,7 @@ SIGNATURES = {
     "cpmcu_tree_attention": (c_int, [_P, _P, _P, _P, _P, c_int, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_float, _P, _P, c_size_t, c_int, _P]),
     "cpmcu_tree_attention_rope": (c_int, [_P, _P, _P, _P, _P, c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_float, _P, _P, c_size_t, c_int, _P]),
     "cpmcu_tree_attention_window": (c_int, [_P, _P, _P, _P, _P, c_int, _P, _P, _P, c_int, _P, c_int, c_int, c_int, c_int, c_int, c_float, _P, _P, c_size_t, c_int, _P]),
+    "cpmcu_tree_attention_plan": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_char_p, c_size_t, ctypes.POINTER(c_int), ctypes.POINTER(c_int), ctypes.POINTER(c_int)]),
     "cpmcu_rope_table": (c_int, [_P, _P, c_int, _P, _P]),
     "cpmcu_rope_apply": (c_int, [_P, c_int, c_int, c_int, _P, _P, _P]),
     "cpmcu_gather_rows": (c_int, [_P, _P, c_int, c_int, _P, _P]),
@@ -55,6 +57,7 @@ SIGNATURES = {
     "cpmcu_head_weight_tile": (c_int, [_P, _P, c_int, c_int, _P, _P]),
     "cpmcu_frspec_head_topk": (c_int, [_P, _P, c_int, _P, c_int, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, c_size_t, _P]),
     "cpmcu_lm_head_argmax": (c_int, [_P, _P, c_int, c_int, c_int, c_int, c_int, c_float, _P, _P, _P, c_size_t, _P]),
+    "cpmcu_head_plan": (c_int, [c_int, c_int, c_int, c_int, c_char_p, c_size_t, ctypes.POINTER(c_int)]),
     "cpmcu_lm_head_partials": (c_int, [_P, _P, c_int, c_int, c_int, c_int, c_int, c_float, _P, _P, c_size_t, ctypes.POINTER(c_int), ctypes.POINTER(c_int), _P]),
     "cpmcu_lm_head_argmax_static_scratch_bytes": (c_size_t, []),
     "cpmcu_lm_head_argmax_static": (c_int, [_P, _P, c_int, c_int, c_int, c_int, c_int, c_float, _P, _P, _P]),

@@ -77,6 +77,10 @@ class PathModel:
                            p(accepted_ids), p(prev_hidden), p(next_position_ids), p(result), 1 if advance_length else 0,
                            1 if cuda_graph else 0)
 
+    def stream(self):
+        """The library's stream as a torch stream object (events recorded on it time the library's launches)."""
+        return torch.cuda.ExternalStream(self.L.raw.cpmcu_stream())
+
     def synchronize(self):
         self.L.synchronize()
 

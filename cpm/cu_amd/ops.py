@@ -338,3 +338,22 @@ class DraftTree:
         _lib().draft_tree_finish(_ptr(self.state), self.k, self.num_iter, T, _ptr(cache_length), _ptr(self.remap),
                                  _ptr(tree_draft_ids), _ptr(pos), _ptr(mask), _ptr(parent), _stream())
         return tree_draft_ids, pos, mask, parent
+
+
+def attention_plan(T, Hq, Hkv, max_kv_len, rope=False, block_window_size=0, num_splits=0):
+    """(kernel names, KV splits, KV groups per workgroup, workgroups) of a tree-attention call of this shape."""
+    buf = ctypes.create_string_buffer(160)
+    ns, g, wg = ctypes.c_int(0), ctypes.c_int(0), ctypes.c_int(0)
+    _lib().tree_attention_plan(T, Hq, Hkv, int(max_kv_len), 1 if rope else 0, int(block_window_size), int(num_splits), buf, 160,
+                               ctypes.byref(ns), ctypes.byref(g), ctypes.byref(wg))
+    return buf.value.decode(), ns.value, g.value, wg.value
+
+
+def head_plan(n, w):
+    """(GEMM kernel name, workgroups) of a head call with n hidden rows on weight matrix w."""
+    _, layout, V = _weight(w)
+    H = w.H if isinstance(w, TiledWeight) else w.shape[1]
+    buf = ctypes.create_string_buffer(96)
+    wg = ctypes.c_int(0)
+    _lib().head_plan(n, V, H, layout, buf, 96, ctypes.byref(wg))
+    return buf.value.decode(), wg.value

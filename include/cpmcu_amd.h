@@ -207,6 +207,9 @@ int cpmcu_set_block_table(const int32_t* host_table, int n);
  * num_hidden_layers + drafter num_layers) are the drafter's own caches. */
 int cpmcu_model_pointers(int layer, uint64_t* k_pool, uint64_t* v_pool, uint64_t* block_table, int* num_pages);
 
+/* No reference counterpart: the library's own stream (a hipStream_t as an integer; created on first use), for
+ * harnesses that record events on it or order their own streams against it.  0 if it cannot be created. */
+uint64_t cpmcu_stream(void);
 /* Synchronise the library's stream. */
 int cpmcu_synchronize(void);
 /* Free everything the global model owns (the reference never frees). */
@@ -260,6 +263,13 @@ int cpmcu_tree_attention(const void* q, void* k_pool, void* v_pool, const int32_
                          const uint64_t* mask, int mask_words, int mask_k_range, int T, int Hq, int Hkv, float scale,
                          void* out,
                          void* workspace, size_t workspace_bytes, int num_splits_override, void* stream);
+
+/* No reference counterpart: which kernels a cpmcu_tree_attention* call of this shape launches, without
+ * launching -- for reports that must name the instantiation actually taken.  kernel_names receives e.g.
+ * "tree_attn_split_kernel<2,false>+tree_attn_combine_kernel"; the outputs may each be NULL. */
+int cpmcu_tree_attention_plan(int T, int Hq, int Hkv, int max_kv_len, int with_rope, int block_window_size,
+                              int num_splits_override, char* kernel_names, size_t kernel_names_bytes, int* num_splits,
+                              int* kv_groups, int* num_workgroups);
 
 /* Rotary embedding of the T tree rows -- RotaryEmbedding::prefill / rotary_embedding_kernel,
  * src/model/rotary.cuh:7-34,61-63, which Attention::decode runs on q and k before the append
@@ -341,6 +351,10 @@ int cpmcu_frspec_head_topk(const void* hidden, const void* w, int w_layout, cons
 int cpmcu_lm_head_argmax(const void* hidden, const void* w, int w_layout, int n, int V, int H, int apply_scale,
                          float head_scale, void* logits, int32_t* gt, void* workspace,
                          size_t workspace_bytes, void* stream);
+
+/* No reference counterpart: the GEMM kernel a head call of this shape launches (e.g.
+ * "head_gemm_chunked_kernel<4,4,256,2>") and its workgroup count, without launching. */
+int cpmcu_head_plan(int n, int V, int H, int w_layout, char* kernel_name, size_t kernel_name_bytes, int* num_workgroups);
 
 /* The target head's GEMM without its finishing launch: the per-workgroup arg-max partials stay in
  * `workspace` (same size as for cpmcu_lm_head_argmax) and are finished by cpmcu_verify_tail, which is their
