@@ -65,9 +65,13 @@ def parse_args():
     return ap.parse_args()
 
 
-def timed_torch(torch, fn, steps, warmup, use_graph=True):
-    """Operator timings on a torch side stream: fn() captured once into a graph (unless disabled), `warmup` untimed and
-    exactly `steps` timed calls between two events on that stream.  fn may be a list: the calls cycle through it."""
+WARM_MS = 40.0  # operator timings first replay for this long: clocks settle over tens of milliseconds after a change of kernel mix
+
+
+def timed_torch(torch, fn, steps, warmup, use_graph=True, warm_ms=0.0):
+    """Operator timings on a torch side stream: fn() captured once into a graph (unless disabled), `warmup` untimed calls
+    (and further ones until warm_ms have passed) and exactly `steps` timed calls between two events on that stream.
+    fn may be a list: the calls cycle through it."""
     fns = list(fn) if isinstance(fn, (list, tuple)) else [fn]
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
@@ -85,6 +89,11 @@ def timed_torch(torch, fn, steps, warmup, use_graph=True):
         for i in range(warmup):
             runs[i % len(runs)]()
         stream.synchronize()
+        t_w = time.perf_counter()
+        while (time.perf_counter() - t_w) * 1e3 < warm_ms:
+            for i in range(len(runs)):
+                runs[i]()
+            stream.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
         e0.record(stream)
@@ -334,10 +343,32 @@ def main():
         HEAD_REP, TAIL_REP = 4, 8  # several repetitions per graph, so that the graph launch itself does not dominate
         head_name = ops.head_plan(T, w_t)[0]
 
-        def head_only():
+        def timed_model(fn, n_rep):
+            """fn(): model-level calls, recorded into a library graph and replayed on the library's stream."""
+            gid = model.capture(fn)
+            st_ = model.stream()
+            t_w = time.perf_counter()
+            while (time.perf_counter() - t_w) * 1e3 < WARM_MS:  # (the first replays run at ramping clocks)
+                model.replay(gid)
+                model.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(st_)
+            for _ in range(n_rep):
+                model.replay(gid)
+            e1.record(st_)
+            model.synchronize()
+            return e0.elapsed_time(e1) / n_rep
+
+        # the target head on the library's own copy of the weights (cpmcu_decode_lm_head: GEMM + arg-max finish)
+        def head_model():
+            for _ in range(HEAD_REP):
+                model.L.decode_lm_head(T, bufs.hidden.data_ptr(), 0, bufs.gt.data_ptr())
+        ms_head_model = timed_model(head_model, reps) / HEAD_REP
+
+        def head_only():  # the GEMM alone, on a separately allocated copy of the tiled weights
             for _ in range(HEAD_REP):
                 ops.lm_head_partials(bufs.hidden, w_t)
-        ms_head = timed_torch(torch, head_only, reps, 5) / HEAD_REP  # (the first replays run at ramping clocks)
+        ms_head = timed_torch(torch, head_only, reps, 2, warm_ms=WARM_MS) / HEAD_REP
         parts = ops.lm_head_partials(bufs.hidden, w_t)
         best = torch.zeros(2, dtype=torch.int32, device="cuda")
         path = torch.zeros(T, dtype=torch.int32, device="cuda")
@@ -346,15 +377,22 @@ def main():
             for _ in range(TAIL_REP):
                 ops.verify_tail(cache0, bufs.draft_ids, parts, pos, clen, mask, parent, gt_out=bufs.gt, best=best, path=path,
                                 accepted_ids=bufs.accepted)
-        ms_tail = timed_torch(torch, tail_only, reps, 2) / TAIL_REP
+        ms_tail = timed_torch(torch, tail_only, reps, 2, warm_ms=WARM_MS) / TAIL_REP
         head_gbs = bytes_head / (ms_head * 1e-3) / 1e9
         head_tail_gbs = bytes_head / ((ms_head + ms_tail) * 1e-3) / 1e9
         tail_bytes = 2 * a_gpu * 2 * L * Hkv * D * 2  # compaction: a rows, read + written, in every K and V cache
+        head_model_gbs = bytes_head / (ms_head_model * 1e-3) / 1e9
         kernels.append(dict(kernel=head_name, launches_per_step=1, us_per_launch=round(ms_head * 1e3, 2), bound="hbm",
                             achieved=round(head_gbs, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(head_gbs / HBM_PEAK_GBS, 4), traffic=None,
                             frac_with_tail_launch=round(head_tail_gbs / HBM_PEAK_GBS, 4),
-                            note="the target head's GEMM; its arg-max is finished inside the tail launch (frac_with_tail_launch "
-                                 "charges that whole launch -- acceptance and compaction included -- to the head)"))
+                            note="the target head's GEMM on a separately allocated copy of the weights; in the step its arg-max is "
+                                 "finished inside the tail launch (frac_with_tail_launch charges that whole launch -- acceptance and "
+                                 "compaction included -- to the head)"))
+        kernels.append(dict(kernel=head_name + "+head_argmax_finalize_kernel", launches_per_step=0, us_per_launch=round(ms_head_model * 1e3, 2),
+                            bound="hbm", achieved=round(head_model_gbs, 1), peak=HBM_PEAK_GBS, unit="GB/s",
+                            frac=round(head_model_gbs / HBM_PEAK_GBS, 4), traffic=None,
+                            note="the target head with its arg-max as an operator of its own (cpmcu_decode_lm_head on the library's "
+                                 "weights, two launches); not part of the step, which finishes the arg-max in its tail"))
         kernels.append(dict(kernel="verify_tail_kernel", launches_per_step=1, us_per_launch=round(ms_tail * 1e3, 2), bound="hbm",
                             achieved=round(tail_bytes / (ms_tail * 1e-3) / 1e9, 2), peak=HBM_PEAK_GBS, unit="GB/s",
                             frac=round(tail_bytes / (ms_tail * 1e-3) / 1e9 / HBM_PEAK_GBS, 5), traffic=None,
@@ -394,18 +432,30 @@ def main():
         def fr_head():
             for _ in range(HEAD_REP):
                 ops.frspec_head_topk(hid10, w_subs[0], remap, 10)
-        ms_fr = timed_torch(torch, fr_head, reps, 5) / HEAD_REP
+        ms_fr = timed_torch(torch, fr_head, reps, 2, warm_ms=WARM_MS) / HEAD_REP
         fr_bytes = shp["frspec_vocab"] * H * 2.0 + 10 * H * 2.0 + 10 * 10 * 6.0
         fr_gbs = fr_bytes / (ms_fr * 1e-3) / 1e9
         frspec = dict(kernel=fr_name, us_per_call=round(ms_fr * 1e3, 2), bound="hbm", achieved=round(fr_gbs, 1), peak=HBM_PEAK_GBS,
                       unit="GB/s", frac=round(fr_gbs / HBM_PEAK_GBS, 4))
+
+        # through the library's own sub-matrix and buffers (cpmcu_draft_head)
+        fr_val = torch.zeros((10, 10), dtype=torch.float16, device="cuda")
+        fr_pos = torch.zeros((10, 10), dtype=torch.int32, device="cuda")
+        fr_ids = torch.zeros((10, 10), dtype=torch.int32, device="cuda")
+
+        def fr_model():
+            for _ in range(HEAD_REP):
+                model.L.draft_head(10, hid10.data_ptr(), fr_val.data_ptr(), fr_pos.data_ptr(), fr_ids.data_ptr())
+        ms_fr_model = timed_model(fr_model, reps) / HEAD_REP
+        frspec["model_level_us_per_call"] = round(ms_fr_model * 1e3, 2)
+        frspec["model_level_frac"] = round(fr_bytes / (ms_fr_model * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)
 
         # the same head from a cold cache: its matrix (268 MB) nearly fits the last-level cache, so replays on one copy are
         # partly served from it; here every replay walks several distinct copies, so each pass misses
         def fr_cold():
             for w in w_subs:
                 ops.frspec_head_topk(hid10, w, remap, 10)
-        ms_fr_cold = timed_torch(torch, fr_cold, reps, 5) / FR_SETS
+        ms_fr_cold = timed_torch(torch, fr_cold, reps, 2, warm_ms=WARM_MS) / FR_SETS
         cold = {"frspec_head_us_per_call": round(ms_fr_cold * 1e3, 2), "frspec_weight_copies_rotated": FR_SETS,
                 "frspec_frac_hbm": round(fr_bytes / (ms_fr_cold * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                 "note": "the FR-Spec head with every replay walking distinct copies of its matrix, so that no pass is served "
@@ -437,10 +487,45 @@ def main():
                 r = ops.frspec_head_topk(hid10, w_subs[d % FR_SETS], remap, k_it)
                 dtree.extend(d, r["val"], r["pos"])
             dtree.finish(T, clen, tree_draft_ids=tree_ids)
-        ms_draft = timed_torch(torch, draft_path, reps, 2)
-        draft = {"us_per_draft": round(ms_draft * 1e3, 1), "rounds": n_it, "topk_per_round": k_it, "tree_size": T,
+        ms_draft_cold = timed_torch(torch, draft_path, reps, 2)
+
+        # the same draft through the library's own model-level calls (drafter state, FR-Spec sub-matrix and the drafter
+        # layer's cache owned by the library), recorded once into a library graph and replayed on the library's stream.
+        # One copy of the matrix here: part of it stays in the last-level cache from round to round.
+        next_ids = torch.zeros(k_it, dtype=torch.int32, device="cuda")
+        prows = torch.zeros(k_it, dtype=torch.int32, device="cuda")
+        dmask = torch.zeros(k_it, dtype=torch.int64, device="cuda")
+        t_pos = torch.zeros(T, dtype=torch.int32, device="cuda")
+        t_mask = torch.zeros(T, dtype=torch.int64, device="cuda")
+        t_par = torch.zeros(T, dtype=torch.int32, device="cuda")
+        model.set_block_table(main_run["tables"][0])
+        torch.cuda.synchronize()
+
+        def draft_model_level():
+            model.draft_round(0, hid1, next_ids, None, dmask)
+            for d in range(1, n_it):
+                model.draft_attention(0, k_it, padded, qd, kd, vd, d_len[d], dmask, k_it * d, d_out)
+                model.draft_round(d, hid10, next_ids, prows, dmask)
+            model.draft_finish(tree_ids, t_pos, clen, t_mask, t_par)
+        gid = model.capture(draft_model_level)
+        lib_stream = model.stream()
+        for _ in range(3):
+            model.replay(gid)
+        model.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(lib_stream)
+        for _ in range(reps):
+            model.replay(gid)
+        e1.record(lib_stream)
+        model.synchronize()
+        ms_draft = e0.elapsed_time(e1) / reps
+        draft = {"us_per_draft": round(ms_draft * 1e3, 1), "us_per_draft_cold_matrix": round(ms_draft_cold * 1e3, 1),
+                 "rounds": n_it, "topk_per_round": k_it, "tree_size": T,
                  "operators": "6 x (FR-Spec head + log-softmax + top-10 + id map-back) + 5 x drafter-layer attention "
-                              "(window 1024) + tree bookkeeping (begin, 5 x extend, finish)"}
+                              "(window 1024) + tree bookkeeping (begin, 5 x extend, finish)",
+                 "note": "us_per_draft: cpmcu_draft_round / cpmcu_draft_attention / cpmcu_draft_finish on the library's model, "
+                         "replayed as a library graph; us_per_draft_cold_matrix: the same operators with every round reading a "
+                         "different copy of the FR-Spec matrix (as after the drafter layer's dense weights)"}
         del w_subs, dtree, dcache, w_t
         torch.cuda.empty_cache()
 
@@ -450,7 +535,7 @@ def main():
             if kib is not None:
                 k["traffic"] = kib * 1024
                 k["traffic_unit"] = "bytes/launch"
-    dominant = max(kernels, key=lambda k: k["us_per_launch"] * k["launches_per_step"])
+    dominant = max(kernels, key=lambda k: k["us_per_launch"] * k["launches_per_step"])  # (operators outside the step count 0)
     roofline = {k: dominant[k] for k in ("bound", "achieved", "peak", "unit", "frac", "traffic")}
     roofline["kernel"] = dominant["kernel"]
     roofline["us_per_launch"] = dominant["us_per_launch"]

@@ -127,6 +127,15 @@ PYBIND11_MODULE(C, m) {
               check(cpmcu_draft_head(n, hidden, topk_val, topk_pos, topk_ids));
           },
           "FR-Spec draft head + log-softmax + top-k + id map-back");
+    m.def("draft_round",
+          [](int d, std::uintptr_t hidden, std::uintptr_t next_ids, std::uintptr_t parent_rows, std::uintptr_t draft_mask) {
+              check(cpmcu_draft_round(d, hidden, next_ids, parent_rows, draft_mask));
+          },
+          "One round of draft() without the drafter's dense layers: FR-Spec head + log-softmax + top-k + tree bookkeeping");
+    m.def("draft_finish",
+          [](std::uintptr_t tree_draft_ids, std::uintptr_t tree_position_ids, std::uintptr_t cache_length, std::uintptr_t attn_mask,
+             std::uintptr_t tree_parent) { check(cpmcu_draft_finish(tree_draft_ids, tree_position_ids, cache_length, attn_mask, tree_parent)); },
+          "The end of draft(): the final selection and the tree the verify step consumes");
     m.def("verify_step",
           [](int num_tokens, int padded_length, std::vector<std::uintptr_t> q, std::vector<std::uintptr_t> k_new,
              std::vector<std::uintptr_t> v_new, std::vector<std::uintptr_t> attn_out, std::uintptr_t hidden, std::uintptr_t draft_ids,

@@ -88,6 +88,13 @@ struct Model {
     size_t head_ws_bytes = 0;
     f16* draft_logits = nullptr;  // [16][frspec_vocab]
     float* row_stats = nullptr;   // [16][2]
+    // the drafter's tree bookkeeping between the rounds of one draft (tried_history_*, eagle_mask_2d and the
+    // running log-probs of src/model/minicpm4/minicpm4_eagle.cuh:158-170) and the head's top-k of the round
+    void* draft_state = nullptr;
+    f16* topk_val = nullptr;      // [16][topk_per_iter]
+    int32_t* topk_pos = nullptr;  // [16][topk_per_iter]
+    int32_t* topk_ids = nullptr;  // [16][topk_per_iter]
+    int draft_rounds_done = 0;    // rounds of the current draft that have run (0 .. num_iter)
     int32_t* d_best = nullptr;
     int32_t* d_ids = nullptr;     // [64] accepted ids of the last verify
     int32_t* h_result = nullptr;  // pinned, device-visible: (a, ids) of the last verify
@@ -102,6 +109,9 @@ struct Model {
         uint64_t signature = 0;
     };
     std::map<std::pair<int, int>, std::vector<StepGraph>> step_graphs;
+    // sequences of model-level calls captured by the caller (cpmcu_capture_begin / _end)
+    std::vector<StepGraph> user_graphs;
+    bool capturing = false;
 };
 
 Model* g_model = nullptr;
@@ -123,7 +133,7 @@ struct PerfScope {
     hipEvent_t e0 = nullptr, e1 = nullptr;
     hipStream_t st;
     PerfScope(const char* l, hipStream_t s) : label(l), st(s) {
-        if (g_model && g_model->perf) {
+        if (g_model && g_model->perf && !g_model->capturing) {  // (a capture records launches, it does not run them)
             (void)hipEventCreate(&e0);
             (void)hipEventCreate(&e1);
             (void)hipEventRecord(e0, st);
@@ -274,6 +284,10 @@ extern "C" int cpmcu_init_storage(int* max_context) {
     if (m.drafter) {
         if ((rc = alloc((void**)&m.draft_logits, (size_t)16 * m.frspec_vocab * 2))) return rc;
         if ((rc = alloc((void**)&m.row_stats, 16 * 2 * sizeof(float)))) return rc;
+        if ((rc = alloc(&m.draft_state, cpmcu_draft_tree_state_bytes(m.topk_per_iter, m.num_iter)))) return rc;
+        if ((rc = alloc((void**)&m.topk_val, (size_t)16 * m.topk_per_iter * sizeof(f16)))) return rc;
+        if ((rc = alloc((void**)&m.topk_pos, (size_t)16 * m.topk_per_iter * sizeof(int32_t)))) return rc;
+        if ((rc = alloc((void**)&m.topk_ids, (size_t)16 * m.topk_per_iter * sizeof(int32_t)))) return rc;
     }
     if ((rc = alloc((void**)&m.d_best, 2 * sizeof(int32_t)))) return rc;
     if ((rc = alloc((void**)&m.d_ids, 64 * sizeof(int32_t)))) return rc;
@@ -342,8 +356,13 @@ extern "C" int cpmcu_set_block_table(const int32_t* host_table, int n) {
                         "set_block_table: entry %d = %d is out of range or repeated", i, host_table[i]);
         seen[host_table[i]] = 1;
     }
+    // The logical pages behind the n given ones take the physical pages that are left, in ascending order: the table
+    // stays a permutation of all pages, so a context that grows past the given prefix never lands on a page twice.
+    std::vector<int32_t> full(host_table, host_table + n);
+    for (int pg = 0; pg < m.num_pages; ++pg)
+        if (!seen[pg]) full.push_back(pg);
     CPMCU_HIP(hipStreamSynchronize(resolve_stream(nullptr)));
-    CPMCU_HIP(hipMemcpy(m.block_table, host_table, n * sizeof(int32_t), hipMemcpyHostToDevice));
+    CPMCU_HIP(hipMemcpy(m.block_table, full.data(), full.size() * sizeof(int32_t), hipMemcpyHostToDevice));
     return CPMCU_OK;
 }
 
@@ -482,6 +501,62 @@ extern "C" int cpmcu_draft_head(int n, uint64_t hidden, uint64_t topk_val, uint6
                                   (void*)topk_val, (int32_t*)topk_pos, (int32_t*)topk_ids, m.head_ws, m.head_ws_bytes, st);
 }
 
+// One round of draft() without the drafter's dense layers (src/model/minicpm4/minicpm4_eagle.cuh:319-382): the
+// FR-Spec head on the round's hidden rows, log-softmax, top-k and the tree bookkeeping, with the state kept here.
+extern "C" int cpmcu_draft_round(int d, uint64_t hidden, uint64_t next_ids, uint64_t parent_rows, uint64_t draft_mask) {
+    int rc = require_model(true);
+    if (rc) return rc;
+    Model& m = *g_model;
+    if (!m.drafter) {
+        set_error("draft_round: no drafter configured");  // src/model/model.cuh:172-173
+        return CPMCU_ERR_RUNTIME;
+    }
+    CPMCU_CHECK_ARG(m.lm_head_loaded, "draft_round: lm_head.weight has not been loaded");
+    CPMCU_CHECK_ARG(d >= 0 && d < m.num_iter, "draft_round: round %d outside [0, %d)", d, m.num_iter);
+    CPMCU_CHECK_ARG(d == 0 || d == m.draft_rounds_done, "draft_round: round %d out of order (%d rounds of this draft have run)", d,
+                    m.draft_rounds_done);
+    CPMCU_CHECK_ARG(hidden && next_ids, "draft_round: null pointer argument");
+    hipStream_t st = resolve_stream(nullptr);
+    PerfScope perf("DRAFT_ROUND", st);
+    const int k = m.topk_per_iter;
+    const int n = d == 0 ? 1 : k;  // the last accepted row, then the k rows of the previous round's picks
+    const int32_t* remap = m.fr_head != m.lm_head ? m.token_id_remap : nullptr;
+    rc = cpmcu_frspec_head_topk((const void*)hidden, m.fr_head, CPMCU_W_TILED, remap, n, m.frspec_vocab, m.hidden, k, m.draft_logits,
+                                m.row_stats, m.topk_val, m.topk_pos, m.topk_ids, m.head_ws, m.head_ws_bytes, st);
+    if (rc) return rc;
+    if (d == 0)
+        rc = cpmcu_draft_tree_begin(m.draft_state, k, m.num_iter, m.topk_val, m.topk_pos, remap, (int32_t*)next_ids, (uint64_t*)draft_mask, st);
+    else
+        rc = cpmcu_draft_tree_extend(m.draft_state, k, m.num_iter, d, m.topk_val, m.topk_pos, remap, (int32_t*)next_ids,
+                                     (int32_t*)parent_rows, (uint64_t*)draft_mask, st);
+    if (rc) return rc;
+    m.draft_rounds_done = d + 1;
+    return CPMCU_OK;
+}
+
+// The end of draft() (src/model/minicpm4/minicpm4_eagle.cuh:385-393): the tree_size - 1 best candidates of the
+// rounds become the tree the verify step consumes.
+extern "C" int cpmcu_draft_finish(uint64_t tree_draft_ids, uint64_t tree_position_ids, uint64_t cache_length, uint64_t tree_attn_mask,
+                                  uint64_t tree_parent) {
+    int rc = require_model(true);
+    if (rc) return rc;
+    Model& m = *g_model;
+    if (!m.drafter) {
+        set_error("draft_finish: no drafter configured");
+        return CPMCU_ERR_RUNTIME;
+    }
+    CPMCU_CHECK_ARG(m.draft_rounds_done == m.num_iter, "draft_finish: %d of %d rounds have run", m.draft_rounds_done, m.num_iter);
+    CPMCU_CHECK_ARG(tree_draft_ids && tree_position_ids && cache_length && tree_attn_mask && tree_parent, "draft_finish: null pointer argument");
+    hipStream_t st = resolve_stream(nullptr);
+    PerfScope perf("DRAFT_FINISH", st);
+    const int32_t* remap = m.fr_head != m.lm_head ? m.token_id_remap : nullptr;
+    rc = cpmcu_draft_tree_finish(m.draft_state, m.topk_per_iter, m.num_iter, m.tree_size, (const int32_t*)cache_length, remap,
+                                 (int32_t*)tree_draft_ids, (int32_t*)tree_position_ids, (uint64_t*)tree_attn_mask, (int32_t*)tree_parent, st);
+    if (rc) return rc;
+    m.draft_rounds_done = 0;
+    return CPMCU_OK;
+}
+
 extern "C" int cpmcu_verify_and_fix(int num_tokens, uint64_t pred, uint64_t gt, uint64_t position_ids,
                                     uint64_t cache_length, uint64_t attn_mask, uint64_t tree_parent,
                                     int* accept_length) {
@@ -492,6 +567,7 @@ extern "C" int cpmcu_verify_and_fix(int num_tokens, uint64_t pred, uint64_t gt, 
         set_error("verify is not supported: no drafter configured");  // src/model/model.cuh:172-173
         return CPMCU_ERR_RUNTIME;
     }
+    CPMCU_CHECK_ARG(!m.capturing, "verify_and_fix synchronises: it cannot be part of a capture");
     CPMCU_CHECK_ARG(num_tokens >= 1 && num_tokens <= 64, "verify_and_fix: num_tokens=%d outside [1, 64]", num_tokens);
     CPMCU_CHECK_ARG(pred && gt && position_ids && cache_length && attn_mask && tree_parent, "verify_and_fix: null pointer argument");
     hipStream_t st = resolve_stream(nullptr);
@@ -577,6 +653,11 @@ void destroy_step_graphs(Model& m) {
             if (g.graph) (void)hipGraphDestroy(g.graph);
         }
     m.step_graphs.clear();
+    for (auto& g : m.user_graphs) {
+        if (g.exec) (void)hipGraphExecDestroy(g.exec);
+        if (g.graph) (void)hipGraphDestroy(g.graph);
+    }
+    m.user_graphs.clear();
 }
 
 }  // namespace
@@ -611,6 +692,7 @@ extern "C" int cpmcu_verify_step(int num_layers, int num_tokens, int padded_leng
         PerfScope perf("VERIFY_STEP", st);
         return enqueue_verify_step(m, a, st);
     }
+    CPMCU_CHECK_ARG(!m.capturing, "verify_step: cuda_graph inside an open capture (pass cuda_graph = 0 there)");
     // Graph path, as decode(..., cuda_graph = true) of the reference: captured once per (padded_length, num_tokens)
     // -- and per set of addresses, which a graph bakes in -- and replayed afterwards.  Every length the kernels
     // need is read from device memory, so the same graph serves every step of that padded length.
@@ -637,6 +719,48 @@ extern "C" int cpmcu_verify_step(int num_layers, int num_tokens, int padded_leng
     CPMCU_HIP(hipGraphInstantiate(&g.exec, g.graph, nullptr, nullptr, 0));
     bucket.push_back(g);
     CPMCU_HIP(hipGraphLaunch(g.exec, st));
+    return CPMCU_OK;
+}
+
+// The same mechanism for any sequence of the model-level calls that only enqueue (decode_attention, draft_attention,
+// decode_lm_head, draft_head, draft_round, draft_finish, verify_step without cuda_graph): what is called between
+// capture_begin and capture_end is recorded on the library's stream instead of run, and replayed as one graph.
+extern "C" int cpmcu_capture_begin(void) {
+    int rc = require_model(true);
+    if (rc) return rc;
+    Model& m = *g_model;
+    CPMCU_CHECK_ARG(!m.capturing, "capture_begin: a capture is already open");
+    CPMCU_HIP(hipStreamBeginCapture(resolve_stream(nullptr), hipStreamCaptureModeRelaxed));
+    m.capturing = true;
+    return CPMCU_OK;
+}
+
+extern "C" int cpmcu_capture_end(int* graph_id) {
+    int rc = require_model(true);
+    if (rc) return rc;
+    Model& m = *g_model;
+    CPMCU_CHECK_ARG(m.capturing, "capture_end: no capture is open");
+    CPMCU_CHECK_ARG(graph_id, "capture_end: null pointer argument");
+    m.capturing = false;
+    Model::StepGraph g;
+    const hipError_t e = hipStreamEndCapture(resolve_stream(nullptr), &g.graph);
+    if (e != hipSuccess || g.graph == nullptr) {
+        set_error("capture_end: stream capture failed: %s", hipGetErrorString(e));
+        return CPMCU_ERR_HIP;
+    }
+    CPMCU_HIP(hipGraphInstantiate(&g.exec, g.graph, nullptr, nullptr, 0));
+    m.user_graphs.push_back(g);
+    *graph_id = (int)m.user_graphs.size() - 1;
+    return CPMCU_OK;
+}
+
+extern "C" int cpmcu_graph_replay(int graph_id) {
+    int rc = require_model(true);
+    if (rc) return rc;
+    Model& m = *g_model;
+    CPMCU_CHECK_ARG(graph_id >= 0 && graph_id < (int)m.user_graphs.size(), "graph_replay: unknown graph %d", graph_id);
+    CPMCU_CHECK_ARG(!m.capturing, "graph_replay: a capture is open");
+    CPMCU_HIP(hipGraphLaunch(m.user_graphs[graph_id].exec, resolve_stream(nullptr)));
     return CPMCU_OK;
 }
 
@@ -692,6 +816,10 @@ extern "C" int cpmcu_shutdown(void) {
     (void)hipFree(m.head_ws);
     (void)hipFree(m.draft_logits);
     (void)hipFree(m.row_stats);
+    (void)hipFree(m.draft_state);
+    (void)hipFree(m.topk_val);
+    (void)hipFree(m.topk_pos);
+    (void)hipFree(m.topk_ids);
     (void)hipFree(m.d_best);
     (void)hipFree(m.d_ids);
     (void)hipFree(m.chain_mask);

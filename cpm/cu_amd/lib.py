@@ -33,11 +33,16 @@ SIGNATURES = {
     "cpmcu_draft": (c_int, [c_u64] * 5),
     "cpmcu_verify_and_fix": (c_int, [c_int, c_u64, c_u64, c_u64, c_u64, c_u64, c_u64, ctypes.POINTER(c_int)]),
     "cpmcu_verify_step": (c_int, [c_int, c_int, c_int, _P, _P, _P, _P] + [c_u64] * 13 + [c_int, c_int]),
+    "cpmcu_capture_begin": (c_int, []),
+    "cpmcu_capture_end": (c_int, [ctypes.POINTER(c_int)]),
+    "cpmcu_graph_replay": (c_int, [c_int]),
     "cpmcu_print_perf_summary": (c_int, []),
     "cpmcu_decode_attention": (c_int, [c_int, c_int, c_int, c_u64, c_u64, c_u64, c_u64, c_u64, c_u64]),
     "cpmcu_draft_attention": (c_int, [c_int, c_int, c_int, c_u64, c_u64, c_u64, c_u64, c_u64, c_int, c_u64]),
     "cpmcu_decode_lm_head": (c_int, [c_int, c_u64, c_u64, c_u64]),
     "cpmcu_draft_head": (c_int, [c_int, c_u64, c_u64, c_u64, c_u64]),
+    "cpmcu_draft_round": (c_int, [c_int, c_u64, c_u64, c_u64, c_u64]),
+    "cpmcu_draft_finish": (c_int, [c_u64] * 5),
     "cpmcu_set_block_table": (c_int, [_P, c_int]),
     "cpmcu_model_pointers": (c_int, [c_int, ctypes.POINTER(c_u64), ctypes.POINTER(c_u64), ctypes.POINTER(c_u64), ctypes.POINTER(c_int)]),
     "cpmcu_stream": (c_u64, []),

@@ -77,6 +77,38 @@ class PathModel:
                            p(accepted_ids), p(prev_hidden), p(next_position_ids), p(result), 1 if advance_length else 0,
                            1 if cuda_graph else 0)
 
+    def draft_round(self, d, hidden, next_ids, parent_rows=None, draft_mask=None):
+        """Round d of draft() without the dense layers (cpmcu_draft_round); tensors are the caller's static buffers."""
+        p = lambda t: 0 if t is None else t.data_ptr()
+        self.L.draft_round(int(d), p(hidden), p(next_ids), p(parent_rows), p(draft_mask))
+
+    def draft_finish(self, tree_draft_ids, tree_position_ids, cache_length, tree_attn_mask, tree_parent):
+        self.L.draft_finish(tree_draft_ids.data_ptr(), tree_position_ids.data_ptr(), cache_length.data_ptr(), tree_attn_mask.data_ptr(),
+                            tree_parent.data_ptr())
+
+    def draft_attention(self, draft_layer, n, padded_length, q, k_new, v_new, cache_length, mask, mask_k_range, out):
+        self.L.draft_attention(int(draft_layer), int(n), int(padded_length), q.data_ptr(), k_new.data_ptr(), v_new.data_ptr(),
+                               cache_length.data_ptr(), 0 if mask is None else mask.data_ptr(), int(mask_k_range), out.data_ptr())
+
+    def set_block_table(self, table):
+        """Install a logical -> physical page table (a full permutation of the model's pages, or a prefix of one whose
+        remaining pages follow in ascending order); `table`: int32 tensor or array."""
+        t = np.ascontiguousarray(table.cpu().numpy() if hasattr(table, "cpu") else table, np.int32)
+        self.L.set_block_table(t.ctypes.data_as(ctypes.c_void_p), t.size)
+
+    def capture(self, fn):
+        """Record the model-level calls fn() makes into a library-owned graph; returns its id for replay()."""
+        self.L.capture_begin()
+        try:
+            fn()
+        finally:
+            gid = ctypes.c_int(-1)
+            self.L.capture_end(ctypes.byref(gid))
+        return gid.value
+
+    def replay(self, graph_id):
+        self.L.graph_replay(int(graph_id))
+
     def stream(self):
         """The library's stream as a torch stream object (events recorded on it time the library's launches)."""
         return torch.cuda.ExternalStream(self.L.raw.cpmcu_stream())

@@ -157,6 +157,16 @@ int cpmcu_verify_step(int num_layers, int num_tokens, int padded_length, const u
                       uint64_t gt_out, uint64_t accepted_ids, uint64_t prev_hidden, uint64_t next_position_ids,
                       uint64_t result, int flags, int cuda_graph);
 
+/* No reference counterpart (the reference captures decode only, src/entry.cu:475-492): the same graph mechanism
+ * for any sequence of the model-level calls that only enqueue -- cpmcu_decode_attention, cpmcu_draft_attention,
+ * cpmcu_decode_lm_head, cpmcu_draft_head, cpmcu_draft_round, cpmcu_draft_finish, cpmcu_verify_step with
+ * cuda_graph = 0.  Calls made between capture_begin and capture_end are recorded on the library's stream instead
+ * of run; capture_end hands back an id, cpmcu_graph_replay enqueues the recorded launches as one graph.  The
+ * addresses passed during the capture are baked in; lengths are read from device memory at replay, as always. */
+int cpmcu_capture_begin(void);
+int cpmcu_capture_end(int* graph_id);
+int cpmcu_graph_replay(int graph_id);
+
 /* src/entry.cu:506-508 print_perf_summary: prints the per-operator event timings
  * collected when CPMCU_PERF=1 is set in the environment. */
 int cpmcu_print_perf_summary(void);
@@ -198,8 +208,26 @@ int cpmcu_decode_lm_head(int input_length, uint64_t hidden, uint64_t logits, uin
  *   (FR-Spec indices), topk_ids [n][k] int32 (full-vocabulary ids). */
 int cpmcu_draft_head(int n, uint64_t hidden, uint64_t topk_val, uint64_t topk_pos, uint64_t topk_ids);
 
-/* No reference counterpart: install a logical -> physical page permutation (host int32[n], a
- * partial permutation of [0, num_pages)); the default table is the identity. */
+/* draft() without the drafter's dense layers (src/model/minicpm4/minicpm4_eagle.cuh:304-396): what runs between
+ * them, with the drafter's state (tried_history_*, eagle_mask_2d, running log-probs) kept by the library.
+ *   cpmcu_draft_round(d, ...), d = 0 .. num_iter - 1 in order: FR-Spec head on hidden (1 row at d = 0: the last
+ *       accepted row of the drafter's output, :320; topk_per_iter rows afterwards, :366), log-softmax, top-k, and the
+ *       tree bookkeeping of the round (:321-332 / :367-382).  next_ids int32[topk_per_iter] out: the token ids to
+ *       embed for the next round (full-vocabulary ids); parent_rows int32[topk_per_iter] out (d >= 1; may be 0): the
+ *       row of the previous hidden states each pick continues (remap_hidden, :377); draft_mask uint64[topk_per_iter]
+ *       out (may be 0): Mask(eagle_mask_2d, k, k * (d + 1)) for cpmcu_draft_attention of the next round.
+ *   cpmcu_draft_finish (:385-393): tree_draft_ids[1 .. tree_size) (entry 0, the root, is the caller's),
+ *       tree_position_ids / tree_attn_mask (one uint64 per row) / tree_parent [tree_size]; cache_length is the
+ *       device scalar P (the reference copies it to the host first, :305; here it is read on the device).
+ * Both only enqueue on the library's stream.  A round out of order or a finish before the last round is
+ * CPMCU_ERR_INVALID_ARGUMENT. */
+int cpmcu_draft_round(int d, uint64_t hidden, uint64_t next_ids, uint64_t parent_rows, uint64_t draft_mask);
+int cpmcu_draft_finish(uint64_t tree_draft_ids, uint64_t tree_position_ids, uint64_t cache_length, uint64_t tree_attn_mask,
+                       uint64_t tree_parent);
+
+/* No reference counterpart: install a logical -> physical page permutation (host int32[n], distinct entries of
+ * [0, num_pages)); the logical pages behind the n given ones take the remaining physical pages in ascending
+ * order, so the table is always a permutation of all pages.  The default table is the identity. */
 int cpmcu_set_block_table(const int32_t* host_table, int n);
 
 /* No reference counterpart: device addresses of the model's storage, for harnesses that fill the

@@ -264,3 +264,69 @@ def test_library_graph_replays_equal_eager_steps(gpu, orc):
         assert np.array_equal(o1.view(np.uint16), o2.view(np.uint16))  # same launches, same split geometry: same bits
     for (k1, v1), (k2, v2) in zip(kv_e, kv_g):
         assert np.array_equal(k1.view(np.uint16), k2.view(np.uint16)) and np.array_equal(v1.view(np.uint16), v2.view(np.uint16))
+
+
+def test_model_level_draft_rounds(gpu, orc):
+    """cpmcu_draft_round / cpmcu_draft_finish (the drafter's state owned by the library, driven through the pybind module)
+    against (1) the operator-level chain on an independently built sub-matrix, bit for bit, and (2) the oracle's tree
+    bookkeeping fed with the device's per-round top-k, which pins ids, positions, masks and parents of the final tree."""
+    from cpm.cu_amd import C, ops
+    torch = gpu
+    V, Vs, H, T, K, N, P = 5000, 2048, 512, 60, 10, 6, 777
+    w = synth.normal_f16((V, H), 41, 2, std=0.05)
+    remap = synth.frspec_remap(V, Vs, 41)
+    C.init_base_model(0.01, V, 1, H, 1024, HQ, HKV, D, 1e-5, 0, 2048, 1.0, 1.0, 1.0)
+    C.init_minicpm4_eagle_model(1, N, K, T, 0, False, 128, 1024, Vs, 1.0, True, True)
+    C.init_storage()
+    C.load_model("eagle.token_id_remap", remap.ctypes.data)
+    C.load_model("lm_head.weight", w.ctypes.data)
+    try:
+        hid = [to_dev(torch, synth.normal_f16((1 if d == 0 else K, H), 41, 100 + d)) for d in range(N)]
+        next_ids = torch.zeros(K, dtype=torch.int32, device="cuda")
+        rows = torch.zeros(K, dtype=torch.int32, device="cuda")
+        dmask = torch.zeros(K, dtype=torch.int64, device="cuda")
+        with pytest.raises(ValueError, match="out of order"):
+            C.draft_round(2, hid[2].data_ptr(), next_ids.data_ptr(), rows.data_ptr(), dmask.data_ptr())
+        trace = []
+        for d in range(N):
+            C.draft_round(d, hid[d].data_ptr(), next_ids.data_ptr(), rows.data_ptr() if d else 0, dmask.data_ptr())
+            C.synchronize()
+            trace.append((to_np(next_ids).copy(), to_np(rows).copy(), to_np(dmask).view(np.uint64).copy()))
+            if d == 1:
+                with pytest.raises(ValueError, match="rounds have run"):
+                    C.draft_finish(1, 1, 1, 1, 1)
+        ids = torch.full((T,), -1, dtype=torch.int32, device="cuda")
+        ids[0] = 4321  # the root token is the caller's
+        tpos = torch.zeros(T, dtype=torch.int32, device="cuda")
+        tmask = torch.zeros(T, dtype=torch.int64, device="cuda")
+        tpar = torch.zeros(T, dtype=torch.int32, device="cuda")
+        cl = torch.tensor([P], dtype=torch.int32, device="cuda")
+        torch.cuda.synchronize()
+        C.draft_finish(ids.data_ptr(), tpos.data_ptr(), cl.data_ptr(), tmask.data_ptr(), tpar.data_ptr())
+        C.synchronize()
+    finally:
+        C.shutdown()
+    # (1) the operator-level chain
+    d_remap = to_dev(torch, remap)
+    sub = ops.tile_head_weight(to_dev(torch, w), d_remap)
+    t = ops.DraftTree(K, N, d_remap)
+    o_tree = orc.DraftTree(K, N, remap)
+    for d in range(N):
+        r = ops.frspec_head_topk(hid[d], sub, d_remap, K)
+        torch.cuda.synchronize()
+        val_np, pos_np = to_np(r["val"]).copy(), to_np(r["pos"]).copy()
+        if d == 0:
+            got = to_np(t.begin(r["val"][0], r["pos"][0])).copy()
+            assert np.array_equal(trace[0][0], got)
+            assert np.array_equal(got, o_tree.begin(val_np[0], pos_np[0]))
+        else:
+            g_ids, g_rows, g_mask = t.extend(d, r["val"], r["pos"])
+            torch.cuda.synchronize()
+            assert np.array_equal(trace[d][0], to_np(g_ids)) and np.array_equal(trace[d][1], to_np(g_rows))
+            assert np.array_equal(trace[d][2], to_np(g_mask).view(np.uint64))
+            o_ids, o_rows, _ = o_tree.extend(d, val_np, pos_np)  # (2) the oracle on the device's top-k of the round
+            assert np.array_equal(trace[d][0], o_ids) and np.array_equal(trace[d][1], o_rows) and np.array_equal(trace[d][2], o_tree.mask)
+    o_ids, o_pos, o_mask, o_par = o_tree.finish(T, P)
+    assert int(to_np(ids)[0]) == 4321 and np.array_equal(to_np(ids)[1:], o_ids[1:])
+    assert np.array_equal(to_np(tpos), o_pos) and np.array_equal(to_np(tpar), o_par)
+    assert np.array_equal(to_np(tmask).view(np.uint64), o_mask[:, 0])
