@@ -12,6 +12,10 @@ struct Options {
 };
 Options& options();
 
+// tree_attention.hip -- an attention launch whose device-side length lay outside [max(T, mask_k_range), max_kv_len]
+// worked on the clamped length and left the offending value behind; this reads and clears it (synchronising).
+int attention_take_bad_length(int* value);
+
 // lm_head.hip -- the streaming GEMM with its two epilogues.
 constexpr int kHeadModeStats = 0;
 constexpr int kHeadModeArgmax = 1;

@@ -154,6 +154,19 @@ struct PerfScope {
     }
 };
 
+// After a synchronisation: did an attention launch see a length outside what the host had promised?
+int check_device_errors() {
+    int bad = 0;
+    int rc = attention_take_bad_length(&bad);
+    if (rc) return rc;
+    if (bad != 0) {
+        set_error("a tree-attention launch read a KV length of %d from device memory, outside [rows, max_kv_len] of its call; "
+                  "it ran on the clamped length and its output is not valid", bad < 0 ? 0 : bad);
+        return CPMCU_ERR_RUNTIME;
+    }
+    return CPMCU_OK;
+}
+
 int check_dtype(int torch_dtype) {
     if (torch_dtype != 0) {  // 0 = fp16, 1 = bf16 (cpmcu/llm.py:11-14)
         set_error("dtype %d is not compiled into this library (fp16 only)", torch_dtype);
@@ -252,11 +265,80 @@ extern "C" int cpmcu_init_minicpm4_eagle_model(int num_layers, int num_iter, int
     return CPMCU_OK;
 }
 
+namespace {
+
+void destroy_step_graphs(Model& m) {
+    for (auto& kv : m.step_graphs)
+        for (auto& g : kv.second) {
+            if (g.exec) (void)hipGraphExecDestroy(g.exec);
+            if (g.graph) (void)hipGraphDestroy(g.graph);
+        }
+    m.step_graphs.clear();
+    for (auto& g : m.user_graphs) {
+        if (g.exec) (void)hipGraphExecDestroy(g.exec);
+        if (g.graph) (void)hipGraphDestroy(g.graph);
+    }
+    m.user_graphs.clear();
+}
+
+// Frees everything init_storage allocates and forgets it (also after a failure half-way, so that a retry starts clean).
+void release_storage(Model& m) {
+    destroy_step_graphs(m);
+    if (m.fr_head && m.fr_head != m.lm_head) (void)hipFree(m.fr_head);
+    (void)hipFree(m.lm_head);
+    (void)hipFree(m.token_id_remap);
+    for (void* p : m.k_pools) (void)hipFree(p);
+    for (void* p : m.v_pools) (void)hipFree(p);
+    (void)hipFree(m.d_k_pools);
+    (void)hipFree(m.d_v_pools);
+    (void)hipFree(m.block_table);
+    (void)hipFree(m.attn_ws);
+    (void)hipFree(m.head_ws);
+    (void)hipFree(m.draft_logits);
+    (void)hipFree(m.row_stats);
+    (void)hipFree(m.draft_state);
+    (void)hipFree(m.topk_val);
+    (void)hipFree(m.topk_pos);
+    (void)hipFree(m.topk_ids);
+    (void)hipFree(m.d_best);
+    (void)hipFree(m.d_ids);
+    (void)hipFree(m.chain_mask);
+    if (m.h_result) (void)hipHostFree(m.h_result);
+    m.lm_head = m.fr_head = nullptr;
+    m.token_id_remap = nullptr;
+    m.k_pools.clear();
+    m.v_pools.clear();
+    m.d_k_pools = m.d_v_pools = nullptr;
+    m.block_table = nullptr;
+    m.attn_ws = m.head_ws = m.draft_state = nullptr;
+    m.draft_logits = nullptr;
+    m.row_stats = nullptr;
+    m.topk_val = nullptr;
+    m.topk_pos = m.topk_ids = nullptr;
+    m.d_best = m.d_ids = m.h_result = nullptr;
+    m.chain_mask = nullptr;
+    m.storage = m.remap_loaded = m.lm_head_loaded = false;
+    m.num_pages = 0;
+}
+
+int init_storage_impl(Model& m, int* max_context);
+
+}  // namespace
+
 extern "C" int cpmcu_init_storage(int* max_context) {
     int rc = require_model(false);
     if (rc) return rc;
     Model& m = *g_model;
     CPMCU_CHECK_ARG(!m.storage, "init_storage: already initialised");
+    rc = init_storage_impl(m, max_context);
+    if (rc) release_storage(m);  // nothing of a failed attempt stays allocated
+    return rc;
+}
+
+namespace {
+
+int init_storage_impl(Model& m, int* max_context) {
+    int rc = CPMCU_OK;
     size_t free_b = 0, total_b = 0;
     CPMCU_HIP(hipMemGetInfo(&free_b, &total_b));
     const size_t budget = (size_t)((double)total_b * m.memory_limit);
@@ -298,11 +380,13 @@ extern "C" int cpmcu_init_storage(int* max_context) {
         for (int i = 0; i < 64; ++i) rows[i] = i == 63 ? ~0ull : ((2ull << i) - 1ull);
         CPMCU_HIP(hipMemcpy(m.chain_mask, rows, sizeof(rows), hipMemcpyHostToDevice));
     }
+    // load_model passes lm_head.weight through a row-major staging buffer of its full size: keep room for it
+    used += align_up((size_t)m.vocab * m.hidden * sizeof(f16), 256);
     // KV pools take what is left of the budget, in whole pages (the reference gives the KV cache
     // all remaining pool memory, src/model/kvcache.cuh:50).
     const size_t page_bytes = (size_t)m.kv_heads * kPage * kHeadDim * 2;  // one of K/V, one layer
     const int all_layers = m.layers + m.draft_layers;  // the drafter's layers keep caches of the same length (src/model/minicpm4/minicpm4_eagle.cuh:76,183-184)
-    const size_t per_page_all = page_bytes * 2 * all_layers + 4;
+    const size_t per_page_all = page_bytes * 2 * all_layers + sizeof(int32_t);  // + the page's block-table entry
     const size_t remaining = budget > used ? budget - used : 0;
     const size_t free_now = free_b > used ? free_b - used : 0;
     size_t pages = std::min(remaining, (size_t)(free_now * 0.95)) / per_page_all;
@@ -343,6 +427,8 @@ extern "C" int cpmcu_init_storage(int* max_context) {
     if (max_context) *max_context = (int)std::min<size_t>(pages * kPage, 0x7fffffff);
     return CPMCU_OK;
 }
+
+}  // namespace
 
 // Extension (no reference counterpart): install a logical -> physical page permutation.
 extern "C" int cpmcu_set_block_table(const int32_t* host_table, int n) {
@@ -585,7 +671,7 @@ extern "C" int cpmcu_verify_and_fix(int num_tokens, uint64_t pred, uint64_t gt, 
     if (rc) return rc;
     CPMCU_HIP(hipStreamSynchronize(st));
     if (accept_length) *accept_length = m.h_result[0];
-    return CPMCU_OK;
+    return check_device_errors();
 }
 
 namespace {
@@ -646,19 +732,6 @@ uint64_t step_signature(const Model& m, const StepArgs& a) {
     return h;
 }
 
-void destroy_step_graphs(Model& m) {
-    for (auto& kv : m.step_graphs)
-        for (auto& g : kv.second) {
-            if (g.exec) (void)hipGraphExecDestroy(g.exec);
-            if (g.graph) (void)hipGraphDestroy(g.graph);
-        }
-    m.step_graphs.clear();
-    for (auto& g : m.user_graphs) {
-        if (g.exec) (void)hipGraphExecDestroy(g.exec);
-        if (g.graph) (void)hipGraphDestroy(g.graph);
-    }
-    m.user_graphs.clear();
-}
 
 }  // namespace
 
@@ -796,34 +869,14 @@ extern "C" uint64_t cpmcu_stream(void) { return (uint64_t)(uintptr_t)resolve_str
 
 extern "C" int cpmcu_synchronize(void) {
     CPMCU_HIP(hipStreamSynchronize(resolve_stream(nullptr)));
-    return CPMCU_OK;
+    return check_device_errors();
 }
 
 extern "C" int cpmcu_shutdown(void) {
     if (!g_model) return CPMCU_OK;
     Model& m = *g_model;
     if (g_stream) (void)hipStreamSynchronize(g_stream);
-    destroy_step_graphs(m);
-    if (m.fr_head && m.fr_head != m.lm_head) (void)hipFree(m.fr_head);
-    (void)hipFree(m.lm_head);
-    (void)hipFree(m.token_id_remap);
-    for (void* p : m.k_pools) (void)hipFree(p);
-    for (void* p : m.v_pools) (void)hipFree(p);
-    (void)hipFree(m.d_k_pools);
-    (void)hipFree(m.d_v_pools);
-    (void)hipFree(m.block_table);
-    (void)hipFree(m.attn_ws);
-    (void)hipFree(m.head_ws);
-    (void)hipFree(m.draft_logits);
-    (void)hipFree(m.row_stats);
-    (void)hipFree(m.draft_state);
-    (void)hipFree(m.topk_val);
-    (void)hipFree(m.topk_pos);
-    (void)hipFree(m.topk_ids);
-    (void)hipFree(m.d_best);
-    (void)hipFree(m.d_ids);
-    (void)hipFree(m.chain_mask);
-    if (m.h_result) (void)hipHostFree(m.h_result);
+    release_storage(m);
     delete g_model;
     g_model = nullptr;
     return CPMCU_OK;

@@ -62,6 +62,11 @@ constexpr float kLazyLog2 = 8.f;  // slack of the lazily updated softmax referen
 
 typedef __attribute__((address_space(3))) void* lds_ptr_t;
 
+// Set by a launch whose device-side length does not fit what the host promised (above max_kv_len, or shorter
+// than the query rows / the masked range): the launch then works on the length clamped into that range -- every
+// access stays inside the page table -- and this word keeps the offending length for the next synchronising call.
+__device__ int g_attn_bad_length;
+
 struct AttnParams {
     const f16* q;
     const f16* k_pool;
@@ -81,6 +86,7 @@ struct AttnParams {
     int ntiles_max;  // tiles the split partition spans: ceil(max_kv_len / 64), fixed by the host-side bound
                      // (with a window: the most tiles a window can hold, counted from its first tile)
     int table_pages;    // entries of block_table the caller guarantees: ceil(max_kv_len / 256)
+    int max_kv_len;     // the host-side bound of *kv_len the launch geometry was derived from
     int window_blocks;  // block sliding window in blocks of 128 keys (0 = none): key blocks below
                         // ceil(P / 128) - window_blocks are not visited (src/flash_attn/src/flash_blockmask.h:32,43-46)
     float scale_log2;
@@ -262,7 +268,14 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
         // (a window's last tile slot can lie past the host bound; it is never consumed, and the table is not read there)
         for (int i = tid; i < npg; i += kThreads) s_pages[i] = p.block_table[min(pg0 + i, p.table_pages - 1)];
     }
-    const int S = p.kv_len[0];
+    int S = p.kv_len[0];
+    {
+        const int lo = max(p.T, p.mask_k_range);
+        if (S > p.max_kv_len || S < lo) {
+            if (wg == 0 && tid == 0) g_attn_bad_length = S == 0 ? -1 : S;
+            S = min(max(S, lo), p.max_kv_len);
+        }
+    }
     const int P = S - p.T;              // the T query tokens are the last T keys
     const int Pm = S - p.mask_k_range;  // first key column governed by the mask bits (mask.h: mask_k_begin)
     const int ntiles = (S + kTileN - 1) / kTileN;
@@ -788,6 +801,20 @@ extern "C" int cpmcu_tree_attention_plan(int T, int Hq, int Hkv, int max_kv_len,
     return CPMCU_OK;
 }
 
+namespace cpmcu {
+// Reads and clears the bad-length word of the current device (a synchronising copy); 0 = none.
+int attention_take_bad_length(int* value) {
+    int v = 0;
+    CPMCU_HIP(hipMemcpyFromSymbol(&v, HIP_SYMBOL(g_attn_bad_length), sizeof(int)));
+    if (v != 0) {
+        const int zero = 0;
+        CPMCU_HIP(hipMemcpyToSymbol(HIP_SYMBOL(g_attn_bad_length), &zero, sizeof(int)));
+    }
+    *value = v;
+    return CPMCU_OK;
+}
+}  // namespace cpmcu
+
 extern "C" size_t cpmcu_tree_attention_workspace_bytes(int T, int Hq, int Hkv, int max_kv_len) {
     (void)max_kv_len;
     if (T <= 0 || Hkv <= 0 || Hq <= 0 || Hq % Hkv) return 0;
@@ -847,6 +874,7 @@ static int tree_attention_impl(const void* q, void* k_pool, void* v_pool,
     CPMCU_CHECK_ARG(p.num_splits <= kMaxSplits, "tree_attention: max_kv_len=%d is beyond the supported context", max_kv_len);
     p.ntiles_max = ceil_div(span, kTileN);
     p.table_pages = ceil_div(max_kv_len, kPage);
+    p.max_kv_len = max_kv_len;
     p.scale_log2 = scale * 1.4426950408889634f;
     p.out = (f16*)out;
     p.o_part = nullptr;

@@ -49,6 +49,9 @@ class VerifyStep:
         self.attn_out = None
         self.commit = bool(commit)
         self.fused = bool(fused)
+        # only the fused tail advances the tree positions with the lengths; the operator-by-operator tail would leave
+        # them behind the device-side prefix length from the second step on
+        assert self.fused or not self.commit, "commit=True needs the fused tail"
         self.path = torch.zeros(self.T, dtype=torch.int32, device=dev)
         if self.commit:
             self.prev_hidden = None  # allocated at the first step, when the hidden size is known

@@ -238,7 +238,9 @@ int cpmcu_model_pointers(int layer, uint64_t* k_pool, uint64_t* v_pool, uint64_t
 /* No reference counterpart: the library's own stream (a hipStream_t as an integer; created on first use), for
  * harnesses that record events on it or order their own streams against it.  0 if it cannot be created. */
 uint64_t cpmcu_stream(void);
-/* Synchronise the library's stream. */
+/* Synchronise the library's stream.  Also reports (CPMCU_ERR_RUNTIME) an attention launch since the last check whose
+ * device-side KV length lay outside what its call had promised -- above max_kv_len / padded_length, or shorter than
+ * its rows: such a launch runs on the clamped length (no access leaves the page table) and its output is not valid. */
 int cpmcu_synchronize(void);
 /* Free everything the global model owns (the reference never frees). */
 int cpmcu_shutdown(void);
@@ -328,7 +330,10 @@ int cpmcu_tree_attention_rope(const void* q, void* k_pool, void* v_pool, const i
  *           128 * that block index on, under the same mask and causal rules as above.
  *   rope_cos_sin: as for cpmcu_tree_attention_rope, or NULL for inputs that are already rotated.
  * The kernel starts its KV stream at the window's first block, so the cost follows the window, not
- * the context; max_kv_len still bounds *kv_len and the page table. */
+ * the context; max_kv_len still bounds *kv_len and the page table.  With more than 64 rows the window start is
+ * taken once, from the first row, for all rows; the reference derives it per 64-row block of queries
+ * (src/flash_attn/src/flash_blockmask.h:32) but asserts tree_size <= 64, so that case lies beyond it and is not
+ * pinned against anything. */
 int cpmcu_tree_attention_window(const void* q, void* k_pool, void* v_pool, const int32_t* block_table,
                                 const int32_t* kv_len, int max_kv_len, const void* k_new, const void* v_new,
                                 const float* rope_cos_sin, int block_window_size,

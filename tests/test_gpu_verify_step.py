@@ -330,3 +330,125 @@ def test_model_level_draft_rounds(gpu, orc):
     assert int(to_np(ids)[0]) == 4321 and np.array_equal(to_np(ids)[1:], o_ids[1:])
     assert np.array_equal(to_np(tpos), o_pos) and np.array_equal(to_np(tpar), o_par)
     assert np.array_equal(to_np(tmask).view(np.uint64), o_mask[:, 0])
+
+
+def test_c2_full_size_step_on_the_library_graph(gpu, orc):
+    """Config 2 as the benchmark runs it: 32 layers, 4096-token prefix, 60-node tree, the 73448 x 4096 head, one
+    cpmcu_verify_step on the library's storage replayed from the library's graph.  Accept length, ids and the compacted
+    rows of all 64 caches bit-exact against the oracle, the arg-max staged on the oracle's logits of the same head,
+    attention of two sampled layers within the fp16 tolerance."""
+    from cpm.cu_amd.model import PathModel
+    torch = gpu
+    cfg, shp = synth.CONFIGS["c2_verify_4k"], synth.MINICPM4_8B
+    L, P, T, V, H = cfg["layers"], cfg["prefix"], cfg["T"], shp["vocab"], shp["hidden"]
+    S = P + T
+    tree = synth.eagle_tree(cfg["num_iter"], cfg["topk"], T, cfg["seed"])
+    g = torch.Generator(device="cuda")
+    g.manual_seed(2)
+    w = (torch.randn(V, H, device="cuda", generator=g) * 0.02).to(torch.float16).cpu().numpy()
+    npages = (S + 255) // 256 + 1
+    m = PathModel(V, L, H, HQ, HKV, memory_limit=0.02, tree_size=T, num_iter=cfg["num_iter"], topk=cfg["topk"])
+    try:
+        m.load_head(w)
+        table = to_dev(torch, synth.rng(0, 4).permutation(npages).astype(np.int32))
+        cache = m.cache(block_table=table)
+        for l in range(L):
+            m._k[l][:npages].normal_(generator=g)
+            m._v[l][:npages].normal_(generator=g)
+        rn = lambda *s: torch.randn(*s, device="cuda", generator=g).to(torch.float16)
+        q, kn, vn = [rn(T, HQ, D) for _ in range(L)], [rn(T, HKV, D) for _ in range(L)], [rn(T, HKV, D) for _ in range(L)]
+        out = [torch.zeros(T, HQ, D, dtype=torch.float16, device="cuda") for _ in range(L)]
+        hidden = rn(T, H)
+        sampled = (3, 30)
+        before = {l: tuple(to_np(t) for t in cache.read_logical(l, 0, P)) for l in sampled}
+        draft = torch.zeros(T, dtype=torch.int32, device="cuda")
+        gt = torch.zeros(T, dtype=torch.int32, device="cuda")
+        ids = torch.zeros(T, dtype=torch.int32, device="cuda")
+        result = torch.zeros(1 + T, dtype=torch.int32).pin_memory()
+        clen = torch.tensor([P], dtype=torch.int32, device="cuda")
+        kvlen = torch.tensor([S], dtype=torch.int32, device="cuda")
+        pos, mask, parent = to_dev(torch, tree.positions(P)), to_dev(torch, tree.mask), to_dev(torch, tree.parent)
+        padded = (S + 127) // 128 * 128
+        torch.cuda.synchronize()
+        step = lambda: m.verify_step(T, padded, q, kn, vn, out, hidden, draft, pos, clen, kvlen, mask, parent, ids, gt_out=gt,
+                                     result=result, block_table=table, cuda_graph=True)
+        step()  # captures; the target arg-max of this pass rigs the draft ids
+        m.synchronize()
+        gt_np = to_np(gt)
+        z_ref = orc.lm_head(to_np(hidden), w)
+        gt_ref = orc.argmax(z_ref)
+        for i in np.nonzero(gt_np != gt_ref)[0]:  # only inside the logit tolerance
+            assert float(z_ref[i, gt_ref[i]]) - float(z_ref[i, gt_np[i]]) <= 4e-2
+        for depth in (0, 3, int(tree.depth.max())):
+            pred, leaf = synth.draft_ids_for_accept(tree, gt_np, depth, V, 7 + depth)
+            draft.copy_(to_dev(torch, pred))
+            torch.cuda.synchronize()
+            step()  # a replay
+            m.synchronize()
+            a = int(result[0])
+            a_ref, _, path = orc.tree_accept(pred, gt_np, tree.positions(P), P, tree.mask, tree.parent)
+            assert a == a_ref == depth + 1 and np.array_equal(result[1:1 + a].numpy(), gt_np[path])
+            for l in range(L):
+                kd, vd = cache.read_logical(l, P, a)
+                assert np.array_equal(to_np(kd).reshape(a, -1).view(np.uint16), to_np(kn[l]).reshape(T, -1)[path].view(np.uint16)), (depth, l)
+                assert np.array_equal(to_np(vd).reshape(a, -1).view(np.uint16), to_np(vn[l]).reshape(T, -1)[path].view(np.uint16)), (depth, l)
+        for l in sampled:
+            kp, vp = before[l]
+            ref = orc.tree_attention(to_np(q[l]), np.concatenate([kp, to_np(kn[l])]), np.concatenate([vp, to_np(vn[l])]), tree.mask, P)
+            assert_close_f16(to_np(out[l]), ref, "config 2 step on the library graph, attention of layer %d" % l)
+            kd, vd = cache.read_logical(l, 0, P)
+            assert np.array_equal(to_np(kd).view(np.uint16), kp.view(np.uint16)) and np.array_equal(to_np(vd).view(np.uint16), vp.view(np.uint16))
+    finally:
+        m.close()
+
+
+def test_device_side_length_outside_the_promised_bound_is_reported(gpu):
+    """A KV length read from device memory that exceeds the call's max_kv_len (a stale padded length under a replayed
+    graph, say) must not walk off the page table: the launch clamps it, and the next synchronising call says so."""
+    from cpm.cu_amd import lib as libmod, ops
+    from cpm.cu_amd.kvcache import PagedKVCache
+    torch = gpu
+    L = libmod.get()
+    T, P = 8, 300
+    cache = PagedKVCache(1, HKV, 3)
+    q = torch.randn(T, HQ, D, device="cuda").to(torch.float16)
+    L.synchronize()  # clears anything an earlier test left
+    kv_len = torch.tensor([P + T + 200], dtype=torch.int32, device="cuda")  # beyond the max_kv_len promised below
+    out = ops.tree_attention(q, cache, 0, kv_len, P + T, None)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out.float()).all()
+    with pytest.raises(RuntimeError, match="KV length of 508"):
+        L.synchronize()
+    L.synchronize()  # reported once
+    kv_len.fill_(4)  # shorter than the query rows
+    ops.tree_attention(q, cache, 0, kv_len, P + T, None)
+    torch.cuda.synchronize()
+    with pytest.raises(RuntimeError, match="KV length of 4"):
+        L.synchronize()
+
+
+def test_init_storage_failure_leaves_nothing_behind(gpu):
+    """An init_storage that cannot fit its budget fails with an error and frees what it had taken: the retry with a
+    workable budget starts clean."""
+    from cpm.cu_amd import lib as libmod
+    import ctypes
+    torch = gpu
+    L = libmod.get()
+    free0 = torch.cuda.mem_get_info()[0]
+    total = torch.cuda.mem_get_info()[1]
+    V, H = 40000, 2048
+    L.init_base_model(ctypes.c_float(200e6 / total), V, 2, H, 4 * H, HQ, HKV, D, ctypes.c_float(1e-5), 0, 2048, ctypes.c_float(1.0),
+                      ctypes.c_float(1.0), ctypes.c_float(1.0))  # 200 MB: the head fits, its staging buffer and the pools do not
+    L.init_minicpm4_eagle_model(1, 6, 10, 60, 0, 0, 128, 1024, 0, ctypes.c_float(1.0), 1, 1)
+    ctx = ctypes.c_int(0)
+    with pytest.raises(RuntimeError, match="budget"):
+        L.init_storage(ctypes.byref(ctx))
+    free1 = torch.cuda.mem_get_info()[0]
+    assert free0 - free1 < 64 << 20, "a failed init_storage kept %d MB" % ((free0 - free1) >> 20)
+    L.shutdown()
+    L.init_base_model(ctypes.c_float(2e9 / total), V, 2, H, 4 * H, HQ, HKV, D, ctypes.c_float(1e-5), 0, 2048, ctypes.c_float(1.0),
+                      ctypes.c_float(1.0), ctypes.c_float(1.0))
+    L.init_minicpm4_eagle_model(1, 6, 10, 60, 0, 0, 128, 1024, 0, ctypes.c_float(1.0), 1, 1)
+    L.init_storage(ctypes.byref(ctx))
+    assert ctx.value >= 4096
+    L.shutdown()
