@@ -54,7 +54,6 @@ constexpr int kStages = 4;
 constexpr int kKTileBytes = kTileN * kHeadDim * 2;  // 16 KB, row = one key (256 B)
 constexpr int kVTileBytes = kHeadDim * kTileN * 2;  // 16 KB, row = one dim (128 B)
 constexpr int kStageBytes = kKTileBytes + kVTileBytes;
-constexpr int kMaxPagesPerSplit = 1024;
 constexpr int kVStageRows = 64;  // appended V rows staged in LDS ahead of their transposition
 constexpr int kMaxSplits = 128;
 constexpr int kXcds = 8;
@@ -82,6 +81,7 @@ struct AttnParams {
     int mask_words;
     int mask_k_range;  // trailing key columns the mask bits refer to (>= T; = T for the verify tree)
     int T, Hq, Hkv, group;
+    int group_shift, hkv_shift;  // log2 of group / Hkv when they are powers of two (the usual case), else -1: plain division
     int num_splits, num_mtiles, rows_pad;
     int ntiles_max;  // tiles the split partition spans: ceil(max_kv_len / 64), fixed by the host-side bound
                      // (with a window: the most tiles a window can hold, counted from its first tile)
@@ -139,6 +139,19 @@ __device__ inline void load_to_lds16_v(const void* gptr, const char* lds_dst) {
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gptr), "s"(lds_addr) : "memory", "m0");
 }
 
+// Scalar loads of wave-uniform int32 values, issued and awaited in place: an entry of the page table when a tile is
+// requested (consecutive entries share a cache line, so after the first one of a page run these are scalar-cache
+// hits), and the KV length together with the first page id at the start of the kernel, where a vector load would
+// queue behind the Q rows.  Nothing else of this wave's scalar or LDS traffic is outstanding at those points.
+__device__ inline int scalar_load(const int32_t* ptr) {
+    int v;
+    asm volatile("s_load_dword %0, %1, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=s"(v) : "s"(ptr) : "memory");
+    return v;
+}
+__device__ inline void scalar_load2(const int32_t* pa, const int32_t* pb, int& a, int& b) {
+    asm volatile("s_load_dword %0, %2, 0x0\n\ts_load_dword %1, %3, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=&s"(a), "=&s"(b) : "s"(pa), "s"(pb) : "memory");
+}
+
 // Per-thread byte offsets of its pieces inside a K tile and a V^T tile of a page (second piece of each:
 // + 32 keys = 8192 bytes for K, + 64 dims = 64 * 512 bytes for V^T; the swizzle terms do not change).
 __device__ inline uint32_t k_piece_off(int wave, int lane) {
@@ -193,19 +206,22 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
     constexpr int kRowsPerWg = kRowWaves * kRowsPerWave;
     constexpr int kDepth = kStages / G - 1;  // iterations in flight behind the one being consumed
     __shared__ __attribute__((aligned(1024))) char ring[kStages * kStageBytes];
-    __shared__ int32_t s_pages[kMaxPagesPerSplit];
     __shared__ __attribute__((aligned(1024))) char vstage[kVStageRows * kHeadDim * 2];  // first appended V rows, row-major
 
-    // XCD-aware work mapping: consecutive workgroup ids go to consecutive XCDs, so
-    // id % 8 picks the XCD; all M-tiles of one (split, kv head) pair share an XCD.
-    const int wg = blockIdx.x;
-    const int xcd = wg % kXcds;
-    const int jj = wg / kXcds;
-    const int sh = xcd + kXcds * (jj / p.num_mtiles);
-    const int mt = jj % p.num_mtiles;
+    // XCD-aware work mapping: the grid is (splits x KV heads, padded to a multiple of the XCD count) x M-tiles.
+    // Workgroups are numbered x first and consecutive numbers go to consecutive XCDs, so x % 8 picks the XCD:
+    // all M-tiles of one (split, kv head) pair share an XCD and the K/V pages they stream meet in its L2.
+    // All launch arguments are fetched in one go, up front: left alone, the compiler fetches them in three batches as
+    // the code first needs them, and each batch is a memory round trip of its own in front of the first K/V request.
+    asm volatile("" ::"s"(p.q), "s"(p.k_pool), "s"(p.v_pool), "s"(p.block_table), "s"(p.kv_len), "s"(p.k_new), "s"(p.v_new), "s"(p.rope),
+                 "s"(p.mask), "s"(p.mask_words), "s"(p.mask_k_range), "s"(p.T), "s"(p.Hq), "s"(p.Hkv), "s"(p.group), "s"(p.group_shift),
+                 "s"(p.hkv_shift), "s"(p.num_splits), "s"(p.num_mtiles), "s"(p.ntiles_max), "s"(p.table_pages), "s"(p.window_blocks),
+                 "s"(p.max_kv_len));
+    const int sh = blockIdx.x;
+    const int mt = blockIdx.y;
     if (sh >= p.num_splits * p.Hkv) return;
-    const int g = sh % p.Hkv;
-    const int split = sh / p.Hkv;
+    const int g = p.hkv_shift >= 0 ? sh & (p.Hkv - 1) : sh % p.Hkv;
+    const int split = p.hkv_shift >= 0 ? sh >> p.hkv_shift : sh / p.Hkv;
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6;
@@ -217,35 +233,40 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
 
     const int R = mt * kRowsPerWg + rw * kRowsPerWave + qcol;  // packed row
     const bool row_ok = R < p.group * p.T;
-    const int node = row_ok ? R / p.group : 0;
-    const int head = g * p.group + (row_ok ? R % p.group : 0);
+    const int node = !row_ok ? 0 : p.group_shift >= 0 ? R >> p.group_shift : R / p.group;
+    const int head = g * p.group + (!row_ok ? 0 : p.group_shift >= 0 ? R & (p.group - 1) : R % p.group);
 
     // Loads that do not depend on the KV length go first.
-    // Q as the B operand of S^T = K.Q^T: lane (qcol, hf) holds d = 16*ks + 8*hf + [0,8).
-    f16x8 qreg[8];
-    {
-        const f16* qrow = p.q + ((size_t)node * p.Hq + head) * kHeadDim + hf * 8;
-#pragma unroll
-        for (int ks = 0; ks < 8; ++ks)
-            qreg[ks] = row_ok ? *reinterpret_cast<const f16x8*>(qrow + ks * 16) : zero8();
-    }
-    // Tree mask row of this lane's node with the causal bound j <= node folded in
-    // (src/flash_attn/src/mask.h:185-198).
-    uint64_t mw0, mw1 = 0;
+    // Tree mask row of this lane's node (src/flash_attn/src/mask.h:185-198).  The loads are issued here and
+    // awaited together with the Q rows below (loads return in order): written as assembly so that no wait of the
+    // compiler's own lands between the requests of this prologue.
+    uint64_t mw0 = ~0ull, mw1 = ~0ull;
     if (p.mask) {
-        mw0 = p.mask[(size_t)node * p.mask_words];
-        if (p.mask_words > 1) mw1 = p.mask[(size_t)node * p.mask_words + 1];
-    } else {
-        mw0 = ~0ull;
-        mw1 = ~0ull;
+        const uint64_t* mrow = p.mask + (size_t)node * p.mask_words;
+        asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(mw0) : "v"(mrow) : "memory");
+        if (p.mask_words > 1) asm volatile("global_load_dwordx2 %0, %1, off offset:8" : "=v"(mw1) : "v"(mrow) : "memory");
+        else mw1 = 0;
     }
+    // The workgroup's Q rows go to LDS first, as whole 256-byte rows (four rows per wave instruction), into the
+    // ring stages the first tile requests leave free, and are read from there into the B-operand registers:
+    // fetched straight into that layout -- every lane 16 bytes of a row of its own -- a wave instruction touches
+    // 32 cache lines for 1 KB and the eight of them hold the CU's address path for 1.5 us ahead of the first K/V
+    // tile.  Both KV groups read the same copy.
+    constexpr int kQStages = kRowsPerWg * kHeadDim * 2 / kStageBytes;  // ring stages the Q rows occupy
+    char* const qstage = ring + (kStages - kQStages) * kStageBytes;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
     {
-        // mask column of the query's own key: the causal bound keeps columns up to and including it
-        const int own = p.mask_k_range - p.T + node;
-        const uint64_t c0 = own >= 63 ? ~0ull : ((2ull << own) - 1ull);
-        const uint64_t c1 = own >= 127 ? ~0ull : (own < 64 ? 0ull : ((2ull << (own - 64)) - 1ull));
-        mw0 &= c0;
-        mw1 &= c1;
+        const int last_row = p.group * p.T - 1;
+#pragma unroll
+        for (int x = 0; x < kRowsPerWg / (4 * kWaves); ++x) {
+            const int inst = x * kWaves + wave_u;  // 1 KB of the staging area: rows 4 * inst .. + 3
+            const int r = inst * 4 + (lane >> 4);
+            const int Rr = min(mt * kRowsPerWg + r, last_row);  // rows past the end re-read the last one (zeroed below)
+            const int nr = p.group_shift >= 0 ? Rr >> p.group_shift : Rr / p.group;
+            const int hr = g * p.group + (p.group_shift >= 0 ? Rr & (p.group - 1) : Rr % p.group);
+            const int piece = (lane & 15) ^ (r & 15);  // the K tile's swizzle: the reads below are conflict-free
+            load_to_lds16_v(p.q + ((size_t)nr * p.Hq + hr) * kHeadDim + piece * 8, qstage + inst * 1024);
+        }
     }
 
     // The split's tile range is fixed by the host-side bound, so the page ids can be fetched without
@@ -256,23 +277,33 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
     // A block sliding window moves the start of the stream to its first visible tile, which depends on
     // the device-side length: such calls (the drafter's own layer, a few tiles in all) pay the extra
     // round trip in front of the page ids.
-    int tile_lo = 0;
-    if (p.window_blocks > 0)
-        tile_lo = max((p.kv_len[0] - p.T + 127) / 128 - p.window_blocks, 0) * (128 / kTileN);
     const int vtiles = p.ntiles_max + (p.k_new != nullptr && p.num_splits > 1 ? (ROPE ? 3 : 2) : 0);
-    const int t0 = tile_lo + min((int)(((long long)split * vtiles) / p.num_splits), p.ntiles_max);
-    const int t1_max = tile_lo + min((int)(((long long)(split + 1) * vtiles) / p.num_splits), p.ntiles_max);
-    const int pg0 = (t0 * kTileN) / kPage;
-    if (t1_max > t0) {
-        const int npg = ((t1_max * kTileN - 1) / kPage) - pg0 + 1;
-        // (a window's last tile slot can lie past the host bound; it is never consumed, and the table is not read there)
-        for (int i = tid; i < npg; i += kThreads) s_pages[i] = p.block_table[min(pg0 + i, p.table_pages - 1)];
+    const int r0 = min((int)(((long long)split * vtiles) / p.num_splits), p.ntiles_max);
+    const int r1 = min((int)(((long long)(split + 1) * vtiles) / p.num_splits), p.ntiles_max);
+    // The device-side length and the page id of the split's first tile come through scalar loads, together: the
+    // Q rows requested above are still on their way, and a vector load of these few bytes would return behind them.
+    int S, first_page;
+    int tile_lo = 0;
+    if (p.window_blocks > 0) {  // the window's first tile depends on the length: one more round trip for the page id
+        S = scalar_load(p.kv_len);
+        tile_lo = max((S - p.T + 127) / 128 - p.window_blocks, 0) * (128 / kTileN);
+        first_page = scalar_load(p.block_table + min(((tile_lo + r0) * kTileN) / kPage, p.table_pages - 1));
+    } else {
+        scalar_load2(p.kv_len, p.block_table + min((r0 * kTileN) / kPage, p.table_pages - 1), S, first_page);
     }
-    int S = p.kv_len[0];
+    const int t0 = tile_lo + r0;
+    const int t1_max = tile_lo + r1;
+    const int pg0 = (t0 * kTileN) / kPage;
+    // page of a tile: a scalar load of its table entry (the first one is already here)
+    // (a window's last tile slot can lie past the host bound; it is never consumed, and the table is not read there)
+    auto page_of_tile = [&](int tile) {
+        const int pg = (tile * kTileN) / kPage;
+        return pg == pg0 ? first_page : scalar_load(p.block_table + min(pg, p.table_pages - 1));
+    };
     {
         const int lo = max(p.T, p.mask_k_range);
         if (S > p.max_kv_len || S < lo) {
-            if (wg == 0 && tid == 0) g_attn_bad_length = S == 0 ? -1 : S;
+            if (sh == 0 && mt == 0 && tid == 0) g_attn_bad_length = S == 0 ? -1 : S;
             S = min(max(S, lo), p.max_kv_len);
         }
     }
@@ -282,23 +313,20 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
     const int t1 = min(t1_max, ntiles);
     const int n = max(t1 - t0, 0);
     const int niter = (n + G - 1) / G;  // one iteration consumes G tiles, one per KV group
-    __syncthreads();
 
-    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
     const uint32_t koff = k_piece_off(wave, lane), voff = v_piece_off(wave, lane);
+    auto issue_tile_i = [&](int i) {  // the i-th tile of this workgroup's range, into its ring stage
+        const int tile = t0 + i;
+        const int page = page_of_tile(tile);
+        if (p.k_new != nullptr && (tile + 1) * kTileN > P)
+            issue_tile_append(p, g, tile, page, ring + (i % kStages) * kStageBytes, wave_u, lane, koff, voff, P, S);
+        else
+            issue_tile(p, g, tile, page, ring + (i % kStages) * kStageBytes, wave_u, koff, voff);
+    };
     auto issue_iter = [&](int it) {
 #pragma unroll
-        for (int e = 0; e < G; ++e) {
-            const int i = it * G + e;
-            if (i < n) {
-                const int tile = t0 + i;
-                const int page = __builtin_amdgcn_readfirstlane(s_pages[(tile * kTileN) / kPage - pg0]);
-                if (p.k_new != nullptr && (tile + 1) * kTileN > P)
-                    issue_tile_append(p, g, tile, page, ring + (i % kStages) * kStageBytes, wave_u, lane, koff, voff, P, S);
-                else
-                    issue_tile(p, g, tile, page, ring + (i % kStages) * kStageBytes, wave_u, koff, voff);
-            }
-        }
+        for (int e = 0; e < G; ++e)
+            if (it * G + e < n) issue_tile_i(it * G + e);
     };
 
     f32x16 oacc[4];
@@ -326,9 +354,42 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
             load_to_lds16_v(p.v_new + ((size_t)r * p.Hkv + g) * kHeadDim + (lane & 15) * 8, vstage + inst * 1024);
         }
     }
+    // The first tiles are requested into the stages the Q rows do not occupy ...
+    constexpr int kPrologueTiles = (kDepth + 1) * G;  // = kStages
+    constexpr int kEarlyTiles = kStages - kQStages;
+    const int n_early = min(n, kEarlyTiles);
 #pragma unroll
-    for (int d = 0; d <= kDepth; ++d)
-        if (d < niter) issue_iter(d);
+    for (int i = 0; i < kEarlyTiles; ++i)
+        if (i < n) issue_tile_i(i);
+    // ... then the Q rows (and the mask words, older still) are awaited: everything requested after them may stay in flight
+    // (4 loads per thread and tile; the two staged V requests, where issued, are waited for as well).
+    switch (n_early) {
+        case 0: asm volatile("s_waitcnt vmcnt(0)" : "+v"(mw0), "+v"(mw1)::"memory"); break;
+        case 1: asm volatile("s_waitcnt vmcnt(4)" : "+v"(mw0), "+v"(mw1)::"memory"); break;
+        case 2: asm volatile("s_waitcnt vmcnt(8)" : "+v"(mw0), "+v"(mw1)::"memory"); break;
+        default: asm volatile("s_waitcnt vmcnt(12)" : "+v"(mw0), "+v"(mw1)::"memory"); break;
+    }
+    __syncthreads();
+    // Q as the B operand of S^T = K.Q^T: lane (qcol, hf) holds d = 16*ks + 8*hf + [0,8).
+    f16x8 qreg[8];
+#pragma unroll
+    for (int ks = 0; ks < 8; ++ks) {
+        const f16x8 v = *reinterpret_cast<const f16x8*>(qstage + k_lds_off(rw * kRowsPerWave + qcol, 2 * ks + hf));
+        qreg[ks] = row_ok ? v : zero8();
+    }
+    __syncthreads();  // the stages are free for tiles
+#pragma unroll
+    for (int i = kEarlyTiles; i < kPrologueTiles; ++i)
+        if (i < n) issue_tile_i(i);
+    {
+        // the causal bound j <= node folded into the mask row: the mask column of the query's own key is kept,
+        // every column above it cleared
+        const int own = p.mask_k_range - p.T + node;
+        const uint64_t c0 = own >= 63 ? ~0ull : ((2ull << own) - 1ull);
+        const uint64_t c1 = own >= 127 ? ~0ull : (own < 64 ? 0ull : ((2ull << (own - 64)) - 1ull));
+        mw0 &= c0;
+        mw1 &= c1;
+    }
 
     // Fused rotary embedding of the query (rotary_embedding_kernel, src/model/rotary.cuh:11-22), placed behind
     // the first tile requests so that its table reads and arithmetic run under their latency: the pair
@@ -387,7 +448,7 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
                 if (ie >= n) continue;
                 char* st = ring + (ie % kStages) * kStageBytes;
                 const bool append = p.k_new != nullptr && ce + kTileN > P;
-                const int pg = append ? s_pages[(ce + kTileN - 1) / kPage - pg0] : 0;  // a tile lies inside one page
+                const int pg = append ? p.block_table[min((ce + kTileN - 1) / kPage, p.table_pages - 1)] : 0;  // a tile lies inside one page
                 if (ROPE && append) {
                     // Fused rotary embedding of the appended K rows (src/model/rotary.cuh:23-33): the tile holds
                     // them as fetched from k_new; one thread per (key, 16-byte piece of the lower half) rotates
@@ -775,9 +836,6 @@ LaunchPlan plan_launch(int T, int group, int Hkv, int max_kv_len, int block_wind
     pl.kv_groups = choose_groups(T, group, Hkv, pl.span);
     pl.num_mtiles = ceil_div(group * T, rows_per_wg(pl.kv_groups));
     pl.num_splits = num_splits_override > 0 ? num_splits_override : choose_splits(T, group, Hkv, pl.span, pl.kv_groups);
-    // a split keeps the physical page ids of its range in LDS
-    const int min_splits = ceil_div(ceil_div(pl.span, kPage) + 2, kMaxPagesPerSplit - 2);
-    if (pl.num_splits < min_splits) pl.num_splits = min_splits;
     return pl;
 }
 
@@ -864,6 +922,13 @@ static int tree_attention_impl(const void* q, void* k_pool, void* v_pool,
     p.Hq = Hq;
     p.Hkv = Hkv;
     p.group = group;
+    auto log2_or_minus1 = [](int v) {
+        int sft = 0;
+        while ((1 << sft) < v) ++sft;
+        return (1 << sft) == v ? sft : -1;
+    };
+    p.group_shift = log2_or_minus1(group);
+    p.hkv_shift = log2_or_minus1(Hkv);
     p.window_blocks = block_window_size / 128;
     const LaunchPlan plan = plan_launch(T, group, Hkv, max_kv_len, block_window_size, num_splits_override);
     const int span = plan.span;
@@ -889,13 +954,13 @@ static int tree_attention_impl(const void* q, void* k_pool, void* v_pool,
     }
     hipStream_t st = resolve_stream(stream);
     const int nsh = p.num_splits * Hkv;
-    const int grid = kXcds * ceil_div(nsh, kXcds) * p.num_mtiles;
+    const dim3 grid(kXcds * ceil_div(nsh, kXcds), p.num_mtiles);
     if (p.rope != nullptr) {
-        if (G == 1) hipLaunchKernelGGL((tree_attn_split_kernel<1, true>), dim3(grid), dim3(kThreads), 0, st, p);
-        else hipLaunchKernelGGL((tree_attn_split_kernel<2, true>), dim3(grid), dim3(kThreads), 0, st, p);
+        if (G == 1) hipLaunchKernelGGL((tree_attn_split_kernel<1, true>), grid, dim3(kThreads), 0, st, p);
+        else hipLaunchKernelGGL((tree_attn_split_kernel<2, true>), grid, dim3(kThreads), 0, st, p);
     } else {
-        if (G == 1) hipLaunchKernelGGL((tree_attn_split_kernel<1, false>), dim3(grid), dim3(kThreads), 0, st, p);
-        else hipLaunchKernelGGL((tree_attn_split_kernel<2, false>), dim3(grid), dim3(kThreads), 0, st, p);
+        if (G == 1) hipLaunchKernelGGL((tree_attn_split_kernel<1, false>), grid, dim3(kThreads), 0, st, p);
+        else hipLaunchKernelGGL((tree_attn_split_kernel<2, false>), grid, dim3(kThreads), 0, st, p);
     }
     CPMCU_LAUNCH_CHECK();
     if (p.num_splits > 1) {
