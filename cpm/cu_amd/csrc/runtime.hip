@@ -48,6 +48,7 @@ Options& options() {
             if (e[0] == '2' && e[1] == 0) o.attn_kv_groups = 2;
         }
         if (getenv("CPMCU_HEAD_NO_SHARE") != nullptr) o.head_share_last_pass = 0;
+        if (getenv("CPMCU_ATTN_SEPARATE_MERGE") != nullptr) o.attn_merge_in_launch = 0;
         return o;
     }();
     return opt;
@@ -159,6 +160,11 @@ int check_device_errors() {
     int bad = 0;
     int rc = attention_take_bad_length(&bad);
     if (rc) return rc;
+    if (bad == INT32_MIN) {
+        set_error("a tree-attention launch gave up waiting for the other workgroups of its merge (20 ms): part of its output was "
+                  "not written");
+        return CPMCU_ERR_RUNTIME;
+    }
     if (bad != 0) {
         set_error("a tree-attention launch read a KV length of %d from device memory, outside [rows, max_kv_len] of its call; "
                   "it ran on the clamped length and its output is not valid", bad < 0 ? 0 : bad);
@@ -192,6 +198,9 @@ extern "C" int cpmcu_set_option(const char* name, int value) {
     } else if (nm == "head_share_last_pass") {
         CPMCU_CHECK_ARG(value == 0 || value == 1, "set_option: head_share_last_pass=%d must be 0 or 1", value);
         options().head_share_last_pass = value;
+    } else if (nm == "attn_merge_in_launch") {
+        CPMCU_CHECK_ARG(value == 0 || value == 1, "set_option: attn_merge_in_launch=%d must be 0 or 1", value);
+        options().attn_merge_in_launch = value;
     } else {
         set_error("set_option: unknown option %s", name);
         return CPMCU_ERR_INVALID_ARGUMENT;

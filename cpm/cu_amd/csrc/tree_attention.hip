@@ -35,7 +35,10 @@
 #include "common.h"
 #include "internal.h"
 
+#include <map>
+#include <mutex>
 #include <type_traits>
+#include <utility>
 
 namespace cpmcu {
 namespace {
@@ -98,7 +101,95 @@ struct AttnParams {
     //   ml_part [Hkv][num_splits][rows_pad] x float2 (max * scale_log2, sum)
     float* o_part;
     float* ml_part;
+    // Merge inside the split launch (null: the separate combine kernel does it): one {arrivals, generation} pair
+    // per (KV head, M-tile) unit.  Between launches arrivals is 0; the last workgroup of a unit to arrive sets it
+    // back and bumps the generation, which the others wait for.
+    uint32_t* merge_ctr;
 };
+
+constexpr int kMergeUnitWords = 128;  // the two words of a unit sit in 256-byte lines of their own: every poll and every
+                                      // arrival is a memory transaction, and those on one line queue behind each other
+constexpr int kMergeWaitExpired = INT32_MIN;  // value of g_attn_bad_length after a merge wait ran into its limit
+constexpr unsigned long long kMergeWaitTicks = 2000000ull;  // 20 ms of the 100 MHz wall clock
+
+// Loads and stores that other XCDs' workgroups of the same launch see: device-scope accesses go past the
+// (per-XCD, mutually incoherent) L2.
+__device__ inline uint64_t load_dev64(const void* ptr) {
+    return __hip_atomic_load(reinterpret_cast<const uint64_t*>(ptr), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ inline void store_dev64(void* ptr, uint64_t v) {
+    __hip_atomic_store(reinterpret_cast<uint64_t*>(ptr), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <typename To, typename From>
+__device__ inline To bits_as(const From& v) {
+    static_assert(sizeof(To) == sizeof(From), "bits_as: size mismatch");
+    return __builtin_bit_cast(To, v);
+}
+
+// Merge of the split partials of one 32-row block and one quad of output dims (one wave; lane = accumulator lane):
+// M = max_s m_s, L = sum_s l_s 2^(m_s - M), O = sum_s l_s 2^(m_s - M) (O_s / l_s) / L -- the log-sum-exp merge of
+// src/flash_attn/src/flash_fwd_kernel.h:2392-2472 in base-2 form.  The statistics and the O partials of up to 16
+// splits are all requested before any is used, so a block pays one memory round trip, not one per split.
+// DEV: the partials were written by other workgroups of this launch (device-scope loads).
+constexpr int kCombineBatch = 16;
+template <bool DEV>
+__device__ inline void combine_block(const AttnParams& p, int g, int rb, int quad, int lane) {
+    const int nrb = p.rows_pad / kRowsPerWave;  // 32-row blocks per kv head
+    const int qcol = lane & 31, hf = lane >> 5;
+    const int R = rb * kRowsPerWave + qcol;
+    if (R >= p.group * p.T) return;
+    const int node = p.group_shift >= 0 ? R >> p.group_shift : R / p.group;
+    const int head = g * p.group + (p.group_shift >= 0 ? R & (p.group - 1) : R % p.group);
+    const int d0 = (quad >> 2) * 32 + (quad & 3) * 8 + hf * 4;
+    const float2* ml = reinterpret_cast<const float2*>(p.ml_part) + (size_t)g * p.num_splits * p.rows_pad + R;
+    const f16x4* op = reinterpret_cast<const f16x4*>(p.o_part) +
+                      (((size_t)g * p.num_splits) * nrb + rb) * 16 * 64 + quad * 64 + lane;
+    const size_t ml_stride = (size_t)p.rows_pad;
+    const size_t o_stride = (size_t)nrb * 16 * 64;
+
+    float M = -INFINITY, L = 0.f;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < p.num_splits; s0 += kCombineBatch) {
+        float2 v[kCombineBatch];
+        f16x4 o[kCombineBatch];
+#pragma unroll
+        for (int u = 0; u < kCombineBatch; ++u) {
+            const int s = min(s0 + u, p.num_splits - 1);  // clamp: repeats are ignored below
+            if (DEV) {
+                const uint64_t mlw = load_dev64(&ml[s * ml_stride]);
+                v[u] = make_float2(__uint_as_float((uint32_t)mlw), __uint_as_float((uint32_t)(mlw >> 32)));
+                o[u] = bits_as<f16x4>(load_dev64(&op[s * o_stride]));
+            } else {
+                v[u] = ml[s * ml_stride];
+                o[u] = op[s * o_stride];
+            }
+        }
+        float Mb = M;
+#pragma unroll
+        for (int u = 0; u < kCombineBatch; ++u)
+            if (s0 + u < p.num_splits && v[u].y > 0.f) Mb = fmaxf(Mb, v[u].x);
+        if (Mb == -INFINITY) continue;  // nothing but empty splits so far
+        const float resc = __builtin_amdgcn_exp2f(M - Mb);  // 0 when M was -inf
+        L *= resc;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] *= resc;
+        M = Mb;
+#pragma unroll
+        for (int u = 0; u < kCombineBatch; ++u) {
+            // an empty split (l == 0) has no meaningful O partial: select it away, never scale it
+            if (!(s0 + u < p.num_splits && v[u].y > 0.f)) continue;
+            const float w = __builtin_amdgcn_exp2f(v[u].x - M) * v[u].y;  // partials are stored normalised
+            L += w;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[e] += w * (float)o[u][e];
+        }
+    }
+    const float inv = (L == 0.f || L != L) ? 1.f : 1.f / L;
+    f16x4 o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = (f16)(acc[e] * inv);
+    *reinterpret_cast<f16x4*>(p.out + ((size_t)node * p.Hq + head) * kHeadDim + d0) = o;
+}
 
 // One rotary pair: (a, b) -> (a cos - b sin, a sin + b cos), every product and sum rounded on its own
 // (no fused multiply-add), so the result does not depend on how a compiler contracts the expression.
@@ -131,6 +222,12 @@ __device__ inline int v_lds_off(int d, int piece) { return kKTileBytes + d * 128
 __device__ inline void load_to_lds16(const void* base, uint32_t byte_off, const char* lds_dst) {
     const uint32_t lds_addr = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)lds_dst);
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(byte_off), "s"(base), "s"(lds_addr) : "memory", "m0");
+}
+
+// Four bytes per lane (256 bytes per wave instruction), full per-lane address.
+__device__ inline void load_to_lds4_v(const void* gptr, const char* lds_dst) {
+    const uint32_t lds_addr = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_ptr_t)lds_dst);
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off" : : "v"(gptr), "s"(lds_addr) : "memory", "m0");
 }
 
 // Same, with a full per-lane address (used where lanes of one instruction read from different buffers).
@@ -207,6 +304,7 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
     constexpr int kDepth = kStages / G - 1;  // iterations in flight behind the one being consumed
     __shared__ __attribute__((aligned(1024))) char ring[kStages * kStageBytes];
     __shared__ __attribute__((aligned(1024))) char vstage[kVStageRows * kHeadDim * 2];  // first appended V rows, row-major
+    __shared__ uint64_t s_mask[kMaxTree * 2];                                            // the tree mask as handed in
 
     // XCD-aware work mapping: the grid is (splits x KV heads, padded to a multiple of the XCD count) x M-tiles.
     // Workgroups are numbered x first and consecutive numbers go to consecutive XCDs, so x % 8 picks the XCD:
@@ -226,6 +324,9 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
     const int tid = threadIdx.x;
     const int wave = tid >> 6;
     const int lane = tid & 63;
+    // merge inside the launch: the unit's arrivals word and, 256 bytes on, its generation word
+    uint32_t* const unit_ctr = p.merge_ctr ? p.merge_ctr + kMergeUnitWords * (g * p.num_mtiles + mt) : nullptr;
+    uint32_t* const unit_gen = unit_ctr + kMergeUnitWords / 2;
     const int grp = wave / kRowWaves;  // KV group: takes tiles grp, grp + G, ...
     const int rw = wave % kRowWaves;
     const int qcol = lane & 31;
@@ -237,15 +338,13 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
     const int head = g * p.group + (!row_ok ? 0 : p.group_shift >= 0 ? R & (p.group - 1) : R % p.group);
 
     // Loads that do not depend on the KV length go first.
-    // Tree mask row of this lane's node (src/flash_attn/src/mask.h:185-198).  The loads are issued here and
-    // awaited together with the Q rows below (loads return in order): written as assembly so that no wait of the
-    // compiler's own lands between the requests of this prologue.
-    uint64_t mw0 = ~0ull, mw1 = ~0ull;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+    // The tree mask (src/flash_attn/src/mask.h:185-198; at most 128 rows of two words) goes to LDS whole, one request
+    // per wave, and is awaited together with the Q rows below (requests return in order): a load into registers here
+    // would have the compiler wait for everything in flight at the mask's first use.
     if (p.mask) {
-        const uint64_t* mrow = p.mask + (size_t)node * p.mask_words;
-        asm volatile("global_load_dwordx2 %0, %1, off" : "=v"(mw0) : "v"(mrow) : "memory");
-        if (p.mask_words > 1) asm volatile("global_load_dwordx2 %0, %1, off offset:8" : "=v"(mw1) : "v"(mrow) : "memory");
-        else mw1 = 0;
+        const int ndw = p.T * p.mask_words * 2;
+        load_to_lds4_v(reinterpret_cast<const uint32_t*>(p.mask) + min(wave_u * 64 + lane, ndw - 1), reinterpret_cast<const char*>(s_mask) + wave_u * 256);
     }
     // The workgroup's Q rows go to LDS first, as whole 256-byte rows (four rows per wave instruction), into the
     // ring stages the first tile requests leave free, and are read from there into the B-operand registers:
@@ -254,8 +353,7 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
     // tile.  Both KV groups read the same copy.
     constexpr int kQStages = kRowsPerWg * kHeadDim * 2 / kStageBytes;  // ring stages the Q rows occupy
     char* const qstage = ring + (kStages - kQStages) * kStageBytes;
-    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-    {
+    auto issue_q = [&]()     {
         const int last_row = p.group * p.T - 1;
 #pragma unroll
         for (int x = 0; x < kRowsPerWg / (4 * kWaves); ++x) {
@@ -267,7 +365,7 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
             const int piece = (lane & 15) ^ (r & 15);  // the K tile's swizzle: the reads below are conflict-free
             load_to_lds16_v(p.q + ((size_t)nr * p.Hq + hr) * kHeadDim + piece * 8, qstage + inst * 1024);
         }
-    }
+    };
 
     // The split's tile range is fixed by the host-side bound, so the page ids can be fetched without
     // waiting for the device-side length; the length only clips the range.
@@ -358,18 +456,28 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
     constexpr int kPrologueTiles = (kDepth + 1) * G;  // = kStages
     constexpr int kEarlyTiles = kStages - kQStages;
     const int n_early = min(n, kEarlyTiles);
+    constexpr int kFirstTiles = G;  // the first iteration's tiles go ahead of the Q rows
 #pragma unroll
-    for (int i = 0; i < kEarlyTiles; ++i)
+    for (int i = 0; i < kFirstTiles; ++i)
+        if (i < n) issue_tile_i(i);
+    issue_q();
+#pragma unroll
+    for (int i = kFirstTiles; i < kEarlyTiles; ++i)
         if (i < n) issue_tile_i(i);
     // ... then the Q rows (and the mask words, older still) are awaited: everything requested after them may stay in flight
     // (4 loads per thread and tile; the two staged V requests, where issued, are waited for as well).
-    switch (n_early) {
-        case 0: asm volatile("s_waitcnt vmcnt(0)" : "+v"(mw0), "+v"(mw1)::"memory"); break;
-        case 1: asm volatile("s_waitcnt vmcnt(4)" : "+v"(mw0), "+v"(mw1)::"memory"); break;
-        case 2: asm volatile("s_waitcnt vmcnt(8)" : "+v"(mw0), "+v"(mw1)::"memory"); break;
-        default: asm volatile("s_waitcnt vmcnt(12)" : "+v"(mw0), "+v"(mw1)::"memory"); break;
+    switch (n_early - min(n, kFirstTiles)) {
+        case 0: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+        case 1: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
+        case 2: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+        default: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
     }
     __syncthreads();
+    uint64_t mw0 = ~0ull, mw1 = ~0ull;
+    if (p.mask) {
+        mw0 = s_mask[node * p.mask_words];
+        mw1 = p.mask_words > 1 ? s_mask[node * p.mask_words + 1] : 0ull;
+    }
     // Q as the B operand of S^T = K.Q^T: lane (qcol, hf) holds d = 16*ks + 8*hf + [0,8).
     f16x8 qreg[8];
 #pragma unroll
@@ -646,6 +754,10 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
         }
     }
 
+    // Merge inside the launch: the unit's generation as it stands before this workgroup has arrived (it moves only
+    // once all of the unit's workgroups have), requested here so that it is back by the time the partials are stored.
+    uint32_t gen0 = 0;
+    if (unit_ctr != nullptr && tid == 0) gen0 = __hip_atomic_load(unit_gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     // ---- merge the two KV groups through LDS (lane-private layout: [row wave][value][lane]) ----
     if constexpr (G == 2) {
     __syncthreads();  // ring no longer read
@@ -664,8 +776,8 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
         xch[xbase + 16 * 64] = f32x4{m_ref, l_run, 0.f, 0.f};
     }
     __syncthreads();
-    if (grp == 1) return;
-    {
+    if (grp == 1 && unit_ctr == nullptr) return;  // (with the merge in the launch, group 1 stays for its share of it)
+    if (grp == 0) {
         const f32x4 ml1 = xch[xbase + 16 * 64];
         const float m1 = ml1[0], l1 = ml1[1];
         const float m_new = fmaxf(m_ref, m1);
@@ -687,6 +799,7 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
 
     // oacc[db][r] is O[query qcol][d = db*32 + 8*(r/4) + 4*hf + r%4], unnormalised.
     const float l_tot = l_run + __shfl_xor(l_run, 32);
+    const bool owner = G == 1 || grp == 0;  // this wave holds the workgroup's result for its rows
     if (p.num_splits == 1) {
         if (!row_ok) return;
         const float inv = (l_tot == 0.f || l_tot != l_tot) ? 1.f : 1.f / l_tot;
@@ -708,6 +821,7 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
         const float inv = (l_tot == 0.f || l_tot != l_tot) ? 0.f : 1.f / l_tot;
         f16x4* op = reinterpret_cast<f16x4*>(p.o_part) +
                     ((((size_t)g * p.num_splits + split) * p.num_mtiles + mt) * kRowWaves + rw) * 16 * 64 + lane;
+        if (owner)
 #pragma unroll
         for (int db = 0; db < 4; ++db)
 #pragma unroll
@@ -715,78 +829,63 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
                 f16x4 o;
 #pragma unroll
                 for (int e = 0; e < 4; ++e) o[e] = (f16)(oacc[db][rq * 4 + e] * inv);
-                __builtin_nontemporal_store(o, &op[(db * 4 + rq) * 64]);  // streamed: nothing left to flush at kernel end
+                if (unit_ctr != nullptr) store_dev64(&op[(db * 4 + rq) * 64], bits_as<uint64_t>(o));
+                else __builtin_nontemporal_store(o, &op[(db * 4 + rq) * 64]);  // streamed: nothing left to flush at kernel end
             }
-        if (hf == 0 && row_ok) {
-            p.ml_part[prow * 2 + 0] = m_ref;
-            p.ml_part[prow * 2 + 1] = l_tot;
+        if (owner && hf == 0 && row_ok) {
+            if (unit_ctr != nullptr) {
+                store_dev64(&p.ml_part[prow * 2], (uint64_t)__float_as_uint(m_ref) | ((uint64_t)__float_as_uint(l_tot) << 32));
+            } else {
+                p.ml_part[prow * 2 + 0] = m_ref;
+                p.ml_part[prow * 2 + 1] = l_tot;
+            }
         }
+        if (unit_ctr == nullptr) return;
+        // ---- merge inside the launch ----
+        // Every workgroup of the unit (same KV head and M-tile, one per split) announces its partials once they
+        // have reached memory; when all have, each merges a share of the unit's 32-row x 4-dim-quad blocks.
+        // The last to arrive never waits; the others wait for it, with a limit: a launch whose workgroups cannot all
+        // be resident at once would otherwise wait on workgroups that cannot start (the host only picks this path
+        // when they fit; a wait that runs out leaves its blocks unmerged and is reported at the next synchronisation).
+        __shared__ int s_merge_go;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0) {
+            int go = 1;
+            const uint32_t arrived = __hip_atomic_fetch_add(unit_ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (arrived == (uint32_t)p.num_splits - 1u) {
+                __hip_atomic_store(unit_ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                __hip_atomic_store(unit_gen, gen0 + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            } else {
+                const unsigned long long t_begin = wall_clock64();
+                while (__hip_atomic_load(unit_gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == gen0) {
+                    if (wall_clock64() - t_begin > kMergeWaitTicks) {
+                        g_attn_bad_length = kMergeWaitExpired;
+                        go = 0;
+                        break;
+                    }
+                    __builtin_amdgcn_s_sleep(8);
+                }
+            }
+            s_merge_go = go;
+        }
+        __syncthreads();
+        if (!s_merge_go) return;
+        const int nblocks = kRowWaves * 16;
+        for (int b = split + p.num_splits * wave; b < nblocks; b += p.num_splits * kWaves)
+            combine_block<true>(p, g, mt * kRowWaves + (b >> 4), b & 15, lane);
     }
 }
 
-// Merge of the split partials: M = max_s m_s, L = sum_s l_s 2^(m_s - M),
-// O = sum_s l_s 2^(m_s - M) (O_s / l_s) / L  -- the log-sum-exp merge of
-// src/flash_attn/src/flash_fwd_kernel.h:2392-2472 in base-2 form.
-// One thread per (packed row, 4 output dims).  The statistics and the O partials of up to 16 splits
-// are all requested before any is used, so the kernel pays one memory round trip, not one per split.
-constexpr int kCombineBatch = 16;
+// The merge as a launch of its own: one wave per (kv head, 32-row block, quad), in the partial layout's own order.
 __global__ __launch_bounds__(256) void tree_attn_combine_kernel(AttnParams p) {
-    // thread -> (kv head, 32-row block, quad, lane) in the partial layout's own order
     const int idx = blockIdx.x * 256 + threadIdx.x;
     const int lane = idx & 63;
     const int quad = (idx >> 6) & 15;
     const int nrb = p.rows_pad / kRowsPerWave;  // 32-row blocks per kv head (16 * 64 = 1024 threads each)
     const int grb = idx >> 10;
     if (grb >= p.Hkv * nrb) return;
-    const int g = grb / nrb, rb = grb % nrb;
-    const int qcol = lane & 31, hf = lane >> 5;
-    const int R = rb * kRowsPerWave + qcol;
-    if (R >= p.group * p.T) return;
-    const int node = R / p.group;
-    const int head = g * p.group + R % p.group;
-    const int d0 = (quad >> 2) * 32 + (quad & 3) * 8 + hf * 4;
-    const float2* ml = reinterpret_cast<const float2*>(p.ml_part) + (size_t)g * p.num_splits * p.rows_pad + R;
-    const f16x4* op = reinterpret_cast<const f16x4*>(p.o_part) +
-                      (((size_t)g * p.num_splits) * nrb + rb) * 16 * 64 + quad * 64 + lane;
-    const size_t ml_stride = (size_t)p.rows_pad;
-    const size_t o_stride = (size_t)nrb * 16 * 64;
-
-    float M = -INFINITY, L = 0.f;
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-    for (int s0 = 0; s0 < p.num_splits; s0 += kCombineBatch) {
-        float2 v[kCombineBatch];
-        f16x4 o[kCombineBatch];
-#pragma unroll
-        for (int u = 0; u < kCombineBatch; ++u) {
-            const int s = min(s0 + u, p.num_splits - 1);  // clamp: repeats are ignored below
-            v[u] = ml[s * ml_stride];
-            o[u] = op[s * o_stride];
-        }
-        float Mb = M;
-#pragma unroll
-        for (int u = 0; u < kCombineBatch; ++u)
-            if (s0 + u < p.num_splits && v[u].y > 0.f) Mb = fmaxf(Mb, v[u].x);
-        if (Mb == -INFINITY) continue;  // nothing but empty splits so far
-        const float resc = __builtin_amdgcn_exp2f(M - Mb);  // 0 when M was -inf
-        L *= resc;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) acc[e] *= resc;
-        M = Mb;
-#pragma unroll
-        for (int u = 0; u < kCombineBatch; ++u) {
-            // an empty split (l == 0) has no meaningful O partial: select it away, never scale it
-            if (!(s0 + u < p.num_splits && v[u].y > 0.f)) continue;
-            const float w = __builtin_amdgcn_exp2f(v[u].x - M) * v[u].y;  // partials are stored normalised
-            L += w;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) acc[e] += w * (float)o[u][e];
-        }
-    }
-    const float inv = (L == 0.f || L != L) ? 1.f : 1.f / L;
-    f16x4 o;
-#pragma unroll
-    for (int e = 0; e < 4; ++e) o[e] = (f16)(acc[e] * inv);
-    *reinterpret_cast<f16x4*>(p.out + ((size_t)node * p.Hq + head) * kHeadDim + d0) = o;
+    combine_block<false>(p, grb / nrb, grb % nrb, quad, lane);
 }
 
 int choose_splits(int T, int group, int Hkv, int max_kv_len, int G) {
@@ -827,7 +926,61 @@ struct LaunchPlan {
     int span;        // keys the stream can hold: the whole context, or with a window its blocks plus the T new rows
                      // (the window starts on a block boundary at or above P - block_window_size)
     int kv_groups, num_mtiles, num_splits;
+    bool merge_in_launch;  // the split workgroups merge their own partials (no combine launch)
 };
+
+// Counters of the in-launch merge.  They live in the library (zero when it is loaded, and back at zero arrivals after
+// every launch), in blocks handed out per workspace: calls that may overlap use different workspaces and so different
+// counters, and nothing has to be cleared or allocated per call.
+constexpr int kMergeUnits = 256;    // (KV head, M-tile) units a launch may have on this path
+constexpr int kMergeBlocks = 32;    // workspaces that get a block; further ones use the combine launch
+constexpr int kMergeMaxSplits = 32; // arrivals on one counter serialise, about 0.15 us each
+__device__ __align__(256) uint32_t g_merge_ctr[kMergeBlocks][kMergeUnits * kMergeUnitWords];
+
+int device_cu_count() {
+    static int cus[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    if (cus[dev] == 0) {
+        int v = 0;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+        cus[dev] = v;
+    }
+    return cus[dev];
+}
+
+// The split workgroups can merge in the launch when they are all resident at once (one per CU: a workgroup that
+// waits for the others must not keep them from starting) and few enough per counter.
+bool can_merge_in_launch(int Hkv, int num_mtiles, int num_splits) {
+    if (!options().attn_merge_in_launch || num_splits < 2 || num_splits > kMergeMaxSplits) return false;
+    if (Hkv * num_mtiles > kMergeUnits) return false;
+    return kXcds * ceil_div(num_splits * Hkv, kXcds) * num_mtiles <= device_cu_count();
+}
+
+// The counter block of a workspace on the current device (null: none left, or the lookup failed).
+uint32_t* merge_counters_for(const void* workspace) {
+    static std::mutex mu;
+    static std::map<std::pair<int, const void*>, int> blocks;
+    static int next_block[64] = {0};
+    static uint32_t* base[64] = {nullptr};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+    std::lock_guard<std::mutex> lock(mu);
+    if (base[dev] == nullptr) {
+        void* ptr = nullptr;
+        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_merge_ctr)) != hipSuccess) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
+        base[dev] = (uint32_t*)ptr;
+    }
+    auto it = blocks.find({dev, workspace});
+    if (it == blocks.end()) {
+        if (next_block[dev] >= kMergeBlocks) return nullptr;
+        it = blocks.emplace(std::make_pair(dev, workspace), next_block[dev]++).first;
+    }
+    return base[dev] + (size_t)it->second * kMergeUnits * kMergeUnitWords;
+}
 LaunchPlan plan_launch(int T, int group, int Hkv, int max_kv_len, int block_window_size, int num_splits_override) {
     LaunchPlan pl;
     const int window_blocks = block_window_size / 128;
@@ -836,6 +989,7 @@ LaunchPlan plan_launch(int T, int group, int Hkv, int max_kv_len, int block_wind
     pl.kv_groups = choose_groups(T, group, Hkv, pl.span);
     pl.num_mtiles = ceil_div(group * T, rows_per_wg(pl.kv_groups));
     pl.num_splits = num_splits_override > 0 ? num_splits_override : choose_splits(T, group, Hkv, pl.span, pl.kv_groups);
+    pl.merge_in_launch = can_merge_in_launch(Hkv, pl.num_mtiles, pl.num_splits);
     return pl;
 }
 
@@ -852,7 +1006,7 @@ extern "C" int cpmcu_tree_attention_plan(int T, int Hq, int Hkv, int max_kv_len,
     const LaunchPlan pl = plan_launch(T, Hq / Hkv, Hkv, max_kv_len, block_window_size, num_splits_override);
     if (kernel_names && kernel_names_bytes > 0)
         snprintf(kernel_names, kernel_names_bytes, "tree_attn_split_kernel<%d,%s>%s", pl.kv_groups, with_rope ? "true" : "false",
-                 pl.num_splits > 1 ? "+tree_attn_combine_kernel" : "");
+                 pl.num_splits > 1 && !pl.merge_in_launch ? "+tree_attn_combine_kernel" : "");
     if (num_splits) *num_splits = pl.num_splits;
     if (kv_groups) *kv_groups = pl.kv_groups;
     if (num_workgroups) *num_workgroups = kXcds * ceil_div(pl.num_splits * Hkv, kXcds) * pl.num_mtiles;
@@ -944,6 +1098,7 @@ static int tree_attention_impl(const void* q, void* k_pool, void* v_pool,
     p.out = (f16*)out;
     p.o_part = nullptr;
     p.ml_part = nullptr;
+    p.merge_ctr = nullptr;
     if (p.num_splits > 1) {
         const size_t o_bytes = align_up((size_t)Hkv * p.num_splits * p.rows_pad * kHeadDim * sizeof(f16), 256);
         const size_t ml_bytes = (size_t)Hkv * p.num_splits * p.rows_pad * 2 * sizeof(float);
@@ -951,6 +1106,7 @@ static int tree_attention_impl(const void* q, void* k_pool, void* v_pool,
                         "tree_attention: workspace of %zu bytes needed, %zu given", o_bytes + ml_bytes, workspace_bytes);
         p.o_part = (float*)workspace;
         p.ml_part = (float*)((char*)workspace + o_bytes);
+        if (plan.merge_in_launch) p.merge_ctr = merge_counters_for(workspace);
     }
     hipStream_t st = resolve_stream(stream);
     const int nsh = p.num_splits * Hkv;
@@ -963,7 +1119,7 @@ static int tree_attention_impl(const void* q, void* k_pool, void* v_pool,
         else hipLaunchKernelGGL((tree_attn_split_kernel<2, false>), grid, dim3(kThreads), 0, st, p);
     }
     CPMCU_LAUNCH_CHECK();
-    if (p.num_splits > 1) {
+    if (p.num_splits > 1 && p.merge_ctr == nullptr) {
         const int threads_total = Hkv * (p.rows_pad / kRowsPerWave) * 16 * 64;
         hipLaunchKernelGGL(tree_attn_combine_kernel, dim3(ceil_div(threads_total, 256)), dim3(256), 0, st, p);
         CPMCU_LAUNCH_CHECK();

@@ -73,7 +73,10 @@ const char* cpmcu_version(void);
  *   "attn_kv_groups"        0 = chosen per call (default), 1 / 2 = force the 256-row / the two-KV-group
  *                           shape of the tree-attention kernel (CPMCU_ATTN_KV_GROUPS=1|2);
  *   "head_share_last_pass"  1 = the waves of a workgroup share the row blocks of a partly filled last pass
- *                           of the head GEMM (default), 0 = plain mapping (CPMCU_HEAD_NO_SHARE set). */
+ *                           of the head GEMM (default), 0 = plain mapping (CPMCU_HEAD_NO_SHARE set);
+ *   "attn_merge_in_launch"  1 = the workgroups of a split tree-attention launch merge their own partials when the
+ *                           launch fits the GPU's CUs and has at most 32 splits (default), 0 = always the separate
+ *                           merge launch (CPMCU_ATTN_SEPARATE_MERGE set). */
 int cpmcu_set_option(const char* name, int value);
 
 /* ------------------------------------------------------------------------- */

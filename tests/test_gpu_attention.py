@@ -398,3 +398,50 @@ def test_randomised_shape_sweep(gpu, orc, P, T, mode, splits, slack, seed):
         kc, vc = cache.read_logical(0, 0, S)
         assert np.array_equal(to_np(kc).view(np.uint16), k_ref.view(np.uint16))
         assert np.array_equal(to_np(vc).view(np.uint16), v.view(np.uint16))
+
+
+@pytest.mark.parametrize("P,T,splits,fused_append,rope", [
+    (4096, 60, 0, True, False),    # the verify step's shape: 16 splits (two groups) / 32 splits (one group), 256 workgroups
+    (4096, 60, 0, True, True),
+    (33000, 60, 0, False, False),
+    (700, 128, 3, True, False),
+    (1500, 60, 7, False, False),   # a split count that does not divide the blocks of a unit evenly
+    (250, 16, 2, True, False),
+])
+def test_merge_in_launch_equals_separate_merge(gpu, set_option, P, T, splits, fused_append, rope):
+    """The split workgroups' own merge (device-scope partials, per-unit arrival counters) and the combine launch run the
+    same arithmetic on the same partials: outputs must be bit-identical.  Each path is called three times in a row, then
+    with another split count on the same workspace, so that the counters are seen to come back to rest."""
+    torch = gpu
+    from cpm.cu_amd import ops
+    from cpm.cu_amd.kvcache import PagedKVCache
+    tree = synth.eagle_tree(6, 10, T, seed=P) if T > 16 else synth.eagle_tree(3, 4, T, seed=P)
+    S = P + T
+    q = to_dev(torch, synth.normal_f16((T, HQ, D), P, 1))
+    k = synth.normal_f16((S, HKV, D), P, 2)
+    v = synth.normal_f16((S, HKV, D), P, 3)
+    npages = (S + 255) // 256 + 1
+    table = synth.rng(P, 4).permutation(npages).astype(np.int32)
+    mask = to_dev(torch, tree.mask)
+    kv_len = torch.tensor([S], dtype=torch.int32, device="cuda")
+    table_rope = None
+    if rope:
+        pos = torch.arange(P, P + T, dtype=torch.int32, device="cuda")
+        inv_freq = to_dev(torch, (1.0 / (10000.0 ** (np.arange(0, D, 2, dtype=np.float32) / D))).astype(np.float32))
+        table_rope = ops.rope_table(pos, inv_freq)
+    outs = {}
+    for mode in (0, 1):
+        set_option("attn_merge_in_launch", mode)
+        got = []
+        for rep, sp in enumerate((splits, splits, splits, 4, splits)):
+            cache = PagedKVCache(1, HKV, npages, block_table=table, fill=float("nan"))
+            n_cached = P if fused_append else S
+            cache.write_logical(0, 0, to_dev(torch, k[:n_cached]), to_dev(torch, v[:n_cached]))
+            kw = dict(k_new=to_dev(torch, k[P:]), v_new=to_dev(torch, v[P:])) if fused_append else {}
+            out = ops.tree_attention(q, cache, 0, kv_len, S, mask, num_splits=sp, rope=table_rope, **kw)
+            torch.cuda.synchronize()
+            got.append(to_np(out))
+        outs[mode] = got
+    for a, b in zip(outs[0], outs[1]):
+        assert np.all(np.isfinite(a.astype(np.float32)))
+        assert np.array_equal(a.view(np.uint16), b.view(np.uint16))
