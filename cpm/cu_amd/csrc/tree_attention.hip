@@ -101,14 +101,14 @@ struct AttnParams {
     //   ml_part [Hkv][num_splits][rows_pad] x float2 (max * scale_log2, sum)
     float* o_part;
     float* ml_part;
-    // Merge inside the split launch (null: the separate combine kernel does it): one {arrivals, generation} pair
-    // per (KV head, M-tile) unit.  Between launches arrivals is 0; the last workgroup of a unit to arrive sets it
-    // back and bumps the generation, which the others wait for.
+    // Merge inside the split launch (null: the separate combine kernel does it): one word per (KV head, M-tile)
+    // unit, arrivals in its low 16 bits, a generation count above them.  Between launches arrivals is 0; the last
+    // workgroup of a unit to arrive turns the full count into the next generation.
     uint32_t* merge_ctr;
 };
 
-constexpr int kMergeUnitWords = 128;  // the two words of a unit sit in 256-byte lines of their own: every poll and every
-                                      // arrival is a memory transaction, and those on one line queue behind each other
+constexpr int kMergeUnitWords = 64;  // a unit's word sits in a 256-byte line of its own: every poll and every arrival is
+                                     // a memory transaction, and those on one line queue behind each other
 constexpr int kMergeWaitExpired = INT32_MIN;  // value of g_attn_bad_length after a merge wait ran into its limit
 constexpr unsigned long long kMergeWaitTicks = 2000000ull;  // 20 ms of the 100 MHz wall clock
 
@@ -324,9 +324,7 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
     const int tid = threadIdx.x;
     const int wave = tid >> 6;
     const int lane = tid & 63;
-    // merge inside the launch: the unit's arrivals word and, 256 bytes on, its generation word
-    uint32_t* const unit_ctr = p.merge_ctr ? p.merge_ctr + kMergeUnitWords * (g * p.num_mtiles + mt) : nullptr;
-    uint32_t* const unit_gen = unit_ctr + kMergeUnitWords / 2;
+    uint32_t* const unit_ctr = p.merge_ctr ? p.merge_ctr + kMergeUnitWords * (g * p.num_mtiles + mt) : nullptr;  // merge inside the launch
     const int grp = wave / kRowWaves;  // KV group: takes tiles grp, grp + G, ...
     const int rw = wave % kRowWaves;
     const int qcol = lane & 31;
@@ -754,10 +752,6 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
         }
     }
 
-    // Merge inside the launch: the unit's generation as it stands before this workgroup has arrived (it moves only
-    // once all of the unit's workgroups have), requested here so that it is back by the time the partials are stored.
-    uint32_t gen0 = 0;
-    if (unit_ctr != nullptr && tid == 0) gen0 = __hip_atomic_load(unit_gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     // ---- merge the two KV groups through LDS (lane-private layout: [row wave][value][lane]) ----
     if constexpr (G == 2) {
     __syncthreads();  // ring no longer read
@@ -852,19 +846,24 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
         __syncthreads();
         if (tid == 0) {
             int go = 1;
-            const uint32_t arrived = __hip_atomic_fetch_add(unit_ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (arrived == (uint32_t)p.num_splits - 1u) {
-                __hip_atomic_store(unit_ctr, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                __hip_atomic_store(unit_gen, gen0 + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            // The word as this workgroup's arrival found it: the generation of this launch above, the arrivals before it below.
+            const uint32_t before = __hip_atomic_fetch_add(unit_ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const uint32_t full = (before & 0xffff0000u) + (uint32_t)p.num_splits;
+            if (before + 1u == full) {
+                // last to arrive: full count -> next generation, no arrivals (nobody needs the result of this one)
+                __hip_atomic_fetch_add(unit_ctr, 0x10000u - (uint32_t)p.num_splits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             } else {
+                // the others see either the full count or, once the last one has moved it on, the next generation
                 const unsigned long long t_begin = wall_clock64();
-                while (__hip_atomic_load(unit_gen, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == gen0) {
+                while (true) {
+                    const uint32_t now = __hip_atomic_load(unit_ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if (now == full || (now & 0xffff0000u) != (before & 0xffff0000u)) break;
                     if (wall_clock64() - t_begin > kMergeWaitTicks) {
                         g_attn_bad_length = kMergeWaitExpired;
                         go = 0;
                         break;
                     }
-                    __builtin_amdgcn_s_sleep(8);
+                    __builtin_amdgcn_s_sleep(4);
                 }
             }
             s_merge_go = go;
