@@ -16,6 +16,9 @@ Options& options();
 // tree_attention.hip -- an attention launch whose device-side length lay outside [max(T, mask_k_range), max_kv_len]
 // worked on the clamped length and left the offending value behind; this reads and clears it (synchronising).
 int attention_take_bad_length(int* value);
+// Assigns the counters of the in-launch merge to a workspace on the current device (otherwise done by the first
+// launch that uses it outside a stream capture).
+void attention_prepare_workspace(const void* workspace);
 
 // lm_head.hip -- the streaming GEMM with its two epilogues.
 constexpr int kHeadModeStats = 0;

@@ -413,6 +413,7 @@ int init_storage_impl(Model& m, int* max_context) {
     }
     pages -= ws_pages;
     CPMCU_HIP(hipMalloc(&m.attn_ws, m.attn_ws_bytes));
+    attention_prepare_workspace(m.attn_ws);  // its merge counters are assigned now, ahead of any captured launch
     m.num_pages = (int)pages;
     m.k_pools.assign(all_layers, nullptr);
     m.v_pools.assign(all_layers, nullptr);

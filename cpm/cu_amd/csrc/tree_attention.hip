@@ -374,8 +374,9 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
     // the device-side length: such calls (the drafter's own layer, a few tiles in all) pay the extra
     // round trip in front of the page ids.
     const int vtiles = p.ntiles_max + (p.k_new != nullptr && p.num_splits > 1 ? (ROPE ? 3 : 2) : 0);
-    const int r0 = min((int)(((long long)split * vtiles) / p.num_splits), p.ntiles_max);
-    const int r1 = min((int)(((long long)(split + 1) * vtiles) / p.num_splits), p.ntiles_max);
+    // (32-bit arithmetic: at most 128 splits times at most 2^24 tiles; a 64-bit division is a long scalar routine)
+    const int r0 = min((int)(((uint32_t)split * (uint32_t)vtiles) / (uint32_t)p.num_splits), p.ntiles_max);
+    const int r1 = min((int)(((uint32_t)(split + 1) * (uint32_t)vtiles) / (uint32_t)p.num_splits), p.ntiles_max);
     // The device-side length and the page id of the split's first tile come through scalar loads, together: the
     // Q rows requested above are still on their way, and a vector load of these few bytes would return behind them.
     int S, first_page;
@@ -957,7 +958,7 @@ bool can_merge_in_launch(int Hkv, int num_mtiles, int num_splits) {
 }
 
 // The counter block of a workspace on the current device (null: none left, or the lookup failed).
-uint32_t* merge_counters_for(const void* workspace) {
+uint32_t* merge_counters_for(const void* workspace, hipStream_t st) {
     static std::mutex mu;
     static std::map<std::pair<int, const void*>, int> blocks;
     static int next_block[64] = {0};
@@ -966,6 +967,13 @@ uint32_t* merge_counters_for(const void* workspace) {
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
     std::lock_guard<std::mutex> lock(mu);
     if (base[dev] == nullptr) {
+        // The address of the counters is looked up once per device, outside any stream capture (a launch that is being
+        // captured before the first eager one uses the combine launch).
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(st, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
+            (void)hipGetLastError();
+            return nullptr;
+        }
         void* ptr = nullptr;
         if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_merge_ctr)) != hipSuccess) {
             (void)hipGetLastError();
@@ -1013,6 +1021,8 @@ extern "C" int cpmcu_tree_attention_plan(int T, int Hq, int Hkv, int max_kv_len,
 }
 
 namespace cpmcu {
+void attention_prepare_workspace(const void* workspace) { (void)merge_counters_for(workspace, nullptr); }
+
 // Reads and clears the bad-length word of the current device (a synchronising copy); 0 = none.
 int attention_take_bad_length(int* value) {
     int v = 0;
@@ -1046,6 +1056,7 @@ static int tree_attention_impl(const void* q, void* k_pool, void* v_pool,
     CPMCU_CHECK_ARG(T >= 1 && T <= kMaxTree, "tree_attention: T=%d outside [1, %d]", T, kMaxTree);
     CPMCU_CHECK_ARG(Hkv >= 1 && Hq >= Hkv && Hq % Hkv == 0, "tree_attention: Hq=%d must be a multiple of Hkv=%d", Hq, Hkv);
     CPMCU_CHECK_ARG(max_kv_len >= T, "tree_attention: max_kv_len=%d < T=%d", max_kv_len, T);
+    CPMCU_CHECK_ARG(max_kv_len <= (1 << 30), "tree_attention: max_kv_len=%d is beyond the supported context of 2^30 keys", max_kv_len);
     if (mask_k_range == 0 || mask == nullptr) mask_k_range = T;
     CPMCU_CHECK_ARG(mask_k_range >= T && mask_k_range <= kMaxTree && mask_k_range <= max_kv_len,
                     "tree_attention: mask_k_range=%d outside [T=%d, min(%d, max_kv_len)]", mask_k_range, T, kMaxTree);
@@ -1095,6 +1106,7 @@ static int tree_attention_impl(const void* q, void* k_pool, void* v_pool,
     p.max_kv_len = max_kv_len;
     p.scale_log2 = scale * 1.4426950408889634f;
     p.out = (f16*)out;
+    hipStream_t st = resolve_stream(stream);
     p.o_part = nullptr;
     p.ml_part = nullptr;
     p.merge_ctr = nullptr;
@@ -1105,9 +1117,8 @@ static int tree_attention_impl(const void* q, void* k_pool, void* v_pool,
                         "tree_attention: workspace of %zu bytes needed, %zu given", o_bytes + ml_bytes, workspace_bytes);
         p.o_part = (float*)workspace;
         p.ml_part = (float*)((char*)workspace + o_bytes);
-        if (plan.merge_in_launch) p.merge_ctr = merge_counters_for(workspace);
+        if (plan.merge_in_launch) p.merge_ctr = merge_counters_for(workspace, st);
     }
-    hipStream_t st = resolve_stream(stream);
     const int nsh = p.num_splits * Hkv;
     const dim3 grid(kXcds * ceil_div(nsh, kXcds), p.num_mtiles);
     if (p.rope != nullptr) {
