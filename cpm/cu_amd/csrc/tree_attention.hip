@@ -753,61 +753,82 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
         }
     }
 
-    // ---- merge the two KV groups through LDS (lane-private layout: [row wave][value][lane]) ----
+    // ---- the two KV groups meet through LDS ----
+    // Each wave keeps half of the output dims of its rows (group 0: d < 64, group 1: d >= 64) and hands the other half
+    // to the wave of the other group with the same rows, so that the exchange, the merge and the stores behind it are
+    // spread over all eight waves.  The exchange area is the two ring stages the last iteration does not read (the
+    // previous iteration's tiles, which every wave has left; no request is in flight into them) and, for (max, sum),
+    // the appended-row staging area (last read ahead of a barrier inside the iteration): a wave writes as soon as its
+    // own last tile is done, whatever the other group is still doing.
     if constexpr (G == 2) {
-    __syncthreads();  // ring no longer read
-    f32x4* xch = reinterpret_cast<f32x4*>(ring);           // [row wave][17 quads][64 lanes]
-    const int xbase = rw * 17 * 64 + lane;
-    if (grp == 1) {
+        const int i_last = niter > 0 ? 2 * (niter - 1) : 0;
+        f32x4* xch = reinterpret_cast<f32x4*>(ring + ((i_last + 2) % kStages) * kStageBytes);  // [wave][8 quads][64 lanes]
+        float2* xml = reinterpret_cast<float2*>(vstage);                                        // [wave][64 lanes]
+        auto send = [&](auto db0_c) {
+            constexpr int DB0 = decltype(db0_c)::value;
 #pragma unroll
-        for (int db = 0; db < 4; ++db)
+            for (int db = 0; db < 2; ++db)
 #pragma unroll
-            for (int rq = 0; rq < 4; ++rq) {
-                f32x4 o;
+                for (int rq = 0; rq < 4; ++rq) {
+                    f32x4 o;
 #pragma unroll
-                for (int e = 0; e < 4; ++e) o[e] = oacc[db][rq * 4 + e];
-                xch[xbase + (db * 4 + rq) * 64] = o;
-            }
-        xch[xbase + 16 * 64] = f32x4{m_ref, l_run, 0.f, 0.f};
-    }
-    __syncthreads();
-    if (grp == 1 && unit_ctr == nullptr) return;  // (with the merge in the launch, group 1 stays for its share of it)
-    if (grp == 0) {
-        const f32x4 ml1 = xch[xbase + 16 * 64];
-        const float m1 = ml1[0], l1 = ml1[1];
-        const float m_new = fmaxf(m_ref, m1);
+                    for (int e = 0; e < 4; ++e) o[e] = oacc[DB0 + db][rq * 4 + e];
+                    xch[(wave * 8 + db * 4 + rq) * 64 + lane] = o;
+                }
+        };
+        if (grp == 0) send(std::integral_constant<int, 2>{});
+        else send(std::integral_constant<int, 0>{});
+        xml[wave * 64 + lane] = make_float2(m_ref, l_run);
+        __syncthreads();
+        const int other = wave ^ kRowWaves;  // same rows, other group
+        const float2 ml1 = xml[other * 64 + lane];
+        const float m_new = fmaxf(m_ref, ml1.x);
         const float m_scaled = (m_new == -INFINITY) ? 0.f : m_new;
         const float a0 = __builtin_amdgcn_exp2f(m_ref - m_scaled);
-        const float a1 = __builtin_amdgcn_exp2f(m1 - m_scaled);
+        const float a1 = __builtin_amdgcn_exp2f(ml1.x - m_scaled);
+        auto receive = [&](auto db0_c) {
+            constexpr int DB0 = decltype(db0_c)::value;
 #pragma unroll
-        for (int db = 0; db < 4; ++db)
+            for (int db = 0; db < 2; ++db)
 #pragma unroll
-            for (int rq = 0; rq < 4; ++rq) {
-                const f32x4 o = xch[xbase + (db * 4 + rq) * 64];
+                for (int rq = 0; rq < 4; ++rq) {
+                    const f32x4 o = xch[(other * 8 + db * 4 + rq) * 64 + lane];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) oacc[db][rq * 4 + e] = oacc[db][rq * 4 + e] * a0 + o[e] * a1;
-            }
-        l_run = l_run * a0 + l1 * a1;
+                    for (int e = 0; e < 4; ++e) oacc[DB0 + db][rq * 4 + e] = oacc[DB0 + db][rq * 4 + e] * a0 + o[e] * a1;
+                }
+        };
+        if (grp == 0) receive(std::integral_constant<int, 0>{});
+        else receive(std::integral_constant<int, 2>{});
+        l_run = l_run * a0 + ml1.y * a1;
         m_ref = m_new;
     }
-    }
 
-    // oacc[db][r] is O[query qcol][d = db*32 + 8*(r/4) + 4*hf + r%4], unnormalised.
+    // oacc[db][r] is O[query qcol][d = db*32 + 8*(r/4) + 4*hf + r%4], unnormalised; with two KV groups a wave now holds
+    // the d blocks [2 * grp, 2 * grp + 2) of its rows.
     const float l_tot = l_run + __shfl_xor(l_run, 32);
-    const bool owner = G == 1 || grp == 0;  // this wave holds the workgroup's result for its rows
+    // stores db blocks [DB0, DB0 + NDB) of this wave's rows through `put(db, rq, values)`
+    auto for_my_blocks = [&](auto&& put) {
+        auto run = [&](auto db0_c, auto ndb_c) {
+            constexpr int DB0 = decltype(db0_c)::value, NDB = decltype(ndb_c)::value;
+#pragma unroll
+            for (int db = DB0; db < DB0 + NDB; ++db)
+#pragma unroll
+                for (int rq = 0; rq < 4; ++rq) put(db, rq, oacc[db]);
+        };
+        if constexpr (G == 1) run(std::integral_constant<int, 0>{}, std::integral_constant<int, 4>{});
+        else if (grp == 0) run(std::integral_constant<int, 0>{}, std::integral_constant<int, 2>{});
+        else run(std::integral_constant<int, 2>{}, std::integral_constant<int, 2>{});
+    };
     if (p.num_splits == 1) {
         if (!row_ok) return;
         const float inv = (l_tot == 0.f || l_tot != l_tot) ? 1.f : 1.f / l_tot;
         f16* orow = p.out + ((size_t)node * p.Hq + head) * kHeadDim;
+        for_my_blocks([&](int db, int rq, const f32x16& acc) {
+            f16x4 o;
 #pragma unroll
-        for (int db = 0; db < 4; ++db)
-#pragma unroll
-            for (int rq = 0; rq < 4; ++rq) {
-                f16x4 o;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) o[e] = (f16)(oacc[db][rq * 4 + e] * inv);
-                *reinterpret_cast<f16x4*>(orow + db * 32 + rq * 8 + hf * 4) = o;
-            }
+            for (int e = 0; e < 4; ++e) o[e] = (f16)(acc[rq * 4 + e] * inv);
+            *reinterpret_cast<f16x4*>(orow + db * 32 + rq * 8 + hf * 4) = o;
+        });
     } else {
         const size_t prow = ((size_t)g * p.num_splits + split) * p.rows_pad + R;
         // Partials leave the kernel normalised (O / l) and rounded to fp16 -- the precision of the
@@ -816,18 +837,14 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
         const float inv = (l_tot == 0.f || l_tot != l_tot) ? 0.f : 1.f / l_tot;
         f16x4* op = reinterpret_cast<f16x4*>(p.o_part) +
                     ((((size_t)g * p.num_splits + split) * p.num_mtiles + mt) * kRowWaves + rw) * 16 * 64 + lane;
-        if (owner)
+        for_my_blocks([&](int db, int rq, const f32x16& acc) {
+            f16x4 o;
 #pragma unroll
-        for (int db = 0; db < 4; ++db)
-#pragma unroll
-            for (int rq = 0; rq < 4; ++rq) {
-                f16x4 o;
-#pragma unroll
-                for (int e = 0; e < 4; ++e) o[e] = (f16)(oacc[db][rq * 4 + e] * inv);
-                if (unit_ctr != nullptr) store_dev64(&op[(db * 4 + rq) * 64], bits_as<uint64_t>(o));
-                else __builtin_nontemporal_store(o, &op[(db * 4 + rq) * 64]);  // streamed: nothing left to flush at kernel end
-            }
-        if (owner && hf == 0 && row_ok) {
+            for (int e = 0; e < 4; ++e) o[e] = (f16)(acc[rq * 4 + e] * inv);
+            if (unit_ctr != nullptr) store_dev64(&op[(db * 4 + rq) * 64], bits_as<uint64_t>(o));
+            else __builtin_nontemporal_store(o, &op[(db * 4 + rq) * 64]);  // streamed: nothing left to flush at kernel end
+        });
+        if (grp == 0 && hf == 0 && row_ok) {
             if (unit_ctr != nullptr) {
                 store_dev64(&p.ml_part[prow * 2], (uint64_t)__float_as_uint(m_ref) | ((uint64_t)__float_as_uint(l_tot) << 32));
             } else {
