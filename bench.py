@@ -370,6 +370,24 @@ def main():
             for _ in range(HEAD_REP):
                 ops.lm_head_partials(bufs.hidden, w_t)
         ms_head = timed_torch(torch, head_only, reps, 2, warm_ms=WARM_MS) / HEAD_REP
+        # the same GEMM where the step has it, behind the 32 attention launches (every K/V set in turn): replays of the head
+        # alone keep HBM at its limit without a pause, and the head then runs slower than it does inside a step
+        all_caches = main_run["caches"]
+
+        def attn_layers(c):
+            for l in range(L):
+                ops.tree_attention(bufs.q[l], c, l, kvlen, padded, mask, out=bufs.attn_out[l], k_new=bufs.k_new[l], v_new=bufs.v_new[l])
+
+        def attn_then_head():
+            for c in all_caches:
+                attn_layers(c)
+                ops.lm_head_partials(bufs.hidden, w_t)
+
+        def attn_without_head():
+            for c in all_caches:
+                attn_layers(c)
+        ms_head_in_step = (timed_torch(torch, attn_then_head, reps, 2, warm_ms=WARM_MS) -
+                           timed_torch(torch, attn_without_head, reps, 2, warm_ms=WARM_MS)) / len(all_caches)
         parts = ops.lm_head_partials(bufs.hidden, w_t)
         best = torch.zeros(2, dtype=torch.int32, device="cuda")
         path = torch.zeros(T, dtype=torch.int32, device="cuda")
@@ -386,9 +404,13 @@ def main():
         kernels.append(dict(kernel=head_name, launches_per_step=1, us_per_launch=round(ms_head * 1e3, 2), bound="hbm",
                             achieved=round(head_gbs, 1), peak=HBM_PEAK_GBS, unit="GB/s", frac=round(head_gbs / HBM_PEAK_GBS, 4), traffic=None,
                             frac_with_tail_launch=round(head_tail_gbs / HBM_PEAK_GBS, 4),
-                            note="the target head's GEMM on a separately allocated copy of the weights; in the step its arg-max is "
+                            us_behind_attention=round(ms_head_in_step * 1e3, 2),
+                            frac_behind_attention=round(bytes_head / (ms_head_in_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
+                            note="the target head's GEMM on a separately allocated copy of the weights, replayed back to back "
+                                 "(us_per_launch, frac) and where the step has it (us_behind_attention: a graph of the %d attention "
+                                 "launches + the GEMM minus the same graph without it, over every K/V set); in the step its arg-max is "
                                  "finished inside the tail launch (frac_with_tail_launch charges that whole launch -- acceptance and "
-                                 "compaction included -- to the head)"))
+                                 "compaction included -- to the back-to-back figure)" % L))
         kernels.append(dict(kernel=head_name + "+head_argmax_finalize_kernel", launches_per_step=0, us_per_launch=round(ms_head_model * 1e3, 2),
                             bound="hbm", achieved=round(head_model_gbs, 1), peak=HBM_PEAK_GBS, unit="GB/s",
                             frac=round(head_model_gbs / HBM_PEAK_GBS, 4), traffic=None,
