@@ -950,7 +950,7 @@ struct LaunchPlan {
 // every launch), in blocks handed out per workspace: calls that may overlap use different workspaces and so different
 // counters, and nothing has to be cleared or allocated per call.
 constexpr int kMergeUnits = 256;    // (KV head, M-tile) units a launch may have on this path
-constexpr int kMergeBlocks = 32;    // workspaces that get a block; further ones use the combine launch
+constexpr int kMergeBlocks = 32;    // blocks per device (see merge_counters_for)
 constexpr int kMergeMaxSplits = 32; // arrivals on one counter serialise, about 0.15 us each
 __device__ __align__(256) uint32_t g_merge_ctr[kMergeBlocks][kMergeUnits * kMergeUnitWords];
 
@@ -974,11 +974,19 @@ bool can_merge_in_launch(int Hkv, int num_mtiles, int num_splits) {
     return kXcds * ceil_div(num_splits * Hkv, kXcds) * num_mtiles <= device_cu_count();
 }
 
-// The counter block of a workspace on the current device (null: none left, or the lookup failed).
+// The counter block of a workspace on the current device (null: the lookup of the counters' address failed or has to
+// wait).  When all blocks are taken, the one whose workspace has gone unused the longest moves on to the new workspace:
+// between launches a block is at rest, so this is safe as long as no more than kMergeBlocks workspaces have launches in
+// flight on one device at the same time.
 uint32_t* merge_counters_for(const void* workspace, hipStream_t st) {
+    struct Block {
+        int index;
+        unsigned long long last_use;
+    };
     static std::mutex mu;
-    static std::map<std::pair<int, const void*>, int> blocks;
+    static std::map<std::pair<int, const void*>, Block> blocks;
     static int next_block[64] = {0};
+    static unsigned long long use_clock = 0;
     static uint32_t* base[64] = {nullptr};
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
@@ -1000,10 +1008,20 @@ uint32_t* merge_counters_for(const void* workspace, hipStream_t st) {
     }
     auto it = blocks.find({dev, workspace});
     if (it == blocks.end()) {
-        if (next_block[dev] >= kMergeBlocks) return nullptr;
-        it = blocks.emplace(std::make_pair(dev, workspace), next_block[dev]++).first;
+        int index;
+        if (next_block[dev] < kMergeBlocks) {
+            index = next_block[dev]++;
+        } else {
+            auto oldest = blocks.end();
+            for (auto b = blocks.begin(); b != blocks.end(); ++b)
+                if (b->first.first == dev && (oldest == blocks.end() || b->second.last_use < oldest->second.last_use)) oldest = b;
+            index = oldest->second.index;
+            blocks.erase(oldest);
+        }
+        it = blocks.emplace(std::make_pair(dev, workspace), Block{index, 0}).first;
     }
-    return base[dev] + (size_t)it->second * kMergeUnits * kMergeUnitWords;
+    it->second.last_use = ++use_clock;
+    return base[dev] + (size_t)it->second.index * kMergeUnits * kMergeUnitWords;
 }
 LaunchPlan plan_launch(int T, int group, int Hkv, int max_kv_len, int block_window_size, int num_splits_override) {
     LaunchPlan pl;

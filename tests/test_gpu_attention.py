@@ -445,3 +445,35 @@ def test_merge_in_launch_equals_separate_merge(gpu, set_option, P, T, splits, fu
     for a, b in zip(outs[0], outs[1]):
         assert np.all(np.isfinite(a.astype(np.float32)))
         assert np.array_equal(a.view(np.uint16), b.view(np.uint16))
+
+
+def test_merge_counter_blocks_move_on_to_new_workspaces(gpu):
+    """The library hands a block of merge counters to each workspace pointer it meets (a fixed number per device) and,
+    when they run out, passes the one unused the longest on to the newcomer: every call must give the same bits."""
+    torch = gpu
+    from cpm.cu_amd import ops
+    from cpm.cu_amd.kvcache import PagedKVCache
+    T, P = 60, 2000
+    tree = synth.eagle_tree(6, 10, T, seed=3)
+    S = P + T
+    q = to_dev(torch, synth.normal_f16((T, HQ, D), 7, 1))
+    k = synth.normal_f16((S, HKV, D), 7, 2)
+    v = synth.normal_f16((S, HKV, D), 7, 3)
+    npages = (S + 255) // 256 + 1
+    cache = PagedKVCache(1, HKV, npages)
+    cache.write_logical(0, 0, to_dev(torch, k), to_dev(torch, v))
+    mask = to_dev(torch, tree.mask)
+    kv_len = torch.tensor([S], dtype=torch.int32, device="cuda")
+    ref = None
+    keep = []
+    for i in range(40):  # more distinct workspaces than the library has counter blocks; each is used twice in a row
+        ops._workspaces.pop(("attn", q.device), None)
+        for rep in range(2):
+            out = ops.tree_attention(q, cache, 0, kv_len, S, mask)
+            torch.cuda.synchronize()
+            got = to_np(out)
+            if ref is None:
+                ref = got
+            assert np.array_equal(got.view(np.uint16), ref.view(np.uint16)), "call %d.%d" % (i, rep)
+        keep.append(ops._workspaces[("attn", q.device)])  # kept alive: every call sees a new address
+    assert len({t.data_ptr() for t in keep}) == 40
