@@ -1,6 +1,8 @@
 // Tree-verify flash attention for gfx950 (MI355X): tree-masked draft queries
 // against the paged prefix KV plus the in-tree KV, GQA-packed, fp16 MFMA with
-// fp32 accumulation, split over the KV stream and merged by a second kernel.
+// fp32 accumulation, split over the KV stream; the split workgroups merge their
+// partial results themselves (a second kernel does it for launches that do not
+// fit the GPU's CUs or have more than 32 splits).
 //
 // What it computes is the dense tree-mask path of the reference's
 // mha_fwd_kvcache (src/flash_attn/flash_api.hpp:292-392, kernel body
@@ -30,6 +32,8 @@
 //    the ring and are merged through LDS at the end -- half the partial traffic
 //    of splitting the same work over two workgroups.  For long contexts they
 //    are 8 row waves over 256 packed rows, every tile feeding all of them.
+//  * The Q rows and the tree mask reach the registers through LDS (whole rows,
+//    coalesced), not through per-lane fetches in the MFMA operand layout.
 //  * Workgroups are mapped so that all M-tiles that stream the same KV range
 //    land on the same XCD (workgroup id modulo 8) and share its L2.
 #include "common.h"
