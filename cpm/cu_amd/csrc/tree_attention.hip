@@ -63,6 +63,8 @@ constexpr int kVTileBytes = kHeadDim * kTileN * 2;  // 16 KB, row = one dim (128
 constexpr int kStageBytes = kKTileBytes + kVTileBytes;
 constexpr int kVStageRows = 64;  // appended V rows staged in LDS ahead of their transposition
 constexpr int kMaxSplits = 128;
+constexpr int kMergeMaxSplits = 32;  // most splits of a launch that merges its own partials: arrivals on one counter
+                                     // serialise, about 0.15 us each
 constexpr int kXcds = 8;
 constexpr float kLazyLog2 = 8.f;  // slack of the lazily updated softmax reference, in log2 units
 
@@ -912,10 +914,21 @@ __global__ __launch_bounds__(256) void tree_attn_combine_kernel(AttnParams p) {
 int choose_splits(int T, int group, int Hkv, int max_kv_len, int G) {
     const int num_mtiles = ceil_div(group * T, rows_per_wg(G));
     const int ntiles = ceil_div(max_kv_len, kTileN);
-    // One workgroup per CU (256 CUs); every split should get at least one tile per KV group.
+    // One workgroup per CU (256 CUs).
     int splits = 256 / (num_mtiles * Hkv);
     if (splits < 1) splits = 1;
-    if (splits > ntiles / G) splits = ntiles / G > 0 ? ntiles / G : 1;
+    const bool merge = options().attn_merge_in_launch != 0;
+    // One or two row units (plain decode, trees of up to 32 nodes) could take 64 or 128 splits; up to about 28K context
+    // they do better on at most 32, which the launch can merge itself: 16 while a split still gets about four tiles,
+    // 32 beyond.  One query, us per call, 16 / 32 splits merged in the launch against the split count below with its
+    // second launch: 13.3 / 13.8 vs 17.5 at 4K, 17.3 / 15.1 vs 20.9 at 8K, 24.9 / 18.9 vs 21.8 at 16K, 32.8 / 22.8 vs 24.0
+    // at 24K, - / 27.2 vs 25.9 at 32K.
+    constexpr int kShortContextTiles = 448;
+    if (merge && splits > kMergeMaxSplits && ntiles <= kShortContextTiles) splits = std::min(kMergeMaxSplits, std::max(16, ntiles / 4));
+    // Every split gets at least one tile -- one per KV group when a second launch merges: a launch that merges itself does
+    // better on more, shorter splits at short contexts (60-node tree at 512 tokens: 12.7 us on 10 splits, 16.2 on 4).
+    const int tile_cap = merge && splits <= kMergeMaxSplits ? ntiles : ntiles / G;
+    if (splits > tile_cap) splits = tile_cap > 0 ? tile_cap : 1;
     // More than 64 splits (one or two row units: plain decode, trees of up to 8 nodes) pay for their partials
     // and per-workgroup latencies only when every KV group still gets a run of 8 tiles: with one query,
     // 128 against 64 splits take 50.7 vs 55.0 us per layer at 128K context, but 38.1 vs 34.8 at 64K and
@@ -955,7 +968,6 @@ struct LaunchPlan {
 // counters, and nothing has to be cleared or allocated per call.
 constexpr int kMergeUnits = 256;    // (KV head, M-tile) units a launch may have on this path
 constexpr int kMergeBlocks = 32;    // blocks per device (see merge_counters_for)
-constexpr int kMergeMaxSplits = 32; // arrivals on one counter serialise, about 0.15 us each
 __device__ __align__(256) uint32_t g_merge_ctr[kMergeBlocks][kMergeUnits * kMergeUnitWords];
 
 int device_cu_count() {
