@@ -289,8 +289,14 @@ size_t cpmcu_tree_attention_workspace_bytes(int T, int Hq, int Hkv, int max_kv_l
  *           mask = NULL: causal chain.  mask_words = ceil(mask_k_range / 64).
  *   scale: softmax scale (1/sqrt(128) in the reference, flash_api.hpp:360).
  *   workspace: device scratch of at least ..._workspace_bytes(), may be NULL
- *           when that is 0.
- *   num_splits_override: 0 = choose from max_kv_len; >0 forces the KV split count. */
+ *           when that is 0.  Calls that may overlap on one GPU must use different
+ *           workspaces: the split partials live there, and the library keys the
+ *           arrival counters of the in-launch merge by this pointer (a launch with at
+ *           most 32 splits and at most one workgroup per CU merges its own partials;
+ *           its workgroups wait for each other, which needs them all resident -- see
+ *           "attn_merge_in_launch" above).
+ *   num_splits_override: 0 = choose from max_kv_len; >0 forces the KV split count.
+ * max_kv_len is limited to 2^30. */
 int cpmcu_tree_attention(const void* q, void* k_pool, void* v_pool, const int32_t* block_table,
                          const int32_t* kv_len, int max_kv_len, const void* k_new, const void* v_new,
                          const uint64_t* mask, int mask_words, int mask_k_range, int T, int Hq, int Hkv, float scale,
