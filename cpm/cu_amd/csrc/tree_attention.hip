@@ -338,6 +338,10 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
 
     const int R = mt * kRowsPerWg + rw * kRowsPerWave + qcol;  // packed row
     const bool row_ok = R < p.group * p.T;
+    // A wave whose 32 rows all lie past the last packed row (the tail of the last M-tile: two of its eight waves for a
+    // 60-node tree) has nothing to compute: it still requests its share of every tile and meets every barrier, but
+    // skips the tile arithmetic -- 6 % of the launch's matrix and vector work at that tree size.
+    const bool wave_has_rows = __builtin_amdgcn_readfirstlane(mt * kRowsPerWg + rw * kRowsPerWave) < p.group * p.T;
     const int node = !row_ok ? 0 : p.group_shift >= 0 ? R >> p.group_shift : R / p.group;
     const int head = g * p.group + (!row_ok ? 0 : p.group_shift >= 0 ? R & (p.group - 1) : R % p.group);
 
@@ -645,7 +649,7 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
             }
             __syncthreads();
         }
-        if (i < n) {
+        if (i < n && wave_has_rows) {
             // ---- S^T = K.Q^T : two 32-key blocks.  All 16 operand reads are issued before the first
             // MFMA: LDS returns in order, so MFMA i only waits for read i. ----
             f32x16 sacc[2];
