@@ -10,6 +10,7 @@ struct Options {
     int attn_kv_groups = 0;        // 0 = chosen per call; 1 / 2 force that tree-attention kernel shape
     int head_share_last_pass = 1;  // 0 keeps the plain row-block mapping of the head GEMM
     int attn_merge_in_launch = 1;  // 0: the split partials of tree attention are always merged by a launch of their own
+    int attn_merge_wait_us = 2000; // longest wait of a workgroup for the others of its merge before it abandons its share
 };
 Options& options();
 

@@ -111,12 +111,11 @@ struct AttnParams {
     // unit, arrivals in its low 16 bits, a generation count above them.  Between launches arrivals is 0; the last
     // workgroup of a unit to arrive turns the full count into the next generation.
     uint32_t* merge_ctr;
+    uint32_t merge_wait_ticks;  // longest wait for the other workgroups of a unit, in ticks of the 100 MHz wall clock
 };
 
 constexpr int kMergeUnitWords = 64;  // a unit's word sits in a 256-byte line of its own: every poll and every arrival is
                                      // a memory transaction, and those on one line queue behind each other
-constexpr int kMergeWaitExpired = INT32_MIN;  // value of g_attn_bad_length after a merge wait ran into its limit
-constexpr unsigned long long kMergeWaitTicks = 2000000ull;  // 20 ms of the 100 MHz wall clock
 
 // Loads and stores that other XCDs' workgroups of the same launch see: device-scope accesses go past the
 // (per-XCD, mutually incoherent) L2.
@@ -865,42 +864,66 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
         if (unit_ctr == nullptr) return;
         // ---- merge inside the launch ----
         // Every workgroup of the unit (same KV head and M-tile, one per split) announces its partials once they
-        // have reached memory; when all have, each merges a share of the unit's 32-row x 4-dim-quad blocks.
-        // The last to arrive never waits; the others wait for it, with a limit: a launch whose workgroups cannot all
-        // be resident at once would otherwise wait on workgroups that cannot start (the host only picks this path
-        // when they fit; a wait that runs out leaves its blocks unmerged and is reported at the next synchronisation).
-        __shared__ int s_merge_go;
+        // have reached memory; when all have, each merges its share of the unit's 32-row x 4-dim-quad blocks
+        // (share s: the blocks b with b % splits == s).
+        // The last to arrive never waits; the others wait for it, with a limit -- workgroups that wait for each other
+        // must all be resident, which the host checks against the CU count but cannot promise when another launch
+        // holds CUs (two such launches on one GPU could wait for each other's unstarted workgroups).  A workgroup
+        // whose wait runs out marks its share as abandoned and leaves, which frees its CU; the last to arrive merges
+        // the abandoned shares after its own, so the output is complete either way.
+        __shared__ int s_merge_go, s_merge_last;
+        __shared__ uint32_t s_merge_abandoned;
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
+        uint32_t* const unit_abandoned = unit_ctr + 1;  // one bit per share; zero between launches
         if (tid == 0) {
-            int go = 1;
+            int go = 1, last = 0;
             // The word as this workgroup's arrival found it: the generation of this launch above, the arrivals before it below.
             const uint32_t before = __hip_atomic_fetch_add(unit_ctr, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             const uint32_t full = (before & 0xffff0000u) + (uint32_t)p.num_splits;
+            auto all_arrived = [&]() {  // either the full count or, once the last one has moved it on, the next generation
+                const uint32_t now = __hip_atomic_load(unit_ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                return now == full || (now & 0xffff0000u) != (before & 0xffff0000u);
+            };
             if (before + 1u == full) {
                 // last to arrive: full count -> next generation, no arrivals (nobody needs the result of this one)
                 __hip_atomic_fetch_add(unit_ctr, 0x10000u - (uint32_t)p.num_splits, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                last = 1;
             } else {
-                // the others see either the full count or, once the last one has moved it on, the next generation
                 const unsigned long long t_begin = wall_clock64();
-                while (true) {
-                    const uint32_t now = __hip_atomic_load(unit_ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    if (now == full || (now & 0xffff0000u) != (before & 0xffff0000u)) break;
-                    if (wall_clock64() - t_begin > kMergeWaitTicks) {
-                        g_attn_bad_length = kMergeWaitExpired;
-                        go = 0;
+                while (!all_arrived()) {
+                    if (wall_clock64() - t_begin >= p.merge_wait_ticks) {
+                        // The mark is in memory before this workgroup looks once more: if the others have all arrived by
+                        // then, the last of them may have read the marks already, and this workgroup merges its share
+                        // itself (twice the same values at worst); if not, the last one will find the mark.
+                        const uint32_t marks = __hip_atomic_fetch_or(unit_abandoned, 1u << split, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        asm volatile("" ::"v"(marks));  // (the mark has been made once its old value is back)
+                        go = all_arrived() ? 1 : 0;
                         break;
                     }
                     __builtin_amdgcn_s_sleep(4);
                 }
             }
             s_merge_go = go;
+            s_merge_last = last;
         }
         __syncthreads();
         if (!s_merge_go) return;
+        const bool last = s_merge_last != 0;
+        // the last one collects the abandoned shares while it merges its own
+        uint32_t abandoned = 0;
+        if (last && tid == 0) abandoned = __hip_atomic_exchange(unit_abandoned, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         const int nblocks = kRowWaves * 16;
-        for (int b = split + p.num_splits * wave; b < nblocks; b += p.num_splits * kWaves)
-            combine_block<true>(p, g, mt * kRowWaves + (b >> 4), b & 15, lane);
+        auto merge_share = [&](int share) {
+            for (int b = share + p.num_splits * wave; b < nblocks; b += p.num_splits * kWaves)
+                combine_block<true>(p, g, mt * kRowWaves + (b >> 4), b & 15, lane);
+        };
+        merge_share(split);
+        if (last) {
+            if (tid == 0) s_merge_abandoned = abandoned;
+            __syncthreads();
+            for (uint32_t m = s_merge_abandoned; m != 0; m &= m - 1) merge_share(__builtin_ctz(m));
+        }
     }
 }
 
@@ -1165,6 +1188,7 @@ static int tree_attention_impl(const void* q, void* k_pool, void* v_pool,
     p.o_part = nullptr;
     p.ml_part = nullptr;
     p.merge_ctr = nullptr;
+    p.merge_wait_ticks = 0;
     if (p.num_splits > 1) {
         const size_t o_bytes = align_up((size_t)Hkv * p.num_splits * p.rows_pad * kHeadDim * sizeof(f16), 256);
         const size_t ml_bytes = (size_t)Hkv * p.num_splits * p.rows_pad * 2 * sizeof(float);
@@ -1173,6 +1197,7 @@ static int tree_attention_impl(const void* q, void* k_pool, void* v_pool,
         p.o_part = (float*)workspace;
         p.ml_part = (float*)((char*)workspace + o_bytes);
         if (plan.merge_in_launch) p.merge_ctr = merge_counters_for(workspace, st);
+        p.merge_wait_ticks = (uint32_t)options().attn_merge_wait_us * 100u;
     }
     const int nsh = p.num_splits * Hkv;
     const dim3 grid(kXcds * ceil_div(nsh, kXcds), p.num_mtiles);

@@ -76,7 +76,9 @@ const char* cpmcu_version(void);
  *                           of the head GEMM (default), 0 = plain mapping (CPMCU_HEAD_NO_SHARE set);
  *   "attn_merge_in_launch"  1 = the workgroups of a split tree-attention launch merge their own partials when the
  *                           launch fits the GPU's CUs and has at most 32 splits (default), 0 = always the separate
- *                           merge launch (CPMCU_ATTN_SEPARATE_MERGE set). */
+ *                           merge launch (CPMCU_ATTN_SEPARATE_MERGE set);
+ *   "attn_merge_wait_us"    longest time a workgroup of such a launch waits for the others of its merge before it
+ *                           leaves its share to the last one to arrive (default 2000; 0 = never wait). */
 int cpmcu_set_option(const char* name, int value);
 
 /* ------------------------------------------------------------------------- */

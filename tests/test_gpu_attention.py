@@ -477,3 +477,34 @@ def test_merge_counter_blocks_move_on_to_new_workspaces(gpu):
             assert np.array_equal(got.view(np.uint16), ref.view(np.uint16)), "call %d.%d" % (i, rep)
         keep.append(ops._workspaces[("attn", q.device)])  # kept alive: every call sees a new address
     assert len({t.data_ptr() for t in keep}) == 40
+
+
+@pytest.mark.parametrize("P,T", [(4096, 60), (33000, 60), (700, 128)])
+def test_merge_wait_that_runs_out_leaves_the_share_to_the_last_arrival(gpu, set_option, P, T):
+    """With the wait limit at zero every workgroup but the last of a unit gives up at once (unless everyone has
+    arrived already), marks its share as abandoned and leaves; the last arrival merges those shares.  The output must be
+    what the separate merge launch gives, bit for bit, and the marks must be gone for the next call."""
+    torch = gpu
+    from cpm.cu_amd import ops
+    from cpm.cu_amd.kvcache import PagedKVCache
+    tree = synth.eagle_tree(6, 10, T, seed=P)
+    S = P + T
+    q = to_dev(torch, synth.normal_f16((T, HQ, D), P, 1))
+    k = synth.normal_f16((S, HKV, D), P, 2)
+    v = synth.normal_f16((S, HKV, D), P, 3)
+    npages = (S + 255) // 256 + 1
+    cache = PagedKVCache(1, HKV, npages)
+    cache.write_logical(0, 0, to_dev(torch, k), to_dev(torch, v))
+    mask = to_dev(torch, tree.mask)
+    kv_len = torch.tensor([S], dtype=torch.int32, device="cuda")
+    names, splits, _, _ = ops.attention_plan(T, HQ, HKV, S)  # the split count a self-merging launch of this shape takes
+    assert "combine" not in names and splits > 1
+    set_option("attn_merge_in_launch", 0)
+    ref = to_np(ops.tree_attention(q, cache, 0, kv_len, S, mask, num_splits=splits))
+    set_option("attn_merge_in_launch", 1)
+    for wait_us in (0, 0, 2000, 0):
+        set_option("attn_merge_wait_us", wait_us)
+        out = torch.full_like(q, float("nan"))  # a share nobody merged would stay NaN
+        ops.tree_attention(q, cache, 0, kv_len, S, mask, num_splits=splits, out=out)
+        torch.cuda.synchronize()
+        assert np.array_equal(to_np(out).view(np.uint16), ref.view(np.uint16)), "wait %d us" % wait_us
