@@ -508,3 +508,59 @@ def test_merge_wait_that_runs_out_leaves_the_share_to_the_last_arrival(gpu, set_
         ops.tree_attention(q, cache, 0, kv_len, S, mask, num_splits=splits, out=out)
         torch.cuda.synchronize()
         assert np.array_equal(to_np(out).view(np.uint16), ref.view(np.uint16)), "wait %d us" % wait_us
+
+
+def test_two_self_merging_launches_side_by_side(gpu):
+    """Attention calls on two streams with a workspace each (the condition under which calls may overlap on one GPU):
+    whether the launches run one after the other or share the CUs, every output must carry the bits of the same call
+    made alone."""
+    torch = gpu
+    from cpm.cu_amd import lib, ops
+    from cpm.cu_amd.kvcache import PagedKVCache
+    T, P, layers = 60, 4096, 3
+    tree = synth.eagle_tree(6, 10, T, seed=11)
+    S = P + T
+    mask = to_dev(torch, tree.mask)
+    kv_len = torch.tensor([S], dtype=torch.int32, device="cuda")
+    npages = (S + 255) // 256 + 1
+    need = lib.get().raw.cpmcu_tree_attention_workspace_bytes(T, HQ, HKV, S)
+    sides = []
+    for i in range(2):
+        cache = PagedKVCache(layers, HKV, npages)
+        for l in range(layers):
+            cache.write_logical(l, 0, to_dev(torch, synth.normal_f16((S, HKV, D), 20 + i, 2 + l)),
+                                to_dev(torch, synth.normal_f16((S, HKV, D), 30 + i, 2 + l)))
+        sides.append(dict(q=to_dev(torch, synth.normal_f16((T, HQ, D), 40 + i, 1)), cache=cache,
+                          ws=torch.empty(need, dtype=torch.uint8, device="cuda"), stream=torch.cuda.Stream()))
+    key = ("attn", sides[0]["q"].device)
+    saved = ops._workspaces.get(key)
+
+    def call(side, l, out):
+        ops._workspaces[key] = side["ws"]
+        ops.tree_attention(side["q"], side["cache"], l, kv_len, S, mask, out=out)
+    try:
+        refs = []
+        for side in sides:
+            row = []
+            for l in range(layers):
+                o = torch.empty_like(side["q"])
+                call(side, l, o)
+                torch.cuda.synchronize()
+                row.append(to_np(o))
+            refs.append(row)
+        for rep in range(10):
+            outs = [[torch.full_like(side["q"], float("nan")) for _ in range(layers)] for side in sides]
+            torch.cuda.synchronize()
+            for l in range(layers):
+                for i, side in enumerate(sides):
+                    with torch.cuda.stream(side["stream"]):
+                        call(side, l, outs[i][l])
+            torch.cuda.synchronize()
+            for i in range(2):
+                for l in range(layers):
+                    assert np.array_equal(to_np(outs[i][l]).view(np.uint16), refs[i][l].view(np.uint16)), (rep, i, l)
+    finally:
+        if saved is None:
+            ops._workspaces.pop(key, None)
+        else:
+            ops._workspaces[key] = saved
