@@ -9,6 +9,7 @@ namespace cpmcu {
 struct Options {
     int attn_kv_groups = 0;        // 0 = chosen per call; 1 / 2 force that tree-attention kernel shape
     int head_share_last_pass = 1;  // 0 keeps the plain row-block mapping of the head GEMM
+    int head_stream_kernel = 1;    // 0 keeps tiled weights on the K-chunked kernel (tests compare the two)
     int attn_merge_in_launch = 1;  // 0: the split partials of tree attention are always merged by a launch of their own
     int attn_merge_wait_us = 2000; // longest wait of a workgroup for the others of its merge before it abandons its share
 };
@@ -24,9 +25,17 @@ void attention_prepare_workspace(const void* workspace);
 // lm_head.hip -- the streaming GEMM with its two epilogues.
 constexpr int kHeadModeStats = 0;
 constexpr int kHeadModeArgmax = 1;
-// (row-walking kernel by row blocks of hidden, or the K-chunked kernel <NB, NP, KC, NBUF>)
+// The streaming kernel <NB, FP, KC> (tiled weights, one sweep): NB 16-row blocks of hidden rows, FP full passes, KC-column chunks.
+#define CPMCU_HEAD_STREAM_SHAPES(X)                                                                           \
+    X(1, 1, 512) X(1, 2, 256) X(1, 3, 256) X(1, 4, 256) X(2, 1, 512) X(2, 2, 256) X(2, 3, 256) X(2, 4, 128) \
+    X(4, 1, 256) X(4, 2, 256) X(4, 3, 128) X(4, 4, 128) X(8, 1, 128) X(8, 2, 128)
+// (row-walking kernel by row blocks of hidden, the K-chunked kernel <NB, NP, KC, NBUF>, or the streaming kernel)
 enum class HeadShape { Row1, Row2, Row4, Row8, C_1_2_512_2, C_1_4_256_2, C_2_4_256_4, C_2_4_256_2, C_4_4_256_4, C_4_4_256_2, C_8_4_128_2,
-                       C_2_4_512_2, C_4_4_128_4, C_8_2_128_2 };
+                       C_2_4_512_2, C_4_4_128_4, C_8_2_128_2,
+#define CPMCU_X(nb, fp, kc) S_##nb##_##fp##_##kc,
+                       CPMCU_HEAD_STREAM_SHAPES(CPMCU_X)
+#undef CPMCU_X
+};
 const char* head_shape_name(HeadShape s);
 // dry_run: only choose the kernel shape and grid (reported through shape_out / grid_out), launch nothing.
 int launch_head_gemm(const void* hidden, const void* w, int w_layout, int n, int V, int H, int apply_scale, float head_scale,

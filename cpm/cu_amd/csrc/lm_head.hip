@@ -26,6 +26,7 @@
 //     filled last pass are dealt round-robin to the workgroups and several waves share each of
 //     them, every one taking a subset of the K chunks; their partial sums meet in LDS.
 #include <mutex>
+#include <type_traits>
 
 #include "common.h"
 #include "internal.h"
@@ -50,6 +51,7 @@ struct HeadParams {
     // complete passes, rem_blocks = row blocks left for the last one; 0 = plain mapping.
     int full_passes;
     int rem_blocks;
+    int last_share;  // streaming kernel: waves that share one row block of the last pass (power of two)
     int apply_scale;
     float head_scale;
     int mode;
@@ -530,6 +532,191 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_chunked_kernel(HeadPar
     head_finish<NB>(p, ea, eb, red_a, red_b, tid, wave, lane, c);
 }
 
+// Tiled weights whose row blocks fit one sweep: FP full passes (every wave one whole row block each) and at most
+// one partly filled last pass.  The wave's W stream is a ring of 1 KB fragments held in registers and refilled
+// fragment by fragment: as soon as the MFMAs of a (row block, K step) have read their fragment, the same registers
+// are requested again for the same position of the NEXT chunk, so a wave keeps about one chunk's worth of W
+// (FP row blocks x KC columns, + its slice of the last pass) in flight at all times.  The loop body is straight-line
+// code (FP is a template parameter, the refills are unconditional, the last chunk -- which refills nothing -- is a
+// second instance of the body) so that the compiler's own vmcnt bookkeeping is exact: with loads inside
+// wave-uniform branches, as in the kernel above, it has to assume the fewest loads in flight, waits for the
+// newest group before it computes on the one before, and load and compute take turns.  The scheduling fence
+// after every K step keeps the refills where they are written; without it they are sunk below the MFMAs
+// that follow, to shorten register live ranges.  Against the kernel above, same GPU, 73448 x 4096 head:
+// 103.1 -> 96.2 us with 60 hidden rows, 100.5 -> 95.1 with 33, 92.7 -> 90.3 with 16 or 1.  (Refilling a row
+// block's K steps of a chunk in one burst behind its MFMAs instead: 98.7 / 97.4 / 92.0 us.)
+//   A K step reads its hidden-row operands from LDS once and uses them for all FP row blocks.
+//   Last pass: the workgroup's row blocks of it are shared by `share` waves each (a power of two, the same for
+//   the whole launch), and every wave takes `PD / share` K steps of EVERY chunk (slice `wave % share`), so its
+//   stream has the same length in every chunk; the partial sums meet in LDS after the loop.  These loads sit in
+//   wave-uniform branches (their count is a run-time value); the ring has PD extra slots for them, and what the
+//   compiler has to assume about them costs the full passes at most that many fragments of look-ahead.
+//   The hidden chunk is brought in as in the kernel above (direct-to-LDS, double buffered, XOR-swizzled).
+template <int NB, int FP, int KC>
+__global__ __launch_bounds__(kHeadThreads) void head_gemm_stream_kernel(HeadParams p) {
+    constexpr int PD = KC / 32;              // 1 KB W fragments per row block and chunk
+    constexpr int R = (FP + 1) * PD;         // ring slots
+    constexpr int ROWB = KC * 2;
+    constexpr int BUF = NB * 16 * ROWB;
+    constexpr int PR = KC / 8;               // 16-byte pieces per hidden row chunk
+    constexpr int NINST = BUF / 1024 / kHeadWaves;  // 1 KB DMA instructions per wave and chunk
+    static_assert(NINST >= 1 && PD % 4 == 0 && FP >= 1 && FP * PD <= 63, "shape limits (swizzle groups of 4 K steps, vmcnt immediate)");
+    __shared__ __attribute__((aligned(1024))) char lds[2 * BUF];
+    __shared__ float red_a[kHeadWaves][NB * 16];
+    __shared__ float red_b[kHeadWaves][NB * 16];
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    const int l16 = lane & 15;
+    const int kgp = lane >> 4;
+    const int G = gridDim.x;
+    const int c = blockIdx.x;
+    const int H = p.H;
+    const int nch = H / KC;
+    const int rotc = c % nch;  // workgroups start their K walk at different chunks (HBM channel spread)
+    const f16 sc = (f16)p.head_scale;
+
+    // last pass: block `my_last` of this workgroup's share of it, K slice `my_sub` of every chunk
+    const int share = p.last_share;
+    const int my_last = wave / share, my_sub = wave % share;
+    const bool last_active = p.rem_blocks > 0 && c + my_last * G < p.rem_blocks;
+    const int sl = last_active ? PD / share : 0;  // K steps per chunk
+    const int rb_last = FP * kHeadWaves * G + c + my_last * G;
+
+    auto chunk_of = [&](int q) { const int x = q + rotc; return x >= nch ? x - nch : x; };
+    auto issue_hidden = [&](int q) {
+        const int k0 = chunk_of(q) * KC;
+#pragma unroll
+        for (int j = 0; j < NINST; ++j) {
+            const int inst = wave * NINST + j;
+            const int row = inst * (64 / PR) + lane / PR;
+            const int piece = (lane % PR) ^ (row & 15);
+            const int rc = row < p.n ? row : p.n - 1;  // rows past n: any valid data, their results are dropped
+            const f16* src = p.hidden + (size_t)rc * H + k0 + piece * 8;
+            const uint32_t dst = __builtin_amdgcn_readfirstlane(
+                (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)(lds + (q & 1) * BUF + inst * 1024));
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(src), "s"(dst) : "memory", "m0");
+        }
+    };
+    // fragment (row block, 32-column step) of the tiled matrix: 512 halves, this lane's 8 at lane * 8
+    const f16* wfull[FP];
+#pragma unroll
+    for (int pl = 0; pl < FP; ++pl) wfull[pl] = p.w + (size_t)((pl * kHeadWaves + wave) * G + c) * (H / 32) * 512 + lane * 8;
+    const f16* wlast = p.w + (size_t)(last_active ? rb_last : 0) * (H / 32) * 512 + lane * 8;
+    auto load_frag = [&](const f16* base, int step) { return __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(base + (size_t)step * 512)); };
+
+    f32x4 acc[FP + 1][NB];
+#pragma unroll
+    for (int pl = 0; pl <= FP; ++pl)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) acc[pl][nb][r] = 0.f;
+    float ea[NB], eb[NB];
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+        ea[nb] = -INFINITY;
+        eb[nb] = p.mode == kHeadModeStats ? 0.f : __int_as_float(0x7fffffff);
+    }
+    const int xl = (kgp ^ (l16 & 3)) << 4, hi = l16 >> 2;
+
+    // ring slot ks * FP + pl: K step ks of full pass pl; slot FP * PD + j: step j of the last-pass slice
+    f16x8 ring[R];
+    issue_hidden(0);
+    {
+        const int s0 = chunk_of(0) * PD;
+#pragma unroll
+        for (int ks = 0; ks < PD; ++ks)
+#pragma unroll
+            for (int pl = 0; pl < FP; ++pl) ring[ks * FP + pl] = load_frag(wfull[pl], s0 + ks);
+#pragma unroll
+        for (int j = 0; j < PD; ++j)
+            if (j < sl) ring[FP * PD + j] = load_frag(wlast, s0 + my_sub * sl + j);
+    }
+    // One chunk: `refill` = request the same ring positions for the next chunk (everywhere but in the last one).
+    auto chunk_body = [&](int q, auto refill) {
+        // Chunk q of the hidden rows was requested before the FP * PD (+ sl) fragments that were requested since
+        // (memory operations return in order).
+        asm volatile("s_waitcnt vmcnt(%0)" : : "n"(FP * PD) : "memory");
+        if (p.apply_scale) {  // fp16 pre-scale of the hidden rows (src/model/linear.cuh:82-101): own pieces, in place
+#pragma unroll
+            for (int j = 0; j < NINST; ++j) {
+                f16x8* px = reinterpret_cast<f16x8*>(lds + (q & 1) * BUF + (wave * NINST + j) * 1024 + lane * 16);
+                f16x8 x = *px;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x[e] = (f16)((float)x[e] * (float)sc);
+                *px = x;
+            }
+        }
+        __syncthreads();  // chunk q visible to all waves; all waves are done with the other buffer
+        if (refill) issue_hidden(q + 1);
+        const int sn = chunk_of(q + 1) * PD;
+        const char* base = lds + (q & 1) * BUF + l16 * ROWB + xl;
+        f16x8 b[2][NB];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) b[0][nb] = *reinterpret_cast<const f16x8*>(base + ((0 ^ hi) << 6) + nb * 16 * ROWB);
+#pragma unroll
+        for (int ks = 0; ks < PD; ++ks) {
+            if (ks + 1 < PD) {
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb)
+                    b[(ks + 1) & 1][nb] = *reinterpret_cast<const f16x8*>(base + (((ks + 1) ^ hi) << 6) + nb * 16 * ROWB);
+            }
+#pragma unroll
+            for (int pl = 0; pl < FP; ++pl)
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb)
+                    acc[pl][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ring[ks * FP + pl], b[ks & 1][nb], acc[pl][nb], 0, 0, 0);
+            if (refill) {
+#pragma unroll
+                for (int pl = 0; pl < FP; ++pl) ring[ks * FP + pl] = load_frag(wfull[pl], sn + ks);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int j = 0; j < PD; ++j) {
+            if (j < sl) {
+                const int ksl = my_sub * sl + j;
+                f16x8 bl[NB];
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) bl[nb] = *reinterpret_cast<const f16x8*>(base + ((ksl ^ hi) << 6) + nb * 16 * ROWB);
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb)
+                    acc[FP][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ring[FP * PD + j], bl[nb], acc[FP][nb], 0, 0, 0);
+                if (refill) ring[FP * PD + j] = load_frag(wlast, sn + ksl);
+            }
+        }
+    };
+    for (int q = 0; q + 1 < nch; ++q) chunk_body(q, std::true_type{});
+    chunk_body(nch - 1, std::false_type{});
+#pragma unroll
+    for (int pl = 0; pl < FP; ++pl) head_epilogue<NB>(p, acc[pl], ((pl * kHeadWaves + wave) * G + c) * 16 + kgp * 4, l16, ea, eb);
+    if (p.rem_blocks > 0) {
+        // The waves that shared a block of the last pass hold partial sums over their K slices: they meet in LDS
+        // (the hidden buffers are free now) and the first wave of each group adds them up in wave order.
+        __syncthreads();
+        f32x4* xch = reinterpret_cast<f32x4*>(lds);  // [wave][NB][64 lanes]
+        if (last_active && share > 1) {
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) xch[(wave * NB + nb) * 64 + lane] = acc[FP][nb];
+        }
+        __syncthreads();
+        if (last_active && my_sub == 0) {
+            for (int o = 1; o < share; ++o) {
+#pragma unroll
+                for (int nb = 0; nb < NB; ++nb) {
+                    const f32x4 x = xch[((wave + o) * NB + nb) * 64 + lane];
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) acc[FP][nb][r] += x[r];
+                }
+            }
+            head_epilogue<NB>(p, acc[FP], rb_last * 16 + kgp * 4, l16, ea, eb);
+        }
+    }
+    head_finish<NB>(p, ea, eb, red_a, red_b, tid, wave, lane, c);
+}
+
 // Final arg-max over the per-workgroup partials: one block per hidden row.  Largest value, lowest
 // index among equals: one 64-bit key (ordered image of the float, complemented index) per partial,
 // reduced per wave on the DPP path and across the four waves through LDS.
@@ -588,6 +775,10 @@ const char* head_shape_name(HeadShape s) {
         case HeadShape::C_2_4_512_2: return "head_gemm_chunked_kernel<2,4,512,2>";
         case HeadShape::C_4_4_128_4: return "head_gemm_chunked_kernel<4,4,128,4>";
         case HeadShape::C_8_2_128_2: return "head_gemm_chunked_kernel<8,2,128,2>";
+#define CPMCU_X(nb, fp, kc) \
+    case HeadShape::S_##nb##_##fp##_##kc: return "head_gemm_stream_kernel<" #nb "," #fp "," #kc ">";
+            CPMCU_HEAD_STREAM_SHAPES(CPMCU_X)
+#undef CPMCU_X
     }
     return "?";
 }
@@ -666,7 +857,30 @@ int launch_head_gemm(const void* hidden, const void* w, int w_layout, int n, int
     CPMCU_CHECK_ARG(G <= head_max_grid(), "lm_head: %d workgroups exceed the %d rows of the partial planes", G, head_max_grid());
     *grid_out = G;
     *stride_out = NB * 16;
-    const HeadShape shape = pick_head_shape(NB, H, p.w_tiled, p.nch, p.npasses, nrb, G, &p.full_passes, &p.rem_blocks);
+    p.last_share = 1;
+    HeadShape shape = pick_head_shape(NB, H, p.w_tiled, p.nch, p.npasses, nrb, G, &p.full_passes, &p.rem_blocks);
+    // Tiled weights with 1..4 full passes (1..2 for 65-128 hidden rows) and at most one partly filled pass: the streaming kernel.
+    int stream_kc = 0;
+    if (p.w_tiled && options().head_stream_kernel) {
+        const int slots = G * kHeadWaves;
+        const int full = nrb / slots, rem = nrb % slots;
+#define CPMCU_X(nb, fp, kc)                                \
+    if (NB == nb && full == fp && H % kc == 0) {           \
+        shape = HeadShape::S_##nb##_##fp##_##kc;           \
+        stream_kc = kc;                                    \
+    }
+        CPMCU_HEAD_STREAM_SHAPES(CPMCU_X)
+#undef CPMCU_X
+        if (stream_kc) {
+            p.full_passes = full;
+            p.rem_blocks = rem;
+            if (rem > 0 && options().head_share_last_pass) {
+                // the busiest workgroup has r_max blocks of the last pass; share * r_max waves work on them
+                const int r_max = ceil_div(rem, G);
+                while (p.last_share * 2 * r_max <= kHeadWaves && p.last_share * 2 <= stream_kc / 32) p.last_share *= 2;
+            }
+        }
+    }
     if (shape_out) *shape_out = shape;
     if (dry_run) return CPMCU_OK;
 #define CPMCU_HEAD_ROW(nb) hipLaunchKernelGGL(head_gemm_kernel<nb>, dim3(G), dim3(kHeadThreads), 0, st, p)
@@ -686,6 +900,10 @@ int launch_head_gemm(const void* hidden, const void* w, int w_layout, int n, int
         case HeadShape::C_2_4_512_2: CPMCU_HEAD_CHUNKED(2, 4, 512, 2); break;
         case HeadShape::C_4_4_128_4: CPMCU_HEAD_CHUNKED(4, 4, 128, 4); break;
         case HeadShape::C_8_2_128_2: CPMCU_HEAD_CHUNKED(8, 2, 128, 2); break;
+#define CPMCU_X(nb, fp, kc) \
+    case HeadShape::S_##nb##_##fp##_##kc: hipLaunchKernelGGL((head_gemm_stream_kernel<nb, fp, kc>), dim3(G), dim3(kHeadThreads), 0, st, p); break;
+            CPMCU_HEAD_STREAM_SHAPES(CPMCU_X)
+#undef CPMCU_X
     }
 #undef CPMCU_HEAD_ROW
 #undef CPMCU_HEAD_CHUNKED

@@ -48,6 +48,7 @@ Options& options() {
             if (e[0] == '2' && e[1] == 0) o.attn_kv_groups = 2;
         }
         if (getenv("CPMCU_HEAD_NO_SHARE") != nullptr) o.head_share_last_pass = 0;
+        if (getenv("CPMCU_HEAD_NO_STREAM") != nullptr) o.head_stream_kernel = 0;
         if (getenv("CPMCU_ATTN_SEPARATE_MERGE") != nullptr) o.attn_merge_in_launch = 0;
         return o;
     }();
@@ -190,6 +191,9 @@ extern "C" int cpmcu_set_option(const char* name, int value) {
     if (nm == "attn_kv_groups") {
         CPMCU_CHECK_ARG(value >= 0 && value <= 2, "set_option: attn_kv_groups=%d outside [0, 2]", value);
         options().attn_kv_groups = value;
+    } else if (nm == "head_stream_kernel") {
+        CPMCU_CHECK_ARG(value == 0 || value == 1, "set_option: head_stream_kernel=%d must be 0 or 1", value);
+        options().head_stream_kernel = value;
     } else if (nm == "head_share_last_pass") {
         CPMCU_CHECK_ARG(value == 0 || value == 1, "set_option: head_share_last_pass=%d must be 0 or 1", value);
         options().head_share_last_pass = value;

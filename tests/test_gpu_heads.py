@@ -399,3 +399,72 @@ def test_tiled_frspec_head_with_fused_gather(gpu, orc):
     val_s, pos_s = orc.topk(lp, k)
     assert np.array_equal(to_np(b["pos"]), pos_s) and np.array_equal(to_np(b["val"]).view(np.uint16), val_s.view(np.uint16))
     assert np.array_equal(to_np(b["ids"]), remap[pos_s])
+
+
+# (rows, vocabulary, hidden, head_scale) -> streaming kernel <NB, FP, KC>, waves per shared last-pass block
+_STREAM_SHAPES = [
+    (60, 73448, 4096, None),      # <4,2,256>, 4
+    (10, 32768, 4096, None),      # <1,1,512>, no last pass
+    (1, 32768 + 16 * 300, 512, None),   # <1,1,512>, 4; a single K chunk
+    (33, 36000, 512, 0.3125),     # <4,1,256>, 8
+    (64, 50000, 512, None),       # <4,1,256>, 1 (five blocks of the last pass per workgroup)
+    (20, 45000, 1024, None),      # <2,1,512>, 2
+    (100, 40000, 512, None),      # <8,1,128>, 4
+    (128, 70000, 512, 2.0),       # <8,2,128>, 4
+    (16, 122753, 1024, None),     # <1,3,256>, 1
+    (32, 110000, 512, None),      # <2,3,256>, 2
+    (60, 100000, 512, None),      # <4,3,128>, 4
+    (17, 151936, 512, None),      # <2,4,128>, 1
+    (60, 140000, 512, 0.3125),    # <4,4,128>, 2
+    (7, 140000, 512, None),       # <1,4,256>, 2
+    (40, 65536, 512, None),       # <4,2,256>, no last pass
+    (24, 65536 + 16 * 2047, 1024, None),  # <2,2,256>, 1: all but one wave slot of the last pass filled
+]
+
+
+@pytest.mark.parametrize("n,V,H,scale", _STREAM_SHAPES)
+def test_streaming_head_kernel_equals_chunked_kernel(gpu, orc, set_option, n, V, H, scale):
+    """Tiled weights with one to four full passes run the streaming kernel (register ring refilled fragment by
+    fragment, last pass shared by K slices).  Every (row blocks, full passes) shape it is built for, with 1, 2,
+    4 and 8 waves per last-pass block and without a last pass: same logits as the K-chunked kernel up to the
+    fp32 summation order, both within tolerance of the oracle, arg-max exact on each kernel's own logits."""
+    from cpm.cu_amd import ops
+    torch = gpu
+    hid = synth.normal_f16((n, H), V + n, 1)
+    w = synth.normal_f16((V, H), V + n, 2, std=0.02)
+    d_hid = to_dev(torch, hid)
+    wt = ops.tile_head_weight(to_dev(torch, w))
+    assert "head_gemm_stream_kernel" in ops.head_plan(n, wt)[0]
+    gt_s, z_s = ops.lm_head_argmax(d_hid, wt, head_scale=scale, want_logits=True)
+    gt_s2 = ops.lm_head_argmax(d_hid, wt, head_scale=scale)
+    torch.cuda.synchronize()
+    set_option("head_stream_kernel", 0)
+    assert "head_gemm_stream_kernel" not in ops.head_plan(n, wt)[0]
+    gt_c, z_c = ops.lm_head_argmax(d_hid, wt, head_scale=scale, want_logits=True)
+    torch.cuda.synchronize()
+    assert_close_f16(to_np(z_s), to_np(z_c), "streaming vs chunked kernel", atol=8e-3, rtol=2e-3)
+    z_ref = orc.lm_head(hid, w, head_scale=scale)
+    assert_close_f16(to_np(z_s), z_ref, "streaming kernel vs oracle")
+    assert np.array_equal(to_np(gt_s), to_np(gt_s2))
+    for z, gt in ((to_np(z_s), to_np(gt_s)), (to_np(z_c), to_np(gt_c))):
+        assert np.array_equal(gt, orc.argmax(z))  # staged: the kernel's own logits decide
+
+
+def test_streaming_head_kernel_plain_last_pass(gpu, orc, set_option):
+    """head_share_last_pass = 0 on the streaming kernel: whole row blocks per wave in the last pass."""
+    from cpm.cu_amd import ops
+    torch = gpu
+    n, V, H = 60, 73448, 512
+    hid = synth.normal_f16((n, H), 5, 1)
+    w = synth.normal_f16((V, H), 5, 2, std=0.02)
+    d_hid = to_dev(torch, hid)
+    wt = ops.tile_head_weight(to_dev(torch, w))
+    gt_s, z_s = ops.lm_head_argmax(d_hid, wt, want_logits=True)
+    torch.cuda.synchronize()
+    set_option("head_share_last_pass", 0)
+    assert "head_gemm_stream_kernel" in ops.head_plan(n, wt)[0]
+    gt_p, z_p = ops.lm_head_argmax(d_hid, wt, want_logits=True)
+    torch.cuda.synchronize()
+    assert_close_f16(to_np(z_s), to_np(z_p), "shared vs plain last pass", atol=8e-3, rtol=2e-3)
+    assert_close_f16(to_np(z_p), orc.lm_head(hid, w), "plain last pass vs oracle")
+    assert np.array_equal(to_np(gt_p), orc.argmax(to_np(z_p)))
