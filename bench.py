@@ -43,7 +43,7 @@ MEASURED_TRAFFIC = {
     "measured_at_commit": "779ad85",  # the library the counters were read on (git rev-parse --short HEAD of that run)
     "kib_per_launch": {
         "tree_attn_split_kernel<2,false>": 15154 + 9463,  # the merge of the split partials runs inside the launch
-        "head_gemm_chunked_kernel<4,4,256,2>": 592010 + 128,
+        "head_gemm_stream_kernel<4,2,256>": 592010 + 128,
     },
 }
 

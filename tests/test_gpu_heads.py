@@ -124,6 +124,16 @@ def test_frspec_tiled_chunk_rotation_shapes(gpu, orc):
     _frspec_check(gpu, orc, n=7, V=40000, Vs=32768, H=1024, k=32, seed=12, tiled=True)
 
 
+@pytest.mark.parametrize("n,V,Vs,H,k", [(10, 73448, 32768 + 16 * 300, 1024, 10), (16, 60000, 50000, 512, 10), (3, 73448, 70000, 512, 32),
+                                        (12, 50000, 36000, 512, 5)])
+def test_frspec_streaming_kernel_with_a_shared_last_pass(gpu, orc, n, V, Vs, H, k):
+    """Sub-vocabularies that are not a whole number of passes: the streaming GEMM with its statistics epilogue, the
+    last pass shared by 4, 1, 4 (behind two full passes) and 8 waves."""
+    from cpm.cu_amd import ops
+    assert "head_gemm_stream_kernel" in ops.head_plan(n, ops.tile_head_weight(to_dev(gpu, np.zeros((Vs, H), np.float16))))[0]
+    _frspec_check(gpu, orc, n=n, V=V, Vs=Vs, H=H, k=k, seed=Vs % 97, tiled=True)
+
+
 def test_frspec_subset_vs_full_head(gpu, orc):
     """If the full-vocab top-k ids all lie in the subset, the mapped subset top-k is the full-vocab top-k."""
     from cpm.cu_amd import ops
