@@ -77,6 +77,22 @@ struct HeadCfg {
 template <int NB>
 __device__ inline void head_epilogue(const HeadParams& p, const f32x4 (&acc)[NB], int vrow0, int l16, float (&ea)[NB], float (&eb)[NB]) {
     const int V = p.V;
+    if (p.mode == kHeadModeArgmax && p.logits == nullptr) {
+        // The verify step's case (arg-max only), without a branch per value: the same comparisons as below as selects.
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+            const bool row_in = nb * 16 + l16 < p.n;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float x = (float)(f16)acc[nb][r];
+                const int idx = vrow0 + r;
+                const bool take = row_in && idx < V && (x > ea[nb] || (x == ea[nb] && idx < __float_as_int(eb[nb])));
+                ea[nb] = take ? x : ea[nb];
+                eb[nb] = take ? __int_as_float(idx) : eb[nb];
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
         const int hrow = nb * 16 + l16;
