@@ -168,6 +168,64 @@ def test_frspec_subset_vs_full_head(gpu, orc):
         assert clear <= set(int(t) for t in sub_ids[i])
 
 
+def test_frspec_c3_full_size_against_the_full_vocabulary_head(gpu, orc):
+    """Config 3 as stated: the 32768-row FR-Spec head (gathered and tiled out of the 73448 x 4096 head, the layout the
+    benchmark runs) beside the full-vocabulary head on the same 10 hidden rows.  The subset's raw logits are the full
+    head's logits of the remapped rows; log-probabilities are rounded to fp16 (one ulp = 2^-6 below 16 in magnitude)
+    before ranking and the two heads normalise differently, so what must hold is: every id the subset returns is a
+    member of the subset and ranks, among the subset's members, no lower than the k-th best of them in the full head's
+    logits (within that rounding); every clear winner among the subset's members is returned; and a row whose
+    full-vocabulary top-k all lie in the subset returns the full head's ids."""
+    from cpm.cu_amd import ops
+    torch = gpu
+    n, V, Vs, H, k = 10, 73448, 32768, 4096, 10
+    hid = synth.normal_f16((n, H), 0, 1)
+    w = synth.normal_f16((V, H), 0, 2, std=0.02)
+    remap = synth.frspec_remap(V, Vs, 0)
+    d_hid, d_w, d_remap = to_dev(torch, hid), to_dev(torch, w), to_dev(torch, remap)
+    full = ops.frspec_head_topk(d_hid, ops.tile_head_weight(d_w), None, k)
+    sub = ops.frspec_head_topk(d_hid, ops.tile_head_weight(d_w, d_remap), d_remap, k)
+    torch.cuda.synchronize()
+    z_full, z_sub = to_np(full["logits"]), to_np(sub["logits"])
+    assert_close_f16(z_full, orc.lm_head(hid, w), "full-vocabulary logits")
+    # the two launches walk K in the same chunk order per row block, but in different kernels: logits to an fp16 ulp
+    assert_close_f16(z_sub, z_full[:, remap], "subset logits vs the full head's remapped rows", atol=8e-3, rtol=2e-3)
+    full_ids, sub_ids = to_np(full["ids"]), to_np(sub["ids"])
+    assert np.array_equal(full_ids, to_np(full["pos"]))  # no map: ids are positions
+    in_subset = np.zeros(V, bool)
+    in_subset[remap] = True
+    zf = z_full.astype(np.float32)
+    ulp = 2.0 ** -6
+    rows_inside = 0
+    for i in range(n):
+        assert in_subset[sub_ids[i]].all()
+        members = np.where(in_subset, zf[i], -np.inf)
+        kth = np.sort(members)[-k]
+        assert np.all(zf[i, sub_ids[i]] >= kth - 2 * ulp), "row %d: a returned id ranks below the subset's k-th" % i
+        clear = set(np.nonzero(members > kth + 2 * ulp)[0].tolist())
+        assert clear <= set(sub_ids[i].tolist()), "row %d: a clear winner of the subset is missing" % i
+        if in_subset[full_ids[i]].all():
+            rows_inside += 1
+            gaps = -np.diff(zf[i, full_ids[i]])
+            if gaps.min() > 2 * ulp:
+                assert np.array_equal(sub_ids[i], full_ids[i]), "row %d" % i
+    print("c3: rows whose full-vocabulary top-%d lies inside the subset: %d of %d" % (k, rows_inside, n))
+    # a subset that holds every row's full-vocabulary winners returns exactly the full head's ids
+    winners = np.unique(full_ids)
+    rest = np.setdiff1d(np.arange(V), winners)
+    remap2 = np.concatenate([winners, rest[: Vs - len(winners)]]).astype(np.int32)
+    synth.rng(0, 9).shuffle(remap2)
+    d_remap2 = to_dev(torch, remap2)
+    sub2 = ops.frspec_head_topk(d_hid, ops.tile_head_weight(d_w, d_remap2), d_remap2, k)
+    torch.cuda.synchronize()
+    sub2_ids = to_np(sub2["ids"])
+    for i in range(n):
+        kth = zf[i, full_ids[i]].min()
+        assert np.all(zf[i, sub2_ids[i]] >= kth - 2 * ulp)
+        clear = set(int(t) for t in full_ids[i] if zf[i, t] > kth + 2 * ulp)
+        assert clear <= set(int(t) for t in sub2_ids[i])
+
+
 def _argmax_check(torch, orc, n, V, H, seed, scale=None, plant=None, tiled=False):
     from cpm.cu_amd import ops
     hid = synth.normal_f16((n, H), seed, 1)
@@ -258,6 +316,16 @@ def test_row_major_head_with_many_k_chunks(gpu, orc, n, H):
 def test_target_head_c2_full_size(gpu, orc):
     """Config 2 head: 60 tree rows against the 73448x4096 head."""
     _argmax_check(gpu, orc, 60, V=73448, H=4096, seed=0)
+
+
+def test_target_head_c5_full_size(gpu, orc):
+    """Config 5 head: 128 tree rows against the 73448x4096 head in the tiled layout -- the 8-row-block streaming
+    kernel at its real K depth (32 chunks of 128 columns, two full passes and a shared last pass)."""
+    from cpm.cu_amd import ops
+    wt = ops.tile_head_weight(to_dev(gpu, np.zeros((73448, 4096), np.float16)))
+    assert "head_gemm_stream_kernel<8,2,128>" in ops.head_plan(128, wt)[0].replace(" ", "")
+    del wt
+    _argmax_check(gpu, orc, 128, V=73448, H=4096, seed=5, tiled=True)
 
 
 @pytest.mark.parametrize("n,dim,top", [(1, 100, 10), (1, 510, 59), (10, 32768, 10), (3, 5000, 32), (2, 2048, 1),

@@ -402,6 +402,82 @@ def test_c2_full_size_step_on_the_library_graph(gpu, orc):
         m.close()
 
 
+def test_128k_step_integer_parity_on_the_library_graph(gpu, orc):
+    """The longest context of the benchmark as a verify step whose results are checked: 3 layers, a 131072-token
+    prefix behind a permuted page table (the tree rows land in logical pages 512-513), 60-node tree, cpmcu_verify_step
+    replayed from the library's graph.  Accept length, ids and the compacted rows of every cache bit-exact against the
+    oracle at three accept depths; the attention of one layer against the oracle's pass over all 131132 keys; the
+    last prefix page of every cache untouched.  The head is reduced (the full-size heads have their own tests)."""
+    from cpm.cu_amd.model import PathModel
+    torch = gpu
+    L, P, T, V, H = 3, 131072, 60, 20000, 1024
+    S = P + T
+    tree = synth.eagle_tree(6, 10, T, seed=11)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(128)
+    w = (torch.randn(V, H, device="cuda", generator=g) * 0.02).to(torch.float16).cpu().numpy()
+    npages = (S + 255) // 256 + 1
+    m = PathModel(V, L, H, HQ, HKV, memory_limit=0.01, tree_size=T, num_iter=6, topk=10)
+    try:
+        assert m.max_context >= S
+        m.load_head(w)
+        table = to_dev(torch, synth.rng(128, 4).permutation(npages).astype(np.int32))
+        cache = m.cache(block_table=table)
+        for l in range(L):
+            m._k[l][:npages].normal_(generator=g)
+            m._v[l][:npages].normal_(generator=g)
+        rn = lambda *s: torch.randn(*s, device="cuda", generator=g).to(torch.float16)
+        q, kn, vn = [rn(T, HQ, D) for _ in range(L)], [rn(T, HKV, D) for _ in range(L)], [rn(T, HKV, D) for _ in range(L)]
+        out = [torch.zeros(T, HQ, D, dtype=torch.float16, device="cuda") for _ in range(L)]
+        hidden = rn(T, H)
+        tail0 = P - 256
+        before_tail = [cache.read_logical(l, tail0, 256) for l in range(L)]
+        kp, vp = (to_np(t) for t in cache.read_logical(1, 0, P))
+        draft = torch.zeros(T, dtype=torch.int32, device="cuda")
+        gt = torch.zeros(T, dtype=torch.int32, device="cuda")
+        ids = torch.zeros(T, dtype=torch.int32, device="cuda")
+        result = torch.zeros(1 + T, dtype=torch.int32).pin_memory()
+        clen = torch.tensor([P], dtype=torch.int32, device="cuda")
+        kvlen = torch.tensor([S], dtype=torch.int32, device="cuda")
+        pos, mask, parent = to_dev(torch, tree.positions(P)), to_dev(torch, tree.mask), to_dev(torch, tree.parent)
+        padded = (S + 127) // 128 * 128
+        torch.cuda.synchronize()
+        step = lambda: m.verify_step(T, padded, q, kn, vn, out, hidden, draft, pos, clen, kvlen, mask, parent, ids, gt_out=gt,
+                                     result=result, block_table=table, cuda_graph=True)
+        step()  # captures; the target arg-max of this pass rigs the draft ids
+        m.synchronize()
+        gt_np = to_np(gt)
+        z_ref = orc.lm_head(to_np(hidden), w)
+        gt_ref = orc.argmax(z_ref)
+        for i in np.nonzero(gt_np != gt_ref)[0]:  # only inside the logit tolerance
+            assert float(z_ref[i, gt_ref[i]]) - float(z_ref[i, gt_np[i]]) <= 4e-2
+        for depth in (0, 2, int(tree.depth.max())):
+            pred, leaf = synth.draft_ids_for_accept(tree, gt_np, depth, V, 70 + depth)
+            draft.copy_(to_dev(torch, pred))
+            torch.cuda.synchronize()
+            step()  # a replay
+            m.synchronize()
+            a = int(result[0])
+            a_ref, _, path = orc.tree_accept(pred, gt_np, tree.positions(P), P, tree.mask, tree.parent)
+            assert a == a_ref == depth + 1 and list(path) == tree.path_to(leaf)
+            flat = []
+            for l in range(L):
+                flat += [to_np(kn[l]).reshape(T, -1).copy(), to_np(vn[l]).reshape(T, -1).copy()]
+            ids_ref = orc.kv_compact(flat, 0, path, gt_np)
+            assert np.array_equal(result[1:1 + a].numpy(), ids_ref) and np.array_equal(to_np(ids)[:a], ids_ref)
+            for l in range(L):
+                kd, vd = cache.read_logical(l, P, a)
+                assert np.array_equal(to_np(kd).reshape(a, -1).view(np.uint16), flat[2 * l][:a].view(np.uint16)), (depth, l)
+                assert np.array_equal(to_np(vd).reshape(a, -1).view(np.uint16), flat[2 * l + 1][:a].view(np.uint16)), (depth, l)
+        ref = orc.tree_attention(to_np(q[1]), np.concatenate([kp, to_np(kn[1])]), np.concatenate([vp, to_np(vn[1])]), tree.mask, P)
+        assert_close_f16(to_np(out[1]), ref, "128K step on the library graph, attention of layer 1")
+        for l in range(L):
+            kd, vd = cache.read_logical(l, tail0, 256)
+            assert torch.equal(kd, before_tail[l][0]) and torch.equal(vd, before_tail[l][1]), "last prefix page of layer %d changed" % l
+    finally:
+        m.close()
+
+
 def test_device_side_length_outside_the_promised_bound_is_reported(gpu):
     """A KV length read from device memory that exceeds the call's max_kv_len (a stale padded length under a replayed
     graph, say) must not walk off the page table: the launch clamps it, and the next synchronising call says so."""
