@@ -15,12 +15,18 @@ struct Options {
 };
 Options& options();
 
-// tree_attention.hip -- an attention launch whose device-side length lay outside [max(T, mask_k_range), max_kv_len]
-// worked on the clamped length and left the offending value behind; this reads and clears it (synchronising).
-int attention_take_bad_length(int* value);
+// tree_attention.hip -- two things an attention launch can leave behind for the host: a device-side length outside
+// [max(T, mask_k_range), max_kv_len] (the launch worked on the clamped length), and merge waits that ran out.
+// attention_report_enqueue copies both words to pinned host memory in stream order (ahead of a synchronisation, never
+// under a capture); attention_report_take reads that copy afterwards and clears what it found.
+int attention_report_enqueue(hipStream_t st);
+int attention_report_take(int* bad_length, unsigned int* abandoned);
+void attention_merge_reenable();
 // Assigns the counters of the in-launch merge to a workspace on the current device (otherwise done by the first
-// launch that uses it outside a stream capture).
-void attention_prepare_workspace(const void* workspace);
+// launch that uses it outside a stream capture); they stay with it until it is released.
+void attention_prepare_workspace(const void* workspace, void* stream);
+// For a workspace that is about to be freed, with none of its launches in flight or captured.
+void attention_release_workspace(const void* workspace);
 
 // lm_head.hip -- the streaming GEMM with its two epilogues.
 constexpr int kHeadModeStats = 0;

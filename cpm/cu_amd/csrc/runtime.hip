@@ -156,11 +156,19 @@ struct PerfScope {
     }
 };
 
-// After a synchronisation: did an attention launch see a length outside what the host had promised?
-int check_device_errors() {
-    int bad = 0;
-    int rc = attention_take_bad_length(&bad);
+// Synchronises the stream and looks at what attention launches left behind for the host (the report words travel to
+// pinned memory in front of the synchronisation: no round trip of their own): a length outside what the host had
+// promised is an error; merge waits that ran out are counted for the summary.
+long g_abandoned_waits = 0;
+int synchronize_and_check(hipStream_t st) {
+    int rc = attention_report_enqueue(st);
     if (rc) return rc;
+    CPMCU_HIP(hipStreamSynchronize(st));
+    int bad = 0;
+    unsigned int abandoned = 0;
+    rc = attention_report_take(&bad, &abandoned);
+    if (rc) return rc;
+    g_abandoned_waits += abandoned;
     if (bad != 0) {
         set_error("a tree-attention launch read a KV length of %d from device memory, outside [rows, max_kv_len] of its call; "
                   "it ran on the clamped length and its output is not valid", bad < 0 ? 0 : bad);
@@ -203,6 +211,7 @@ extern "C" int cpmcu_set_option(const char* name, int value) {
     } else if (nm == "attn_merge_in_launch") {
         CPMCU_CHECK_ARG(value == 0 || value == 1, "set_option: attn_merge_in_launch=%d must be 0 or 1", value);
         options().attn_merge_in_launch = value;
+        if (value) attention_merge_reenable();  // also for workspaces that went back to the combine launch after an abandoned wait
     } else {
         set_error("set_option: unknown option %s", name);
         return CPMCU_ERR_INVALID_ARGUMENT;
@@ -303,6 +312,7 @@ void release_storage(Model& m) {
     (void)hipFree(m.d_k_pools);
     (void)hipFree(m.d_v_pools);
     (void)hipFree(m.block_table);
+    if (m.attn_ws) attention_release_workspace(m.attn_ws);
     (void)hipFree(m.attn_ws);
     (void)hipFree(m.head_ws);
     (void)hipFree(m.draft_logits);
@@ -415,7 +425,8 @@ int init_storage_impl(Model& m, int* max_context) {
     }
     pages -= ws_pages;
     CPMCU_HIP(hipMalloc(&m.attn_ws, m.attn_ws_bytes));
-    attention_prepare_workspace(m.attn_ws);  // its merge counters are assigned now, ahead of any captured launch
+    // the state of the in-launch merge is made now, ahead of any captured launch
+    attention_prepare_workspace(m.attn_ws, nullptr);
     m.num_pages = (int)pages;
     m.k_pools.assign(all_layers, nullptr);
     m.v_pools.assign(all_layers, nullptr);
@@ -681,9 +692,9 @@ extern "C" int cpmcu_verify_and_fix(int num_tokens, uint64_t pred, uint64_t gt, 
     if (rc) return rc;
     rc = cpmcu_verify_tail_inplace(m.d_best, m.d_ids, num_tokens, (int32_t*)pred, nullptr, nullptr, nullptr, 0, st);
     if (rc) return rc;
-    CPMCU_HIP(hipStreamSynchronize(st));
+    rc = synchronize_and_check(st);
     if (accept_length) *accept_length = m.h_result[0];
-    return check_device_errors();
+    return rc;
 }
 
 namespace {
@@ -858,9 +869,16 @@ extern "C" int cpmcu_print_perf_summary(void) {
     size_t free_b = 0, total_b = 0;
     if (hipMemGetInfo(&free_b, &total_b) == hipSuccess)
         printf("GPU memory: %.1f MiB used of %.1f MiB\n", (total_b - free_b) / 1048576.0, total_b / 1048576.0);
+    printf("attention merge waits that ran out (share left to the last workgroup of its unit): %ld\n", g_abandoned_waits);
     fflush(stdout);
     return CPMCU_OK;
 }
+
+// Extension: merge waits of tree-attention launches that ran out since the library was loaded, as seen by the
+// synchronising calls so far (cpmcu_synchronize, cpmcu_verify_and_fix).  Each is a workgroup that stopped waiting for the
+// others of its unit and left its share of the merge to the last of them: the output was complete, but late, and the
+// device's workspaces have gone back to the separate merge launch (cpmcu_set_option("attn_merge_in_launch", 1) undoes that).
+extern "C" long cpmcu_attention_abandoned_waits(void) { return g_abandoned_waits; }
 
 // Extension: device pointers of the model's storage for harnesses that fill the cache directly.
 extern "C" int cpmcu_model_pointers(int layer, uint64_t* k_pool, uint64_t* v_pool, uint64_t* block_table,
@@ -880,8 +898,8 @@ extern "C" int cpmcu_model_pointers(int layer, uint64_t* k_pool, uint64_t* v_poo
 extern "C" uint64_t cpmcu_stream(void) { return (uint64_t)(uintptr_t)resolve_stream(nullptr); }
 
 extern "C" int cpmcu_synchronize(void) {
-    CPMCU_HIP(hipStreamSynchronize(resolve_stream(nullptr)));
-    return check_device_errors();
+    CPMCU_CHECK_ARG(!(g_model && g_model->capturing), "synchronize: the library's stream is being captured");
+    return synchronize_and_check(resolve_stream(nullptr));
 }
 
 extern "C" int cpmcu_shutdown(void) {

@@ -42,7 +42,9 @@
 #include <map>
 #include <mutex>
 #include <type_traits>
+#include <algorithm>
 #include <utility>
+#include <vector>
 
 namespace cpmcu {
 namespace {
@@ -73,7 +75,13 @@ typedef __attribute__((address_space(3))) void* lds_ptr_t;
 // Set by a launch whose device-side length does not fit what the host promised (above max_kv_len, or shorter
 // than the query rows / the masked range): the launch then works on the length clamped into that range -- every
 // access stays inside the page table -- and this word keeps the offending length for the next synchronising call.
-__device__ int g_attn_bad_length;
+// `abandoned` counts merge waits that ran out (see the merge inside the launch below): workgroups that left their share to
+// the last arrival of their unit (the output was complete, only late).
+struct AttnReport {
+    int bad_length;
+    unsigned int abandoned;
+};
+__device__ AttnReport g_attn_report;
 
 struct AttnParams {
     const f16* q;
@@ -409,7 +417,7 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
     {
         const int lo = max(p.T, p.mask_k_range);
         if (S > p.max_kv_len || S < lo) {
-            if (sh == 0 && mt == 0 && tid == 0) g_attn_bad_length = S == 0 ? -1 : S;
+            if (sh == 0 && mt == 0 && tid == 0) g_attn_report.bad_length = S == 0 ? -1 : S;
             S = min(max(S, lo), p.max_kv_len);
         }
     }
@@ -878,7 +886,8 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
         __shared__ uint32_t s_merge_abandoned;
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        uint32_t* const unit_abandoned = unit_ctr + 1;  // one bit per share; zero between launches
+        uint32_t* const unit_abandoned = unit_ctr + 1;  // one bit per share; zero between launches (a mark that was made just
+                                                        // behind the last arrival's collection is taken back by its maker)
         if (tid == 0) {
             int go = 1, last = 0;
             // The word as this workgroup's arrival found it: the generation of this launch above, the arrivals before it below.
@@ -899,9 +908,15 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
                         // The mark is in memory before this workgroup looks once more: if the others have all arrived by
                         // then, the last of them may have read the marks already, and this workgroup merges its share
                         // itself (twice the same values at worst); if not, the last one will find the mark.
-                        const uint32_t marks = __hip_atomic_fetch_or(unit_abandoned, 1u << split, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        asm volatile("" ::"v"(marks));  // (the mark has been made once its old value is back)
-                        go = all_arrived() ? 1 : 0;
+                        // (acquire-release on the mark, acquire on the look that follows: the two stay in this order)
+                        (void)__hip_atomic_fetch_or(unit_abandoned, 1u << split, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+                        const uint32_t now = __hip_atomic_load(unit_ctr, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+                        go = (now == full || (now & 0xffff0000u) != (before & 0xffff0000u)) ? 1 : 0;
+                        // everyone is there after all: this workgroup merges its share itself and takes its mark back, so that
+                        // no mark outlives the launch (if the last arrival has collected it already, the share is merged twice
+                        // with the same values)
+                        if (go) (void)__hip_atomic_fetch_and(unit_abandoned, ~(1u << split), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        __hip_atomic_fetch_add(&g_attn_report.abandoned, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                         break;
                     }
                     __builtin_amdgcn_s_sleep(4);
@@ -941,11 +956,24 @@ __global__ __launch_bounds__(256) void tree_attn_combine_kernel(AttnParams p) {
     combine_block<false>(p, grb / nrb, grb % nrb, quad, lane);
 }
 
+int device_cu_count() {
+    static int cus[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    if (cus[dev] == 0) {
+        int v = 0;
+        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+        cus[dev] = v;
+    }
+    return cus[dev];
+}
+
 int choose_splits(int T, int group, int Hkv, int max_kv_len, int G) {
     const int num_mtiles = ceil_div(group * T, rows_per_wg(G));
     const int ntiles = ceil_div(max_kv_len, kTileN);
-    // One workgroup per CU (256 CUs).
-    int splits = 256 / (num_mtiles * Hkv);
+    // One workgroup per CU.
+    const int cus = device_cu_count() > 0 ? device_cu_count() : 256;
+    int splits = cus / (num_mtiles * Hkv);
     if (splits < 1) splits = 1;
     const bool merge = options().attn_merge_in_launch != 0;
     // One or two row units (plain decode, trees of up to 32 nodes) could take 64 or 128 splits; up to about 28K context
@@ -994,23 +1022,14 @@ struct LaunchPlan {
 };
 
 // Counters of the in-launch merge.  They live in the library (zero when it is loaded, and back at zero arrivals after
-// every launch), in blocks handed out per workspace: calls that may overlap use different workspaces and so different
-// counters, and nothing has to be cleared or allocated per call.
+// every launch), in blocks handed out per workspace pointer: calls that may overlap use different workspaces and so
+// different counters, and nothing has to be cleared or allocated per call.  A block stays with its workspace until
+// attention_release_workspace: a captured launch keeps its block's address, so a block is never passed on to another
+// workspace.  A launch that cannot have one -- more workspaces than blocks, a first launch under capture -- is merged by
+// the combine launch instead.
 constexpr int kMergeUnits = 256;    // (KV head, M-tile) units a launch may have on this path
-constexpr int kMergeBlocks = 32;    // blocks per device (see merge_counters_for)
+constexpr int kMergeBlocks = 32;    // workspaces with a block per device
 __device__ __align__(256) uint32_t g_merge_ctr[kMergeBlocks][kMergeUnits * kMergeUnitWords];
-
-int device_cu_count() {
-    static int cus[64] = {0};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
-    if (cus[dev] == 0) {
-        int v = 0;
-        if (hipDeviceGetAttribute(&v, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
-        cus[dev] = v;
-    }
-    return cus[dev];
-}
 
 // The split workgroups can merge in the launch when they are all resident at once (one per CU: a workgroup that
 // waits for the others must not keep them from starting) and few enough per counter.
@@ -1020,54 +1039,49 @@ bool can_merge_in_launch(int Hkv, int num_mtiles, int num_splits) {
     return kXcds * ceil_div(num_splits * Hkv, kXcds) * num_mtiles <= device_cu_count();
 }
 
-// The counter block of a workspace on the current device (null: the lookup of the counters' address failed or has to
-// wait).  When all blocks are taken, the one whose workspace has gone unused the longest moves on to the new workspace:
-// between launches a block is at rest, so this is safe as long as no more than kMergeBlocks workspaces have launches in
-// flight on one device at the same time.
+struct MergeState {
+    int block = -1;
+    bool use_combine = false;  // a wait was abandoned on this device: the workspace's launches are merged by the combine launch
+};
+std::mutex g_merge_mu;
+std::map<std::pair<int, const void*>, MergeState> g_merge_states;
+std::vector<int> g_merge_free_blocks[64];
+bool g_merge_blocks_listed[64] = {false};
+uint32_t* g_merge_ctr_base[64] = {nullptr};
+
+// The counter block of a workspace on the current device; null: the launch has to be merged by the combine launch.
 uint32_t* merge_counters_for(const void* workspace, hipStream_t st) {
-    struct Block {
-        int index;
-        unsigned long long last_use;
-    };
-    static std::mutex mu;
-    static std::map<std::pair<int, const void*>, Block> blocks;
-    static int next_block[64] = {0};
-    static unsigned long long use_clock = 0;
-    static uint32_t* base[64] = {nullptr};
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
-    std::lock_guard<std::mutex> lock(mu);
-    if (base[dev] == nullptr) {
-        // The address of the counters is looked up once per device, outside any stream capture (a launch that is being
-        // captured before the first eager one uses the combine launch).
-        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
-        if (hipStreamIsCapturing(st, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
-            (void)hipGetLastError();
-            return nullptr;
+    std::lock_guard<std::mutex> lock(g_merge_mu);
+    auto it = g_merge_states.find({dev, workspace});
+    if (it == g_merge_states.end()) {
+        if (g_merge_ctr_base[dev] == nullptr) {
+            // The address of the counters is looked up once per device, outside any stream capture.
+            hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+            if (hipStreamIsCapturing(st, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
+                (void)hipGetLastError();
+                return nullptr;
+            }
+            void* ptr = nullptr;
+            if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_merge_ctr)) != hipSuccess) {
+                (void)hipGetLastError();
+                return nullptr;
+            }
+            g_merge_ctr_base[dev] = (uint32_t*)ptr;
         }
-        void* ptr = nullptr;
-        if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_merge_ctr)) != hipSuccess) {
-            (void)hipGetLastError();
-            return nullptr;
+        if (!g_merge_blocks_listed[dev]) {
+            for (int b = kMergeBlocks - 1; b >= 0; --b) g_merge_free_blocks[dev].push_back(b);
+            g_merge_blocks_listed[dev] = true;
         }
-        base[dev] = (uint32_t*)ptr;
+        if (g_merge_free_blocks[dev].empty()) return nullptr;
+        MergeState ns;
+        ns.block = g_merge_free_blocks[dev].back();
+        g_merge_free_blocks[dev].pop_back();
+        it = g_merge_states.emplace(std::make_pair(dev, workspace), ns).first;
     }
-    auto it = blocks.find({dev, workspace});
-    if (it == blocks.end()) {
-        int index;
-        if (next_block[dev] < kMergeBlocks) {
-            index = next_block[dev]++;
-        } else {
-            auto oldest = blocks.end();
-            for (auto b = blocks.begin(); b != blocks.end(); ++b)
-                if (b->first.first == dev && (oldest == blocks.end() || b->second.last_use < oldest->second.last_use)) oldest = b;
-            index = oldest->second.index;
-            blocks.erase(oldest);
-        }
-        it = blocks.emplace(std::make_pair(dev, workspace), Block{index, 0}).first;
-    }
-    it->second.last_use = ++use_clock;
-    return base[dev] + (size_t)it->second.index * kMergeUnits * kMergeUnitWords;
+    if (it->second.use_combine) return nullptr;
+    return g_merge_ctr_base[dev] + (size_t)it->second.block * kMergeUnits * kMergeUnitWords;
 }
 LaunchPlan plan_launch(int T, int group, int Hkv, int max_kv_len, int block_window_size, int num_splits_override) {
     LaunchPlan pl;
@@ -1102,20 +1116,86 @@ extern "C" int cpmcu_tree_attention_plan(int T, int Hq, int Hkv, int max_kv_len,
 }
 
 namespace cpmcu {
-void attention_prepare_workspace(const void* workspace) { (void)merge_counters_for(workspace, nullptr); }
+void attention_prepare_workspace(const void* workspace, void* stream) { (void)merge_counters_for(workspace, resolve_stream(stream)); }
 
-// Reads and clears the bad-length word of the current device (a synchronising copy); 0 = none.
-int attention_take_bad_length(int* value) {
-    int v = 0;
-    CPMCU_HIP(hipMemcpyFromSymbol(&v, HIP_SYMBOL(g_attn_bad_length), sizeof(int)));
-    if (v != 0) {
-        const int zero = 0;
-        CPMCU_HIP(hipMemcpyToSymbol(HIP_SYMBOL(g_attn_bad_length), &zero, sizeof(int)));
+// Gives up the counter block of a workspace that is about to be freed (no launch on it may be in flight or captured).
+void attention_release_workspace(const void* workspace) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return;
+    std::lock_guard<std::mutex> lock(g_merge_mu);
+    auto it = g_merge_states.find({dev, workspace});
+    if (it == g_merge_states.end()) return;
+    g_merge_free_blocks[dev].push_back(it->second.block);
+    g_merge_states.erase(it);
+}
+
+// The report words of the current device, read without a round trip of their own: `attention_report_enqueue` puts a copy
+// into pinned host memory in stream order (call it ahead of a synchronisation of that stream, outside any capture),
+// `attention_report_take` looks at that copy afterwards and clears the device words only when something is there.
+// After any abandoned wait every workspace of the device goes back to the combine launch.
+namespace {
+AttnReport* g_report_host[64] = {nullptr};
+}
+int attention_report_enqueue(hipStream_t st) {
+    int dev = 0;
+    CPMCU_HIP(hipGetDevice(&dev));
+    CPMCU_CHECK_ARG(dev >= 0 && dev < 64, "device index %d outside [0, 64)", dev);
+    if (g_report_host[dev] == nullptr) {
+        CPMCU_HIP(hipHostMalloc((void**)&g_report_host[dev], sizeof(AttnReport), hipHostMallocDefault));
+        *g_report_host[dev] = AttnReport{0, 0u};
     }
-    *value = v;
+    CPMCU_HIP(hipMemcpyFromSymbolAsync(g_report_host[dev], HIP_SYMBOL(g_attn_report), sizeof(AttnReport), 0, hipMemcpyDeviceToHost, st));
     return CPMCU_OK;
 }
+int attention_report_take(int* bad_length, unsigned int* abandoned) {
+    int dev = 0;
+    CPMCU_HIP(hipGetDevice(&dev));
+    *bad_length = 0;
+    *abandoned = 0;
+    if (dev < 0 || dev >= 64 || g_report_host[dev] == nullptr) return CPMCU_OK;
+    const AttnReport r = *g_report_host[dev];
+    if (r.bad_length != 0 || r.abandoned != 0) {
+        const AttnReport zero{0, 0u};
+        CPMCU_HIP(hipMemcpyToSymbol(HIP_SYMBOL(g_attn_report), &zero, sizeof(zero)));
+        *g_report_host[dev] = zero;
+        if (r.abandoned != 0) {
+            std::lock_guard<std::mutex> lock(g_merge_mu);
+            for (auto& kv : g_merge_states)
+                if (kv.first.first == dev) kv.second.use_combine = true;
+        }
+    }
+    *bad_length = r.bad_length;
+    *abandoned = r.abandoned;
+    return CPMCU_OK;
+}
+// Lets the workspaces of the current device merge inside the launch again (cpmcu_set_option attn_merge_in_launch = 1).
+void attention_merge_reenable() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return;
+    std::lock_guard<std::mutex> lock(g_merge_mu);
+    for (auto& kv : g_merge_states)
+        if (kv.first.first == dev) kv.second.use_combine = false;
+}
 }  // namespace cpmcu
+
+// 1: a launch on this workspace (outside a stream capture, of a shape that allows it) merges its split partials itself;
+// 0: it is merged by the combine launch (no counter block left for the workspace, or the device has seen an abandoned wait).
+extern "C" int cpmcu_tree_attention_merge_mode(const void* workspace) {
+    int dev = 0;
+    if (workspace == nullptr || hipGetDevice(&dev) != hipSuccess) return 0;
+    {
+        std::lock_guard<std::mutex> lock(g_merge_mu);
+        auto it = g_merge_states.find({dev, workspace});
+        if (it != g_merge_states.end()) return it->second.use_combine || !options().attn_merge_in_launch ? 0 : 1;
+    }
+    return merge_counters_for(workspace, nullptr) != nullptr && options().attn_merge_in_launch ? 1 : 0;
+}
+
+extern "C" int cpmcu_tree_attention_release_workspace(const void* workspace) {
+    CPMCU_CHECK_ARG(workspace, "tree_attention_release_workspace: null pointer argument");
+    attention_release_workspace(workspace);
+    return CPMCU_OK;
+}
 
 extern "C" size_t cpmcu_tree_attention_workspace_bytes(int T, int Hq, int Hkv, int max_kv_len) {
     (void)max_kv_len;

@@ -47,12 +47,15 @@ SIGNATURES = {
     "cpmcu_model_pointers": (c_int, [c_int, ctypes.POINTER(c_u64), ctypes.POINTER(c_u64), ctypes.POINTER(c_u64), ctypes.POINTER(c_int)]),
     "cpmcu_stream": (c_u64, []),
     "cpmcu_synchronize": (c_int, []),
+    "cpmcu_attention_abandoned_waits": (ctypes.c_long, []),
     "cpmcu_shutdown": (c_int, []),
     "cpmcu_kv_append": (c_int, [_P, _P, _P, _P, _P, _P, c_int, c_int, _P]),
     "cpmcu_tree_attention_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "cpmcu_tree_attention": (c_int, [_P, _P, _P, _P, _P, c_int, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_float, _P, _P, c_size_t, c_int, _P]),
     "cpmcu_tree_attention_rope": (c_int, [_P, _P, _P, _P, _P, c_int, _P, _P, _P, _P, c_int, c_int, c_int, c_int, c_int, c_float, _P, _P, c_size_t, c_int, _P]),
     "cpmcu_tree_attention_window": (c_int, [_P, _P, _P, _P, _P, c_int, _P, _P, _P, c_int, _P, c_int, c_int, c_int, c_int, c_int, c_float, _P, _P, c_size_t, c_int, _P]),
+    "cpmcu_tree_attention_merge_mode": (c_int, [_P]),
+    "cpmcu_tree_attention_release_workspace": (c_int, [_P]),
     "cpmcu_tree_attention_plan": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_char_p, c_size_t, ctypes.POINTER(c_int), ctypes.POINTER(c_int), ctypes.POINTER(c_int)]),
     "cpmcu_rope_table": (c_int, [_P, _P, c_int, _P, _P]),
     "cpmcu_rope_apply": (c_int, [_P, c_int, c_int, c_int, _P, _P, _P]),

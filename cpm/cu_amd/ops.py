@@ -42,9 +42,18 @@ def _workspace(kind, nbytes, device):
     key = (kind, device)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
+        if ws is not None and kind == "attn":
+            release_attention_workspace(ws)
         ws = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
+
+
+def release_attention_workspace(ws):
+    """Before an attention workspace tensor is dropped: the library gives its merge counters to another workspace.
+    The device is synchronised first (no launch on the workspace may be in flight)."""
+    torch.cuda.synchronize()
+    _lib().tree_attention_release_workspace(ctypes.c_void_p(ws.data_ptr()))
 
 
 def mask_words(T):

@@ -250,6 +250,13 @@ uint64_t cpmcu_stream(void);
  * device-side KV length lay outside what its call had promised -- above max_kv_len / padded_length, or shorter than
  * its rows: such a launch runs on the clamped length (no access leaves the page table) and its output is not valid. */
 int cpmcu_synchronize(void);
+/* No reference counterpart: merge waits of tree-attention launches that ran out, as counted by the synchronising calls
+ * so far (cpmcu_synchronize, cpmcu_verify_and_fix; also printed by cpmcu_print_perf_summary).  A split workgroup that
+ * has waited attn_merge_wait_us for the other workgroups of its unit leaves its share of the merge to the last of them
+ * and ends: the output is complete, only late.  It happens when the launch's workgroups are not all resident at once,
+ * i.e. when another launch holds CUs.  After the first such wait is seen, the device's workspaces go back to the
+ * separate merge launch; cpmcu_set_option("attn_merge_in_launch", 1) lets them merge inside the launch again. */
+long cpmcu_attention_abandoned_waits(void);
 /* Free everything the global model owns (the reference never frees). */
 int cpmcu_shutdown(void);
 
@@ -307,6 +314,17 @@ int cpmcu_tree_attention(const void* q, void* k_pool, void* v_pool, const int32_
                          const uint64_t* mask, int mask_words, int mask_k_range, int T, int Hq, int Hkv, float scale,
                          void* out,
                          void* workspace, size_t workspace_bytes, int num_splits_override, void* stream);
+
+/* No reference counterpart: whether launches on this workspace merge their split partials themselves (1) or leave it
+ * to the separate merge launch (0).  The library keeps a block of arrival counters per workspace pointer it has met on a
+ * device (32 per device, kept until the library's own workspace is freed at cpmcu_shutdown; further workspaces get
+ * none), and takes every workspace of a device off the in-launch merge once a merge wait has been abandoned there
+ * (see cpmcu_attention_abandoned_waits).  Asking assigns a block to a workspace that has none yet. */
+int cpmcu_tree_attention_merge_mode(const void* workspace);
+/* No reference counterpart: tells the library that an attention workspace is about to be freed, so that its block of
+ * arrival counters can go to another workspace.  None of its launches may be in flight, and no captured graph that holds
+ * one may be replayed afterwards.  A workspace the library has never met is ignored. */
+int cpmcu_tree_attention_release_workspace(const void* workspace);
 
 /* No reference counterpart: which kernels a cpmcu_tree_attention* call of this shape launches, without
  * launching -- for reports that must name the instantiation actually taken.  kernel_names receives e.g.

@@ -447,11 +447,13 @@ def test_merge_in_launch_equals_separate_merge(gpu, set_option, P, T, splits, fu
         assert np.array_equal(a.view(np.uint16), b.view(np.uint16))
 
 
-def test_merge_counter_blocks_move_on_to_new_workspaces(gpu):
-    """The library hands a block of merge counters to each workspace pointer it meets (a fixed number per device) and,
-    when they run out, passes the one unused the longest on to the newcomer: every call must give the same bits."""
+def test_merge_counter_blocks_stay_with_their_workspaces(gpu):
+    """The library hands a block of merge counters to each workspace pointer it meets (a fixed number per device) and
+    never takes one back while the workspace may still be in use: workspaces beyond that number are merged by the
+    separate launch.  Every call must give the same bits whichever way it was merged, and a launch captured early must
+    still own its counters after many other workspaces have come and gone."""
     torch = gpu
-    from cpm.cu_amd import ops
+    from cpm.cu_amd import lib, ops
     from cpm.cu_amd.kvcache import PagedKVCache
     T, P = 60, 2000
     tree = synth.eagle_tree(6, 10, T, seed=3)
@@ -464,19 +466,45 @@ def test_merge_counter_blocks_move_on_to_new_workspaces(gpu):
     cache.write_logical(0, 0, to_dev(torch, k), to_dev(torch, v))
     mask = to_dev(torch, tree.mask)
     kv_len = torch.tensor([S], dtype=torch.int32, device="cuda")
-    ref = None
-    keep = []
+    merge_mode = lib.get().raw.cpmcu_tree_attention_merge_mode
+    # a graph captured on the current workspace (one eager call first: its counters are assigned outside the capture)
+    out_g = torch.empty_like(q)
+    ref = to_np(ops.tree_attention(q, cache, 0, kv_len, S, mask, out=out_g))
+    ws_g = ops._workspaces[("attn", q.device)]
+    in_launch = merge_mode(ws_g.data_ptr())
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            ops.tree_attention(q, cache, 0, kv_len, S, mask, out=out_g)
+    keep, modes = [], []
     for i in range(40):  # more distinct workspaces than the library has counter blocks; each is used twice in a row
         ops._workspaces.pop(("attn", q.device), None)
         for rep in range(2):
             out = ops.tree_attention(q, cache, 0, kv_len, S, mask)
             torch.cuda.synchronize()
-            got = to_np(out)
-            if ref is None:
-                ref = got
-            assert np.array_equal(got.view(np.uint16), ref.view(np.uint16)), "call %d.%d" % (i, rep)
+            assert np.array_equal(to_np(out).view(np.uint16), ref.view(np.uint16)), "call %d.%d" % (i, rep)
         keep.append(ops._workspaces[("attn", q.device)])  # kept alive: every call sees a new address
+        modes.append(merge_mode(keep[-1].data_ptr()))
     assert len({t.data_ptr() for t in keep}) == 40
+    assert modes[-1] == 0, "the library has 32 counter blocks per device: the last of 40 workspaces cannot have one"
+    assert modes == sorted(modes, reverse=True), "a workspace met earlier lost its block to a later one: %s" % modes
+    assert merge_mode(ws_g.data_ptr()) == in_launch
+    # the captured launch replayed next to eager launches on another workspace: same bits
+    for rep in range(5):
+        out_g.fill_(float("nan"))
+        torch.cuda.synchronize()
+        with torch.cuda.stream(side):
+            graph.replay()
+        out = ops.tree_attention(q, cache, 0, kv_len, S, mask)
+        torch.cuda.synchronize()
+        assert np.array_equal(to_np(out_g).view(np.uint16), ref.view(np.uint16)), rep
+        assert np.array_equal(to_np(out).view(np.uint16), ref.view(np.uint16)), rep
+    del graph
+    for t in keep:
+        ops.release_attention_workspace(t)
+    ops._workspaces[("attn", q.device)] = ws_g
 
 
 @pytest.mark.parametrize("P,T", [(4096, 60), (33000, 60), (700, 128)])
@@ -485,7 +513,7 @@ def test_merge_wait_that_runs_out_leaves_the_share_to_the_last_arrival(gpu, set_
     arrived already), marks its share as abandoned and leaves; the last arrival merges those shares.  The output must be
     what the separate merge launch gives, bit for bit, and the marks must be gone for the next call."""
     torch = gpu
-    from cpm.cu_amd import ops
+    from cpm.cu_amd import lib, ops
     from cpm.cu_amd.kvcache import PagedKVCache
     tree = synth.eagle_tree(6, 10, T, seed=P)
     S = P + T
@@ -502,12 +530,31 @@ def test_merge_wait_that_runs_out_leaves_the_share_to_the_last_arrival(gpu, set_
     set_option("attn_merge_in_launch", 0)
     ref = to_np(ops.tree_attention(q, cache, 0, kv_len, S, mask, num_splits=splits))
     set_option("attn_merge_in_launch", 1)
+    L = lib.get()
+    L.synchronize()
+    set_option("attn_merge_in_launch", 1)  # (also puts workspaces back on the in-launch merge after an earlier test's abandoned waits)
+    ws = ops._workspaces[("attn", q.device)].data_ptr()
+    if not L.raw.cpmcu_tree_attention_merge_mode(ws):
+        pytest.skip("this process has used up the library's counter blocks: the workspace is merged by the separate launch")
+    seen0 = L.raw.cpmcu_attention_abandoned_waits()
     for wait_us in (0, 0, 2000, 0):
         set_option("attn_merge_wait_us", wait_us)
         out = torch.full_like(q, float("nan"))  # a share nobody merged would stay NaN
         ops.tree_attention(q, cache, 0, kv_len, S, mask, num_splits=splits, out=out)
         torch.cuda.synchronize()
         assert np.array_equal(to_np(out).view(np.uint16), ref.view(np.uint16)), "wait %d us" % wait_us
+    # the abandoned waits are counted at the next synchronising call of the library, and the device's workspaces go back
+    # to the separate merge launch until the option is set again
+    L.synchronize()
+    assert L.raw.cpmcu_attention_abandoned_waits() > seen0
+    assert L.raw.cpmcu_tree_attention_merge_mode(ws) == 0
+    out = torch.full_like(q, float("nan"))
+    ops.tree_attention(q, cache, 0, kv_len, S, mask, num_splits=splits, out=out)
+    torch.cuda.synchronize()
+    assert np.array_equal(to_np(out).view(np.uint16), ref.view(np.uint16))
+    L.synchronize()
+    set_option("attn_merge_in_launch", 1)
+    assert L.raw.cpmcu_tree_attention_merge_mode(ws) == 1
 
 
 def test_two_self_merging_launches_side_by_side(gpu):
@@ -560,6 +607,8 @@ def test_two_self_merging_launches_side_by_side(gpu):
                 for l in range(layers):
                     assert np.array_equal(to_np(outs[i][l]).view(np.uint16), refs[i][l].view(np.uint16)), (rep, i, l)
     finally:
+        for side in sides:
+            ops.release_attention_workspace(side["ws"])
         if saved is None:
             ops._workspaces.pop(key, None)
         else:
