@@ -1042,12 +1042,19 @@ constexpr int kMaxDevices = 64;
 void* g_scratch_ptr[kMaxDevices] = {};
 std::mutex g_scratch_mutex;
 
-int static_head_scratch(float** out) {
+int static_head_scratch(float** out, hipStream_t st) {
     int dev = -1;
     CPMCU_HIP(hipGetDevice(&dev));
     CPMCU_CHECK_ARG(dev >= 0 && dev < kMaxDevices, "lm_head_argmax_static: device index %d outside [0, %d)", dev, kMaxDevices);
     std::lock_guard<std::mutex> lock(g_scratch_mutex);
     if (g_scratch_ptr[dev] == nullptr) {
+        // The address lookup is not a thing to do while the stream is being captured: the first call on a device has to
+        // come before.
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (hipStreamIsCapturing(st, &capturing) != hipSuccess) (void)hipGetLastError();
+        CPMCU_CHECK_ARG(capturing == hipStreamCaptureStatusNone,
+                        "lm_head_argmax_static: the first call on a device looks up the address of the built-in scratch and cannot be "
+                        "part of a stream capture; make one call outside the capture first");
         void* ptr = nullptr;
         CPMCU_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
         g_scratch_ptr[dev] = ptr;
@@ -1071,7 +1078,7 @@ extern "C" int cpmcu_lm_head_argmax_static(const void* hidden, const void* w, in
                     "lm_head_argmax_static: the built-in scratch of %zu bytes is too small for %d workgroups", kStaticHeadScratchBytes,
                     head_max_grid());
     float* part = nullptr;
-    int rc = static_head_scratch(&part);
+    int rc = static_head_scratch(&part, (hipStream_t)stream);
     if (rc != CPMCU_OK) return rc;
     // NULL selects HIP's null stream here: the library's own stream is created on first use, and this entry
     // point creates nothing

@@ -109,7 +109,9 @@ struct Model {
         hipGraph_t graph = nullptr;
         hipGraphExec_t exec = nullptr;
         uint64_t signature = 0;
+        unsigned long long last_use = 0;
     };
+    unsigned long long graph_clock = 0;
     std::map<std::pair<int, int>, std::vector<StepGraph>> step_graphs;
     // sequences of model-level calls captured by the caller (cpmcu_capture_begin / _end)
     std::vector<StepGraph> user_graphs;
@@ -117,6 +119,7 @@ struct Model {
 };
 
 Model* g_model = nullptr;
+constexpr int kMaxStepGraphs = 16;  // captured verify steps kept at a time (least recently used goes first)
 
 int require_model(bool need_storage) {
     if (!g_model || !g_model->base) {
@@ -458,6 +461,7 @@ extern "C" int cpmcu_set_block_table(const int32_t* host_table, int n) {
     int rc = require_model(true);
     if (rc) return rc;
     Model& m = *g_model;
+    CPMCU_CHECK_ARG(!m.capturing, "set_block_table copies synchronously: it cannot be part of a capture");
     CPMCU_CHECK_ARG(host_table && n >= 1 && n <= m.num_pages, "set_block_table: n=%d outside [1, %d]", n, m.num_pages);
     std::vector<char> seen(m.num_pages, 0);
     for (int i = 0; i < n; ++i) {
@@ -752,6 +756,9 @@ uint64_t step_signature(const Model& m, const StepArgs& a) {
     for (uint64_t v : {a.hidden, a.draft_ids, a.position_ids, a.cache_length, a.kv_length, a.attn_mask, a.tree_parent, a.block_table,
                        a.gt_out, a.accepted_ids, a.prev_hidden, a.next_position_ids, a.result, (uint64_t)a.flags})
         mix(v);
+    // the options decide which kernels a capture records: a graph captured under other settings is another graph
+    const Options& o = options();
+    for (int v : {o.attn_kv_groups, o.head_share_last_pass, o.head_stream_kernel, o.attn_merge_in_launch, o.attn_merge_wait_us}) mix((uint64_t)(uint32_t)v);
     return h;
 }
 
@@ -781,6 +788,7 @@ extern "C" int cpmcu_verify_step(int num_layers, int num_tokens, int padded_leng
     CPMCU_CHECK_ARG(hidden && draft_ids && position_ids && cache_length && kv_length && attn_mask && tree_parent && accepted_ids,
                     "verify_step: null pointer argument");
     CPMCU_CHECK_ARG((flags & ~CPMCU_COMMIT_ADVANCE_LENGTH) == 0, "verify_step: unknown flags 0x%x", flags);
+    CPMCU_CHECK_ARG(prev_hidden == 0 || prev_hidden != hidden, "verify_step: prev_hidden must not alias hidden (rows are gathered by many workgroups)");
     const StepArgs a{num_tokens, padded_length, q, k_new, v_new, attn_out, hidden, draft_ids, position_ids, cache_length, kv_length,
                      attn_mask, tree_parent, block_table, gt_out, accepted_ids, prev_hidden, next_position_ids, result, flags};
     hipStream_t st = resolve_stream(nullptr);
@@ -793,14 +801,39 @@ extern "C" int cpmcu_verify_step(int num_layers, int num_tokens, int padded_leng
     // -- and per set of addresses, which a graph bakes in -- and replayed afterwards.  Every length the kernels
     // need is read from device memory, so the same graph serves every step of that padded length.
     const uint64_t sig = step_signature(m, a);
-    auto& bucket = m.step_graphs[{padded_length, num_tokens}];
-    for (auto& g : bucket)
-        if (g.signature == sig) {
-            CPMCU_HIP(hipGraphLaunch(g.exec, st));
-            return CPMCU_OK;
-        }
+    {
+        auto& bucket = m.step_graphs[{padded_length, num_tokens}];
+        for (auto& g : bucket)
+            if (g.signature == sig) {
+                g.last_use = ++m.graph_clock;
+                CPMCU_HIP(hipGraphLaunch(g.exec, st));
+                return CPMCU_OK;
+            }
+    }
+    // A new graph.  The library keeps at most kMaxStepGraphs of them (the reference keeps one and drops it when the key
+    // changes, src/entry.cu:476-484; a caller that rotates over a few sets of buffers or page tables needs a few): the one
+    // unused the longest goes first, once the stream has drained -- it may still be running.
+    size_t held = 0;
+    for (auto& kv : m.step_graphs) held += kv.second.size();
+    while (held >= (size_t)kMaxStepGraphs) {
+        std::map<std::pair<int, int>, std::vector<Model::StepGraph>>::iterator ob = m.step_graphs.end();
+        size_t oi = 0;
+        for (auto it = m.step_graphs.begin(); it != m.step_graphs.end(); ++it)
+            for (size_t i = 0; i < it->second.size(); ++i)
+                if (ob == m.step_graphs.end() || it->second[i].last_use < ob->second[oi].last_use) {
+                    ob = it;
+                    oi = i;
+                }
+        CPMCU_HIP(hipStreamSynchronize(st));
+        if (ob->second[oi].exec) (void)hipGraphExecDestroy(ob->second[oi].exec);
+        if (ob->second[oi].graph) (void)hipGraphDestroy(ob->second[oi].graph);
+        ob->second.erase(ob->second.begin() + oi);
+        if (ob->second.empty()) m.step_graphs.erase(ob);
+        --held;
+    }
     Model::StepGraph g;
     g.signature = sig;
+    g.last_use = ++m.graph_clock;
     CPMCU_HIP(hipStreamBeginCapture(st, hipStreamCaptureModeRelaxed));
     rc = enqueue_verify_step(m, a, st);
     const hipError_t e = hipStreamEndCapture(st, &g.graph);
@@ -812,8 +845,15 @@ extern "C" int cpmcu_verify_step(int num_layers, int num_tokens, int padded_leng
         set_error("verify_step: stream capture failed: %s", hipGetErrorString(e));
         return CPMCU_ERR_HIP;
     }
-    CPMCU_HIP(hipGraphInstantiate(&g.exec, g.graph, nullptr, nullptr, 0));
-    bucket.push_back(g);
+    {
+        const hipError_t ei = hipGraphInstantiate(&g.exec, g.graph, nullptr, nullptr, 0);
+        if (ei != hipSuccess) {
+            (void)hipGraphDestroy(g.graph);
+            set_error("verify_step: hipGraphInstantiate failed: %s", hipGetErrorString(ei));
+            return CPMCU_ERR_HIP;
+        }
+    }
+    m.step_graphs[{padded_length, num_tokens}].push_back(g);
     CPMCU_HIP(hipGraphLaunch(g.exec, st));
     return CPMCU_OK;
 }
@@ -844,17 +884,54 @@ extern "C" int cpmcu_capture_end(int* graph_id) {
         set_error("capture_end: stream capture failed: %s", hipGetErrorString(e));
         return CPMCU_ERR_HIP;
     }
-    CPMCU_HIP(hipGraphInstantiate(&g.exec, g.graph, nullptr, nullptr, 0));
+    {
+        const hipError_t ei = hipGraphInstantiate(&g.exec, g.graph, nullptr, nullptr, 0);
+        if (ei != hipSuccess) {
+            (void)hipGraphDestroy(g.graph);
+            set_error("capture_end: hipGraphInstantiate failed: %s", hipGetErrorString(ei));
+            return CPMCU_ERR_HIP;
+        }
+    }
+    // a slot freed by cpmcu_graph_destroy is taken again
+    for (size_t i = 0; i < m.user_graphs.size(); ++i)
+        if (m.user_graphs[i].exec == nullptr) {
+            m.user_graphs[i] = g;
+            *graph_id = (int)i;
+            return CPMCU_OK;
+        }
     m.user_graphs.push_back(g);
     *graph_id = (int)m.user_graphs.size() - 1;
     return CPMCU_OK;
+}
+
+extern "C" int cpmcu_graph_destroy(int graph_id) {
+    int rc = require_model(true);
+    if (rc) return rc;
+    Model& m = *g_model;
+    CPMCU_CHECK_ARG(graph_id >= 0 && graph_id < (int)m.user_graphs.size() && m.user_graphs[graph_id].exec != nullptr,
+                    "graph_destroy: unknown graph %d", graph_id);
+    CPMCU_CHECK_ARG(!m.capturing, "graph_destroy: a capture is open");
+    CPMCU_HIP(hipStreamSynchronize(resolve_stream(nullptr)));  // it may still be running
+    (void)hipGraphExecDestroy(m.user_graphs[graph_id].exec);
+    (void)hipGraphDestroy(m.user_graphs[graph_id].graph);
+    m.user_graphs[graph_id] = Model::StepGraph{};
+    return CPMCU_OK;
+}
+
+// Extension for tests and diagnostics: captured verify steps the library holds at the moment.
+extern "C" int cpmcu_step_graph_count(void) {
+    if (!g_model) return 0;
+    int n = 0;
+    for (auto& kv : g_model->step_graphs) n += (int)kv.second.size();
+    return n;
 }
 
 extern "C" int cpmcu_graph_replay(int graph_id) {
     int rc = require_model(true);
     if (rc) return rc;
     Model& m = *g_model;
-    CPMCU_CHECK_ARG(graph_id >= 0 && graph_id < (int)m.user_graphs.size(), "graph_replay: unknown graph %d", graph_id);
+    CPMCU_CHECK_ARG(graph_id >= 0 && graph_id < (int)m.user_graphs.size() && m.user_graphs[graph_id].exec != nullptr,
+                    "graph_replay: unknown graph %d", graph_id);
     CPMCU_CHECK_ARG(!m.capturing, "graph_replay: a capture is open");
     CPMCU_HIP(hipGraphLaunch(m.user_graphs[graph_id].exec, resolve_stream(nullptr)));
     return CPMCU_OK;

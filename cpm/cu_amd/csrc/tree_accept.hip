@@ -480,6 +480,7 @@ extern "C" int cpmcu_accept_commit(void* const* k_pools, void* const* v_pools, i
     CPMCU_CHECK_ARG(num_layers >= 1 && Hkv >= 1, "accept_commit: num_layers=%d Hkv=%d", num_layers, Hkv);
     CPMCU_CHECK_ARG(max_accept >= 1 && max_accept <= kMaxTree, "accept_commit: max_accept=%d outside [1, %d]", max_accept, kMaxTree);
     CPMCU_CHECK_ARG((hidden == nullptr) == (prev_hidden == nullptr), "accept_commit: hidden and prev_hidden go together");
+    CPMCU_CHECK_ARG(hidden == nullptr || hidden != prev_hidden, "accept_commit: prev_hidden must not alias hidden");
     CPMCU_CHECK_ARG(!hidden || (hidden_dim >= 8 && hidden_dim % 8 == 0), "accept_commit: hidden_dim=%d must be a positive multiple of 8", hidden_dim);
     CPMCU_CHECK_ARG((flags & ~(CPMCU_COMMIT_ADVANCE_LENGTH | CPMCU_COMMIT_NEXT_ROOT)) == 0, "accept_commit: unknown flags 0x%x", flags);
     CompactParams p{k_pools, v_pools, block_table, Hkv, pred, cache_length, best, max_accept, num_layers * 2 * Hkv,
@@ -511,6 +512,7 @@ extern "C" int cpmcu_verify_tail(void* const* k_pools, void* const* v_pools, int
                         "verify_tail: %d partials of stride %d do not describe a head launch on %d rows", num_partials, partial_stride, T);
     }
     CPMCU_CHECK_ARG((hidden == nullptr) == (prev_hidden == nullptr), "verify_tail: hidden and prev_hidden go together");
+    CPMCU_CHECK_ARG(hidden == nullptr || hidden != prev_hidden, "verify_tail: prev_hidden must not alias hidden");
     CPMCU_CHECK_ARG(!hidden || (hidden_dim >= 8 && hidden_dim % 8 == 0), "verify_tail: hidden_dim=%d must be a positive multiple of 8", hidden_dim);
     TailParams p;
     p.T = T;

@@ -1227,6 +1227,10 @@ static int tree_attention_impl(const void* q, void* k_pool, void* v_pool,
                     "tree_attention: num_splits_override=%d outside [0, %d]", num_splits_override, kMaxSplits);
     CPMCU_CHECK_ARG(block_window_size == 0 || block_window_size >= 128,
                     "tree_attention: block_window_size=%d must be 0 (no window) or at least one block of 128", block_window_size);
+    // The reference derives the window's first block per 64-row query block (src/flash_attn/src/flash_blockmask.h:16,32:
+    // q_block_idx = m_block + cache length) and never runs a window with more than 64 rows; one start for all rows is
+    // what this kernel has, which is the same thing up to 64 rows.
+    CPMCU_CHECK_ARG(block_window_size == 0 || T <= 64, "tree_attention: a block window with T=%d rows is not supported (at most 64)", T);
     const int group = Hq / Hkv;
     AttnParams p;
     p.q = (const f16*)q;

@@ -36,6 +36,8 @@ SIGNATURES = {
     "cpmcu_capture_begin": (c_int, []),
     "cpmcu_capture_end": (c_int, [ctypes.POINTER(c_int)]),
     "cpmcu_graph_replay": (c_int, [c_int]),
+    "cpmcu_graph_destroy": (c_int, [c_int]),
+    "cpmcu_step_graph_count": (c_int, []),
     "cpmcu_print_perf_summary": (c_int, []),
     "cpmcu_decode_attention": (c_int, [c_int, c_int, c_int, c_u64, c_u64, c_u64, c_u64, c_u64, c_u64]),
     "cpmcu_draft_attention": (c_int, [c_int, c_int, c_int, c_u64, c_u64, c_u64, c_u64, c_u64, c_int, c_u64]),

@@ -174,6 +174,12 @@ int cpmcu_verify_step(int num_layers, int num_tokens, int padded_length, const u
 int cpmcu_capture_begin(void);
 int cpmcu_capture_end(int* graph_id);
 int cpmcu_graph_replay(int graph_id);
+/* Frees a graph made by cpmcu_capture_end (its id may be handed out again); waits for the library's stream first. */
+int cpmcu_graph_destroy(int graph_id);
+/* No reference counterpart: how many captured verify steps (cpmcu_verify_step with cuda_graph = 1) the library holds.
+ * It keeps at most 16 -- one per (padded_length, num_tokens), set of buffer addresses and option settings met -- and
+ * drops the one unused the longest when another is needed (the reference keeps one, src/entry.cu:476-484). */
+int cpmcu_step_graph_count(void);
 
 /* src/entry.cu:506-508 print_perf_summary: prints the per-operator event timings
  * collected when CPMCU_PERF=1 is set in the environment. */

@@ -253,7 +253,7 @@ def test_draft_layer_block_window(gpu, orc, k, d, P0, window, splits, seed):
         assert np.abs(ref.astype(np.float32) - full.astype(np.float32)).max() > 1e-3
 
 
-@pytest.mark.parametrize("P,T,window,rope", [(4096, 60, 1024, False), (4097, 60, 1024, True), (700, 128, 256, True), (33000, 60, 2048, False)])
+@pytest.mark.parametrize("P,T,window,rope", [(4096, 60, 1024, False), (4097, 60, 1024, True), (700, 64, 256, True), (33000, 60, 2048, False)])
 def test_tree_block_window_with_rope(gpu, orc, P, T, window, rope):
     """The window together with a verify-sized tree, the fused append and (optionally) the fused rotary
     embedding: the cost-relevant part is that the stream starts at the window's first block."""
@@ -294,6 +294,11 @@ def test_block_window_argument_checks(gpu):
     for bad in (64, 127, -128):
         with pytest.raises(Exception):
             ops.tree_attention(q, cache, 0, kv_len, 100, None, block_window_size=bad)
+    # more than 64 rows: the reference would start the window per 64-row query block; rejected, not approximated
+    q100 = torch.zeros((100, HQ, D), dtype=torch.float16, device="cuda")
+    kv_len.fill_(300)
+    with pytest.raises(ValueError, match="at most 64"):
+        ops.tree_attention(q100, cache, 0, kv_len, 300, None, block_window_size=128)
 
 
 @pytest.mark.parametrize("T,num_iter,topk", [(60, 6, 10), (128, 8, 16)])

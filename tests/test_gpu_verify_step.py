@@ -266,6 +266,66 @@ def test_library_graph_replays_equal_eager_steps(gpu, orc):
         assert np.array_equal(k1.view(np.uint16), k2.view(np.uint16)) and np.array_equal(v1.view(np.uint16), v2.view(np.uint16))
 
 
+def test_step_graph_cache_is_bounded(gpu, orc):
+    """A caller whose buffers are not static makes cpmcu_verify_step capture a graph per set of addresses: the library keeps
+    the 16 used most recently and frees the rest.  40 sets of addresses, revisited in a different order, give the results of
+    the eager step every time; cpmcu_graph_destroy frees a caller-made graph and its id is handed out again."""
+    from cpm.cu_amd.model import PathModel
+    torch = gpu
+    V, H, LAYERS, T, P = 3000, 512, 1, 12, 300
+    tree = synth.random_tree(T, 5, max_children=3, max_depth=4)
+    w = synth.normal_f16((V, H), 8, 2, std=0.02)
+    m = PathModel(V, LAYERS, H, HQ, HKV, memory_limit=0.005, tree_size=T, num_iter=4, topk=3)
+    try:
+        m.load_head(w)
+        cache = m.cache()
+        cache.write_logical(0, 0, to_dev(torch, synth.normal_f16((P, HKV, D), 8, 10)), to_dev(torch, synth.normal_f16((P, HKV, D), 8, 50)))
+        f16 = dict(dtype=torch.float16, device="cuda")
+        q, kn, vn = [to_dev(torch, synth.normal_f16((T, HQ, D), 8, 3))], [to_dev(torch, synth.normal_f16((T, HKV, D), 8, 4))], \
+            [to_dev(torch, synth.normal_f16((T, HKV, D), 8, 5))]
+        out = [torch.zeros((T, HQ, D), **f16)]
+        hiddens = [to_dev(torch, synth.normal_f16((T, H), 8, 100 + i)) for i in range(40)]
+        draft = torch.zeros(T, dtype=torch.int32, device="cuda")
+        pos, mask, parent = to_dev(torch, tree.positions(P)), to_dev(torch, tree.mask), to_dev(torch, tree.parent)
+        clen = torch.tensor([P], dtype=torch.int32, device="cuda")
+        kvlen = torch.tensor([P + T], dtype=torch.int32, device="cuda")
+        ids = torch.zeros(T, dtype=torch.int32, device="cuda")
+        gt = torch.zeros(T, dtype=torch.int32, device="cuda")
+        result = torch.zeros(1 + T, dtype=torch.int32).pin_memory()
+        padded = (P + T + 127) // 128 * 128
+
+        def step(i, graph):
+            m.verify_step(T, padded, q, kn, vn, out, hiddens[i], draft, pos, clen, kvlen, mask, parent, ids, gt_out=gt, result=result,
+                          cuda_graph=graph)
+            m.synchronize()
+            return int(result[0]), result[1:1 + int(result[0])].numpy().copy(), to_np(gt).copy()
+        count = m.L.raw.cpmcu_step_graph_count
+        ref = [step(i, False) for i in range(40)]
+        assert count() == 0
+        for order in (range(40), reversed(range(40)), [3, 3, 17, 3, 39, 0]):
+            for i in order:
+                a, acc, g = step(i, True)
+                assert a == ref[i][0] and np.array_equal(acc, ref[i][1]) and np.array_equal(g, ref[i][2]), i
+                assert 1 <= count() <= 16
+        assert count() == 16
+        # caller-made graphs: destroy frees the slot, the id comes back
+        g0 = m.capture(lambda: m.L.decode_lm_head(T, hiddens[0].data_ptr(), 0, gt.data_ptr()))
+        g1 = m.capture(lambda: m.L.decode_lm_head(T, hiddens[1].data_ptr(), 0, gt.data_ptr()))
+        m.replay(g0)
+        m.synchronize()
+        assert np.array_equal(to_np(gt), ref[0][2])
+        m.L.graph_destroy(g0)
+        with pytest.raises(ValueError, match="unknown graph"):
+            m.replay(g0)
+        g2 = m.capture(lambda: m.L.decode_lm_head(T, hiddens[2].data_ptr(), 0, gt.data_ptr()))
+        assert g2 == g0 and g1 != g0
+        m.replay(g2)
+        m.synchronize()
+        assert np.array_equal(to_np(gt), ref[2][2])
+    finally:
+        m.close()
+
+
 def test_model_level_draft_rounds(gpu, orc):
     """cpmcu_draft_round / cpmcu_draft_finish (the drafter's state owned by the library, driven through the pybind module)
     against (1) the operator-level chain on an independently built sub-matrix, bit for bit, and (2) the oracle's tree

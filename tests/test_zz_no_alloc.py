@@ -56,6 +56,33 @@ def test_static_scratch_head_matches_workspace_head(gpu, orc):
         assert np.array_equal(z_st.view(np.uint16), z_ws.view(np.uint16))
         # and the shared result is the oracle's arg-max of the device logits (lowest index on ties)
         assert np.array_equal(gt_st, orc.argmax(z_st))
+    # what the entry point is for: it takes no device memory, and it can be part of a stream capture (its first call on the
+    # device, above, was outside one)
+    n, V, H = 60, 40000, 1024
+    hid = to_dev(torch, synth.normal_f16((n, H), 1, 1))
+    tw = ops.tile_head_weight(to_dev(torch, synth.normal_f16((V, H), 1, 2, std=0.02)))
+    gt = torch.full((n,), -7, dtype=torch.int32, device="cuda")
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    call = lambda: L.lm_head_argmax_static(p(hid), p(tw.data), ops.W_TILED, n, V, H, 1, ctypes.c_float(0.5), None, p(gt),
+                                           ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    torch.cuda.synchronize()
+    free0 = torch.cuda.mem_get_info()[0]
+    call()
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0, "the call took device memory"
+    ref = to_np(gt).copy()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            call()
+    for rep in range(3):
+        gt.fill_(-7)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(to_np(gt), ref), rep
     # more rows than the built-in scratch holds: a clear error, nothing launched
     with pytest.raises(ValueError, match="outside \\[1, 128\\]"):
         q = ctypes.c_void_p(16)
