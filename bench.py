@@ -57,7 +57,7 @@ def parse_args():
     ap.add_argument("--no-contexts", action="store_true", help="skip the 32K / 128K context step timings")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true", help="enqueue the step's launches eagerly instead of replaying the library's HIP graph")
-    ap.add_argument("--no-probes", action="store_true", help="skip the MFMA-rate probe of the machine")
+    ap.add_argument("--no-probes", action="store_true", help="skip the MFMA-rate probe of the machine and the power probe of the attention launch")
     ap.add_argument("--no-operators", action="store_true", help="skip the per-operator timings (heads, tail, draft path)")
     ap.add_argument("--accept-depth", type=int, default=3, help="draft tokens the rigged tree gets accepted")
     ap.add_argument("--traffic-probe", action="store_true",
@@ -271,6 +271,95 @@ def machine_probes(torch):
             best = max(best, flops / (e0.elapsed_time(e1) * 1e-3) / 1e12)
         out["mfma_tflops_" + name] = round(best, 1)
     out["note"] = "v_mfma_f32_32x32x16_f16 from registers, 256 workgroups x 8 waves, nothing else in the loop"
+    return out
+
+
+def power_probe(torch, np, synth, seconds=0.6):
+    """The tree-attention launch at 32K and 128K context on all-zero and on random Q/K/V, with the board power read
+    from the driver's hwmon file (every 20 ms) while the launches run: the time of the same launch depends on the
+    data, and the board's power limit is why.  Four layers' pools per context, replayed as one graph."""
+    import glob
+    import threading
+    from cpm.cu_amd import ops
+    from cpm.cu_amd.kvcache import PagedKVCache
+    files = []
+    for h in sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*")):
+        for f in ("power1_average", "power1_input"):
+            if os.path.exists(os.path.join(h, f)):
+                files.append(os.path.join(h, f))
+    cap = None
+    for h in sorted(glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*")):
+        if os.path.exists(os.path.join(h, "power1_cap")):
+            try:
+                cap = int(open(os.path.join(h, "power1_cap")).read()) / 1e6
+            except (OSError, ValueError):
+                pass
+            break
+    shp = synth.MINICPM4_8B
+    T, Hq, Hkv, D, L = 60, shp["q_heads"], shp["kv_heads"], shp["head_dim"], 4
+    tree = synth.eagle_tree(6, 10, T, 0)
+    mask = torch.from_numpy(tree.mask.view(np.int64)).cuda()
+    out = {"power_file": files[0] if files else None, "power_cap_w": cap, "layers_per_graph": L, "contexts": {}}
+    for P in (32768, 131072):
+        S = P + T
+        cache = PagedKVCache(L, Hkv, (S + 255) // 256 + 1)
+        kv_len = torch.tensor([S], dtype=torch.int32, device="cuda")
+        padded = (S + 127) // 128 * 128
+        row = {}
+        for mode in ("zeros", "random"):
+            for l in range(L):
+                if mode == "zeros":
+                    cache.k[l].zero_()
+                    cache.v[l].zero_()
+                else:
+                    cache.k[l].normal_()
+                    cache.v[l].normal_()
+            q = torch.zeros(T, Hq, D, device="cuda").half() if mode == "zeros" else torch.randn(T, Hq, D, device="cuda").half()
+            o = torch.empty_like(q)
+            call = lambda l: ops.tree_attention(q, cache, l, kv_len, padded, mask, out=o)
+            call(0)
+            torch.cuda.synchronize()
+            st = torch.cuda.Stream()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.stream(st):
+                with torch.cuda.graph(g, stream=st):
+                    for l in range(L):
+                        call(l)
+            samples, stop = [], [False]
+
+            def sampler():
+                while not stop[0]:
+                    if files:
+                        try:
+                            samples.append(int(open(files[0]).read()) / 1e6)
+                        except (OSError, ValueError):
+                            pass
+                    time.sleep(0.02)
+            th = threading.Thread(target=sampler)
+            th.start()
+            n = max(20, int(seconds * 1e6 / (150.0 * L * P / 131072 + 15 * L)))
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            with torch.cuda.stream(st):
+                for _ in range(n // 4):
+                    g.replay()
+                e0.record(st)
+                for _ in range(n):
+                    g.replay()
+                e1.record(st)
+            torch.cuda.synchronize()
+            stop[0] = True
+            th.join()
+            us = e0.elapsed_time(e1) * 1e3 / (n * L)
+            tail = sorted(samples[len(samples) // 2:]) if samples else []
+            row[mode] = {"us_per_layer": round(us, 2), "tflops": round(4.0 * Hq * T * D * S / us / 1e6, 1),
+                         "board_power_w_median": round(tail[len(tail) // 2], 0) if tail else None,
+                         "board_power_w_max": round(max(samples), 0) if samples else None, "power_samples": len(samples)}
+            del g
+        out["contexts"][str(P)] = row
+        del cache
+        torch.cuda.empty_cache()
+    out["note"] = ("the same attention launch on all-zero and on random fp16 data; power is the driver's reading over the second half of "
+                   "the run; a zero in every operand draws less, so the clock stays higher")
     return out
 
 
@@ -652,6 +741,7 @@ def main():
 
     # ---- what the matrix pipes sustain on this GPU (last, so that its heat does not touch the figures above) ----
     probes = None if args.no_probes else machine_probes(torch)
+    power = None if args.no_probes else power_probe(torch, np, synth)
     if probes is not None:
         ceiling = probes["mfma_tflops_random_operands"]
         if roofline["bound"] == "mfma":  # the same achieved figure against MFMAs alone on random operands
@@ -680,6 +770,7 @@ def main():
         "us_per_step_one_kv_set": round(main_run["ms_one_set"] * 1e3, 1),
         "roofline": roofline,
         "machine_probes": probes,
+        "power_probe": power,
         "kernels": kernels,
         "traffic_source": MEASURED_TRAFFIC["source"],
         "traffic_measured_at_commit": MEASURED_TRAFFIC["measured_at_commit"],
