@@ -261,6 +261,10 @@ __device__ inline int scalar_load(const int32_t* ptr) {
 __device__ inline void scalar_load2(const int32_t* pa, const int32_t* pb, int& a, int& b) {
     asm volatile("s_load_dword %0, %2, 0x0\n\ts_load_dword %1, %3, 0x0\n\ts_waitcnt lgkmcnt(0)" : "=&s"(a), "=&s"(b) : "s"(pa), "s"(pb) : "memory");
 }
+__device__ inline void scalar_load3(const int32_t* pa, const int32_t* pb, const int32_t* pc, int& a, int& b, int& c) {
+    asm volatile("s_load_dword %0, %3, 0x0\n\ts_load_dword %1, %4, 0x0\n\ts_load_dword %2, %5, 0x0\n\ts_waitcnt lgkmcnt(0)"
+                 : "=&s"(a), "=&s"(b), "=&s"(c) : "s"(pa), "s"(pb), "s"(pc) : "memory");
+}
 
 // Per-thread byte offsets of its pieces inside a K tile and a V^T tile of a page (second piece of each:
 // + 32 keys = 8192 bytes for K, + 64 dims = 64 * 512 bytes for V^T; the swizzle terms do not change).
@@ -382,45 +386,58 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
         }
     };
 
-    // The split's tile range is fixed by the host-side bound, so the page ids can be fetched without
-    // waiting for the device-side length; the length only clips the range.
+    // The split ranges partition the tiles of the stream as the device-side length gives it, so that every split gets its
+    // share of what is really there (a padded host-side bound would leave the last splits short and the others long).
+    // The page id of the split's first tile is still fetched together with the length, not behind it: the exact first
+    // tile can only lie at or below the one the host-side bound gives, almost always on the same page or the one before,
+    // so both table entries are requested with the length; a first tile further away (a bound far above the length)
+    // costs one more scalar load.
     // With the fused append the last split also patches the appended rows into its tiles, which costs
     // about as much as an iteration: the partition counts two tiles' worth of extra work at the end
     // of the stream (three when the appended K rows are also rotated there), so that split gets fewer real tiles.
     // A block sliding window moves the start of the stream to its first visible tile, which depends on
     // the device-side length: such calls (the drafter's own layer, a few tiles in all) pay the extra
-    // round trip in front of the page ids.
-    const int vtiles = p.ntiles_max + (p.k_new != nullptr && p.num_splits > 1 ? (ROPE ? 3 : 2) : 0);
+    // round trip in front of the page ids and keep the partition of the window's bound.
+    const int extra_tiles = p.k_new != nullptr && p.num_splits > 1 ? (ROPE ? 3 : 2) : 0;
     // (32-bit arithmetic: at most 128 splits times at most 2^24 tiles; a 64-bit division is a long scalar routine)
-    const int r0 = min((int)(((uint32_t)split * (uint32_t)vtiles) / (uint32_t)p.num_splits), p.ntiles_max);
-    const int r1 = min((int)(((uint32_t)(split + 1) * (uint32_t)vtiles) / (uint32_t)p.num_splits), p.ntiles_max);
-    // The device-side length and the page id of the split's first tile come through scalar loads, together: the
-    // Q rows requested above are still on their way, and a vector load of these few bytes would return behind them.
+    auto range_begin = [&](int sp, int tiles) { return min((int)(((uint32_t)sp * (uint32_t)(tiles + extra_tiles)) / (uint32_t)p.num_splits), tiles); };
     int S, first_page;
     int tile_lo = 0;
-    if (p.window_blocks > 0) {  // the window's first tile depends on the length: one more round trip for the page id
-        S = scalar_load(p.kv_len);
-        tile_lo = max((S - p.T + 127) / 128 - p.window_blocks, 0) * (128 / kTileN);
-        first_page = scalar_load(p.block_table + min(((tile_lo + r0) * kTileN) / kPage, p.table_pages - 1));
-    } else {
-        scalar_load2(p.kv_len, p.block_table + min((r0 * kTileN) / kPage, p.table_pages - 1), S, first_page);
-    }
-    const int t0 = tile_lo + r0;
-    const int t1_max = tile_lo + r1;
-    const int pg0 = (t0 * kTileN) / kPage;
-    // page of a tile: a scalar load of its table entry (the first one is already here)
-    // (a window's last tile slot can lie past the host bound; it is never consumed, and the table is not read there)
-    auto page_of_tile = [&](int tile) {
-        const int pg = (tile * kTileN) / kPage;
-        return pg == pg0 ? first_page : scalar_load(p.block_table + min(pg, p.table_pages - 1));
-    };
-    {
+    int r0, r1;
+    auto clamp_length = [&]() {
         const int lo = max(p.T, p.mask_k_range);
         if (S > p.max_kv_len || S < lo) {
             if (sh == 0 && mt == 0 && tid == 0) g_attn_report.bad_length = S == 0 ? -1 : S;
             S = min(max(S, lo), p.max_kv_len);
         }
+    };
+    if (p.window_blocks > 0) {  // the window's first tile depends on the length: one more round trip for the page id
+        S = scalar_load(p.kv_len);
+        clamp_length();
+        r0 = range_begin(split, p.ntiles_max);
+        r1 = range_begin(split + 1, p.ntiles_max);
+        tile_lo = max((S - p.T + 127) / 128 - p.window_blocks, 0) * (128 / kTileN);
+        first_page = scalar_load(p.block_table + min(((tile_lo + r0) * kTileN) / kPage, p.table_pages - 1));
+    } else {
+        const int pg_b = min((range_begin(split, p.ntiles_max) * kTileN) / kPage, p.table_pages - 1);
+        int page_b, page_before;
+        scalar_load3(p.kv_len, p.block_table + pg_b, p.block_table + max(pg_b - 1, 0), S, page_b, page_before);
+        clamp_length();
+        const int ntiles_now = (S + kTileN - 1) / kTileN;
+        r0 = range_begin(split, ntiles_now);
+        r1 = range_begin(split + 1, ntiles_now);
+        const int pg = min((r0 * kTileN) / kPage, p.table_pages - 1);
+        first_page = pg == pg_b ? page_b : pg == pg_b - 1 ? page_before : scalar_load(p.block_table + pg);
     }
+    const int t0 = tile_lo + r0;
+    const int t1_max = tile_lo + r1;
+    const int pg0 = min((t0 * kTileN) / kPage, p.table_pages - 1);
+    // page of a tile: a scalar load of its table entry (the first one is already here)
+    // (a window's last tile slot can lie past the host bound; it is never consumed, and the table is not read there)
+    auto page_of_tile = [&](int tile) {
+        const int pg = min((tile * kTileN) / kPage, p.table_pages - 1);
+        return pg == pg0 ? first_page : scalar_load(p.block_table + pg);
+    };
     const int P = S - p.T;              // the T query tokens are the last T keys
     const int Pm = S - p.mask_k_range;  // first key column governed by the mask bits (mask.h: mask_k_begin)
     const int ntiles = (S + kTileN - 1) / kTileN;
