@@ -39,12 +39,14 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 # Counters cannot be read from inside this process, so the figures are carried here as constants, keyed by the kernel
 # names the library reports for the dispatch taken: a different instantiation finds no entry and reports null.
 MEASURED_TRAFFIC = {
-    "source": "profiles/verify_step_hbm_traffic.md",
-    "measured_at_commit": "a4c74a5",  # the library the counters were read on (git rev-parse --short HEAD of that run)
+    "source": "profiles/verify_step_hbm_traffic.md, profiles/tree_attention_long_context_traffic.md",
+    "measured_at_commit": "8907f19",  # the library the counters were read on (git rev-parse --short HEAD of that run)
     "kib_per_launch": {
-        "tree_attn_split_kernel<2,false>": 15154 + 9463,  # the merge of the split partials runs inside the launch
-        "head_gemm_stream_kernel<4,2,256>": 591960 + 128,
+        "tree_attn_split_kernel<2,false>": 15186 + 9463,  # the merge of the split partials runs inside the launch
+        "head_gemm_stream_kernel<4,2,256>": 591857 + 128,
     },
+    # the attention launch at the longer contexts (32 splits of 256-row workgroups), by prefix length
+    "attention_kib_per_launch_by_context": {"32768": 52479 + 17894, "131072": 150801 + 17894},
 }
 
 
@@ -726,6 +728,10 @@ def main():
         tf = flops_attn(Pc) / (r["ms_attn"] * 1e-3) / 1e12
         ctx_attn[str(Pc)] = dict(us_per_layer=round(r["ms_attn"] * 1e3, 2), tflops=round(tf, 1), frac_mfma=round(tf / MFMA_F16_PEAK_TFLOPS, 4),
                                  kernel=r["attn_plan"][0], step_minus_attention_us=round((r["ms_step"] - L * r["ms_attn"]) * 1e3, 1))
+        kib = MEASURED_TRAFFIC["attention_kib_per_launch_by_context"].get(str(Pc))
+        if kib is not None and r["attn_plan"][0] == "tree_attn_split_kernel<1,false>":
+            ctx_attn[str(Pc)]["traffic"] = kib * 1024
+            ctx_attn[str(Pc)]["algorithmic_bytes"] = int(bytes_attn(Pc))
         if parity is not None:  # acceptance on the device's arg-max + compacted rows, as for the headline context
             parity.setdefault("contexts", {})[str(Pc)] = context_parity(np, oracle_mod, r, bufs, tree)
         if cpu is not None:
