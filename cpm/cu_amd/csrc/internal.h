@@ -7,6 +7,8 @@ namespace cpmcu {
 // runtime.hip -- kernel-shape switches, read from the environment once when the library is first used
 // (CPMCU_ATTN_KV_GROUPS=1|2, CPMCU_HEAD_NO_SHARE) and changed afterwards through cpmcu_set_option.
 struct Options {
+    int dtype = 0;                 // element type of the 16-bit tensors handed to the operator-level entry points: 0 = fp16,
+                                   // 1 = bf16 (process-wide, like the reference's model; cpmcu_init_base_model sets it)
     int attn_kv_groups = 0;        // 0 = chosen per call; 1 / 2 force that tree-attention kernel shape
     int head_share_last_pass = 1;  // 0 keeps the plain row-block mapping of the head GEMM
     int head_stream_kernel = 1;    // 0 keeps tiled weights on the K-chunked kernel (tests compare the two)

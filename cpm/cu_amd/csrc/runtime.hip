@@ -199,7 +199,12 @@ extern "C" const char* cpmcu_version(void) { return "cpmcu_amd 0.1 (gfx950)"; }
 extern "C" int cpmcu_set_option(const char* name, int value) {
     CPMCU_CHECK_ARG(name, "set_option: null name");
     const std::string nm(name);
-    if (nm == "attn_kv_groups") {
+    if (nm == "dtype") {
+        // the element type of the 16-bit tensors the operator-level entry points are handed from now on (the model-level
+        // ones follow cpmcu_init_base_model's torch_dtype, which sets the same switch)
+        CPMCU_CHECK_ARG(value == 0 || value == 1, "set_option: dtype=%d must be 0 (fp16) or 1 (bf16)", value);
+        options().dtype = value;
+    } else if (nm == "attn_kv_groups") {
         CPMCU_CHECK_ARG(value >= 0 && value <= 2, "set_option: attn_kv_groups=%d outside [0, 2]", value);
         options().attn_kv_groups = value;
     } else if (nm == "head_stream_kernel") {
@@ -758,7 +763,7 @@ uint64_t step_signature(const Model& m, const StepArgs& a) {
         mix(v);
     // the options decide which kernels a capture records: a graph captured under other settings is another graph
     const Options& o = options();
-    for (int v : {o.attn_kv_groups, o.head_share_last_pass, o.head_stream_kernel, o.attn_merge_in_launch, o.attn_merge_wait_us}) mix((uint64_t)(uint32_t)v);
+    for (int v : {o.dtype, o.attn_kv_groups, o.head_share_last_pass, o.head_stream_kernel, o.attn_merge_in_launch, o.attn_merge_wait_us}) mix((uint64_t)(uint32_t)v);
     return h;
 }
 

@@ -145,8 +145,9 @@ __device__ inline To bits_as(const From& v) {
 // splits are all requested before any is used, so a block pays one memory round trip, not one per split.
 // DEV: the partials were written by other workgroups of this launch (device-scope loads).
 constexpr int kCombineBatch = 16;
-template <bool DEV>
+template <bool DEV, typename E>
 __device__ inline void combine_block(const AttnParams& p, int g, int rb, int quad, int lane) {
+    typedef typename Elem<E>::x4 X4;
     const int nrb = p.rows_pad / kRowsPerWave;  // 32-row blocks per kv head
     const int qcol = lane & 31, hf = lane >> 5;
     const int R = rb * kRowsPerWave + qcol;
@@ -155,7 +156,7 @@ __device__ inline void combine_block(const AttnParams& p, int g, int rb, int qua
     const int head = g * p.group + (p.group_shift >= 0 ? R & (p.group - 1) : R % p.group);
     const int d0 = (quad >> 2) * 32 + (quad & 3) * 8 + hf * 4;
     const float2* ml = reinterpret_cast<const float2*>(p.ml_part) + (size_t)g * p.num_splits * p.rows_pad + R;
-    const f16x4* op = reinterpret_cast<const f16x4*>(p.o_part) +
+    const X4* op = reinterpret_cast<const X4*>(p.o_part) +
                       (((size_t)g * p.num_splits) * nrb + rb) * 16 * 64 + quad * 64 + lane;
     const size_t ml_stride = (size_t)p.rows_pad;
     const size_t o_stride = (size_t)nrb * 16 * 64;
@@ -164,14 +165,14 @@ __device__ inline void combine_block(const AttnParams& p, int g, int rb, int qua
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
     for (int s0 = 0; s0 < p.num_splits; s0 += kCombineBatch) {
         float2 v[kCombineBatch];
-        f16x4 o[kCombineBatch];
+        X4 o[kCombineBatch];
 #pragma unroll
         for (int u = 0; u < kCombineBatch; ++u) {
             const int s = min(s0 + u, p.num_splits - 1);  // clamp: repeats are ignored below
             if (DEV) {
                 const uint64_t mlw = load_dev64(&ml[s * ml_stride]);
                 v[u] = make_float2(__uint_as_float((uint32_t)mlw), __uint_as_float((uint32_t)(mlw >> 32)));
-                o[u] = bits_as<f16x4>(load_dev64(&op[s * o_stride]));
+                o[u] = bits_as<X4>(load_dev64(&op[s * o_stride]));
             } else {
                 v[u] = ml[s * ml_stride];
                 o[u] = op[s * o_stride];
@@ -198,26 +199,28 @@ __device__ inline void combine_block(const AttnParams& p, int g, int rb, int qua
         }
     }
     const float inv = (L == 0.f || L != L) ? 1.f : 1.f / L;
-    f16x4 o;
+    X4 o;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) o[e] = (f16)(acc[e] * inv);
-    *reinterpret_cast<f16x4*>(p.out + ((size_t)node * p.Hq + head) * kHeadDim + d0) = o;
+    for (int e = 0; e < 4; ++e) o[e] = (E)(acc[e] * inv);
+    *reinterpret_cast<X4*>(p.out + ((size_t)node * p.Hq + head) * kHeadDim + d0) = o;
 }
 
 // One rotary pair: (a, b) -> (a cos - b sin, a sin + b cos), every product and sum rounded on its own
 // (no fused multiply-add), so the result does not depend on how a compiler contracts the expression.
-__device__ inline void rotate_pair(f16& a, f16& b, float2 cs) {
+template <typename E>
+__device__ inline void rotate_pair(E& a, E& b, float2 cs) {
 #pragma clang fp contract(off)
     const float fa = (float)a, fb = (float)b;
     const float ac = fa * cs.x, bs = fb * cs.y, as = fa * cs.y, bc = fb * cs.x;
-    a = (f16)(ac - bs);
-    b = (f16)(as + bc);
+    a = (E)(ac - bs);
+    b = (E)(as + bc);
 }
 
-__device__ inline f16x8 zero8() {
-    f16x8 z;
+template <typename E>
+__device__ inline typename Elem<E>::x8 zero8() {
+    typename Elem<E>::x8 z;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) z[i] = (f16)0.f;
+    for (int i = 0; i < 8; ++i) z[i] = (E)0.f;
     return z;
 }
 
@@ -314,8 +317,13 @@ __device__ inline void issue_tile_append(const AttnParams& p, int g, int tile, i
 
 // ROPE: the instantiation that rotates q and the appended K rows (p.rope is set); the plain one carries
 // none of that code, so its registers and schedule are those of a kernel without the feature.
-template <int G, bool ROPE>
-__global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams p) {
+// E: the element type.  The kernels proper are thin wrappers below (`tree_attn_split_kernel<G, ROPE>` for fp16 keeps the name
+// it has in every profile, `tree_attn_split_bf16_kernel<G, ROPE>` for bf16).
+template <int G, bool ROPE, typename E>
+__device__ __forceinline__ void tree_attn_split_body(const AttnParams& p) {
+    typedef typename Elem<E>::x8 X8;
+    typedef typename Elem<E>::x4 X4;
+    typedef typename Elem<E>::x2 X2;
     constexpr int kRowWaves = kWaves / G;
     constexpr int kRowsPerWg = kRowWaves * kRowsPerWave;
     constexpr int kDepth = kStages / G - 1;  // iterations in flight behind the one being consumed
@@ -512,11 +520,11 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
         mw1 = p.mask_words > 1 ? s_mask[node * p.mask_words + 1] : 0ull;
     }
     // Q as the B operand of S^T = K.Q^T: lane (qcol, hf) holds d = 16*ks + 8*hf + [0,8).
-    f16x8 qreg[8];
+    X8 qreg[8];
 #pragma unroll
     for (int ks = 0; ks < 8; ++ks) {
-        const f16x8 v = *reinterpret_cast<const f16x8*>(qstage + k_lds_off(rw * kRowsPerWave + qcol, 2 * ks + hf));
-        qreg[ks] = row_ok ? v : zero8();
+        const X8 v = *reinterpret_cast<const X8*>(qstage + k_lds_off(rw * kRowsPerWave + qcol, 2 * ks + hf));
+        qreg[ks] = row_ok ? v : zero8<E>();
     }
     __syncthreads();  // the stages are free for tiles
 #pragma unroll
@@ -542,7 +550,7 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
         for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                f16 a = qreg[ks][j], b = qreg[ks + 4][j];
+                E a = qreg[ks][j], b = qreg[ks + 4][j];
                 rotate_pair(a, b, cs[ks * 16 + j]);
                 qreg[ks][j] = a;
                 qreg[ks + 4][j] = b;
@@ -602,13 +610,13 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
                         const int key = x >> 3, piece = x & 7;
                         const int c = ce + key;
                         if (c >= P && c < S) {
-                            f16x8* lo = reinterpret_cast<f16x8*>(st + k_lds_off(key, piece));
-                            f16x8* hi = reinterpret_cast<f16x8*>(st + k_lds_off(key, piece + 8));
-                            f16x8 a = *lo, b = *hi;
+                            X8* lo = reinterpret_cast<X8*>(st + k_lds_off(key, piece));
+                            X8* hi = reinterpret_cast<X8*>(st + k_lds_off(key, piece + 8));
+                            X8 a = *lo, b = *hi;
                             const float2* cs = p.rope + (size_t)(c - P) * (kHeadDim / 2) + piece * 8;
 #pragma unroll
                             for (int j = 0; j < 8; ++j) {
-                                f16 ra = a[j], rb = b[j];
+                                E ra = a[j], rb = b[j];
                                 rotate_pair(ra, rb, cs[j]);
                                 a[j] = ra;
                                 b[j] = rb;
@@ -617,8 +625,8 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
                             *hi = b;
                             if (mt == 0) {
                                 f16* row = p.k_pool_w + (((size_t)pg * p.Hkv + g) * kPage + c % kPage) * kHeadDim;
-                                *reinterpret_cast<f16x8*>(row + piece * 8) = a;
-                                *reinterpret_cast<f16x8*>(row + (piece + 8) * 8) = b;
+                                *reinterpret_cast<X8*>(row + piece * 8) = a;
+                                *reinterpret_cast<X8*>(row + (piece + 8) * 8) = b;
                             }
                         }
                     }
@@ -681,12 +689,12 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
             // MFMA: LDS returns in order, so MFMA i only waits for read i. ----
             f32x16 sacc[2];
             {
-                f16x8 kf[16];
+                X8 kf[16];
 #pragma unroll
                 for (int ks = 0; ks < 8; ++ks)
 #pragma unroll
                     for (int kb = 0; kb < 2; ++kb)
-                        kf[ks * 2 + kb] = *reinterpret_cast<const f16x8*>(stage + k_lds_off(kb * 32 + qcol, 2 * ks + hf));
+                        kf[ks * 2 + kb] = *reinterpret_cast<const X8*>(stage + k_lds_off(kb * 32 + qcol, 2 * ks + hf));
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb)
@@ -696,17 +704,17 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
                 for (int ks = 0; ks < 8; ++ks)
 #pragma unroll
                     for (int kb = 0; kb < 2; ++kb)  // two independent accumulation chains, interleaved
-                        sacc[kb] = __builtin_amdgcn_mfma_f32_32x32x16_f16(kf[ks * 2 + kb], qreg[ks], sacc[kb], 0, 0, 0);
+                        sacc[kb] = Elem<E>::mfma_32x32x16(kf[ks * 2 + kb], qreg[ks], sacc[kb]);
                 __builtin_amdgcn_sched_barrier(0);
             }
             // The V^T operands of this tile are requested now, so that they arrive under the softmax
             // arithmetic and the probability MFMAs start without waiting for LDS.
-            f16x8 vf[16];
+            X8 vf[16];
 #pragma unroll
             for (int j = 0; j < 4; ++j)
 #pragma unroll
                 for (int db = 0; db < 4; ++db)
-                    vf[j * 4 + db] = *reinterpret_cast<const f16x8*>(stage + v_lds_off(db * 32 + qcol, 2 * j + hf));
+                    vf[j * 4 + db] = *reinterpret_cast<const X8*>(stage + v_lds_off(db * 32 + qcol, 2 * j + hf));
             __builtin_amdgcn_sched_barrier(0);
             // sacc[kb][r] is the score of key  c0 + kb*32 + 8*(r/4) + 4*hf + r%4  for query qcol.
             if (c0 + kTileN > Pm) {  // tile touches masked columns or the end of the stream
@@ -755,24 +763,24 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
             }
             const float m_scaled = (m_ref == -INFINITY) ? 0.f : m_ref;
             float psum = 0.f;
-            f16x8 pb[4];  // P^T as B operand: k-step j holds keys 16*j + {4hf..4hf+3, 8+4hf..8+4hf+3}
+            X8 pb[4];  // P^T as B operand: k-step j holds keys 16*j + {4hf..4hf+3, 8+4hf..8+4hf+3}
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const float pv = __builtin_amdgcn_exp2f(sacc[kb][r] * p.scale_log2 - m_scaled);
-                    pb[kb * 2 + (r >> 3)][r & 7] = (f16)pv;  // P is rounded to fp16 before P.V
+                    pb[kb * 2 + (r >> 3)][r & 7] = (E)pv;  // P is rounded to the element type before P.V
                 }
             // Row sum of the rounded probabilities, two per instruction (fp32 accumulation): the
             // denominator then weighs exactly the values the numerator's MFMA sees.
             {
-                const f16x2 ones = {(f16)1.f, (f16)1.f};
+                const X2 ones = {(E)1.f, (E)1.f};
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        const f16x2 pp = {pb[j][2 * e], pb[j][2 * e + 1]};
-                        psum = __builtin_amdgcn_fdot2(pp, ones, psum, false);
+                        const X2 pp = {pb[j][2 * e], pb[j][2 * e + 1]};
+                        psum = Elem<E>::dot2_acc(pp, ones, psum);
                     }
             }
             l_run += psum;
@@ -784,7 +792,7 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
                 for (int j = 0; j < 4; ++j)
 #pragma unroll
                     for (int db = 0; db < 4; ++db)  // four independent accumulation chains, interleaved
-                        oacc[db] = __builtin_amdgcn_mfma_f32_32x32x16_f16(vf[j * 4 + db], pb[j], oacc[db], 0, 0, 0);
+                        oacc[db] = Elem<E>::mfma_32x32x16(vf[j * 4 + db], pb[j], oacc[db]);
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
@@ -861,10 +869,10 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
         const float inv = (l_tot == 0.f || l_tot != l_tot) ? 1.f : 1.f / l_tot;
         f16* orow = p.out + ((size_t)node * p.Hq + head) * kHeadDim;
         for_my_blocks([&](int db, int rq, const f32x16& acc) {
-            f16x4 o;
+            X4 o;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) o[e] = (f16)(acc[rq * 4 + e] * inv);
-            *reinterpret_cast<f16x4*>(orow + db * 32 + rq * 8 + hf * 4) = o;
+            for (int e = 0; e < 4; ++e) o[e] = (E)(acc[rq * 4 + e] * inv);
+            *reinterpret_cast<X4*>(orow + db * 32 + rq * 8 + hf * 4) = o;
         });
     } else {
         const size_t prow = ((size_t)g * p.num_splits + split) * p.rows_pad + R;
@@ -872,12 +880,12 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
         // final output -- which halves the dominant extra HBM traffic of the split design; (max, l)
         // stay fp32.  The reference keeps fp32 partials; the difference is far inside the tolerance.
         const float inv = (l_tot == 0.f || l_tot != l_tot) ? 0.f : 1.f / l_tot;
-        f16x4* op = reinterpret_cast<f16x4*>(p.o_part) +
+        X4* op = reinterpret_cast<X4*>(p.o_part) +
                     ((((size_t)g * p.num_splits + split) * p.num_mtiles + mt) * kRowWaves + rw) * 16 * 64 + lane;
         for_my_blocks([&](int db, int rq, const f32x16& acc) {
-            f16x4 o;
+            X4 o;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) o[e] = (f16)(acc[rq * 4 + e] * inv);
+            for (int e = 0; e < 4; ++e) o[e] = (E)(acc[rq * 4 + e] * inv);
             if (unit_ctr != nullptr) store_dev64(&op[(db * 4 + rq) * 64], bits_as<uint64_t>(o));
             else __builtin_nontemporal_store(o, &op[(db * 4 + rq) * 64]);  // streamed: nothing left to flush at kernel end
         });
@@ -951,7 +959,7 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
         const int nblocks = kRowWaves * 16;
         auto merge_share = [&](int share) {
             for (int b = share + p.num_splits * wave; b < nblocks; b += p.num_splits * kWaves)
-                combine_block<true>(p, g, mt * kRowWaves + (b >> 4), b & 15, lane);
+                combine_block<true, E>(p, g, mt * kRowWaves + (b >> 4), b & 15, lane);
         };
         merge_share(split);
         if (last) {
@@ -963,15 +971,27 @@ __global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams
 }
 
 // The merge as a launch of its own: one wave per (kv head, 32-row block, quad), in the partial layout's own order.
-__global__ __launch_bounds__(256) void tree_attn_combine_kernel(AttnParams p) {
+template <int G, bool ROPE>
+__global__ __launch_bounds__(kThreads, 1) void tree_attn_split_kernel(AttnParams p) {
+    tree_attn_split_body<G, ROPE, f16>(p);
+}
+template <int G, bool ROPE>
+__global__ __launch_bounds__(kThreads, 1) void tree_attn_split_bf16_kernel(AttnParams p) {
+    tree_attn_split_body<G, ROPE, bf16>(p);
+}
+
+template <typename E>
+__device__ __forceinline__ void tree_attn_combine_body(const AttnParams& p) {
     const int idx = blockIdx.x * 256 + threadIdx.x;
     const int lane = idx & 63;
     const int quad = (idx >> 6) & 15;
     const int nrb = p.rows_pad / kRowsPerWave;  // 32-row blocks per kv head (16 * 64 = 1024 threads each)
     const int grb = idx >> 10;
     if (grb >= p.Hkv * nrb) return;
-    combine_block<false>(p, grb / nrb, grb % nrb, quad, lane);
+    combine_block<false, E>(p, grb / nrb, grb % nrb, quad, lane);
 }
+__global__ __launch_bounds__(256) void tree_attn_combine_kernel(AttnParams p) { tree_attn_combine_body<f16>(p); }
+__global__ __launch_bounds__(256) void tree_attn_combine_bf16_kernel(AttnParams p) { tree_attn_combine_body<bf16>(p); }
 
 int device_cu_count() {
     static int cus[64] = {0};
@@ -1305,7 +1325,16 @@ static int tree_attention_impl(const void* q, void* k_pool, void* v_pool,
     }
     const int nsh = p.num_splits * Hkv;
     const dim3 grid(kXcds * ceil_div(nsh, kXcds), p.num_mtiles);
-    if (p.rope != nullptr) {
+    const bool is_bf16 = options().dtype == 1;
+    if (is_bf16) {
+        if (p.rope != nullptr) {
+            if (G == 1) hipLaunchKernelGGL((tree_attn_split_bf16_kernel<1, true>), grid, dim3(kThreads), 0, st, p);
+            else hipLaunchKernelGGL((tree_attn_split_bf16_kernel<2, true>), grid, dim3(kThreads), 0, st, p);
+        } else {
+            if (G == 1) hipLaunchKernelGGL((tree_attn_split_bf16_kernel<1, false>), grid, dim3(kThreads), 0, st, p);
+            else hipLaunchKernelGGL((tree_attn_split_bf16_kernel<2, false>), grid, dim3(kThreads), 0, st, p);
+        }
+    } else if (p.rope != nullptr) {
         if (G == 1) hipLaunchKernelGGL((tree_attn_split_kernel<1, true>), grid, dim3(kThreads), 0, st, p);
         else hipLaunchKernelGGL((tree_attn_split_kernel<2, true>), grid, dim3(kThreads), 0, st, p);
     } else {
@@ -1315,7 +1344,8 @@ static int tree_attention_impl(const void* q, void* k_pool, void* v_pool,
     CPMCU_LAUNCH_CHECK();
     if (p.num_splits > 1 && p.merge_ctr == nullptr) {
         const int threads_total = Hkv * (p.rows_pad / kRowsPerWave) * 16 * 64;
-        hipLaunchKernelGGL(tree_attn_combine_kernel, dim3(ceil_div(threads_total, 256)), dim3(256), 0, st, p);
+        if (is_bf16) hipLaunchKernelGGL(tree_attn_combine_bf16_kernel, dim3(ceil_div(threads_total, 256)), dim3(256), 0, st, p);
+        else hipLaunchKernelGGL(tree_attn_combine_kernel, dim3(ceil_div(threads_total, 256)), dim3(256), 0, st, p);
         CPMCU_LAUNCH_CHECK();
     }
     return CPMCU_OK;
@@ -1370,14 +1400,15 @@ __global__ void rope_table_kernel(const int32_t* pos, const float* inv_freq, int
 }
 
 // rotary_embedding_kernel, src/model/rotary.cuh:7-34, from a table: in place on q [T][Hq][128] and k [T][Hkv][128].
-__global__ __launch_bounds__(256) void rope_apply_kernel(const float2* table, int Hq, int Hkv, f16* q, f16* k) {
+template <typename E>
+__global__ __launch_bounds__(256) void rope_apply_kernel(const float2* table, int Hq, int Hkv, E* q, E* k) {
     constexpr int half = kHeadDim / 2;
     const int t = blockIdx.x;
     const float2* cs = table + (size_t)t * half;
     for (int i = threadIdx.x; i < (Hq + Hkv) * half; i += 256) {
         const int row = i / half, col = i % half;
-        f16* x = row < Hq ? q + ((size_t)t * Hq + row) * kHeadDim : k + ((size_t)t * Hkv + (row - Hq)) * kHeadDim;
-        f16 a = x[col], b = x[col + half];
+        E* x = row < Hq ? q + ((size_t)t * Hq + row) * kHeadDim : k + ((size_t)t * Hkv + (row - Hq)) * kHeadDim;
+        E a = x[col], b = x[col + half];
         rotate_pair(a, b, cs[col]);
         x[col] = a;
         x[col + half] = b;
@@ -1399,7 +1430,10 @@ extern "C" int cpmcu_rope_table(const int32_t* position_ids, const float* inv_fr
 extern "C" int cpmcu_rope_apply(const float* cos_sin, int T, int Hq, int Hkv, void* q, void* k, void* stream) {
     CPMCU_CHECK_ARG(cos_sin && q && k, "rope_apply: null pointer argument");
     CPMCU_CHECK_ARG(T >= 1 && Hq >= 1 && Hkv >= 1, "rope_apply: T=%d Hq=%d Hkv=%d", T, Hq, Hkv);
-    hipLaunchKernelGGL(rope_apply_kernel, dim3(T), dim3(256), 0, resolve_stream(stream), (const float2*)cos_sin, Hq, Hkv, (f16*)q, (f16*)k);
+    if (options().dtype == 1)
+        hipLaunchKernelGGL(rope_apply_kernel<bf16>, dim3(T), dim3(256), 0, resolve_stream(stream), (const float2*)cos_sin, Hq, Hkv, (bf16*)q, (bf16*)k);
+    else
+        hipLaunchKernelGGL(rope_apply_kernel<f16>, dim3(T), dim3(256), 0, resolve_stream(stream), (const float2*)cos_sin, Hq, Hkv, (f16*)q, (f16*)k);
     CPMCU_LAUNCH_CHECK();
     return CPMCU_OK;
 }

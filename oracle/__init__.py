@@ -43,6 +43,10 @@ def _load():
         "orc_topk": (None, [c_p, i32, i32, i32, c_p, c_p]),
         "orc_remap": (None, [c_p, i32, c_p, c_p]),
         "orc_argmax": (None, [c_p, i32, i32, c_p]),
+        "orc_set_dtype": (None, [i32]),
+        "orc_get_dtype": (i32, []),
+        "orc_bf16_to_f32": (None, [c_p, c_p, i64]),
+        "orc_f32_to_bf16": (None, [c_p, c_p, i64]),
         "orc_tree_accept": (i32, [i32, i32, c_p, c_p, c_p, i32, c_p, c_p, c_p, c_p]),
         "orc_kv_compact": (None, [c_p, i32, i32, i32, i32, c_p, c_p, c_p]),
         "orc_rope": (None, [i32, i32, i32, i32, c_p, c_p, c_p, c_p, c_p]),
@@ -90,6 +94,44 @@ def f32_to_f16(x, software=False):
     out = np.empty(x.shape, np.uint16)
     (_lib.orc_f32_to_f16_sw if software else _lib.orc_f32_to_f16)(_p(x), _p(out), x.size)
     return out
+
+
+def set_dtype(dtype):
+    """Element type of every 16-bit tensor of the calls that follow: 0 / "f16" = IEEE binary16 (the default), 1 / "bf16" =
+    bfloat16.  In bfloat16 mode the arrays still cross this module as numpy float16 arrays -- numpy has no bfloat16 --
+    whose 16 bits are bfloat16 patterns: `encode` / `decode` convert between such containers and float32 values."""
+    _lib.orc_set_dtype(1 if dtype in (1, "bf16") else 0)
+
+
+def get_dtype():
+    return int(_lib.orc_get_dtype())
+
+
+def bf16_to_f32(bits):
+    bits = _c(bits, np.uint16)
+    out = np.empty(bits.shape, np.float32)
+    _lib.orc_bf16_to_f32(_p(bits), _p(out), bits.size)
+    return out
+
+
+def f32_to_bf16(x):
+    x = _c(x, np.float32)
+    out = np.empty(x.shape, np.uint16)
+    _lib.orc_f32_to_bf16(_p(x), _p(out), x.size)
+    return out
+
+
+def decode(x):
+    """float32 values of a 16-bit container (a numpy float16 array) under the element type in force."""
+    x = np.ascontiguousarray(x)
+    assert x.dtype == np.float16
+    return bf16_to_f32(x.view(np.uint16)) if get_dtype() == 1 else x.astype(np.float32)
+
+
+def encode(x):
+    """The 16-bit container (numpy float16 array) of float32 values under the element type in force, rounded to nearest even."""
+    x = np.ascontiguousarray(x, np.float32)
+    return f32_to_bf16(x).view(np.float16) if get_dtype() == 1 else x.astype(np.float16)
 
 
 def mask_words(T):

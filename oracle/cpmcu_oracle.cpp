@@ -80,20 +80,42 @@ inline uint16_t float_to_half_sw(float f) {
     return (uint16_t)(sign | (base + q));
 }
 
-inline float h2f(uint16_t h) {
+// ---- bfloat16 <-> binary32: the upper half of the binary32 pattern, round to nearest even; a NaN stays a (quiet) NaN ----
+inline float bf16_to_float(uint16_t h) {
+    const uint32_t bits = (uint32_t)h << 16;
+    float f;
+    std::memcpy(&f, &bits, 4);
+    return f;
+}
+inline uint16_t float_to_bf16(float f) {
+    uint32_t x;
+    std::memcpy(&x, &f, 4);
+    if ((x & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((x >> 16) | 0x0040u);
+    x += 0x7FFFu + ((x >> 16) & 1u);
+    return (uint16_t)(x >> 16);
+}
+
+// The 16-bit element type of every tensor that crosses the interface: 0 = IEEE binary16 (the default), 1 = bfloat16
+// (src/entry.cu:26-59 dispatches the reference's templates on the same two).  Set once, ahead of the calls it governs.
+int g_dtype = 0;
+
+inline float half_to_float(uint16_t h) {
 #ifdef __F16C__
     return _cvtsh_ss(h);
 #else
     return half_to_float_sw(h);
 #endif
 }
-inline uint16_t f2h(float f) {
+inline uint16_t float_to_half(float f) {
 #ifdef __F16C__
     return _cvtss_sh(f, _MM_FROUND_TO_NEAREST_INT | _MM_FROUND_NO_EXC);
 #else
     return float_to_half_sw(f);
 #endif
 }
+// the element type in force
+inline float h2f(uint16_t h) { return g_dtype == 1 ? bf16_to_float(h) : half_to_float(h); }
+inline uint16_t f2h(float f) { return g_dtype == 1 ? float_to_bf16(f) : float_to_half(f); }
 
 // dot product with 16 interleaved fp32 partial sums (lane = k mod 16) and a
 // fixed pairwise tree at the end.  n must be a multiple of 16.
@@ -128,10 +150,10 @@ inline int threads() {
 extern "C" {
 
 void orc_f16_to_f32(const uint16_t* in, float* out, int64_t n) {
-    for (int64_t i = 0; i < n; ++i) out[i] = h2f(in[i]);
+    for (int64_t i = 0; i < n; ++i) out[i] = half_to_float(in[i]);
 }
 void orc_f32_to_f16(const float* in, uint16_t* out, int64_t n) {
-    for (int64_t i = 0; i < n; ++i) out[i] = f2h(in[i]);
+    for (int64_t i = 0; i < n; ++i) out[i] = float_to_half(in[i]);
 }
 // software versions, exported so the tests can check the F16C path against them
 void orc_f16_to_f32_sw(const uint16_t* in, float* out, int64_t n) {
@@ -139,6 +161,15 @@ void orc_f16_to_f32_sw(const uint16_t* in, float* out, int64_t n) {
 }
 void orc_f32_to_f16_sw(const float* in, uint16_t* out, int64_t n) {
     for (int64_t i = 0; i < n; ++i) out[i] = float_to_half_sw(in[i]);
+}
+
+void orc_set_dtype(int dtype) { g_dtype = dtype == 1 ? 1 : 0; }
+int orc_get_dtype(void) { return g_dtype; }
+void orc_bf16_to_f32(const uint16_t* in, float* out, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) out[i] = bf16_to_float(in[i]);
+}
+void orc_f32_to_bf16(const float* in, uint16_t* out, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) out[i] = float_to_bf16(in[i]);
 }
 
 int orc_num_threads(void) { return threads(); }

@@ -33,6 +33,16 @@ extern "C" {
 void orc_f16_to_f32(const uint16_t* in, float* out, int64_t n);
 void orc_f32_to_f16(const float* in, uint16_t* out, int64_t n);
 
+/* ---- element type ----
+ * Every 16-bit tensor of the functions below is IEEE binary16 by default; orc_set_dtype(1) makes it bfloat16 for the
+ * calls that follow (0 switches back): the reference builds its templates for both (src/entry.cu:26-59,
+ * torch_dtype 0 / 1).  Rounding is to nearest even in both; sums stay fp32.
+ * pinned by: torch's CPU bfloat16 conversion on all 65536 patterns and on random / boundary floats. */
+void orc_set_dtype(int dtype);
+int orc_get_dtype(void);
+void orc_bf16_to_f32(const uint16_t* in, float* out, int64_t n);
+void orc_f32_to_bf16(const float* in, uint16_t* out, int64_t n);
+
 /* Number of worker threads the threaded entry points will use. */
 int orc_num_threads(void);
 void orc_set_num_threads(int n);
