@@ -42,6 +42,7 @@ struct Elem<f16> {
     __device__ static inline float from_bits(uint16_t h) { return (float)__builtin_bit_cast(f16, h); }
     __device__ static inline uint16_t to_bits(float f) { return __builtin_bit_cast(uint16_t, (f16)f); }
     static constexpr int kMantissaBits = 10, kExponentBits = 5, kExponentBias = 15;
+    static constexpr float kMaxFinite = 65504.f;
 };
 template <>
 struct Elem<bf16> {
@@ -55,6 +56,7 @@ struct Elem<bf16> {
     __device__ static inline float from_bits(uint16_t h) { return __uint_as_float((uint32_t)h << 16); }
     __device__ static inline uint16_t to_bits(float f) { return __builtin_bit_cast(uint16_t, (bf16)f); }
     static constexpr int kMantissaBits = 7, kExponentBits = 8, kExponentBias = 127;
+    static constexpr float kMaxFinite = 3.3895313892515355e38f;
 };
 
 constexpr int kPage = CPMCU_PAGE_SIZE;    // tokens per KV page

@@ -14,6 +14,7 @@
 // done by counting: every entry becomes a unique 32-bit key in LDS, every thread counts the keys above
 // its own, and that count is the entry's place in the sorted order -- no rounds, two barriers.
 #include "common.h"
+#include "internal.h"
 #include "topk_keys.h"
 
 namespace cpmcu {
@@ -88,7 +89,7 @@ __global__ void draft_begin_kernel(DraftState s, int k, const uint16_t* val, con
 
 __global__ __launch_bounds__(kTopkThreads) void draft_extend_kernel(DraftState s, int k, int d, uint16_t* val, const int32_t* pos,
                                                                     const int32_t* remap, int32_t* next_ids, int32_t* parent_rows,
-                                                                    uint64_t* mask_out) {
+                                                                    uint64_t* mask_out, int is_bf16) {
     __shared__ __attribute__((aligned(16))) uint32_t s_keys[kMaxK * kMaxK];
     __shared__ int32_t s_sel[kMaxK];
     __shared__ uint16_t s_val[kMaxK * kMaxK];
@@ -100,9 +101,9 @@ __global__ __launch_bounds__(kTopkThreads) void draft_extend_kernel(DraftState s
     for (int x = tid; x < ((kk + 3) & ~3); x += kTopkThreads) {
         uint32_t key = 0;
         if (x < kk) {
-            const float c = (float)__builtin_bit_cast(f16, s.cum[x / k]);
-            const f16 v = (f16)((float)__builtin_bit_cast(f16, val[x]) + c);  // half += half, rounded to half
-            const uint16_t bits = __builtin_bit_cast(uint16_t, v);
+            // the running log-prob of the parent is added in the element type: 16 bits += 16 bits, rounded to 16 bits
+            const uint16_t bits = is_bf16 ? Elem<bf16>::to_bits(Elem<bf16>::from_bits(val[x]) + Elem<bf16>::from_bits(s.cum[x / k]))
+                                          : Elem<f16>::to_bits(Elem<f16>::from_bits(val[x]) + Elem<f16>::from_bits(s.cum[x / k]));
             val[x] = bits;
             s.tried_val[base + x] = bits;
             s.tried_pos[base + x] = pos[x];
@@ -236,7 +237,7 @@ extern "C" int cpmcu_draft_tree_extend(void* state, int k, int num_iter, int d, 
     if (int rc = check_shape("draft_tree_extend", k, num_iter)) return rc;
     CPMCU_CHECK_ARG(d >= 1 && d < num_iter, "draft_tree_extend: iteration d=%d outside [1, %d)", d, num_iter);
     hipLaunchKernelGGL(draft_extend_kernel, dim3(1), dim3(kTopkThreads), 0, resolve_stream(stream), draft_state(state, k, num_iter), k, d,
-                       (uint16_t*)topk_val, topk_pos, token_id_remap, next_ids, parent_rows, draft_mask);
+                       (uint16_t*)topk_val, topk_pos, token_id_remap, next_ids, parent_rows, draft_mask, options().dtype == 1 ? 1 : 0);
     CPMCU_LAUNCH_CHECK();
     return CPMCU_OK;
 }

@@ -74,7 +74,7 @@ struct HeadCfg {
 
 // Folds one finished 16-row block of W (acc[nb][r] <-> vocab row vrow0 + r, hidden row nb*16 + l16) into
 // the lane's running epilogue state and writes its logits when asked to.
-template <int NB>
+template <int NB, typename E>
 __device__ inline void head_epilogue(const HeadParams& p, const f32x4 (&acc)[NB], int vrow0, int l16, float (&ea)[NB], float (&eb)[NB]) {
     const int V = p.V;
     if (p.mode == kHeadModeArgmax && p.logits == nullptr) {
@@ -84,7 +84,7 @@ __device__ inline void head_epilogue(const HeadParams& p, const f32x4 (&acc)[NB]
             const bool row_in = nb * 16 + l16 < p.n;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const float x = (float)(f16)acc[nb][r];
+                const float x = (float)(E)acc[nb][r];
                 const int idx = vrow0 + r;
                 const bool take = row_in && idx < V && (x > ea[nb] || (x == ea[nb] && idx < __float_as_int(eb[nb])));
                 ea[nb] = take ? x : ea[nb];
@@ -96,17 +96,17 @@ __device__ inline void head_epilogue(const HeadParams& p, const f32x4 (&acc)[NB]
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
         const int hrow = nb * 16 + l16;
-        f16 z[4];
+        E z[4];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) z[r] = (f16)acc[nb][r];
+        for (int r = 0; r < 4; ++r) z[r] = (E)acc[nb][r];
         if (hrow < p.n) {
             if (p.logits) {
-                f16* dst = p.logits + (size_t)hrow * V + vrow0;
+                E* dst = reinterpret_cast<E*>(p.logits) + (size_t)hrow * V + vrow0;
                 if ((V & 3) == 0 && vrow0 + 3 < V) {
-                    f16x4 zz;
+                    typename Elem<E>::x4 zz;
 #pragma unroll
                     for (int r = 0; r < 4; ++r) zz[r] = z[r];
-                    *reinterpret_cast<f16x4*>(dst) = zz;
+                    *reinterpret_cast<typename Elem<E>::x4*>(dst) = zz;
                 } else {
 #pragma unroll
                     for (int r = 0; r < 4; ++r)
@@ -185,8 +185,9 @@ __device__ inline void head_finish(const HeadParams& p, float (&ea)[NB], float (
     }
 }
 
-template <int NB>
-__global__ __launch_bounds__(kHeadThreads) void head_gemm_kernel(HeadParams p) {
+template <int NB, typename E>
+__device__ __forceinline__ void head_gemm_body(const HeadParams& p) {
+    typedef typename Elem<E>::x8 X8;
     using C = HeadCfg<NB>;
     constexpr int PD = C::kDepth;
     constexpr int GK = C::kGroupK;
@@ -212,11 +213,11 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_kernel(HeadParams p) {
     // keep hitting addresses with the same low bits -- the same few HBM channels -- at any instant.
     const int rotc = resident ? 0 : c % nch;
     const int rotg = resident ? (c * kHeadWaves + wave) % gpp : rotc * (kc / GK);
-    const f16 sc = (f16)p.head_scale;
+    const E sc = (E)p.head_scale;
 
     // ---- hidden staging helpers ----
     const int chunks16 = NB * 16 * kc / 8;  // 16-byte pieces per K chunk
-    f16x8 stage[C::kStage];
+    X8 stage[C::kStage];
     auto stage_load = [&](int hchunk) {
 #pragma unroll
         for (int s = 0; s < C::kStage; ++s) {
@@ -224,16 +225,16 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_kernel(HeadParams p) {
             if (i < chunks16) {
                 const int row = i / (kc / 8);
                 const int col = (i % (kc / 8)) * 8;
-                f16x8 x;
+                X8 x;
                 if (row < p.n) {
-                    x = *reinterpret_cast<const f16x8*>(p.hidden + (size_t)row * H + (size_t)hchunk * kc + col);
+                    x = *reinterpret_cast<const X8*>(p.hidden + (size_t)row * H + (size_t)hchunk * kc + col);
                     if (p.apply_scale) {
 #pragma unroll
-                        for (int e = 0; e < 8; ++e) x[e] = (f16)((float)x[e] * (float)sc);
+                        for (int e = 0; e < 8; ++e) x[e] = (E)((float)x[e] * (float)sc);
                     }
                 } else {
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) x[e] = (f16)0.f;
+                    for (int e = 0; e < 8; ++e) x[e] = (E)0.f;
                 }
                 stage[s] = x;
             }
@@ -246,7 +247,7 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_kernel(HeadParams p) {
             if (i < chunks16) {
                 const int row = i / (kc / 8);
                 const int col = (i % (kc / 8)) * 8;
-                *reinterpret_cast<f16x8*>(lds + (size_t)buf * C::kLdsBuf + row * lds_row + col * 2) = stage[s];
+                *reinterpret_cast<X8*>(lds + (size_t)buf * C::kLdsBuf + row * lds_row + col * 2) = stage[s];
             }
         }
     };
@@ -254,7 +255,7 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_kernel(HeadParams p) {
     // ---- W prefetch: group `it` = (pass, k-group) of this wave's row block ----
     const int arow_lane = l16;
     auto row_block = [&](int pass) { return (pass * kHeadWaves + wave) * G + c; };
-    auto load_group = [&](int it, f16x8* buf) {
+    auto load_group = [&](int it, X8* buf) {
         const int pass = it / gpp;
         const int k0 = ((it % gpp + rotg) % gpp) * GK;
         if (p.w_tiled) {  // one contiguous KB per instruction, consecutive steps consecutive in memory
@@ -262,14 +263,14 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_kernel(HeadParams p) {
             rb = rb * 16 < V ? rb : (V - 1) / 16;
             const f16* src = p.w + ((size_t)rb * (H / 32) + k0 / 32) * 512 + lane * 8;
 #pragma unroll
-            for (int ks = 0; ks < PD; ++ks) buf[ks] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(src + ks * 512));
+            for (int ks = 0; ks < PD; ++ks) buf[ks] = __builtin_nontemporal_load(reinterpret_cast<const X8*>(src + ks * 512));
             return;
         }
         int row = row_block(pass) * 16 + arow_lane;
         row = row < V ? row : V - 1;  // clamp: rows past the end are computed and discarded
         const f16* src = p.w + (size_t)row * H + k0 + kgp * 8;
 #pragma unroll
-        for (int ks = 0; ks < PD; ++ks) buf[ks] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(src + ks * 32));
+        for (int ks = 0; ks < PD; ++ks) buf[ks] = __builtin_nontemporal_load(reinterpret_cast<const X8*>(src + ks * 32));
     };
 
     f32x4 acc[NB];
@@ -281,7 +282,7 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_kernel(HeadParams p) {
         eb[nb] = p.mode == kHeadModeStats ? 0.f : __int_as_float(0x7fffffff);  // running sum / best index
     }
 
-    auto epilogue = [&](int pass) { head_epilogue<NB>(p, acc, row_block(pass) * 16 + kgp * 4, l16, ea, eb); };
+    auto epilogue = [&](int pass) { head_epilogue<NB, E>(p, acc, row_block(pass) * 16 + kgp * 4, l16, ea, eb); };
 
     // ---- prologue: hidden into LDS ----
     if (resident) {
@@ -295,7 +296,7 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_kernel(HeadParams p) {
         stage_store(0);
     }
 
-    auto compute_group = [&](int it, const f16x8* buf) {
+    auto compute_group = [&](int it, const X8* buf) {
         const int pass = it / gpp;
         const int kg = it % gpp;                     // position in this wave's K walk
         const int k0 = ((kg + rotg) % gpp) * GK;     // actual K offset (rotated by whole chunks)
@@ -323,8 +324,8 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_kernel(HeadParams p) {
         for (int ks = 0; ks < PD; ++ks) {
 #pragma unroll
             for (int nb = 0; nb < NB; ++nb) {
-                const f16x8 b = *reinterpret_cast<const f16x8*>(brow + nb * 16 * lds_row + ks * 64);
-                acc[nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(buf[ks], b, acc[nb], 0, 0, 0);
+                const X8 b = *reinterpret_cast<const X8*>(brow + nb * 16 * lds_row + ks * 64);
+                acc[nb] = Elem<E>::mfma_16x16x32(buf[ks], b, acc[nb]);
             }
         }
         if (!resident && koff + GK == kc) {
@@ -333,7 +334,7 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_kernel(HeadParams p) {
         if (kg == gpp - 1) epilogue(pass);
     };
 
-    f16x8 buf_a[PD], buf_b[PD];
+    X8 buf_a[PD], buf_b[PD];
     if (total > 0) load_group(0, buf_a);
     for (int it = 0; it < total; it += 2) {
         if (it + 1 < total) load_group(it + 1, buf_b);
@@ -355,8 +356,9 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_kernel(HeadParams p) {
 //   LDS layout of a chunk: [hidden row][KC halves], unpadded; the 16-byte piece index is XORed with
 //   row % 16 (applied through the global address each DMA lane fetches), which makes the B-operand
 //   reads (16 rows x one piece per 16 lanes) conflict-free.
-template <int NB, int NP, int KC, int NBUF>  // KC = halves of K per chunk, NBUF = W register buffers
-__global__ __launch_bounds__(kHeadThreads) void head_gemm_chunked_kernel(HeadParams p) {
+template <int NB, int NP, int KC, int NBUF, typename E>  // KC = halves of K per chunk, NBUF = W register buffers
+__device__ __forceinline__ void head_gemm_chunked_body(const HeadParams& p) {
+    typedef typename Elem<E>::x8 X8;
     constexpr int PD = KC / 32;              // 16-byte W loads in flight per lane and buffer
     constexpr int ROWB = KC * 2;
     constexpr int BUF = NB * 16 * ROWB;
@@ -380,7 +382,7 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_chunked_kernel(HeadPar
     const int nsweeps = (p.npasses + NP - 1) / NP;
     const int total_q = nsweeps * nch;
     const int rotc = c % nch;  // workgroups start their K walk at different chunks (HBM channel spread)
-    const f16 sc = (f16)p.head_scale;
+    const E sc = (E)p.head_scale;
 
     // Shared last pass: this workgroup's r_c blocks of it, `share` waves on each (a power of two that
     // divides the chunk count), wave w on block w / share with the chunks q % share == w % share.
@@ -420,7 +422,7 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_chunked_kernel(HeadPar
         return (pass * kHeadWaves + wave) * G + c;
     };
     int groups_since_dma = 0;  // W groups requested after the newest hidden chunk request
-    auto load_w = [&](int q, int pl, f16x8* buf) {
+    auto load_w = [&](int q, int pl, X8* buf) {
         const int pass = (q / nch) * NP + pl;
         if (!step_active(q, pl)) return;
         ++groups_since_dma;
@@ -429,14 +431,14 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_chunked_kernel(HeadPar
             rb = rb * 16 < V ? rb : (V - 1) / 16;
             const f16* src = p.w + ((size_t)rb * (H / 32) + chunk_of(q) * (KC / 32)) * 512 + lane * 8;
 #pragma unroll
-            for (int ks = 0; ks < PD; ++ks) buf[ks] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(src + ks * 512));
+            for (int ks = 0; ks < PD; ++ks) buf[ks] = __builtin_nontemporal_load(reinterpret_cast<const X8*>(src + ks * 512));
             return;
         }
         int row = row_block(pass) * 16 + l16;
         row = row < V ? row : V - 1;  // clamp: rows past the end are computed and discarded
         const f16* src = p.w + (size_t)row * H + chunk_of(q) * KC + kgp * 8;
 #pragma unroll
-        for (int ks = 0; ks < PD; ++ks) buf[ks] = __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(src + ks * 32));
+        for (int ks = 0; ks < PD; ++ks) buf[ks] = __builtin_nontemporal_load(reinterpret_cast<const X8*>(src + ks * 32));
     };
 
     f32x4 acc[NP][NB];
@@ -449,7 +451,7 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_chunked_kernel(HeadPar
     const int xl = (kgp ^ (l16 & 3)) << 4, hi = l16 >> 2;
 
     // W groups are requested NBUF - 1 steps ahead of their use (a step = one row block x one chunk).
-    f16x8 bufs[NBUF][PD];
+    X8 bufs[NBUF][PD];
     issue_hidden(0);
 #pragma unroll
     for (int s0 = 0; s0 < NBUF - 1; ++s0) load_w(s0 / NP, s0 % NP, bufs[s0 % NBUF]);  // NBUF - 1 <= NP
@@ -476,10 +478,10 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_chunked_kernel(HeadPar
         if (p.apply_scale) {  // fp16 pre-scale of the hidden rows (src/model/linear.cuh:82-101): own pieces, in place
 #pragma unroll
             for (int j = 0; j < NINST; ++j) {
-                f16x8* px = reinterpret_cast<f16x8*>(lds + (q & 1) * BUF + (wave * NINST + j) * 1024 + lane * 16);
-                f16x8 x = *px;
+                X8* px = reinterpret_cast<X8*>(lds + (q & 1) * BUF + (wave * NINST + j) * 1024 + lane * 16);
+                X8 x = *px;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) x[e] = (f16)((float)x[e] * (float)sc);
+                for (int e = 0; e < 8; ++e) x[e] = (E)((float)x[e] * (float)sc);
                 *px = x;
             }
         }
@@ -503,8 +505,8 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_chunked_kernel(HeadPar
                     const char* bk = base + ((ks ^ hi) << 6);
 #pragma unroll
                     for (int nb = 0; nb < NB; ++nb) {
-                        const f16x8 b = *reinterpret_cast<const f16x8*>(bk + nb * 16 * ROWB);
-                        acc[pl][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bufs[pl % NBUF][ks], b, acc[pl][nb], 0, 0, 0);
+                        const X8 b = *reinterpret_cast<const X8*>(bk + nb * 16 * ROWB);
+                        acc[pl][nb] = Elem<E>::mfma_16x16x32(bufs[pl % NBUF][ks], b, acc[pl][nb]);
                     }
                 }
             }
@@ -514,7 +516,7 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_chunked_kernel(HeadPar
             for (int pl = 0; pl < NP; ++pl) {
                 const int pass = (q / nch) * NP + pl;
                 if (pass < (shared_last ? p.full_passes : p.npasses))
-                    head_epilogue<NB>(p, acc[pl], row_block(pass) * 16 + kgp * 4, l16, ea, eb);
+                    head_epilogue<NB, E>(p, acc[pl], row_block(pass) * 16 + kgp * 4, l16, ea, eb);
             }
         }
     }
@@ -543,7 +545,7 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_chunked_kernel(HeadPar
                     for (int r = 0; r < 4; ++r) sum[nb][r] += x[r];
                 }
             }
-            head_epilogue<NB>(p, sum, row_block(p.full_passes) * 16 + kgp * 4, l16, ea, eb);
+            head_epilogue<NB, E>(p, sum, row_block(p.full_passes) * 16 + kgp * 4, l16, ea, eb);
         }
     }
     head_finish<NB>(p, ea, eb, red_a, red_b, tid, wave, lane, c);
@@ -569,8 +571,9 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_chunked_kernel(HeadPar
 //   wave-uniform branches (their count is a run-time value); the ring has PD extra slots for them, and what the
 //   compiler has to assume about them costs the full passes at most that many fragments of look-ahead.
 //   The hidden chunk is brought in as in the kernel above (direct-to-LDS, double buffered, XOR-swizzled).
-template <int NB, int FP, int KC>
-__global__ __launch_bounds__(kHeadThreads) void head_gemm_stream_kernel(HeadParams p) {
+template <int NB, int FP, int KC, typename E>
+__device__ __forceinline__ void head_gemm_stream_body(const HeadParams& p) {
+    typedef typename Elem<E>::x8 X8;
     constexpr int PD = KC / 32;              // 1 KB W fragments per row block and chunk
     constexpr int R = (FP + 1) * PD;         // ring slots
     constexpr int ROWB = KC * 2;
@@ -592,7 +595,7 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_stream_kernel(HeadPara
     const int H = p.H;
     const int nch = H / KC;
     const int rotc = c % nch;  // workgroups start their K walk at different chunks (HBM channel spread)
-    const f16 sc = (f16)p.head_scale;
+    const E sc = (E)p.head_scale;
 
     // last pass: block `my_last` of this workgroup's share of it, K slice `my_sub` of every chunk
     const int share = p.last_share;
@@ -621,7 +624,7 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_stream_kernel(HeadPara
 #pragma unroll
     for (int pl = 0; pl < FP; ++pl) wfull[pl] = p.w + (size_t)((pl * kHeadWaves + wave) * G + c) * (H / 32) * 512 + lane * 8;
     const f16* wlast = p.w + (size_t)(last_active ? rb_last : 0) * (H / 32) * 512 + lane * 8;
-    auto load_frag = [&](const f16* base, int step) { return __builtin_nontemporal_load(reinterpret_cast<const f16x8*>(base + (size_t)step * 512)); };
+    auto load_frag = [&](const f16* base, int step) { return __builtin_nontemporal_load(reinterpret_cast<const X8*>(base + (size_t)step * 512)); };
 
     f32x4 acc[FP + 1][NB];
 #pragma unroll
@@ -639,7 +642,7 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_stream_kernel(HeadPara
     const int xl = (kgp ^ (l16 & 3)) << 4, hi = l16 >> 2;
 
     // ring slot ks * FP + pl: K step ks of full pass pl; slot FP * PD + j: step j of the last-pass slice
-    f16x8 ring[R];
+    X8 ring[R];
     issue_hidden(0);
     {
         const int s0 = chunk_of(0) * PD;
@@ -659,10 +662,10 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_stream_kernel(HeadPara
         if (p.apply_scale) {  // fp16 pre-scale of the hidden rows (src/model/linear.cuh:82-101): own pieces, in place
 #pragma unroll
             for (int j = 0; j < NINST; ++j) {
-                f16x8* px = reinterpret_cast<f16x8*>(lds + (q & 1) * BUF + (wave * NINST + j) * 1024 + lane * 16);
-                f16x8 x = *px;
+                X8* px = reinterpret_cast<X8*>(lds + (q & 1) * BUF + (wave * NINST + j) * 1024 + lane * 16);
+                X8 x = *px;
 #pragma unroll
-                for (int e = 0; e < 8; ++e) x[e] = (f16)((float)x[e] * (float)sc);
+                for (int e = 0; e < 8; ++e) x[e] = (E)((float)x[e] * (float)sc);
                 *px = x;
             }
         }
@@ -670,21 +673,21 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_stream_kernel(HeadPara
         if (refill) issue_hidden(q + 1);
         const int sn = chunk_of(q + 1) * PD;
         const char* base = lds + (q & 1) * BUF + l16 * ROWB + xl;
-        f16x8 b[2][NB];
+        X8 b[2][NB];
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) b[0][nb] = *reinterpret_cast<const f16x8*>(base + ((0 ^ hi) << 6) + nb * 16 * ROWB);
+        for (int nb = 0; nb < NB; ++nb) b[0][nb] = *reinterpret_cast<const X8*>(base + ((0 ^ hi) << 6) + nb * 16 * ROWB);
 #pragma unroll
         for (int ks = 0; ks < PD; ++ks) {
             if (ks + 1 < PD) {
 #pragma unroll
                 for (int nb = 0; nb < NB; ++nb)
-                    b[(ks + 1) & 1][nb] = *reinterpret_cast<const f16x8*>(base + (((ks + 1) ^ hi) << 6) + nb * 16 * ROWB);
+                    b[(ks + 1) & 1][nb] = *reinterpret_cast<const X8*>(base + (((ks + 1) ^ hi) << 6) + nb * 16 * ROWB);
             }
 #pragma unroll
             for (int pl = 0; pl < FP; ++pl)
 #pragma unroll
                 for (int nb = 0; nb < NB; ++nb)
-                    acc[pl][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ring[ks * FP + pl], b[ks & 1][nb], acc[pl][nb], 0, 0, 0);
+                    acc[pl][nb] = Elem<E>::mfma_16x16x32(ring[ks * FP + pl], b[ks & 1][nb], acc[pl][nb]);
             if (refill) {
 #pragma unroll
                 for (int pl = 0; pl < FP; ++pl) ring[ks * FP + pl] = load_frag(wfull[pl], sn + ks);
@@ -695,12 +698,12 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_stream_kernel(HeadPara
         for (int j = 0; j < PD; ++j) {
             if (j < sl) {
                 const int ksl = my_sub * sl + j;
-                f16x8 bl[NB];
+                X8 bl[NB];
 #pragma unroll
-                for (int nb = 0; nb < NB; ++nb) bl[nb] = *reinterpret_cast<const f16x8*>(base + ((ksl ^ hi) << 6) + nb * 16 * ROWB);
+                for (int nb = 0; nb < NB; ++nb) bl[nb] = *reinterpret_cast<const X8*>(base + ((ksl ^ hi) << 6) + nb * 16 * ROWB);
 #pragma unroll
                 for (int nb = 0; nb < NB; ++nb)
-                    acc[FP][nb] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ring[FP * PD + j], bl[nb], acc[FP][nb], 0, 0, 0);
+                    acc[FP][nb] = Elem<E>::mfma_16x16x32(ring[FP * PD + j], bl[nb], acc[FP][nb]);
                 if (refill) ring[FP * PD + j] = load_frag(wlast, sn + ksl);
             }
         }
@@ -708,7 +711,7 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_stream_kernel(HeadPara
     for (int q = 0; q + 1 < nch; ++q) chunk_body(q, std::true_type{});
     chunk_body(nch - 1, std::false_type{});
 #pragma unroll
-    for (int pl = 0; pl < FP; ++pl) head_epilogue<NB>(p, acc[pl], ((pl * kHeadWaves + wave) * G + c) * 16 + kgp * 4, l16, ea, eb);
+    for (int pl = 0; pl < FP; ++pl) head_epilogue<NB, E>(p, acc[pl], ((pl * kHeadWaves + wave) * G + c) * 16 + kgp * 4, l16, ea, eb);
     if (p.rem_blocks > 0) {
         // The waves that shared a block of the last pass hold partial sums over their K slices: they meet in LDS
         // (the hidden buffers are free now) and the first wave of each group adds them up in wave order.
@@ -728,11 +731,25 @@ __global__ __launch_bounds__(kHeadThreads) void head_gemm_stream_kernel(HeadPara
                     for (int r = 0; r < 4; ++r) acc[FP][nb][r] += x[r];
                 }
             }
-            head_epilogue<NB>(p, acc[FP], rb_last * 16 + kgp * 4, l16, ea, eb);
+            head_epilogue<NB, E>(p, acc[FP], rb_last * 16 + kgp * 4, l16, ea, eb);
         }
     }
     head_finish<NB>(p, ea, eb, red_a, red_b, tid, wave, lane, c);
 }
+
+// The kernels proper: fp16 under the names they have in every profile, bf16 beside them.
+template <int NB>
+__global__ __launch_bounds__(kHeadThreads) void head_gemm_kernel(HeadParams p) { head_gemm_body<NB, f16>(p); }
+template <int NB>
+__global__ __launch_bounds__(kHeadThreads) void head_gemm_bf16_kernel(HeadParams p) { head_gemm_body<NB, bf16>(p); }
+template <int NB, int NP, int KC, int NBUF>
+__global__ __launch_bounds__(kHeadThreads) void head_gemm_chunked_kernel(HeadParams p) { head_gemm_chunked_body<NB, NP, KC, NBUF, f16>(p); }
+template <int NB, int NP, int KC, int NBUF>
+__global__ __launch_bounds__(kHeadThreads) void head_gemm_chunked_bf16_kernel(HeadParams p) { head_gemm_chunked_body<NB, NP, KC, NBUF, bf16>(p); }
+template <int NB, int FP, int KC>
+__global__ __launch_bounds__(kHeadThreads) void head_gemm_stream_kernel(HeadParams p) { head_gemm_stream_body<NB, FP, KC, f16>(p); }
+template <int NB, int FP, int KC>
+__global__ __launch_bounds__(kHeadThreads) void head_gemm_stream_bf16_kernel(HeadParams p) { head_gemm_stream_body<NB, FP, KC, bf16>(p); }
 
 // Final arg-max over the per-workgroup partials: one block per hidden row.  Largest value, lowest
 // index among equals: one 64-bit key (ordered image of the float, complemented index) per partial,
@@ -900,8 +917,17 @@ int launch_head_gemm(const void* hidden, const void* w, int w_layout, int n, int
     }
     if (shape_out) *shape_out = shape;
     if (dry_run) return CPMCU_OK;
-#define CPMCU_HEAD_ROW(nb) hipLaunchKernelGGL(head_gemm_kernel<nb>, dim3(G), dim3(kHeadThreads), 0, st, p)
-#define CPMCU_HEAD_CHUNKED(nb, np, kc, nbuf) hipLaunchKernelGGL((head_gemm_chunked_kernel<nb, np, kc, nbuf>), dim3(G), dim3(kHeadThreads), 0, st, p)
+    const bool is_bf16 = options().dtype == 1;
+#define CPMCU_HEAD_ROW(nb)                                                                                   \
+    do {                                                                                                     \
+        if (is_bf16) hipLaunchKernelGGL(head_gemm_bf16_kernel<nb>, dim3(G), dim3(kHeadThreads), 0, st, p);    \
+        else hipLaunchKernelGGL(head_gemm_kernel<nb>, dim3(G), dim3(kHeadThreads), 0, st, p);                 \
+    } while (0)
+#define CPMCU_HEAD_CHUNKED(nb, np, kc, nbuf)                                                                                     \
+    do {                                                                                                                         \
+        if (is_bf16) hipLaunchKernelGGL((head_gemm_chunked_bf16_kernel<nb, np, kc, nbuf>), dim3(G), dim3(kHeadThreads), 0, st, p); \
+        else hipLaunchKernelGGL((head_gemm_chunked_kernel<nb, np, kc, nbuf>), dim3(G), dim3(kHeadThreads), 0, st, p);              \
+    } while (0)
     switch (shape) {
         case HeadShape::Row1: CPMCU_HEAD_ROW(1); break;
         case HeadShape::Row2: CPMCU_HEAD_ROW(2); break;
@@ -917,8 +943,11 @@ int launch_head_gemm(const void* hidden, const void* w, int w_layout, int n, int
         case HeadShape::C_2_4_512_2: CPMCU_HEAD_CHUNKED(2, 4, 512, 2); break;
         case HeadShape::C_4_4_128_4: CPMCU_HEAD_CHUNKED(4, 4, 128, 4); break;
         case HeadShape::C_8_2_128_2: CPMCU_HEAD_CHUNKED(8, 2, 128, 2); break;
-#define CPMCU_X(nb, fp, kc) \
-    case HeadShape::S_##nb##_##fp##_##kc: hipLaunchKernelGGL((head_gemm_stream_kernel<nb, fp, kc>), dim3(G), dim3(kHeadThreads), 0, st, p); break;
+#define CPMCU_X(nb, fp, kc)                                                                                                   \
+    case HeadShape::S_##nb##_##fp##_##kc:                                                                                     \
+        if (is_bf16) hipLaunchKernelGGL((head_gemm_stream_bf16_kernel<nb, fp, kc>), dim3(G), dim3(kHeadThreads), 0, st, p);   \
+        else hipLaunchKernelGGL((head_gemm_stream_kernel<nb, fp, kc>), dim3(G), dim3(kHeadThreads), 0, st, p);                \
+        break;
             CPMCU_HEAD_STREAM_SHAPES(CPMCU_X)
 #undef CPMCU_X
     }

@@ -68,6 +68,7 @@ struct Model {
     float memory_limit = 0.f;
     int vocab = 0, layers = 0, hidden = 0, q_heads = 0, kv_heads = 0, head_dim = 0;
     float scale_lmhead = 1.f;
+    int dtype = 0;  // 0 = fp16, 1 = bf16
     // drafter (init_eagle_model / init_minicpm4_eagle_model)
     bool drafter = false;
     int num_iter = 0, topk_per_iter = 0, tree_size = 0, frspec_vocab = 0;
@@ -181,8 +182,8 @@ int synchronize_and_check(hipStream_t st) {
 }
 
 int check_dtype(int torch_dtype) {
-    if (torch_dtype != 0) {  // 0 = fp16, 1 = bf16 (cpmcu/llm.py:11-14)
-        set_error("dtype %d is not compiled into this library (fp16 only)", torch_dtype);
+    if (torch_dtype != 0 && torch_dtype != 1) {  // 0 = fp16, 1 = bf16 (cpmcu/llm.py:11-14)
+        set_error("dtype %d is not compiled into this library (0 = fp16, 1 = bf16)", torch_dtype);
         return CPMCU_ERR_RUNTIME;  // std::runtime_error in the reference, src/entry.cu:43,52
     }
     return CPMCU_OK;
@@ -251,6 +252,8 @@ extern "C" int cpmcu_init_base_model(float memory_limit, int vocab_size, int num
     m.kv_heads = num_key_value_heads;
     m.head_dim = head_dim;
     m.scale_lmhead = scale_lmhead;
+    m.dtype = torch_dtype;
+    options().dtype = torch_dtype;  // the model's element type is the process's: every kernel launch reads this switch
     const char* pe = getenv("CPMCU_PERF");
     m.perf = pe && pe[0] == '1';
     return CPMCU_OK;
@@ -269,6 +272,8 @@ extern "C" int cpmcu_init_minicpm4_eagle_model(int num_layers, int num_iter, int
     if (rc) return rc;
     rc = check_dtype(torch_dtype);
     if (rc) return rc;
+    CPMCU_CHECK_ARG(torch_dtype == g_model->dtype, "init_minicpm4_eagle_model: dtype %d differs from the base model's %d", torch_dtype,
+                    g_model->dtype);
     if (apply_eagle_quant) {
         set_error("init_minicpm4_eagle_model: quantised EAGLE layers are outside the verify/draft path");
         return CPMCU_ERR_UNSUPPORTED;
@@ -991,5 +996,6 @@ extern "C" int cpmcu_shutdown(void) {
     release_storage(m);
     delete g_model;
     g_model = nullptr;
+    options().dtype = 0;  // the operator-level entry points are back on the default element type
     return CPMCU_OK;
 }

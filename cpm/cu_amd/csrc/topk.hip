@@ -48,8 +48,10 @@ __device__ inline void emit_final(const TopkParams& p, int row, int round, uint6
     if (p.ids) p.ids[o] = p.remap ? p.remap[idx] : idx;
 }
 
-template <bool LOGSOFTMAX>
-__global__ __launch_bounds__(kTopkThreads) void topk_chunk_kernel(TopkParams p) {
+// E: the element type of the values (it matters only with the fused log-softmax, which does arithmetic on them; the raw
+// ranking works on bit patterns whose order is the same for both types).  The kernels proper are thin wrappers below.
+template <bool LOGSOFTMAX, typename E>
+__device__ __forceinline__ void topk_chunk_body(const TopkParams& p) {
     const int chunk = blockIdx.x;
     const int row = blockIdx.y;
     const int tid = threadIdx.x;
@@ -103,9 +105,8 @@ __global__ __launch_bounds__(kTopkThreads) void topk_chunk_kernel(TopkParams p) 
         if (idx < p.dim) {
             uint16_t bits = xr[idx];
             if (LOGSOFTMAX) {
-                const float z = (float)__builtin_bit_cast(f16, bits);
-                const f16 lp = (f16)((z - m) - lse);  // src/model/eagle.cuh:87
-                bits = __builtin_bit_cast(uint16_t, lp);
+                const float z = Elem<E>::from_bits(bits);
+                bits = Elem<E>::to_bits((z - m) - lse);  // src/model/eagle.cuh:87
             }
             key = make_key(bits, idx);
         }
@@ -118,6 +119,10 @@ __global__ __launch_bounds__(kTopkThreads) void topk_chunk_kernel(TopkParams p) 
         select_topk(keys, p.top, [&](int round, uint64_t key) { out[round] = key; });
     }
 }
+
+template <bool LOGSOFTMAX>
+__global__ __launch_bounds__(kTopkThreads) void topk_chunk_kernel(TopkParams p) { topk_chunk_body<LOGSOFTMAX, f16>(p); }
+__global__ __launch_bounds__(kTopkThreads) void topk_chunk_bf16_kernel(TopkParams p) { topk_chunk_body<true, bf16>(p); }
 
 template <bool LOGSOFTMAX>
 __global__ __launch_bounds__(kTopkThreads) void topk_merge_kernel(TopkParams p) {
@@ -162,8 +167,8 @@ constexpr int kRowMaxTop = 64;                         // the wave-level bound n
 typedef int16_t s16x2 __attribute__((ext_vector_type(2)));
 typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
 
-template <bool LOGSOFTMAX>
-__global__ __launch_bounds__(kRowThreads) void topk_row_kernel(TopkParams p) {
+template <bool LOGSOFTMAX, typename E>
+__device__ __forceinline__ void topk_row_body(const TopkParams& p) {
     __shared__ __attribute__((aligned(16))) uint64_t cand[kRowCap];
     __shared__ int rank[kRowCap];
     __shared__ uint64_t wave_best[2][kRowWaves];
@@ -270,13 +275,14 @@ __global__ __launch_bounds__(kRowThreads) void topk_row_kernel(TopkParams p) {
         lse = row_m_lse[1];
         if (bound > 0) {
             const uint16_t zb = (uint16_t)((bound & 0x8000u) ? (bound ^ 0x8000u) : (bound ^ 0xFFFFu));
-            const float zl = (float)__builtin_bit_cast(f16, zb);
-            const f16 y = (f16)((zl - m) - lse);
-            const int e = (__builtin_bit_cast(uint16_t, y) >> 10) & 31;
-            const float zlo = zl - 4.f * ldexpf(1.f, e ? e - 25 : -24);
+            const float zl = Elem<E>::from_bits(zb);
+            const uint16_t y = Elem<E>::to_bits((zl - m) - lse);
+            constexpr int kM = Elem<E>::kMantissaBits, kBias = Elem<E>::kExponentBias, kEmax = (1 << Elem<E>::kExponentBits) - 1;
+            const int e = (y >> kM) & kEmax;
+            const float zlo = zl - 4.f * ldexpf(1.f, e ? e - kBias - kM : 1 - kBias - kM);  // four ulps of the mapped bound
             lo = 0;
-            if (e != 31 && zlo == zlo && fabsf(zlo) <= 65504.f) {  // finite mapped bound, representable lower bound
-                const uint16_t lb = __builtin_bit_cast(uint16_t, (f16)zlo);
+            if (e != kEmax && zlo == zlo && fabsf(zlo) <= Elem<E>::kMaxFinite) {  // finite mapped bound, representable lower bound
+                const uint16_t lb = Elem<E>::to_bits(zlo);
                 const uint32_t o = (uint32_t)(lb ^ ((lb & 0x8000u) ? 0xFFFFu : 0x8000u));
                 lo = o > 2 ? o - 2 : 0;  // one step for the rounding of zlo, one for -0
             }
@@ -286,9 +292,8 @@ __global__ __launch_bounds__(kRowThreads) void topk_row_kernel(TopkParams p) {
     const auto key_from_image = [&](uint32_t o, int idx) -> uint64_t {
         uint16_t bits = (uint16_t)((o & 0x8000u) ? (o ^ 0x8000u) : (o ^ 0xFFFFu));
         if (LOGSOFTMAX) {
-            const float z = (float)__builtin_bit_cast(f16, bits);
-            const f16 lp = (f16)((z - m) - lse);  // src/model/eagle.cuh:87
-            bits = __builtin_bit_cast(uint16_t, lp);
+            const float z = Elem<E>::from_bits(bits);
+            bits = Elem<E>::to_bits((z - m) - lse);  // src/model/eagle.cuh:87
         }
         return make_key(bits, idx);
     };
@@ -412,15 +417,20 @@ __global__ __launch_bounds__(kRowThreads) void topk_row_kernel(TopkParams p) {
     }
 }
 
+template <bool LOGSOFTMAX>
+__global__ __launch_bounds__(kRowThreads) void topk_row_kernel(TopkParams p) { topk_row_body<LOGSOFTMAX, f16>(p); }
+__global__ __launch_bounds__(kRowThreads) void topk_row_bf16_kernel(TopkParams p) { topk_row_body<true, bf16>(p); }
+
 // log_softmax in place (src/model/eagle.cuh:29-89): one workgroup per row.
-__global__ __launch_bounds__(1024) void log_softmax_kernel(uint16_t* x, int dim, float* row_stats) {
+template <typename E>
+__device__ __forceinline__ void log_softmax_body(uint16_t* x, int dim, float* row_stats) {
     __shared__ float red[16];
     const int row = blockIdx.x;
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
     uint16_t* xr = x + (size_t)row * dim;
     float m = -INFINITY;
-    for (int i = tid; i < dim; i += 1024) m = fmaxf(m, (float)__builtin_bit_cast(f16, xr[i]));
+    for (int i = tid; i < dim; i += 1024) m = fmaxf(m, Elem<E>::from_bits(xr[i]));
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
     if (lane == 0) red[wave] = m;
@@ -430,7 +440,7 @@ __global__ __launch_bounds__(1024) void log_softmax_kernel(uint16_t* x, int dim,
     for (int w = 1; w < 16; ++w) m = fmaxf(m, red[w]);
     __syncthreads();
     float s = 0.f;
-    for (int i = tid; i < dim; i += 1024) s += expf((float)__builtin_bit_cast(f16, xr[i]) - m);
+    for (int i = tid; i < dim; i += 1024) s += expf(Elem<E>::from_bits(xr[i]) - m);
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off);
     if (lane == 0) red[wave] = s;
@@ -440,14 +450,16 @@ __global__ __launch_bounds__(1024) void log_softmax_kernel(uint16_t* x, int dim,
     for (int w = 0; w < 16; ++w) s += red[w];
     const float lse = logf(s);
     for (int i = tid; i < dim; i += 1024) {
-        const f16 lp = (f16)(((float)__builtin_bit_cast(f16, xr[i]) - m) - lse);
-        xr[i] = __builtin_bit_cast(uint16_t, lp);
+        xr[i] = Elem<E>::to_bits((Elem<E>::from_bits(xr[i]) - m) - lse);
     }
     if (tid == 0 && row_stats) {
         row_stats[row * 2 + 0] = m;
         row_stats[row * 2 + 1] = lse;
     }
 }
+
+__global__ __launch_bounds__(1024) void log_softmax_kernel(uint16_t* x, int dim, float* row_stats) { log_softmax_body<f16>(x, dim, row_stats); }
+__global__ __launch_bounds__(1024) void log_softmax_bf16_kernel(uint16_t* x, int dim, float* row_stats) { log_softmax_body<bf16>(x, dim, row_stats); }
 
 __global__ void remap_kernel(const int32_t* in, int n, const int32_t* table, int32_t* out) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -485,7 +497,8 @@ int launch_topk(const void* x, int n, int dim, int top, void* val, int32_t* pos,
     p.row_stats = stats ? stats->row_stats : nullptr;
     // rows that fit one workgroup's registers: one launch, no candidate buffer
     if (dim <= kRowMaxDim && dim % 8 == 0 && top <= kRowMaxTop && ((uintptr_t)x & 15) == 0) {
-        if (stats) hipLaunchKernelGGL(topk_row_kernel<true>, dim3(n), dim3(kRowThreads), 0, st, p);
+        if (stats && options().dtype == 1) hipLaunchKernelGGL(topk_row_bf16_kernel, dim3(n), dim3(kRowThreads), 0, st, p);
+        else if (stats) hipLaunchKernelGGL(topk_row_kernel<true>, dim3(n), dim3(kRowThreads), 0, st, p);
         else hipLaunchKernelGGL(topk_row_kernel<false>, dim3(n), dim3(kRowThreads), 0, st, p);
         CPMCU_LAUNCH_CHECK();
         return CPMCU_OK;
@@ -498,7 +511,8 @@ int launch_topk(const void* x, int n, int dim, int top, void* val, int32_t* pos,
     }
     const dim3 grid(p.nchunks, n);
     if (stats) {
-        hipLaunchKernelGGL(topk_chunk_kernel<true>, grid, dim3(kTopkThreads), 0, st, p);
+        if (options().dtype == 1) hipLaunchKernelGGL(topk_chunk_bf16_kernel, grid, dim3(kTopkThreads), 0, st, p);
+        else hipLaunchKernelGGL(topk_chunk_kernel<true>, grid, dim3(kTopkThreads), 0, st, p);
         CPMCU_LAUNCH_CHECK();
         if (p.nchunks > 1) {
             hipLaunchKernelGGL(topk_merge_kernel<true>, dim3(n), dim3(kTopkThreads), 0, st, p);
@@ -535,7 +549,8 @@ extern "C" int cpmcu_topk(const void* x, int n, int dim, int top, void* val, int
 extern "C" int cpmcu_log_softmax(void* x, int n, int dim, float* row_stats, void* stream) {
     CPMCU_CHECK_ARG(x, "log_softmax: null pointer argument");
     CPMCU_CHECK_ARG(n >= 1 && dim >= 1, "log_softmax: bad shape n=%d dim=%d", n, dim);
-    hipLaunchKernelGGL(log_softmax_kernel, dim3(n), dim3(1024), 0, resolve_stream(stream), (uint16_t*)x, dim, row_stats);
+    if (options().dtype == 1) hipLaunchKernelGGL(log_softmax_bf16_kernel, dim3(n), dim3(1024), 0, resolve_stream(stream), (uint16_t*)x, dim, row_stats);
+    else hipLaunchKernelGGL(log_softmax_kernel, dim3(n), dim3(1024), 0, resolve_stream(stream), (uint16_t*)x, dim, row_stats);
     CPMCU_LAUNCH_CHECK();
     return CPMCU_OK;
 }

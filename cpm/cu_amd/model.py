@@ -31,14 +31,15 @@ class PathModel:
     One per process (the library keeps one global model, like the reference); ``close()`` frees it."""
 
     def __init__(self, vocab, layers, hidden, q_heads, kv_heads, memory_limit, scale_lmhead=1.0, frspec_vocab=0,
-                 tree_size=60, num_iter=6, topk=10, draft_layers=1, eagle_window=1024):
+                 tree_size=60, num_iter=6, topk=10, draft_layers=1, eagle_window=1024, dtype=0):
         self.L = _libmod.get()
         self.vocab, self.layers, self.hidden, self.q_heads, self.kv_heads = vocab, layers, hidden, q_heads, kv_heads
         self.tree_size = tree_size
         L = self.L
+        # dtype: 0 = fp16, 1 = bf16 (tensors then hold bfloat16 patterns, whatever 16-bit torch dtype carries them)
         L.init_base_model(ctypes.c_float(memory_limit), vocab, layers, hidden, 4 * hidden, q_heads, kv_heads, HEAD_DIM,
-                          ctypes.c_float(1e-5), 0, 2048, ctypes.c_float(1.0), ctypes.c_float(scale_lmhead), ctypes.c_float(1.0))
-        L.init_minicpm4_eagle_model(draft_layers, num_iter, topk, tree_size, 0, 0, 128, eagle_window, frspec_vocab,
+                          ctypes.c_float(1e-5), int(dtype), 2048, ctypes.c_float(1.0), ctypes.c_float(scale_lmhead), ctypes.c_float(1.0))
+        L.init_minicpm4_eagle_model(draft_layers, num_iter, topk, tree_size, int(dtype), 0, 128, eagle_window, frspec_vocab,
                                     ctypes.c_float(1.0), 1, 1)
         ctx = ctypes.c_int(0)
         L.init_storage(ctypes.byref(ctx))

@@ -20,7 +20,9 @@
  *     RuntimeError, matching how std::invalid_argument / std::runtime_error
  *     cross pybind in the reference.
  *   - "device pointer" = HIP device memory owned by the caller for the duration
- *     of the call; fp16 tensors are IEEE binary16, row-major unless stated.
+ *     of the call; "fp16" tensors are 16-bit floating point in the element type in
+ *     force -- IEEE binary16 by default, bfloat16 under torch_dtype = 1 / the "dtype"
+ *     option below -- row-major unless stated.
  *   - `stream` is a hipStream_t passed as void*; NULL selects the library's own
  *     blocking stream (the counterpart of calc_stream, src/utils.cu:6,19).
  *   - operator-level calls only enqueue work; they never synchronise.
@@ -70,6 +72,12 @@ const char* cpmcu_version(void);
 /* No reference counterpart: kernel-shape switches for tests and tuning (process-wide, not thread-safe
  * against concurrent calls).  Initial values come from the environment, read once when the library is
  * first used.
+ *   "dtype"                 element type of every 16-bit floating-point tensor handed to the entry points from now on:
+ *                           0 = IEEE half (default), 1 = bfloat16 -- the two types the reference builds its
+ *                           templates for (src/entry.cu:26-59, torch_dtype).  Process-wide, like the reference's
+ *                           model: cpmcu_init_base_model sets it from its torch_dtype, cpmcu_shutdown puts it
+ *                           back to 0; the operator-level entry points follow whatever is in force.  Kernels
+ *                           that only move values (append, compaction, gathers, weight tiling) do not care;
  *   "attn_kv_groups"        0 = chosen per call (default), 1 / 2 = force the 256-row / the two-KV-group
  *                           shape of the tree-attention kernel (CPMCU_ATTN_KV_GROUPS=1|2);
  *   "head_share_last_pass"  1 = the waves of a workgroup share the row blocks of a partly filled last pass
@@ -89,8 +97,8 @@ int cpmcu_set_option(const char* name, int value);
 /* ------------------------------------------------------------------------- */
 
 /* src/entry.cu:100-136 init_base_model.  Records the target-model geometry.
- * torch_dtype: 0 = fp16 (1 = bf16 is rejected: "dtype not compiled",
- * src/entry.cu:43,52). */
+ * torch_dtype: 0 = fp16, 1 = bf16 (src/entry.cu:26-59; anything else: "dtype not compiled", :43,52).  It becomes the
+ * element type of every call that follows, model-level and operator-level, until cpmcu_shutdown. */
 int cpmcu_init_base_model(float memory_limit, int vocab_size, int num_hidden_layers, int hidden_size,
                           int intermediate_size, int num_attention_heads, int num_key_value_heads,
                           int head_dim, float rms_norm_eps, int torch_dtype, int chunk_length,

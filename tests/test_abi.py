@@ -70,6 +70,6 @@ def test_pybind_module_has_reference_names():
     with pytest.raises(RuntimeError):
         C.init_minicpm4_model(0.9, 1, 1, 1, 1, 1, 1, 128, 1e-5, 0, 1, 1.0, 1.0, 1.0, 0, 0, 0, 0, False)
     with pytest.raises(RuntimeError, match="dtype"):
-        C.init_base_model(0.5, 100, 1, 512, 1024, 32, 2, 128, 1e-5, 1, 2048, 1.0, 1.0, 1.0)
+        C.init_base_model(0.5, 100, 1, 512, 1024, 32, 2, 128, 1e-5, 2, 2048, 1.0, 1.0, 1.0)
     with pytest.raises(ValueError, match="head_dim"):
         C.init_base_model(0.5, 100, 1, 512, 1024, 32, 2, 64, 1e-5, 0, 2048, 1.0, 1.0, 1.0)

@@ -330,7 +330,7 @@ def test_model_level_entry_points(gpu, orc):
         keep.append(t)
         return t.data_ptr()
     with pytest.raises(RuntimeError):
-        L.init_base_model(0.02, V, layers, H, 1024, HQ, HKV, D, 1e-5, 1, 2048, 1.0, 1.0, 1.0)  # bf16 not compiled
+        L.init_base_model(0.02, V, layers, H, 1024, HQ, HKV, D, 1e-5, 2, 2048, 1.0, 1.0, 1.0)  # neither fp16 (0) nor bf16 (1)
     with pytest.raises(ValueError):
         L.init_base_model(0.02, V, layers, H, 1024, HQ, HKV, 64, 1e-5, 0, 2048, 1.0, 1.0, 1.0)  # head_dim
     L.init_base_model(0.02, V, layers, H, 1024, HQ, HKV, D, 1e-5, 0, 2048, 1.0, 0.5, 1.0)

@@ -434,3 +434,109 @@ def test_rope_against_complex_rotation():
     qt, kt = orc.rope(q, k, table=table)
     assert np.array_equal(qt[..., :half], -q[..., half:]) and np.array_equal(qt[..., half:], q[..., :half])
     assert np.array_equal(kt[..., :half], -k[..., half:]) and np.array_equal(kt[..., half:], k[..., :half])
+
+
+# ----------------------------------------------------------------------------- bfloat16 (torch_dtype = 1)
+@pytest.fixture
+def orc_bf16(orc):
+    orc.set_dtype("bf16")
+    yield orc
+    orc.set_dtype("f16")
+
+
+def test_bf16_conversions_against_torch(orc):
+    """Every bfloat16 pattern to float32, and float32 to bfloat16 on random values over the whole exponent range, on the
+    ties between neighbours and at the edges, against torch's CPU conversion (an independent implementation)."""
+    import torch
+    bits = np.arange(65536, dtype=np.uint16)
+    got = orc.bf16_to_f32(bits)
+    ref = torch.from_numpy(bits.view(np.int16)).view(torch.bfloat16).float().numpy()
+    nan = np.isnan(ref)
+    assert np.array_equal(got.view(np.uint32)[~nan], ref.view(np.uint32)[~nan]) and np.all(np.isnan(got[nan]))
+    g = synth.rng(1, 2)
+    x = np.concatenate([
+        g.standard_normal(300000).astype(np.float32) * np.float32(10.0) ** g.integers(-38, 38, 300000).astype(np.float32),
+        np.array([0.0, -0.0, 3.3895314e38, 3.4e38, np.inf, -np.inf, 1e-40, 1.0, 1.00390625, 1.0078125], np.float32),
+        # exact ties between adjacent bfloat16 values (round to even): 1 + (2i + 1) 2^-8
+        1.0 + (2 * np.arange(0, 64, dtype=np.float32) + 1) * np.float32(2.0 ** -8),
+    ])
+    ref_bits = torch.from_numpy(x).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(orc.f32_to_bf16(x), ref_bits)
+    assert np.isnan(orc.bf16_to_f32(orc.f32_to_bf16(np.array([np.nan], np.float32)))).all()
+
+
+def test_bf16_attention_closed_form(orc_bf16):
+    orc = orc_bf16
+    T, P, Hq, Hkv, seed = 60, 333, 32, 2, 1
+    tree = synth.random_tree(T, seed, max_children=4, max_depth=9)
+    enc = lambda shape, stream: orc.encode(synth.rng(seed, stream).standard_normal(shape, dtype=np.float32))
+    q, k, v = enc((T, Hq, 128), 1), enc((P + T, Hkv, 128), 2), enc((P + T, Hkv, 128), 3)
+    out, lse = orc.tree_attention(q, k, v, tree.mask, P, return_lse=True)
+    ref, lse_ref = _attention_fp64(orc.decode(q), orc.decode(k), orc.decode(v), tree.mask, P)
+    # bfloat16 output and bfloat16 P: a few ulps (2^-8 relative) of values that are O(1)
+    assert np.abs(orc.decode(out).astype(np.float64) - ref).max() < 3e-2
+    assert np.abs(lse - lse_ref).max() < 1e-3
+    # and it is not the fp16 oracle on the same bits
+    orc.set_dtype("f16")
+    assert not np.array_equal(orc.tree_attention(q, k, v, tree.mask, P).view(np.uint16), out.view(np.uint16))
+    orc.set_dtype("bf16")
+
+
+def test_bf16_lm_head_log_softmax_and_rounding(orc_bf16):
+    import torch
+    orc = orc_bf16
+    n, V, H = 7, 900, 256
+    hid = orc.encode(synth.rng(6, 1).standard_normal((n, H), dtype=np.float32))
+    w = orc.encode(synth.rng(6, 2).standard_normal((V, H), dtype=np.float32) * 0.05)
+    z = orc.lm_head(hid, w)
+    ref = orc.decode(hid).astype(np.float64) @ orc.decode(w).astype(np.float64).T
+    assert np.abs(orc.decode(z).astype(np.float64) - ref).max() <= np.abs(ref).max() * 2.0 ** -7
+    # the result is the correctly rounded bfloat16 of an fp32 sum that is within fp32 rounding of the fp64 one
+    near = torch.from_numpy(ref.astype(np.float32)).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert (near == z.view(np.uint16)).mean() > 0.98
+    # head_scale: the hidden rows are pre-scaled and ROUNDED to bfloat16 before the product, the scale itself rounded too
+    sc = 0.3
+    sc_r = orc.decode(orc.encode(np.array([sc], np.float32)))[0]
+    pre = orc.encode(orc.decode(hid) * np.float32(sc_r))
+    assert np.array_equal(orc.lm_head(hid, w, head_scale=sc).view(np.uint16), orc.lm_head(pre, w).view(np.uint16))
+    # log-softmax: rounded once to bfloat16 from (x - m) - lse in fp32
+    x = orc.encode(synth.rng(7, 1).standard_normal((4, 5000), dtype=np.float32) * 2)
+    lp, m, lse = orc.log_softmax(x)
+    xf = orc.decode(x)
+    assert np.array_equal(m, xf.max(1))
+    ref_lp = torch.from_numpy((xf - m[:, None]) - lse[:, None]).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(lp.view(np.uint16), ref_lp)
+    assert np.allclose(lse, scipy.special.logsumexp(xf.astype(np.float64), axis=1) - m, atol=1e-5)
+    # the ranking is on bit patterns: value descending, lower index first among equals, as for fp16
+    val, pos = orc.topk(lp, 10)
+    lpf = orc.decode(lp)
+    ref_pos = np.stack([np.lexsort((np.arange(lpf.shape[1]), -r))[:10] for r in lpf]).astype(np.int32)
+    assert np.array_equal(pos, ref_pos)
+
+
+def test_bf16_rope_and_running_log_probs(orc_bf16):
+    """Rotary pairs and the drafter's running sums are rounded to bfloat16 (torch's conversion as the independent rounding)."""
+    import torch
+    orc = orc_bf16
+    T, Hq, Hkv, Dh = 5, 4, 2, 128
+    q = orc.encode(synth.rng(9, 1).standard_normal((T, Hq, Dh), dtype=np.float32))
+    k = orc.encode(synth.rng(9, 2).standard_normal((T, Hkv, Dh), dtype=np.float32))
+    pos = np.arange(100, 100 + T, dtype=np.int32)
+    inv_freq = (1.0 / (10000.0 ** (np.arange(0, Dh, 2, dtype=np.float32) / Dh))).astype(np.float32)
+    qr, kr = orc.rope(q, k, pos=pos, inv_freq=inv_freq)
+    ang = pos[:, None].astype(np.float32) * inv_freq[None, :]
+    c, s = np.cos(ang).astype(np.float32)[:, None, :], np.sin(ang).astype(np.float32)[:, None, :]
+    qf = orc.decode(q)
+    a, b = qf[..., :64], qf[..., 64:]
+    ref = np.concatenate([a * c - b * s, a * s + b * c], axis=-1).astype(np.float32)
+    ref_bits = torch.from_numpy(ref).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert (ref_bits == qr.view(np.uint16)).mean() > 0.999  # (cos / sin of the host library may differ in their last bit)
+    k_it = 4
+    t = orc.DraftTree(k_it, 3)
+    v0 = orc.encode(np.array([-0.11, -0.7, -1.3, -2.9], np.float32))
+    t.begin(v0, np.arange(k_it, dtype=np.int32))
+    rows = orc.encode(-np.abs(synth.rng(9, 3).standard_normal((k_it, k_it), dtype=np.float32)))
+    rows = orc.encode(-np.sort(-orc.decode(rows), axis=1))
+    _, _, summed = t.extend(1, rows, np.arange(k_it * k_it, dtype=np.int32).reshape(k_it, k_it))
+    ref = torch.from_numpy(orc.decode(rows) + orc.decode(v0)[:, None]).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    assert np.array_equal(summed.view(np.uint16), ref)
