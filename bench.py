@@ -435,7 +435,7 @@ def main():
     bytes_head = V * H * 2.0 + T * H * 2.0 + T * 4.0
 
     # ---- per-operator timings on the main workload (operator level, same pools and buffers, graph-replayed) ----
-    kernels, frspec, cold, draft, rope_cmp = [], None, None, None, None
+    kernels, frspec, cold, draft, rope_cmp, bf16 = [], None, None, None, None, None
     attn_tflops = flops_attn(P) / (ms_attn * 1e-3) / 1e12
     attn_name = main_run["attn_plan"][0]
     kernels.append(dict(kernel=attn_name, launches_per_step=L, us_per_launch=round(ms_attn * 1e3, 2), bound="mfma",
@@ -657,6 +657,31 @@ def main():
                  "note": "us_per_draft: cpmcu_draft_round / cpmcu_draft_attention / cpmcu_draft_finish on the library's model, "
                          "replayed as a library graph; us_per_draft_cold_matrix: the same operators with every round reading a "
                          "different copy of the FR-Spec matrix (as after the drafter layer's dense weights)"}
+        # ---- the same kernels in bfloat16 (torch_dtype = 1): timing only, on the same buffers read as bfloat16 patterns ----
+        lib.get().set_option(b"dtype", 1)
+        try:
+            def attn_bf16():
+                for l in range(L):
+                    ops.tree_attention(bufs.q[l], cache0, l, kvlen, padded, mask, out=bufs.attn_out[l], k_new=bufs.k_new[l], v_new=bufs.v_new[l])
+
+            def head_bf16():
+                for _ in range(HEAD_REP):
+                    ops.lm_head_partials(bufs.hidden, w_t)
+
+            as_bf16 = lambda t: t.to(torch.bfloat16).view(torch.float16)  # the same values, rounded to bfloat16, as 16-bit patterns
+            w_subs_bf16 = [ops.tile_head_weight(as_bf16(w_dev), remap) for _ in range(FR_SETS)]
+            hid10_bf16 = as_bf16(hid10)
+
+            def fr_bf16():
+                for w in w_subs_bf16:
+                    ops.frspec_head_topk(hid10_bf16, w, remap, 10)
+            bf16 = {"attention_us_per_layer_one_kv_set": round(timed_torch(torch, attn_bf16, reps, 2) / L * 1e3, 2),
+                    "target_head_us": round(timed_torch(torch, head_bf16, reps, 2, warm_ms=WARM_MS) / HEAD_REP * 1e3, 2),
+                    "frspec_head_us_per_call_cold": round(timed_torch(torch, fr_bf16, reps, 2, warm_ms=WARM_MS) / FR_SETS * 1e3, 2),
+                    "note": "the bfloat16 instantiations of the same kernels (v_mfma_*_bf16), same shapes; the headline runs in fp16"}
+        finally:
+            lib.get().set_option(b"dtype", 0)
+        del w_subs_bf16
         del w_subs, dtree, dcache, w_t
         torch.cuda.empty_cache()
 
@@ -784,6 +809,7 @@ def main():
         "cold_cache": cold,
         "draft_path": draft,
         "attention_with_rope": rope_cmp,
+        "bf16": bf16,
         "contexts_us_per_step": contexts,
         "attention_by_context": ctx_attn,
         "cpu_baseline": cpu,
