@@ -516,7 +516,7 @@ def test_merge_counter_blocks_stay_with_their_workspaces(gpu):
 def test_merge_wait_that_runs_out_leaves_the_share_to_the_last_arrival(gpu, set_option, P, T):
     """With the wait limit at zero every workgroup but the last of a unit gives up at once (unless everyone has
     arrived already), marks its share as abandoned and leaves; the last arrival merges those shares.  The output must be
-    what the separate merge launch gives, bit for bit, and the marks must be gone for the next call."""
+    what the separate merge launch gives, bit for bit, the counter of abandoned waits must say so, and the next call must be whole again."""
     torch = gpu
     from cpm.cu_amd import lib, ops
     from cpm.cu_amd.kvcache import PagedKVCache
