@@ -558,7 +558,7 @@ def main():
         FR_SETS = 3
         w_subs = [ops.tile_head_weight(w_dev, remap) for _ in range(FR_SETS)]  # remap_copy fused with the re-tiling
         hid10 = bufs.hidden[:10].contiguous()
-        fr_name = ops.head_plan(10, w_subs[0])[0] + "+topk_row_kernel<true>"
+        fr_name = ops.frspec_head_plan(10, w_subs[0], 10)
 
         def fr_head():
             for _ in range(HEAD_REP):
@@ -568,6 +568,13 @@ def main():
         fr_gbs = fr_bytes / (ms_fr * 1e-3) / 1e9
         frspec = dict(kernel=fr_name, us_per_call=round(ms_fr * 1e3, 2), bound="hbm", achieved=round(fr_gbs, 1), peak=HBM_PEAK_GBS,
                       unit="GB/s", frac=round(fr_gbs / HBM_PEAK_GBS, 4))
+
+        # the same call as ONE launch (option frspec_fused: every GEMM workgroup publishes its best keys per row as tagged
+        # words, the first workgroups to finish rank a row each), which is no faster and therefore not the default
+        lib.get().set_option(b"frspec_fused", 1)
+        frspec["one_launch_kernel"] = ops.frspec_head_plan(10, w_subs[0], 10)
+        frspec["one_launch_us_per_call"] = round(timed_torch(torch, fr_head, reps, 2, warm_ms=WARM_MS) / HEAD_REP * 1e3, 2)
+        lib.get().set_option(b"frspec_fused", 0)
 
         # through the library's own sub-matrix and buffers (cpmcu_draft_head)
         fr_val = torch.zeros((10, 10), dtype=torch.float16, device="cuda")
@@ -591,6 +598,10 @@ def main():
                 "frspec_frac_hbm": round(fr_bytes / (ms_fr_cold * 1e-3) / 1e9 / HBM_PEAK_GBS, 4),
                 "note": "the FR-Spec head with every replay walking distinct copies of its matrix, so that no pass is served "
                         "from the 256 MB last-level cache; frspec_head above replays one copy"}
+
+        lib.get().set_option(b"frspec_fused", 1)
+        cold["frspec_one_launch_us_per_call"] = round(timed_torch(torch, fr_cold, reps, 2, warm_ms=WARM_MS) / FR_SETS * 1e3, 2)
+        lib.get().set_option(b"frspec_fused", 0)
 
         # ---- the draft side of the path: one whole draft of the FR-Spec drafter (6 rounds of 10) ----
         # Per round: the drafter layer's own attention (10 queries, mask over 10*d columns, block sliding window of 1024

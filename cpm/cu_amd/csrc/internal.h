@@ -14,6 +14,8 @@ struct Options {
     int head_stream_kernel = 1;    // 0 keeps tiled weights on the K-chunked kernel (tests compare the two)
     int attn_merge_in_launch = 1;  // 0: the split partials of tree attention are always merged by a launch of their own
     int attn_merge_wait_us = 2000; // longest wait of a workgroup for the others of its merge before it abandons its share
+    int frspec_fused = 0;          // 1: the FR-Spec head with its top-k as one launch where the shape allows (measured no faster: off)
+    int frspec_wait_us = 50000;    // longest wait of a finisher of the fused FR-Spec launch for the other workgroups' words
 };
 Options& options();
 
@@ -50,6 +52,18 @@ int launch_head_gemm(const void* hidden, const void* w, int w_layout, int n, int
                      int mode, void* logits, float* part_a, float* part_b, int* grid_out, int* stride_out,
                      hipStream_t st, HeadShape* shape_out = nullptr, bool dry_run = false);
 int head_max_grid();
+// The FR-Spec head with its log-softmax, top-k and id map-back in one launch, when the shape allows it and one of the
+// library's publication states is free for (workspace, grid); *launched = false: the caller runs the two launches.
+int launch_frspec_fused(const void* hidden, const void* w, int w_layout, const int32_t* token_id_remap, int n, int V, int H, int k,
+                        void* logits, float* row_stats, void* topk_val, int32_t* topk_pos, int32_t* topk_ids, const void* workspace,
+                        hipStream_t st, bool* launched, bool dry_run = false);
+void head_fuse_release_workspace(const void* workspace);
+// What fused launches left behind: finishers whose wait ran out (their rows hold -1 / NaN and the call has failed), rows
+// redone from the logits in memory, rows finished from the published candidates.  enqueue: copy to pinned host memory
+// in stream order; take: read that copy after the synchronisation and clear what was found.
+int head_fuse_report_enqueue(hipStream_t st);
+int head_fuse_report_take(unsigned int* timeouts, unsigned int* slow_rows, unsigned int* fused_rows);
+void head_fuse_reenable();
 
 // topk.hip -- exact top-k (value descending, ties -> lower index) with an optional fused
 // log-softmax transform whose row statistics come from the GEMM's per-workgroup partials.

@@ -26,8 +26,11 @@
 //   * when the row blocks do not divide evenly over the wave slots, the blocks of the partly
 //     filled last pass are dealt round-robin to the workgroups and several waves share each of
 //     them, every one taking a subset of the K chunks; their partial sums meet in LDS.
+#include <map>
 #include <mutex>
+#include <tuple>
 #include <type_traits>
+#include <vector>
 
 #include "common.h"
 #include "internal.h"
@@ -71,6 +74,60 @@ struct HeadCfg {
     static constexpr int kLdsBuf = NB * 16 * kLdsRowMax;
     static constexpr int kStage = 8;                     // 16-byte staging registers per thread
 };
+
+// ---- FR-Spec head with its log-softmax / top-k / id map-back in the same launch -------------------------------------
+// (src/model/minicpm4/minicpm4_eagle.cuh:366-372: Linear::prefill, log_softmax, TopK::prefill, remap as four+ launches.)
+// Every GEMM workgroup ranks its own logits of a hidden row first (the k..16 largest as (value, index) keys, ties to
+// the lower index) and publishes them, with the row's partial (max, sum exp), as self-validating 64-bit words: each
+// word carries the generation of its row, is written by one device-scope store and read by one device-scope load, so
+// a reader that sees the generation sees the payload -- no fence, no acknowledged store, no arrival counter between
+// producer and consumer.  The first n workgroups to finish (a ticket each) become the finishers of one row each:
+// they poll that row's words of all workgroups, rank the few candidates at or above a bound exactly as the row
+// kernel of topk.hip does, and write the outputs.  What the words cannot decide -- a workgroup with more candidates
+// than slots (rows dominated by one value) -- is redone from the logits in memory, which every workgroup marks
+// complete after its stores have been acknowledged.
+constexpr int kFuseStates = 8;      // (workspace, grid) pairs per device that can have a launch in flight or captured
+constexpr int kFuseMaxGrid = 256;
+constexpr int kFuseRows = 16;
+constexpr int kFuseSlots = 16;
+constexpr int kFuseCap = kHeadThreads;  // candidate keys a finisher ranks
+constexpr int kFuseIdBits = 20;
+constexpr uint32_t kFuseCandTagMask = 0x7FFFFu;
+
+struct HeadFuseState {
+    unsigned long long tickets;  // never reset: a launch of G workgroups takes G of them, ticket % G is the order of finishing
+    uint32_t gen[kFuseRows];     // generation of each hidden row's words; advanced by the row's finisher
+    uint32_t pad[46];
+    uint64_t done[kFuseMaxGrid];                        // generation of row 0 | this workgroup's logits are in memory
+    uint64_t stats[kFuseRows][kFuseMaxGrid];            // tag:16 | max z (element bits):16 | sum exp (fp32 bits, sign = wide ids)
+    uint64_t cand[kFuseRows][kFuseMaxGrid][kFuseSlots];  // tag:19 | ordered image of z:16 | index within the workgroup:9 | token id:20
+};
+static_assert(sizeof(HeadFuseState) % 256 == 0, "states stay 256-byte aligned");
+__device__ __attribute__((aligned(256))) HeadFuseState g_head_fuse[kFuseStates];
+struct HeadFuseReport {
+    unsigned int timeouts;    // finishers whose wait ran out (their rows were not written)
+    unsigned int slow_rows;   // rows redone from the logits in memory
+    unsigned int fused_rows;  // rows finished from the published candidates
+};
+__device__ HeadFuseReport g_head_fuse_report;
+
+struct FuseParams {
+    HeadFuseState* st;
+    int top;
+    const int32_t* remap;
+    uint16_t* val;
+    int32_t* pos;
+    int32_t* ids;
+    float* row_stats;
+    uint32_t wait_ticks;  // longest wait of a finisher, in ticks of the 100 MHz wall clock
+};
+
+__device__ inline uint64_t fuse_load(const uint64_t* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ inline void fuse_store(uint64_t* p, uint64_t v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+// A workgroup publishes at least this many keys of a row (all it has, if fewer): with small k a few more than k, so that
+// a workgroup whose every published key is a candidate -- the case the finisher cannot decide -- stays rare.
+__device__ inline int fuse_publish_min(int top) { return top > 8 ? top : 8; }
+__device__ inline uint16_t image_to_bits(uint32_t o) { return (uint16_t)((o & 0x8000u) ? (o ^ 0x8000u) : (o ^ 0xFFFFu)); }
 
 // Folds one finished 16-row block of W (acc[nb][r] <-> vocab row vrow0 + r, hidden row nb*16 + l16) into
 // the lane's running epilogue state and writes its logits when asked to.
@@ -140,9 +197,9 @@ __device__ inline void head_epilogue(const HeadParams& p, const f32x4 (&acc)[NB]
 
 // Reduces the epilogue state over the lanes that share a hidden row, then over the waves, and writes
 // the workgroup's partials.
-template <int NB>
-__device__ inline void head_finish(const HeadParams& p, float (&ea)[NB], float (&eb)[NB], float (*red_a)[NB * 16], float (*red_b)[NB * 16],
-                                   int tid, int wave, int lane, int c) {
+template <int NB, typename Write>
+__device__ inline void head_finish_with(const HeadParams& p, float (&ea)[NB], float (&eb)[NB], float (*red_a)[NB * 16], float (*red_b)[NB * 16],
+                                        int tid, int wave, int lane, Write write) {
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
 #pragma unroll
@@ -180,9 +237,16 @@ __device__ inline void head_finish(const HeadParams& p, float (&ea)[NB], float (
                 b = ob;
             }
         }
-        p.part_a[(size_t)c * (NB * 16) + tid] = a;
-        p.part_b[(size_t)c * (NB * 16) + tid] = b;
+        write(tid, a, b);
     }
+}
+template <int NB>
+__device__ inline void head_finish(const HeadParams& p, float (&ea)[NB], float (&eb)[NB], float (*red_a)[NB * 16], float (*red_b)[NB * 16],
+                                   int tid, int wave, int lane, int c) {
+    head_finish_with<NB>(p, ea, eb, red_a, red_b, tid, wave, lane, [&](int row, float a, float b) {
+        p.part_a[(size_t)c * (NB * 16) + row] = a;
+        p.part_b[(size_t)c * (NB * 16) + row] = b;
+    });
 }
 
 template <int NB, typename E>
@@ -551,6 +615,313 @@ __device__ __forceinline__ void head_gemm_chunked_body(const HeadParams& p) {
     head_finish<NB>(p, ea, eb, red_a, red_b, tid, wave, lane, c);
 }
 
+// One finished 16-row block of W in the fused FR-Spec launch: the logits (written through, so that a finisher in another
+// XCD can read them once they are marked complete), the running statistics exactly as head_epilogue's STATS branch
+// keeps them, and one ranking key per element in LDS: ordered image of z << 16 | (0xFFFF - index within the workgroup).
+template <typename E>
+__device__ inline void fuse_epilogue(const HeadParams& p, const f32x4& acc, int vrow0, int lidx0, int l16, float& ea, float& eb,
+                                     uint32_t* keys_row) {
+    if (l16 >= p.n) return;
+    typename Elem<E>::x4 zz;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) zz[r] = (E)acc[r];
+    uint32_t kk[4] = {0u, 0u, 0u, 0u};
+    if (vrow0 < p.V) {  // V % 8 == 0 in this launch: the four rows are inside or outside together
+        fuse_store(reinterpret_cast<uint64_t*>(reinterpret_cast<E*>(p.logits) + (size_t)l16 * p.V + vrow0), __builtin_bit_cast(uint64_t, zz));
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float x = (float)zz[r];
+            kk[r] = (ord16(Elem<E>::to_bits(x)) << 16) | (uint32_t)(0xFFFF - (lidx0 + r));
+            if (x == -INFINITY) continue;
+            if (x > ea) {
+                eb = eb * __expf(ea - x) + 1.f;
+                ea = x;
+            } else {
+                eb += __expf(x - ea);
+            }
+        }
+    }
+    *reinterpret_cast<uint4*>(keys_row + lidx0) = make_uint4(kk[0], kk[1], kk[2], kk[3]);
+}
+
+// The finisher of hidden row R (all threads of one workgroup, after its own words are out).
+template <typename E>
+__device__ __forceinline__ void fuse_finish_row(const HeadParams& p, const FuseParams& fp, int R, uint32_t gen_row, uint32_t gen_done) {
+    __shared__ uint64_t s_cand[kFuseCap];
+    __shared__ uint64_t s_raw[kFuseCap];
+    __shared__ uint16_t s_rslice[kFuseCap];
+    __shared__ int s_rank[kFuseCap];
+    __shared__ uint32_t s_wave_kth[kHeadWaves];
+    __shared__ uint64_t s_wave_best[2][kHeadWaves];
+    __shared__ float s_m_lse[2];
+    __shared__ int s_ncand, s_slow, s_timeout, s_wide;
+    HeadFuseState* st = fp.st;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int G = gridDim.x, top = fp.top, V = p.V;
+    const uint32_t g1 = gen_row + 1;
+    const uint64_t ctag = (uint64_t)(g1 & kFuseCandTagMask);
+    const uint64_t stag = (uint64_t)(g1 & 0xFFFFu);
+    // thread -> (workgroup's slice, half of its slots), from the last thread down: wave 0, which reduces the
+    // statistics while the others search the bound, is the first to go without data when G < 256
+    const int u = kHeadThreads - 1 - tid;
+    const int slice = u >> 1, half = u & 1;
+    const bool have = slice < G;
+    const uint64_t* cw = &st->cand[R][have ? slice : 0][half * 8];
+    if (tid == 0) {
+        s_ncand = 0;
+        s_slow = 0;
+        s_timeout = 0;
+        s_wide = 0;
+    }
+    s_cand[tid] = 0;
+    s_rank[tid] = 0;
+    __syncthreads();
+    uint64_t w[8], sw[4];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) w[i] = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) sw[i] = 0;
+    const unsigned long long t_begin = wall_clock64();
+    bool late = false;
+    for (;;) {
+        bool ok = true;
+        if (have) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) w[i] = fuse_load(cw + i);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) ok = ok && (w[i] >> 45) == ctag;
+        }
+        if (wave == 0) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int c = lane + i * 64;
+                if (c < G) {
+                    sw[i] = fuse_load(&st->stats[R][c]);
+                    ok = ok && (sw[i] >> 48) == stag;
+                }
+            }
+        }
+        if (ok) break;
+        if (wall_clock64() - t_begin >= fp.wait_ticks) {
+            late = true;
+            break;
+        }
+        __builtin_amdgcn_s_sleep(1);  // a thread leaves the loop with its own words, so few keep asking towards the end
+    }
+    if (late) s_timeout = 1;
+    __syncthreads();
+    if (s_timeout) {
+        // some workgroup's words never came (it was not resident within the wait): the row is not written; the host
+        // reads the count at its next synchronisation and reports the call as failed
+        if (tid < top) {
+            fp.val[(size_t)R * top + tid] = 0xFFFFu;
+            fp.pos[(size_t)R * top + tid] = -1;
+            if (fp.ids) fp.ids[(size_t)R * top + tid] = -1;
+        }
+        if (tid == 0) {
+            __hip_atomic_fetch_add(&g_head_fuse_report.timeouts, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            st->gen[R] = g1;
+        }
+        return;
+    }
+    uint32_t img[8], tmax = 0, tmin = 0xFFFFFFFFu;
+    int nonempty = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        img[i] = (uint32_t)(w[i] >> 29) & 0xFFFFu;
+        tmax = img[i] > tmax ? img[i] : tmax;
+        if (img[i]) {
+            tmin = img[i] < tmin ? img[i] : tmin;
+            ++nonempty;
+        }
+    }
+    // k-th largest of this wave's thread maxima (a lower bound of the row's k-th largest value), waves 1..7;
+    // wave 0: the row statistics, in the order topk_row_kernel reduces the same partials
+    uint32_t kth = 0;
+    if (wave != 0) {
+        for (int bit = 15; bit >= 4; --bit) {
+            const uint32_t c = kth | (1u << bit);
+            if (__popcll(__ballot(tmax >= c)) >= top) kth = c;
+        }
+    } else {
+        float pa[4], pb[4];
+        bool wide = false;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const bool in = lane + i * 64 < G;
+            pa[i] = in ? (float)Elem<E>::from_bits((uint16_t)(sw[i] >> 32)) : -INFINITY;
+            pb[i] = in ? __uint_as_float((uint32_t)sw[i] & 0x7FFFFFFFu) : 0.f;
+            wide = wide || (in && ((uint32_t)sw[i] >> 31));
+        }
+        const float a = fmaxf(fmaxf(-INFINITY, fmaxf(pa[0], pa[1])), fmaxf(pa[2], pa[3]));
+        float b = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) b += (pa[i] == -INFINITY) ? 0.f : pb[i] * __expf(pa[i] - a);
+        const float wm = wave_max_f32(a);
+        b = wave_sum_f32((a == -INFINITY) ? 0.f : b * __expf(a - wm));
+        const bool any_wide = __ballot(wide) != 0;
+        if (lane == 0) {
+            const float l = __logf(b);
+            s_m_lse[0] = wm;
+            s_m_lse[1] = l;
+            if (any_wide) s_wide = 1;
+            if (fp.row_stats) {
+                fp.row_stats[R * 2 + 0] = wm;
+                fp.row_stats[R * 2 + 1] = l;
+            }
+        }
+    }
+    if (lane == 0) s_wave_kth[wave] = kth;
+    __syncthreads();
+    uint32_t bound = 0;
+#pragma unroll
+    for (int i = 1; i < kHeadWaves; ++i) bound = s_wave_kth[i] > bound ? s_wave_kth[i] : bound;
+    const float m = s_m_lse[0], lse = s_m_lse[1];
+    const uint32_t lo = mapped_lower_image<E>(bound, m, lse);
+    const auto key_of = [&](uint16_t zbits, int idx) -> uint64_t {
+        const float z = Elem<E>::from_bits(zbits);
+        return make_key(Elem<E>::to_bits((z - m) - lse), idx);  // src/model/eagle.cuh:87
+    };
+    {
+        // A workgroup published its largest keys only (at least fuse_publish_min of them, or all it had).  What it held
+        // back is below all of them, so the candidates of the row are complete unless some workgroup's smallest
+        // published value is itself a candidate.
+        const uint32_t omin = (uint32_t)__shfl_xor((int)tmin, 1);
+        const int ocnt = __shfl_xor(nonempty, 1);
+        const uint32_t smin = omin < tmin ? omin : tmin;
+        if (lo == 0 || (have && nonempty + ocnt >= fuse_publish_min(top) && smin >= lo)) s_slow = 1;
+        // The raw words of everything at or above lo go to LDS: slots by ballot prefix sums, one LDS atomic per wave;
+        // the keys are computed afterwards, one candidate per thread.
+        const uint64_t lanes_below = (1ull << lane) - 1ull;
+        int off[8], total = 0;
+        uint32_t em = 0;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const bool is_cand = lo != 0 && img[i] >= lo;
+            const uint64_t mk = __ballot(is_cand);
+            off[i] = total + __popcll(mk & lanes_below);
+            total += __popcll(mk);
+            em |= is_cand ? (1u << i) : 0u;
+        }
+        int base = 0;
+        if (lane == 0 && total) base = atomicAdd(&s_ncand, total);
+        base = __builtin_amdgcn_readfirstlane(base);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            if ((em & (1u << i)) && base + off[i] < kFuseCap) {
+                s_raw[base + off[i]] = w[i];
+                s_rslice[base + off[i]] = (uint16_t)slice;
+            }
+        }
+    }
+    __syncthreads();
+    const int C = s_ncand;
+    if (!s_slow && C <= kFuseCap) {
+        int32_t mapped = 0;
+        if (tid < C) {
+            const uint64_t x = s_raw[tid];
+            const int lidx = (int)((x >> kFuseIdBits) & 0x1FFu);
+            const int idx = ((lidx >> 4) * G + (int)s_rslice[tid]) * 16 + (lidx & 15);
+            s_cand[tid] = key_of(image_to_bits((uint32_t)(x >> 29) & 0xFFFFu), idx);
+            mapped = (int)((uint32_t)x & ((1u << kFuseIdBits) - 1u));
+            if (s_wide) mapped = fp.remap ? fp.remap[idx] : idx;
+        }
+        __syncthreads();
+        int shift = 6;
+        while ((1 << shift) < C) ++shift;
+        const int i = tid & ((1 << shift) - 1);
+        const int part = tid >> shift, nparts = kHeadThreads >> shift;
+        if (i < C) {
+            // slots from C on hold key 0, so whole groups of eight can be compared
+            const uint64_t my = s_cand[i];
+            const int chunk = ((C + nparts - 1) / nparts + 7) & ~7;
+            int r = 0;
+            for (int j = part * chunk; j < (part + 1) * chunk && j < kFuseCap; j += 8) {
+                uint64_t o[8];
+#pragma unroll
+                for (int q = 0; q < 8; ++q) o[q] = s_cand[j + q];
+#pragma unroll
+                for (int q = 0; q < 8; ++q) r += o[q] > my ? 1 : 0;
+            }
+            if (r) atomicAdd(&s_rank[i], r);
+        }
+        __syncthreads();
+        if (tid < C && s_rank[tid] < top) {
+            const uint64_t key = s_cand[tid];
+            const size_t o = (size_t)R * top + s_rank[tid];
+            fp.val[o] = key_bits(key);
+            fp.pos[o] = key_index(key);
+            if (fp.ids) fp.ids[o] = mapped;
+        }
+        if (tid == 0) {
+            __hip_atomic_fetch_add(&g_head_fuse_report.fused_rows, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            st->gen[R] = g1;
+        }
+        return;
+    }
+    // From the logits in memory: every workgroup marks its part complete once its stores have been acknowledged.
+    {
+        bool late2 = false;
+        if (tid < G) {
+            while (fuse_load(&st->done[tid]) != (uint64_t)(gen_done + 1)) {
+                if (wall_clock64() - t_begin >= fp.wait_ticks) {
+                    late2 = true;
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(8);
+            }
+        }
+        if (late2) s_timeout = 1;
+    }
+    __syncthreads();
+    if (s_timeout) {
+        if (tid < top) {
+            fp.val[(size_t)R * top + tid] = 0xFFFFu;
+            fp.pos[(size_t)R * top + tid] = -1;
+            if (fp.ids) fp.ids[(size_t)R * top + tid] = -1;
+        }
+        if (tid == 0) {
+            __hip_atomic_fetch_add(&g_head_fuse_report.timeouts, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            st->gen[R] = g1;
+        }
+        return;
+    }
+    const uint64_t* xr = reinterpret_cast<const uint64_t*>(reinterpret_cast<const uint16_t*>(p.logits) + (size_t)R * V);
+    const int nquads = V >> 2;
+    uint64_t prev = ~0ull;
+    for (int round = 0; round < top; ++round) {
+        uint64_t mine = 0;
+        for (int q = tid; q < nquads; q += kHeadThreads) {
+            const uint64_t x4 = fuse_load(xr + q);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const uint64_t key = key_of((uint16_t)(x4 >> (16 * e)), q * 4 + e);
+                if (key < prev && key > mine) mine = key;
+            }
+        }
+        const uint64_t wbest = wave_max_u64(mine);
+        uint64_t* wb = s_wave_best[round & 1];
+        if (lane == 0) wb[wave] = wbest;
+        __syncthreads();
+        uint64_t best = wb[0];
+#pragma unroll
+        for (int i = 1; i < kHeadWaves; ++i) best = wb[i] > best ? wb[i] : best;
+        if (tid == 0 && best != 0) {
+            const int idx = key_index(best);
+            const size_t o = (size_t)R * top + round;
+            fp.val[o] = key_bits(best);
+            fp.pos[o] = idx;
+            if (fp.ids) fp.ids[o] = fp.remap ? fp.remap[idx] : idx;
+        }
+        prev = best;
+        if (best == 0) break;
+    }
+    if (tid == 0) {
+        __hip_atomic_fetch_add(&g_head_fuse_report.slow_rows, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        st->gen[R] = g1;
+    }
+}
+
 // Tiled weights whose row blocks fit one sweep: FP full passes (every wave one whole row block each) and at most
 // one partly filled last pass.  The wave's W stream is a ring of 1 KB fragments held in registers and refilled
 // fragment by fragment: as soon as the MFMAs of a (row block, K step) have read their fragment, the same registers
@@ -571,8 +942,8 @@ __device__ __forceinline__ void head_gemm_chunked_body(const HeadParams& p) {
 //   wave-uniform branches (their count is a run-time value); the ring has PD extra slots for them, and what the
 //   compiler has to assume about them costs the full passes at most that many fragments of look-ahead.
 //   The hidden chunk is brought in as in the kernel above (direct-to-LDS, double buffered, XOR-swizzled).
-template <int NB, int FP, int KC, typename E>
-__device__ __forceinline__ void head_gemm_stream_body(const HeadParams& p) {
+template <int NB, int FP, int KC, typename E, bool FUSE = false>
+__device__ __forceinline__ void head_gemm_stream_body(const HeadParams& p, const FuseParams& fp = FuseParams{}) {
     typedef typename Elem<E>::x8 X8;
     constexpr int PD = KC / 32;              // 1 KB W fragments per row block and chunk
     constexpr int R = (FP + 1) * PD;         // ring slots
@@ -584,6 +955,16 @@ __device__ __forceinline__ void head_gemm_stream_body(const HeadParams& p) {
     __shared__ __attribute__((aligned(1024))) char lds[2 * BUF];
     __shared__ float red_a[kHeadWaves][NB * 16];
     __shared__ float red_b[kHeadWaves][NB * 16];
+    // fused FR-Spec launch: ranking keys [hidden row][element of this workgroup] (row stride padded by one 16-byte
+    // piece), token ids of the workgroup's vocabulary rows, the rows' generations, staging of the published slots
+    constexpr int kKeyStride = (FP + 1) * 128 + 4;
+    __shared__ __attribute__((aligned(16))) uint32_t s_keys[FUSE ? kFuseRows * kKeyStride : 4];
+    __shared__ int32_t s_tok[FUSE ? (FP + 1) * 128 : 1];
+    __shared__ uint32_t s_gen[kFuseRows];
+    __shared__ __attribute__((aligned(16))) uint64_t s_out[FUSE ? kHeadWaves : 1][2 * kFuseSlots];
+    __shared__ int s_wave_wide[kHeadWaves];
+    __shared__ uint32_t s_ticket;
+    static_assert(!FUSE || (NB == 1 && (FP + 1) * 128 <= kHeadThreads), "fused launch: one block of hidden rows, one id per thread");
 
     const int tid = threadIdx.x;
     const int wave = tid >> 6;
@@ -596,6 +977,18 @@ __device__ __forceinline__ void head_gemm_stream_body(const HeadParams& p) {
     const int nch = H / KC;
     const int rotc = c % nch;  // workgroups start their K walk at different chunks (HBM channel spread)
     const E sc = (E)p.head_scale;
+
+    int32_t my_tok = 0;
+    uint32_t my_gen = 0;
+    if constexpr (FUSE) {
+        // requested first, so that they return ahead of the W stream: the token id of element `tid` of this workgroup
+        // (row block tid / 16 of its blocks, which are G apart) and the generation of hidden row `tid`
+        if (tid < (FP + 1) * 128) {
+            const int idx = ((tid >> 4) * G + c) * 16 + (tid & 15);
+            my_tok = idx < p.V ? (fp.remap ? fp.remap[idx] : idx) : 0;
+        }
+        if (tid < kFuseRows) my_gen = fp.st->gen[tid];
+    }
 
     // last pass: block `my_last` of this workgroup's share of it, K slice `my_sub` of every chunk
     const int share = p.last_share;
@@ -654,6 +1047,14 @@ __device__ __forceinline__ void head_gemm_stream_body(const HeadParams& p) {
         for (int j = 0; j < PD; ++j)
             if (j < sl) ring[FP * PD + j] = load_frag(wlast, s0 + my_sub * sl + j);
     }
+    if constexpr (FUSE) {
+        for (int i = tid; i < kFuseRows * kKeyStride; i += kHeadThreads) s_keys[i] = 0;
+        if (tid < (FP + 1) * 128) s_tok[tid] = my_tok;
+        if (tid < kFuseRows) s_gen[tid] = my_gen;
+        const bool wide = ((uint32_t)my_tok >> kFuseIdBits) != 0;
+        const bool any_wide = __ballot(wide) != 0;
+        if (lane == 0) s_wave_wide[wave] = any_wide ? 1 : 0;
+    }
     // One chunk: `refill` = request the same ring positions for the next chunk (everywhere but in the last one).
     auto chunk_body = [&](int q, auto refill) {
         // Chunk q of the hidden rows was requested before the FP * PD (+ sl) fragments that were requested since
@@ -710,8 +1111,19 @@ __device__ __forceinline__ void head_gemm_stream_body(const HeadParams& p) {
     };
     for (int q = 0; q + 1 < nch; ++q) chunk_body(q, std::true_type{});
     chunk_body(nch - 1, std::false_type{});
+    unsigned long long ticket = 0;
+    if constexpr (FUSE) {
+        // this workgroup's place in the order of finishing (used at the very end; wave 7 has the least to do after the loop)
+        if (tid == kHeadThreads - 64) ticket = __hip_atomic_fetch_add(&fp.st->tickets, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    const auto epilogue = [&](const f32x4 (&a)[NB], int block_pos) {
+        if constexpr (FUSE)
+            fuse_epilogue<E>(p, a[0], (block_pos * G + c) * 16 + kgp * 4, block_pos * 16 + kgp * 4, l16, ea[0], eb[0], s_keys + l16 * kKeyStride);
+        else
+            head_epilogue<NB, E>(p, a, (block_pos * G + c) * 16 + kgp * 4, l16, ea, eb);
+    };
 #pragma unroll
-    for (int pl = 0; pl < FP; ++pl) head_epilogue<NB, E>(p, acc[pl], ((pl * kHeadWaves + wave) * G + c) * 16 + kgp * 4, l16, ea, eb);
+    for (int pl = 0; pl < FP; ++pl) epilogue(acc[pl], pl * kHeadWaves + wave);
     if (p.rem_blocks > 0) {
         // The waves that shared a block of the last pass hold partial sums over their K slices: they meet in LDS
         // (the hidden buffers are free now) and the first wave of each group adds them up in wave order.
@@ -731,10 +1143,100 @@ __device__ __forceinline__ void head_gemm_stream_body(const HeadParams& p) {
                     for (int r = 0; r < 4; ++r) acc[FP][nb][r] += x[r];
                 }
             }
-            head_epilogue<NB, E>(p, acc[FP], rb_last * 16 + kgp * 4, l16, ea, eb);
+            epilogue(acc[FP], FP * kHeadWaves + my_last);
         }
     }
-    head_finish<NB>(p, ea, eb, red_a, red_b, tid, wave, lane, c);
+    if constexpr (!FUSE) {
+        head_finish<NB>(p, ea, eb, red_a, red_b, tid, wave, lane, c);
+    } else {
+        HeadFuseState* st = fp.st;
+        // the workgroup's (max, sum exp) of every hidden row, as one tagged word
+        head_finish_with<NB>(p, ea, eb, red_a, red_b, tid, wave, lane, [&](int row, float a, float b) {
+            if (row >= p.n) return;
+            int wide = 0;
+#pragma unroll
+            for (int i = 0; i < kHeadWaves; ++i) wide |= s_wave_wide[i];
+            const uint64_t word = ((uint64_t)((s_gen[row] + 1) & 0xFFFFu) << 48) | ((uint64_t)Elem<E>::to_bits(a) << 32) |
+                                  (uint64_t)(__float_as_uint(b) | (wide ? 0x80000000u : 0u));
+            fuse_store(&st->stats[row][c], word);
+        });
+        // (head_finish_with has a barrier in it: every wave's keys are in LDS.)  Two hidden rows per wave, one per half
+        // of its lanes: the threshold that leaves between fuse_publish_min(k) and 16 of the workgroup's keys of the
+        // row, found from the top bit down (keys are unique, so the search ends at exactly that many at the latest).
+        const auto select_rows = [&](auto nkl_tag) {
+            constexpr int NKL = decltype(nkl_tag)::value;  // keys per lane
+            const int half = lane >> 5, l32 = lane & 31;
+            const int row = wave * 2 + half;
+            if (wave * 2 >= p.n) return;
+            uint32_t kk[NKL];
+#pragma unroll
+            for (int j = 0; j < NKL; ++j) kk[j] = s_keys[row * kKeyStride + l32 + 32 * j];  // rows from n on hold zeros
+            const int need = fuse_publish_min(fp.top);
+            uint32_t thr_a = 0, thr_b = 0;
+            bool done_a = false, done_b = false;
+            {
+                int ca = 0, cb = 0;
+#pragma unroll
+                for (int j = 0; j < NKL; ++j) {
+                    const uint64_t mk = __ballot(kk[j] != 0u);
+                    ca += __popc((uint32_t)mk);
+                    cb += __popc((uint32_t)(mk >> 32));
+                }
+                if (ca <= kFuseSlots) { thr_a = 1; done_a = true; }
+                if (cb <= kFuseSlots) { thr_b = 1; done_b = true; }
+            }
+            for (int bit = 31; bit >= 0 && !(done_a && done_b); --bit) {
+                const uint32_t xa = thr_a | (1u << bit), xb = thr_b | (1u << bit);
+                const uint32_t x = half ? xb : xa;
+                int ca = 0, cb = 0;
+#pragma unroll
+                for (int j = 0; j < NKL; ++j) {
+                    const uint64_t mk = __ballot(kk[j] >= x);
+                    ca += __popc((uint32_t)mk);
+                    cb += __popc((uint32_t)(mk >> 32));
+                }
+                if (!done_a && ca >= need) {
+                    thr_a = xa;
+                    done_a = ca <= kFuseSlots;
+                }
+                if (!done_b && cb >= need) {
+                    thr_b = xb;
+                    done_b = cb <= kFuseSlots;
+                }
+            }
+            const uint32_t thr = half ? thr_b : thr_a;
+            const uint64_t tagw = (uint64_t)((s_gen[row & (kFuseRows - 1)] + 1) & kFuseCandTagMask) << 45;
+            uint64_t* outw = s_out[wave] + half * kFuseSlots;
+            if (l32 < kFuseSlots) outw[l32] = tagw;  // empty slot: image 0
+            __builtin_amdgcn_wave_barrier();
+            const uint32_t below = (1u << l32) - 1u;
+            int base = 0;
+#pragma unroll
+            for (int j = 0; j < NKL; ++j) {
+                const bool emit = kk[j] >= thr;
+                const uint64_t mk = __ballot(emit);
+                const uint32_t mh = half ? (uint32_t)(mk >> 32) : (uint32_t)mk;
+                if (emit) {
+                    const int slot = base + __popc(mh & below);
+                    const uint32_t lidx = 0xFFFFu - (kk[j] & 0xFFFFu);
+                    outw[slot] = tagw | ((uint64_t)(kk[j] >> 16) << 29) | ((uint64_t)lidx << kFuseIdBits) |
+                                 (uint64_t)((uint32_t)s_tok[lidx] & ((1u << kFuseIdBits) - 1u));
+                }
+                base += __popc(mh);
+            }
+            __builtin_amdgcn_wave_barrier();
+            if (l32 < kFuseSlots && row < p.n) fuse_store(&st->cand[row][c][l32], outw[l32]);
+        };
+        if (p.rem_blocks > 0) select_rows(std::integral_constant<int, (FP + 1) * 4>{});
+        else select_rows(std::integral_constant<int, FP * 4>{});
+        // every store of this workgroup acknowledged (the logits among them), then its mark; the ticket has long returned
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (tid == kHeadThreads - 64) s_ticket = (uint32_t)(ticket % (unsigned long long)G);
+        __syncthreads();
+        if (tid == 0) fuse_store(&st->done[c], (uint64_t)(s_gen[0] + 1));
+        const int place = (int)s_ticket;
+        if (place < p.n) fuse_finish_row<E>(p, fp, place, s_gen[place], s_gen[0]);
+    }
 }
 
 // The kernels proper: fp16 under the names they have in every profile, bf16 beside them.
@@ -750,6 +1252,11 @@ template <int NB, int FP, int KC>
 __global__ __launch_bounds__(kHeadThreads) void head_gemm_stream_kernel(HeadParams p) { head_gemm_stream_body<NB, FP, KC, f16>(p); }
 template <int NB, int FP, int KC>
 __global__ __launch_bounds__(kHeadThreads) void head_gemm_stream_bf16_kernel(HeadParams p) { head_gemm_stream_body<NB, FP, KC, bf16>(p); }
+// FR-Spec head + log-softmax + top-k + id map-back in one launch (one block of hidden rows).
+template <int FP, int KC>
+__global__ __launch_bounds__(kHeadThreads) void frspec_head_topk_kernel(HeadParams p, FuseParams fp) { head_gemm_stream_body<1, FP, KC, f16, true>(p, fp); }
+template <int FP, int KC>
+__global__ __launch_bounds__(kHeadThreads) void frspec_head_topk_bf16_kernel(HeadParams p, FuseParams fp) { head_gemm_stream_body<1, FP, KC, bf16, true>(p, fp); }
 
 // Final arg-max over the per-workgroup partials: one block per hidden row.  Largest value, lowest
 // index among equals: one 64-bit key (ordered image of the float, complemented index) per partial,
@@ -857,10 +1364,10 @@ HeadShape pick_head_shape(int NB, int H, bool w_tiled, int nch, int npasses, int
 
 }  // namespace
 
-// Shared launcher of the GEMM; returns the grid size used (= number of partial rows) in *grid_out.
-int launch_head_gemm(const void* hidden, const void* w, int w_layout, int n, int V, int H, int apply_scale, float head_scale,
-                     int mode, void* logits, float* part_a, float* part_b, int* grid_out, int* stride_out,
-                     hipStream_t st, HeadShape* shape_out, bool dry_run) {
+namespace {
+// The shape of one head GEMM: kernel parameters, kernel shape and grid.
+int plan_head_gemm(const void* hidden, const void* w, int w_layout, int n, int V, int H, int apply_scale, float head_scale,
+                   int mode, void* logits, float* part_a, float* part_b, HeadParams* p_out, HeadShape* shape_out, int* grid_out) {
     CPMCU_CHECK_ARG(w_layout == CPMCU_W_ROW_MAJOR || w_layout == CPMCU_W_TILED, "lm_head: unknown weight layout %d", w_layout);
     const int NB = pick_nb(n);
     const int kc_max = 2048 / NB;
@@ -890,7 +1397,6 @@ int launch_head_gemm(const void* hidden, const void* w, int w_layout, int n, int
     p.rem_blocks = 0;
     CPMCU_CHECK_ARG(G <= head_max_grid(), "lm_head: %d workgroups exceed the %d rows of the partial planes", G, head_max_grid());
     *grid_out = G;
-    *stride_out = NB * 16;
     p.last_share = 1;
     HeadShape shape = pick_head_shape(NB, H, p.w_tiled, p.nch, p.npasses, nrb, G, &p.full_passes, &p.rem_blocks);
     // Tiled weights with 1..4 full passes (1..2 for 65-128 hidden rows) and at most one partly filled pass: the streaming kernel.
@@ -915,6 +1421,23 @@ int launch_head_gemm(const void* hidden, const void* w, int w_layout, int n, int
             }
         }
     }
+    *shape_out = shape;
+    *p_out = p;
+    return CPMCU_OK;
+}
+}  // namespace
+
+// Shared launcher of the GEMM; returns the grid size used (= number of partial rows) in *grid_out.
+int launch_head_gemm(const void* hidden, const void* w, int w_layout, int n, int V, int H, int apply_scale, float head_scale,
+                     int mode, void* logits, float* part_a, float* part_b, int* grid_out, int* stride_out,
+                     hipStream_t st, HeadShape* shape_out, bool dry_run) {
+    HeadParams p;
+    HeadShape shape;
+    int G = 0;
+    const int rc = plan_head_gemm(hidden, w, w_layout, n, V, H, apply_scale, head_scale, mode, logits, part_a, part_b, &p, &shape, &G);
+    if (rc != CPMCU_OK) return rc;
+    *grid_out = G;
+    *stride_out = pick_nb(n) * 16;
     if (shape_out) *shape_out = shape;
     if (dry_run) return CPMCU_OK;
     const bool is_bf16 = options().dtype == 1;
@@ -958,6 +1481,161 @@ int launch_head_gemm(const void* hidden, const void* w, int w_layout, int n, int
 }
 
 int head_max_grid() { return 1024; }
+
+// ---- host side of the fused FR-Spec launch -----------------------------------------------------------------------
+namespace {
+constexpr int kFuseDevices = 64;
+std::mutex g_fuse_mu;
+struct FuseKey {
+    int dev;
+    const void* workspace;
+    int grid;
+    bool operator<(const FuseKey& o) const { return std::tie(dev, workspace, grid) < std::tie(o.dev, o.workspace, o.grid); }
+};
+std::map<FuseKey, int> g_fuse_states;         // -> index into the device's g_head_fuse
+std::vector<int> g_fuse_free[kFuseDevices];
+bool g_fuse_listed[kFuseDevices] = {false};
+bool g_fuse_off[kFuseDevices] = {false};      // a finisher's wait ran out on this device: back to two launches
+HeadFuseState* g_fuse_base[kFuseDevices] = {nullptr};
+HeadFuseReport* g_fuse_report_host[kFuseDevices] = {nullptr};
+
+// The state a (workspace, grid) pair publishes its words through, on the current device; null: none left, or the
+// first use on the device falls inside a stream capture (the address lookup does not belong there).  States stay with
+// their pair until the workspace is released: launches that were captured into a graph keep using them.
+HeadFuseState* fuse_state_for(const void* workspace, int grid, hipStream_t st, bool create) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kFuseDevices) return nullptr;
+    std::lock_guard<std::mutex> lock(g_fuse_mu);
+    if (g_fuse_off[dev]) return nullptr;
+    auto it = g_fuse_states.find({dev, workspace, grid});
+    if (it == g_fuse_states.end()) {
+        if (!create) return nullptr;
+        if (g_fuse_base[dev] == nullptr) {
+            hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+            if (hipStreamIsCapturing(st, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) {
+                (void)hipGetLastError();
+                return nullptr;
+            }
+            void* ptr = nullptr;
+            if (hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_head_fuse)) != hipSuccess) {
+                (void)hipGetLastError();
+                return nullptr;
+            }
+            g_fuse_base[dev] = (HeadFuseState*)ptr;
+        }
+        if (!g_fuse_listed[dev]) {
+            for (int b = kFuseStates - 1; b >= 0; --b) g_fuse_free[dev].push_back(b);
+            g_fuse_listed[dev] = true;
+        }
+        if (g_fuse_free[dev].empty()) return nullptr;
+        const int b = g_fuse_free[dev].back();
+        g_fuse_free[dev].pop_back();
+        it = g_fuse_states.emplace(FuseKey{dev, workspace, grid}, b).first;
+    }
+    return g_fuse_base[dev] + it->second;
+}
+
+// Whether this call takes the one-launch form, and with which kernel.
+bool fuse_eligible(const HeadParams& p, HeadShape shape, int G, int k, const void* logits) {
+    if (!options().frspec_fused || !options().head_stream_kernel) return false;
+    if (shape != HeadShape::S_1_1_512 && shape != HeadShape::S_1_2_256) return false;
+    return G >= kFuseRows && G <= kFuseMaxGrid && p.n <= kFuseRows && k <= kFuseSlots && p.V % 8 == 0 && p.V <= (1 << kFuseIdBits) &&
+           ((uintptr_t)logits & 7) == 0;
+}
+}  // namespace
+
+// FR-Spec head + log-softmax + top-k + id map-back as one launch when the shape allows it (tiled weights, <= 16 hidden
+// rows, k <= 16, one or two full passes of row blocks) and a state is to be had; *launched says whether it was.
+int launch_frspec_fused(const void* hidden, const void* w, int w_layout, const int32_t* token_id_remap, int n, int V, int H, int k,
+                        void* logits, float* row_stats, void* topk_val, int32_t* topk_pos, int32_t* topk_ids, const void* workspace,
+                        hipStream_t st, bool* launched, bool dry_run) {
+    *launched = false;
+    if (w_layout != CPMCU_W_TILED || n > kFuseRows) return CPMCU_OK;
+    HeadParams p;
+    HeadShape shape;
+    int G = 0;
+    const int rc = plan_head_gemm(hidden, w, w_layout, n, V, H, 0, 1.f, kHeadModeStats, logits, nullptr, nullptr, &p, &shape, &G);
+    if (rc != CPMCU_OK) return rc;
+    if (!fuse_eligible(p, shape, G, k, logits)) return CPMCU_OK;
+    HeadFuseState* state = fuse_state_for(workspace, G, st, true);
+    if (state == nullptr) return CPMCU_OK;
+    *launched = true;
+    if (dry_run) return CPMCU_OK;
+    FuseParams fp;
+    fp.st = state;
+    fp.top = k;
+    fp.remap = token_id_remap;
+    fp.val = (uint16_t*)topk_val;
+    fp.pos = topk_pos;
+    fp.ids = topk_ids;
+    fp.row_stats = row_stats;
+    fp.wait_ticks = (uint32_t)options().frspec_wait_us * 100u;
+    const bool is_bf16 = options().dtype == 1;
+    if (shape == HeadShape::S_1_1_512) {
+        if (is_bf16) hipLaunchKernelGGL((frspec_head_topk_bf16_kernel<1, 512>), dim3(G), dim3(kHeadThreads), 0, st, p, fp);
+        else hipLaunchKernelGGL((frspec_head_topk_kernel<1, 512>), dim3(G), dim3(kHeadThreads), 0, st, p, fp);
+    } else {
+        if (is_bf16) hipLaunchKernelGGL((frspec_head_topk_bf16_kernel<2, 256>), dim3(G), dim3(kHeadThreads), 0, st, p, fp);
+        else hipLaunchKernelGGL((frspec_head_topk_kernel<2, 256>), dim3(G), dim3(kHeadThreads), 0, st, p, fp);
+    }
+    CPMCU_LAUNCH_CHECK();
+    return CPMCU_OK;
+}
+
+// Gives back the states of a workspace that is about to be freed (none of its launches in flight or captured).
+void head_fuse_release_workspace(const void* workspace) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kFuseDevices) return;
+    std::lock_guard<std::mutex> lock(g_fuse_mu);
+    for (auto it = g_fuse_states.begin(); it != g_fuse_states.end();) {
+        if (it->first.dev == dev && it->first.workspace == workspace) {
+            g_fuse_free[dev].push_back(it->second);
+            it = g_fuse_states.erase(it);
+        } else {
+            ++it;
+        }
+    }
+}
+
+// The report words of the current device, copied to pinned host memory in stream order (ahead of a synchronisation,
+// never under a capture) and looked at afterwards; a wait that ran out switches the device back to two launches.
+int head_fuse_report_enqueue(hipStream_t st) {
+    int dev = 0;
+    CPMCU_HIP(hipGetDevice(&dev));
+    CPMCU_CHECK_ARG(dev >= 0 && dev < kFuseDevices, "device index %d outside [0, %d)", dev, kFuseDevices);
+    if (g_fuse_report_host[dev] == nullptr) {
+        CPMCU_HIP(hipHostMalloc((void**)&g_fuse_report_host[dev], sizeof(HeadFuseReport), hipHostMallocDefault));
+        *g_fuse_report_host[dev] = HeadFuseReport{0u, 0u, 0u};
+    }
+    CPMCU_HIP(hipMemcpyFromSymbolAsync(g_fuse_report_host[dev], HIP_SYMBOL(g_head_fuse_report), sizeof(HeadFuseReport), 0, hipMemcpyDeviceToHost, st));
+    return CPMCU_OK;
+}
+int head_fuse_report_take(unsigned int* timeouts, unsigned int* slow_rows, unsigned int* fused_rows) {
+    int dev = 0;
+    CPMCU_HIP(hipGetDevice(&dev));
+    *timeouts = *slow_rows = *fused_rows = 0;
+    if (dev < 0 || dev >= kFuseDevices || g_fuse_report_host[dev] == nullptr) return CPMCU_OK;
+    const HeadFuseReport r = *g_fuse_report_host[dev];
+    if (r.timeouts != 0 || r.slow_rows != 0 || r.fused_rows != 0) {
+        const HeadFuseReport zero{0u, 0u, 0u};
+        CPMCU_HIP(hipMemcpyToSymbol(HIP_SYMBOL(g_head_fuse_report), &zero, sizeof(zero)));
+        *g_fuse_report_host[dev] = zero;
+        if (r.timeouts != 0) {
+            std::lock_guard<std::mutex> lock(g_fuse_mu);
+            g_fuse_off[dev] = true;
+        }
+    }
+    *timeouts = r.timeouts;
+    *slow_rows = r.slow_rows;
+    *fused_rows = r.fused_rows;
+    return CPMCU_OK;
+}
+void head_fuse_reenable() {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kFuseDevices) return;
+    std::lock_guard<std::mutex> lock(g_fuse_mu);
+    g_fuse_off[dev] = false;
+}
 
 }  // namespace cpmcu
 

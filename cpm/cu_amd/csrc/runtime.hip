@@ -164,8 +164,12 @@ struct PerfScope {
 // pinned memory in front of the synchronisation: no round trip of their own): a length outside what the host had
 // promised is an error; merge waits that ran out are counted for the summary.
 long g_abandoned_waits = 0;
+// Fused FR-Spec launches: rows finished from the published candidates, rows redone from the logits, waits that ran out.
+long g_frspec_fused_rows = 0, g_frspec_slow_rows = 0, g_frspec_timeouts = 0;
 int synchronize_and_check(hipStream_t st) {
     int rc = attention_report_enqueue(st);
+    if (rc) return rc;
+    rc = head_fuse_report_enqueue(st);
     if (rc) return rc;
     CPMCU_HIP(hipStreamSynchronize(st));
     int bad = 0;
@@ -173,6 +177,17 @@ int synchronize_and_check(hipStream_t st) {
     rc = attention_report_take(&bad, &abandoned);
     if (rc) return rc;
     g_abandoned_waits += abandoned;
+    unsigned int fr_timeouts = 0, fr_slow = 0, fr_fused = 0;
+    rc = head_fuse_report_take(&fr_timeouts, &fr_slow, &fr_fused);
+    if (rc) return rc;
+    g_frspec_fused_rows += fr_fused;
+    g_frspec_slow_rows += fr_slow;
+    g_frspec_timeouts += fr_timeouts;
+    if (fr_timeouts != 0) {
+        set_error("%u row(s) of a one-launch FR-Spec head were not finished: the workgroups of the launch were not all resident within "
+                  "the wait (frspec_wait_us); those rows hold index -1, and the head runs as two launches from now on", fr_timeouts);
+        return CPMCU_ERR_RUNTIME;
+    }
     if (bad != 0) {
         set_error("a tree-attention launch read a KV length of %d from device memory, outside [rows, max_kv_len] of its call; "
                   "it ran on the clamped length and its output is not valid", bad < 0 ? 0 : bad);
@@ -221,6 +236,13 @@ extern "C" int cpmcu_set_option(const char* name, int value) {
         CPMCU_CHECK_ARG(value == 0 || value == 1, "set_option: attn_merge_in_launch=%d must be 0 or 1", value);
         options().attn_merge_in_launch = value;
         if (value) attention_merge_reenable();  // also for workspaces that went back to the combine launch after an abandoned wait
+    } else if (nm == "frspec_fused") {
+        CPMCU_CHECK_ARG(value == 0 || value == 1, "set_option: frspec_fused=%d must be 0 or 1", value);
+        options().frspec_fused = value;
+        if (value) head_fuse_reenable();  // also after a wait that ran out
+    } else if (nm == "frspec_wait_us") {
+        CPMCU_CHECK_ARG(value >= 0 && value <= 1000000, "set_option: frspec_wait_us=%d outside [0, 1000000]", value);
+        options().frspec_wait_us = value;
     } else {
         set_error("set_option: unknown option %s", name);
         return CPMCU_ERR_INVALID_ARGUMENT;
@@ -326,6 +348,7 @@ void release_storage(Model& m) {
     (void)hipFree(m.d_v_pools);
     (void)hipFree(m.block_table);
     if (m.attn_ws) attention_release_workspace(m.attn_ws);
+    if (m.head_ws) head_fuse_release_workspace(m.head_ws);
     (void)hipFree(m.attn_ws);
     (void)hipFree(m.head_ws);
     (void)hipFree(m.draft_logits);
@@ -404,6 +427,8 @@ int init_storage_impl(Model& m, int* max_context) {
         if ((rc = alloc((void**)&m.topk_val, (size_t)16 * m.topk_per_iter * sizeof(f16)))) return rc;
         if ((rc = alloc((void**)&m.topk_pos, (size_t)16 * m.topk_per_iter * sizeof(int32_t)))) return rc;
         if ((rc = alloc((void**)&m.topk_ids, (size_t)16 * m.topk_per_iter * sizeof(int32_t)))) return rc;
+        // the state of the one-launch draft head is assigned now, ahead of any captured launch
+        (void)cpmcu_frspec_head_mode(m.head_ws, CPMCU_W_TILED, 1, m.frspec_vocab, m.hidden, m.topk_per_iter);
     }
     if ((rc = alloc((void**)&m.d_best, 2 * sizeof(int32_t)))) return rc;
     if ((rc = alloc((void**)&m.d_ids, 64 * sizeof(int32_t)))) return rc;
@@ -768,7 +793,7 @@ uint64_t step_signature(const Model& m, const StepArgs& a) {
         mix(v);
     // the options decide which kernels a capture records: a graph captured under other settings is another graph
     const Options& o = options();
-    for (int v : {o.dtype, o.attn_kv_groups, o.head_share_last_pass, o.head_stream_kernel, o.attn_merge_in_launch, o.attn_merge_wait_us}) mix((uint64_t)(uint32_t)v);
+    for (int v : {o.dtype, o.attn_kv_groups, o.head_share_last_pass, o.head_stream_kernel, o.attn_merge_in_launch, o.attn_merge_wait_us, o.frspec_fused, o.frspec_wait_us}) mix((uint64_t)(uint32_t)v);
     return h;
 }
 
@@ -957,6 +982,8 @@ extern "C" int cpmcu_print_perf_summary(void) {
     if (hipMemGetInfo(&free_b, &total_b) == hipSuccess)
         printf("GPU memory: %.1f MiB used of %.1f MiB\n", (total_b - free_b) / 1048576.0, total_b / 1048576.0);
     printf("attention merge waits that ran out (share left to the last workgroup of its unit): %ld\n", g_abandoned_waits);
+    printf("one-launch FR-Spec heads: %ld rows from the published candidates, %ld redone from the logits, %ld not finished\n",
+           g_frspec_fused_rows, g_frspec_slow_rows, g_frspec_timeouts);
     fflush(stdout);
     return CPMCU_OK;
 }
@@ -966,6 +993,16 @@ extern "C" int cpmcu_print_perf_summary(void) {
 // others of its unit and left its share of the merge to the last of them: the output was complete, but late, and the
 // device's workspaces have gone back to the separate merge launch (cpmcu_set_option("attn_merge_in_launch", 1) undoes that).
 extern "C" long cpmcu_attention_abandoned_waits(void) { return g_abandoned_waits; }
+
+// Rows of one-launch FR-Spec heads seen by the library's synchronisations so far: finished from the published candidates,
+// redone from the logits in memory (tie-heavy rows), and not finished because a wait ran out (an error at that
+// synchronisation).  Any of the pointers may be null.
+extern "C" int cpmcu_frspec_fused_rows(long* fused_rows, long* slow_rows, long* timeouts) {
+    if (fused_rows) *fused_rows = g_frspec_fused_rows;
+    if (slow_rows) *slow_rows = g_frspec_slow_rows;
+    if (timeouts) *timeouts = g_frspec_timeouts;
+    return CPMCU_OK;
+}
 
 // Extension: device pointers of the model's storage for harnesses that fill the cache directly.
 extern "C" int cpmcu_model_pointers(int layer, uint64_t* k_pool, uint64_t* v_pool, uint64_t* block_table,

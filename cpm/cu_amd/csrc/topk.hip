@@ -273,20 +273,7 @@ __device__ __forceinline__ void topk_row_body(const TopkParams& p) {
     if (LOGSOFTMAX) {
         m = row_m_lse[0];
         lse = row_m_lse[1];
-        if (bound > 0) {
-            const uint16_t zb = (uint16_t)((bound & 0x8000u) ? (bound ^ 0x8000u) : (bound ^ 0xFFFFu));
-            const float zl = Elem<E>::from_bits(zb);
-            const uint16_t y = Elem<E>::to_bits((zl - m) - lse);
-            constexpr int kM = Elem<E>::kMantissaBits, kBias = Elem<E>::kExponentBias, kEmax = (1 << Elem<E>::kExponentBits) - 1;
-            const int e = (y >> kM) & kEmax;
-            const float zlo = zl - 4.f * ldexpf(1.f, e ? e - kBias - kM : 1 - kBias - kM);  // four ulps of the mapped bound
-            lo = 0;
-            if (e != kEmax && zlo == zlo && fabsf(zlo) <= Elem<E>::kMaxFinite) {  // finite mapped bound, representable lower bound
-                const uint16_t lb = Elem<E>::to_bits(zlo);
-                const uint32_t o = (uint32_t)(lb ^ ((lb & 0x8000u) ? 0xFFFFu : 0x8000u));
-                lo = o > 2 ? o - 2 : 0;  // one step for the rounding of zlo, one for -0
-            }
-        }
+        if (bound > 0) lo = mapped_lower_image<E>(bound, m, lse);
     }
 
     const auto key_from_image = [&](uint32_t o, int idx) -> uint64_t {
@@ -581,6 +568,10 @@ extern "C" int cpmcu_frspec_head_topk(const void* hidden, const void* w, int w_l
     CPMCU_CHECK_ARG(workspace && workspace_bytes >= cpmcu_head_workspace_bytes(n, V),
                     "frspec_head_topk: workspace of %zu bytes needed, %zu given", cpmcu_head_workspace_bytes(n, V), workspace_bytes);
     hipStream_t st = resolve_stream(stream);
+    bool fused = false;
+    int rc0 = launch_frspec_fused(hidden, w, w_layout, token_id_remap, n, V, H, k, logits, row_stats, topk_val, topk_pos, topk_ids, workspace,
+                                  st, &fused);
+    if (rc0 != CPMCU_OK || fused) return rc0;
     float* part_a = (float*)workspace;
     float* part_b = part_a + (size_t)head_max_grid() * 128;
     const size_t parts_bytes = align_up((size_t)2 * head_max_grid() * 128 * sizeof(float), 256);
@@ -590,4 +581,23 @@ extern "C" int cpmcu_frspec_head_topk(const void* hidden, const void* w, int w_l
     TopkStatsSource src{part_a, part_b, G, stride, row_stats};
     return launch_topk(logits, n, V, k, topk_val, topk_pos, topk_ids, token_id_remap, &src,
                        (char*)workspace + parts_bytes, workspace_bytes - parts_bytes, st);
+}
+
+// 1: a call of cpmcu_frspec_head_topk with this shape on this workspace runs as one launch (and a publication state of
+// the library is now assigned to the pair, if it had none); 0: as GEMM launch + top-k launch.
+extern "C" int cpmcu_frspec_head_mode(const void* workspace, int w_layout, int n, int V, int H, int k) {
+    if (workspace == nullptr || n < 1 || n > 16 || k < 1 || V < 1 || H < 1) return 0;
+    bool fused = false;
+    // the planning needs a non-null, 8-byte aligned logits pointer only to check alignment
+    if (launch_frspec_fused(workspace, workspace, w_layout, nullptr, n, V, H, k, (void*)workspace, nullptr, nullptr, nullptr, nullptr, workspace,
+                            nullptr, &fused, true) != CPMCU_OK)
+        return 0;
+    return fused ? 1 : 0;
+}
+
+// Gives back the library-side states of a head workspace that is about to be freed (no launch on it in flight or captured).
+extern "C" int cpmcu_head_release_workspace(const void* workspace) {
+    CPMCU_CHECK_ARG(workspace, "head_release_workspace: null pointer argument");
+    head_fuse_release_workspace(workspace);
+    return CPMCU_OK;
 }

@@ -79,6 +79,28 @@ __device__ inline uint64_t wave_max_u64(uint64_t v) {
     return best;
 }
 
+// The fused log-softmax ranks f16((z - max) - ln sum) (src/model/eagle.cuh:87), a monotone map of z that merges
+// neighbours.  Given the ordered 16-bit image `bound` of a z that has at least k elements at or above it, this is the
+// lowest image whose z can still map to the mapped bound's value or above: four ulps of the mapped bound below it, one
+// step more for the rounding of that difference and one for -0.  0: no usable bound (every element is a candidate).
+template <typename E>
+__device__ inline uint32_t mapped_lower_image(uint32_t bound, float m, float lse) {
+    if (bound == 0) return 0;
+    const uint16_t zb = (uint16_t)((bound & 0x8000u) ? (bound ^ 0x8000u) : (bound ^ 0xFFFFu));
+    const float zl = Elem<E>::from_bits(zb);
+    const uint16_t y = Elem<E>::to_bits((zl - m) - lse);
+    constexpr int kM = Elem<E>::kMantissaBits, kBias = Elem<E>::kExponentBias, kEmax = (1 << Elem<E>::kExponentBits) - 1;
+    const int e = (y >> kM) & kEmax;
+    const int e4 = (e ? e - kBias - kM : 1 - kBias - kM) + 2;  // exponent of four ulps of the mapped bound
+    const float zlo = zl - (e4 >= -126 ? __uint_as_float((uint32_t)(e4 + 127) << 23) : ldexpf(1.f, e4));
+    if (e != kEmax && zlo == zlo && fabsf(zlo) <= Elem<E>::kMaxFinite) {  // finite mapped bound, representable lower bound
+        const uint16_t lb = Elem<E>::to_bits(zlo);
+        const uint32_t o = (uint32_t)(lb ^ ((lb & 0x8000u) ? 0xFFFFu : 0x8000u));
+        return o > 2 ? o - 2 : 0;
+    }
+    return 0;
+}
+
 // k rounds of workgroup-wide max over the keys held in registers; round j's winner goes to
 // emit(j, key), called by thread 0.  Keys equal to 0 are empty slots.  One barrier per round: the
 // per-wave maxima alternate between two LDS buffers, so a wave that runs ahead into the next round

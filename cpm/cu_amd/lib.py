@@ -58,6 +58,9 @@ SIGNATURES = {
     "cpmcu_tree_attention_window": (c_int, [_P, _P, _P, _P, _P, c_int, _P, _P, _P, c_int, _P, c_int, c_int, c_int, c_int, c_int, c_float, _P, _P, c_size_t, c_int, _P]),
     "cpmcu_tree_attention_merge_mode": (c_int, [_P]),
     "cpmcu_tree_attention_release_workspace": (c_int, [_P]),
+    "cpmcu_frspec_head_mode": (c_int, [_P, c_int, c_int, c_int, c_int, c_int]),
+    "cpmcu_head_release_workspace": (c_int, [_P]),
+    "cpmcu_frspec_fused_rows": (c_int, [ctypes.POINTER(ctypes.c_long), ctypes.POINTER(ctypes.c_long), ctypes.POINTER(ctypes.c_long)]),
     "cpmcu_tree_attention_plan": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_char_p, c_size_t, ctypes.POINTER(c_int), ctypes.POINTER(c_int), ctypes.POINTER(c_int)]),
     "cpmcu_rope_table": (c_int, [_P, _P, c_int, _P, _P]),
     "cpmcu_rope_apply": (c_int, [_P, c_int, c_int, c_int, _P, _P, _P]),

@@ -44,6 +44,8 @@ def _workspace(kind, nbytes, device):
     if ws is None or ws.numel() < nbytes:
         if ws is not None and kind == "attn":
             release_attention_workspace(ws)
+        if ws is not None and kind == "head":
+            release_head_workspace(ws)
         ws = torch.empty(max(int(nbytes), 256), dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
@@ -54,6 +56,13 @@ def release_attention_workspace(ws):
     The device is synchronised first (no launch on the workspace may be in flight)."""
     torch.cuda.synchronize()
     _lib().tree_attention_release_workspace(ctypes.c_void_p(ws.data_ptr()))
+
+
+def release_head_workspace(ws):
+    """Before a head workspace tensor is dropped: the library takes back the states its one-launch FR-Spec head
+    publishes through.  The device is synchronised first (no launch on the workspace may be in flight)."""
+    torch.cuda.synchronize()
+    _lib().head_release_workspace(ctypes.c_void_p(ws.data_ptr()))
 
 
 def mask_words(T):
@@ -189,6 +198,19 @@ def frspec_head_topk(hidden, w, token_id_remap, k):
     _lib().frspec_head_topk(_ptr(hidden), _ptr(w), layout, _ptr(token_id_remap), n, V, H, k, _ptr(logits), _ptr(stats),
                             _ptr(val), _ptr(pos), _ptr(ids), _ptr(ws), ws.numel(), _stream())
     return dict(logits=logits, row_stats=stats, val=val, pos=pos, ids=ids)
+
+
+def frspec_head_plan(n, w, k):
+    """Kernel name(s) of a frspec_head_topk call with n hidden rows on matrix w: the one-launch kernel when the shape
+    allows it and the library has a publication state for the head workspace, else GEMM + top-k."""
+    w_, layout, V = _weight(w)
+    H = w.H if isinstance(w, TiledWeight) else w.shape[1]
+    gemm = head_plan(n, w)[0]
+    ws = _workspace("head", _lib().raw.cpmcu_head_workspace_bytes(n, V), w_.device)
+    if _lib().raw.cpmcu_frspec_head_mode(ctypes.c_void_p(ws.data_ptr()), layout, n, V, H, k) == 1:
+        nb, fp, kc = gemm[gemm.index("<") + 1:-1].split(",")
+        return "frspec_head_topk_kernel<%s,%s>" % (fp, kc)
+    return gemm + ("+topk_row_kernel<true>" if V <= 32768 and V % 8 == 0 else "+topk_chunk_kernel<true>+topk_merge_kernel<true>")
 
 
 def lm_head_argmax(hidden, w, head_scale=None, want_logits=False, gt=None):

@@ -422,6 +422,23 @@ int cpmcu_frspec_head_topk(const void* hidden, const void* w, int w_layout, cons
                            int H, int k, void* logits, float* row_stats, void* topk_val, int32_t* topk_pos,
                            int32_t* topk_ids, void* workspace, size_t workspace_bytes, void* stream);
 
+/* The call above runs as ONE launch when the shape allows it (CPMCU_W_TILED weights, k <= 16, V a multiple of 8 with one
+ * or two full passes of 16-row blocks over the GPU -- the FR-Spec vocabulary of 32768 is one) and one of the library's 8
+ * publication states per device is free for (workspace, grid size): every GEMM workgroup publishes its k..16 best
+ * (value, index, token id) per hidden row as tagged 64-bit words, and the first n workgroups to finish rank one row
+ * each.  Same outputs, bit for bit, as the two-launch form (cpmcu_set_option("frspec_fused", 0)); logits are complete
+ * when the launch ends.  A state stays with its (workspace, grid) until cpmcu_head_release_workspace; calls that
+ * overlap on one GPU must use different workspaces, as before.  A finisher waits at most frspec_wait_us (option,
+ * default 50000) for the other workgroups of its launch to become resident; if that runs out its row holds index -1,
+ * the next synchronising call of the library returns CPMCU_ERR_RUNTIME, and the device goes back to two launches.
+ * No counterpart in the reference, which runs these steps as separate kernels (minicpm4_eagle.cuh:366-372).
+ * cpmcu_frspec_head_mode: 1 if a call of this shape on this workspace is one launch (assigns a state if needed), else 0.
+ * cpmcu_frspec_fused_rows: rows seen by the library's synchronisations so far -- finished from the published words,
+ * redone from the logits in memory (rows dominated by equal values), not finished (wait ran out); pointers may be NULL. */
+int cpmcu_frspec_head_mode(const void* workspace, int w_layout, int n, int V, int H, int k);
+int cpmcu_head_release_workspace(const void* workspace);
+int cpmcu_frspec_fused_rows(long* fused_rows, long* slow_rows, long* timeouts);
+
 /* Target head with fused arg-max -- LMHead::prefill (src/model/linear.cuh:82-101;
  * fp16 pre-scale by head_scale when apply_scale != 0) + torch argmax
  * (cpmcu/speculative/tree_drafter.py:153,233; lowest index on ties).
