@@ -129,70 +129,74 @@ __device__ inline void fuse_store(uint64_t* p, uint64_t v) { __hip_atomic_store(
 __device__ inline int fuse_publish_min(int top) { return top > 8 ? top : 8; }
 __device__ inline uint16_t image_to_bits(uint32_t o) { return (uint16_t)((o & 0x8000u) ? (o ^ 0x8000u) : (o ^ 0xFFFFu)); }
 
-// Folds one finished 16-row block of W (acc[nb][r] <-> vocab row vrow0 + r, hidden row nb*16 + l16) into
-// the lane's running epilogue state and writes its logits when asked to.
-template <int NB, typename E>
-__device__ inline void head_epilogue(const HeadParams& p, const f32x4 (&acc)[NB], int vrow0, int l16, float (&ea)[NB], float (&eb)[NB]) {
+// Folds the part of one finished 16-row block of W that belongs to hidden-row block nb (acc[r] <-> vocab row vrow0 + r,
+// hidden row nb*16 + l16) into the lane's running epilogue state and writes its logits when asked to.
+// ASCENDING: the caller hands a lane its vocabulary rows in ascending order and has preset the state to (-inf, the
+// lane's first row), so "lowest index among equals" needs no comparison of indices here: a later equal value never
+// replaces an earlier one.  (Five vector instructions per value instead of nine in the arg-max-only case, which is
+// what the verify step's 60-row head spends its last microseconds on.)
+template <typename E, bool ASCENDING>
+__device__ inline void head_epilogue_block(const HeadParams& p, const f32x4& acc, int nb, int vrow0, int l16, float& ea, float& eb) {
     const int V = p.V;
     if (p.mode == kHeadModeArgmax && p.logits == nullptr) {
-        // The verify step's case (arg-max only), without a branch per value: the same comparisons as below as selects.
+        // The verify step's case (arg-max only), without a branch per value: the comparisons below as selects.
+        const bool row_in = nb * 16 + l16 < p.n;
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-            const bool row_in = nb * 16 + l16 < p.n;
-#pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                const float x = (float)(E)acc[nb][r];
-                const int idx = vrow0 + r;
-                const bool take = row_in && idx < V && (x > ea[nb] || (x == ea[nb] && idx < __float_as_int(eb[nb])));
-                ea[nb] = take ? x : ea[nb];
-                eb[nb] = take ? __int_as_float(idx) : eb[nb];
-            }
+        for (int r = 0; r < 4; ++r) {
+            const float x = (float)(E)acc[r];
+            const int idx = vrow0 + r;
+            const bool better = ASCENDING ? x > ea : (x > ea || (x == ea && idx < __float_as_int(eb)));
+            const bool take = row_in && idx < V && better;
+            ea = take ? x : ea;
+            eb = take ? __int_as_float(idx) : eb;
         }
         return;
     }
+    const int hrow = nb * 16 + l16;
+    E z[4];
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb) {
-        const int hrow = nb * 16 + l16;
-        E z[4];
+    for (int r = 0; r < 4; ++r) z[r] = (E)acc[r];
+    if (hrow < p.n) {
+        if (p.logits) {
+            E* dst = reinterpret_cast<E*>(p.logits) + (size_t)hrow * V + vrow0;
+            if ((V & 3) == 0 && vrow0 + 3 < V) {
+                typename Elem<E>::x4 zz;
 #pragma unroll
-        for (int r = 0; r < 4; ++r) z[r] = (E)acc[nb][r];
-        if (hrow < p.n) {
-            if (p.logits) {
-                E* dst = reinterpret_cast<E*>(p.logits) + (size_t)hrow * V + vrow0;
-                if ((V & 3) == 0 && vrow0 + 3 < V) {
-                    typename Elem<E>::x4 zz;
+                for (int r = 0; r < 4; ++r) zz[r] = z[r];
+                *reinterpret_cast<typename Elem<E>::x4*>(dst) = zz;
+            } else {
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) zz[r] = z[r];
-                    *reinterpret_cast<typename Elem<E>::x4*>(dst) = zz;
-                } else {
-#pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        if (vrow0 + r < V) dst[r] = z[r];
-                }
+                for (int r = 0; r < 4; ++r)
+                    if (vrow0 + r < V) dst[r] = z[r];
             }
+        }
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-                if (vrow0 + r >= V) continue;
-                const float x = (float)z[r];
-                if (p.mode == kHeadModeStats) {
-                    if (x == -INFINITY) continue;  // contributes exp(-inf) = 0
-                    if (x > ea[nb]) {
-                        eb[nb] = eb[nb] * __expf(ea[nb] - x) + 1.f;
-                        ea[nb] = x;
-                    } else {
-                        eb[nb] += __expf(x - ea[nb]);
-                    }
+        for (int r = 0; r < 4; ++r) {
+            if (vrow0 + r >= V) continue;
+            const float x = (float)z[r];
+            if (p.mode == kHeadModeStats) {
+                if (x == -INFINITY) continue;  // contributes exp(-inf) = 0
+                if (x > ea) {
+                    eb = eb * __expf(ea - x) + 1.f;
+                    ea = x;
                 } else {
-                    const int idx = vrow0 + r;
-                    const int bidx = __float_as_int(eb[nb]);
-                    if (x > ea[nb] || (x == ea[nb] && idx < bidx)) {
-                        ea[nb] = x;
-                        eb[nb] = __int_as_float(idx);
-                    }
+                    eb += __expf(x - ea);
+                }
+            } else {
+                const int idx = vrow0 + r;
+                const int bidx = __float_as_int(eb);
+                if (x > ea || (!ASCENDING && x == ea && idx < bidx)) {
+                    ea = x;
+                    eb = __int_as_float(idx);
                 }
             }
         }
     }
+}
+template <int NB, typename E, bool ASCENDING = false>
+__device__ inline void head_epilogue(const HeadParams& p, const f32x4 (&acc)[NB], int vrow0, int l16, float (&ea)[NB], float (&eb)[NB]) {
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) head_epilogue_block<E, ASCENDING>(p, acc[nb], nb, vrow0, l16, ea[nb], eb[nb]);
 }
 
 // Reduces the epilogue state over the lanes that share a hidden row, then over the waves, and writes
@@ -1030,7 +1034,10 @@ __device__ __forceinline__ void head_gemm_stream_body(const HeadParams& p, const
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
         ea[nb] = -INFINITY;
-        eb[nb] = p.mode == kHeadModeStats ? 0.f : __int_as_float(0x7fffffff);
+        // arg-max: the lane's first vocabulary row stands in until something larger than -inf comes (its rows come in
+        // ascending order, so "lowest index among equals" then takes no index comparisons)
+        const int first_row = (wave * G + c) * 16 + kgp * 4;
+        eb[nb] = p.mode == kHeadModeStats ? 0.f : __int_as_float(first_row < p.V ? first_row : 0x7fffffff);
     }
     const int xl = (kgp ^ (l16 & 3)) << 4, hi = l16 >> 2;
 
@@ -1120,7 +1127,7 @@ __device__ __forceinline__ void head_gemm_stream_body(const HeadParams& p, const
         if constexpr (FUSE)
             fuse_epilogue<E>(p, a[0], (block_pos * G + c) * 16 + kgp * 4, block_pos * 16 + kgp * 4, l16, ea[0], eb[0], s_keys + l16 * kKeyStride);
         else
-            head_epilogue<NB, E>(p, a, (block_pos * G + c) * 16 + kgp * 4, l16, ea, eb);
+            head_epilogue<NB, E, true>(p, a, (block_pos * G + c) * 16 + kgp * 4, l16, ea, eb);
     };
 #pragma unroll
     for (int pl = 0; pl < FP; ++pl) epilogue(acc[pl], pl * kHeadWaves + wave);
@@ -1134,16 +1141,34 @@ __device__ __forceinline__ void head_gemm_stream_body(const HeadParams& p, const
             for (int nb = 0; nb < NB; ++nb) xch[(wave * NB + nb) * 64 + lane] = acc[FP][nb];
         }
         __syncthreads();
-        if (last_active && my_sub == 0) {
-            for (int o = 1; o < share; ++o) {
+        if (FUSE || share == 1) {
+            if (last_active && my_sub == 0) {
+                for (int o = 1; o < share; ++o) {
 #pragma unroll
-                for (int nb = 0; nb < NB; ++nb) {
-                    const f32x4 x = xch[((wave + o) * NB + nb) * 64 + lane];
+                    for (int nb = 0; nb < NB; ++nb) {
+                        const f32x4 x = xch[((wave + o) * NB + nb) * 64 + lane];
 #pragma unroll
-                    for (int r = 0; r < 4; ++r) acc[FP][nb][r] += x[r];
+                        for (int r = 0; r < 4; ++r) acc[FP][nb][r] += x[r];
+                    }
+                }
+                epilogue(acc[FP], FP * kHeadWaves + my_last);
+            }
+        } else if (last_active) {
+            // every wave of the group takes the blocks of hidden rows nb = my_sub, my_sub + share, ...: the same sums in
+            // the same order (slice 0 + slice 1 + ...), a share-th of the additions and of the epilogue each
+            const int w0 = wave - my_sub;
+#pragma unroll
+            for (int nb = 0; nb < NB; ++nb) {
+                if ((nb % share) == my_sub) {   // share is a power of two
+                    f32x4 x = xch[(w0 * NB + nb) * 64 + lane];
+                    for (int o = 1; o < share; ++o) {
+                        const f32x4 y = xch[((w0 + o) * NB + nb) * 64 + lane];
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) x[r] += y[r];
+                    }
+                    head_epilogue_block<E, true>(p, x, nb, ((FP * kHeadWaves + my_last) * G + c) * 16 + kgp * 4, l16, ea[nb], eb[nb]);
                 }
             }
-            epilogue(acc[FP], FP * kHeadWaves + my_last);
         }
     }
     if constexpr (!FUSE) {
