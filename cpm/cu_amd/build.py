@@ -21,6 +21,8 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 ARCH = "gfx950"
 
 HIP_SOURCES = ["runtime.hip", "tree_attention.hip", "lm_head.hip", "topk.hip", "tree_accept.hip", "draft_tree.hip"]
+TIMELINE_SOURCES = ["tree_attention.hip", "lm_head.hip"]  # kernels with optional wall-clock stamps (csrc/timeline.h)
+TIMELINE_LIB_PATH = os.path.join(HERE, "libcpmcu_amd_timeline.so")  # loaded only by `python -m cpm.cu_amd.timeline`
 HEADERS = sorted(f for f in os.listdir(CSRC) if f.endswith(".h"))
 
 # packed fp32 VALU ops stay off for every device translation unit
@@ -61,12 +63,25 @@ def build_all(force=False, verbose=False):
         objs.append(o)
         if force or _stale(o, [s] + common_deps):
             jobs.append([HIPCC] + HIP_FLAGS + ["-c", s, "-o", o])
+    # the same two kernels files once more with wall-clock stamps compiled in (csrc/timeline.h), for a library of their own
+    tl_objs = []
+    for src in HIP_SOURCES:
+        if src in TIMELINE_SOURCES:
+            s = os.path.join(CSRC, src)
+            o = os.path.join(OBJ_DIR, src.replace(".hip", "_timeline.o"))
+            tl_objs.append(o)
+            if force or _stale(o, [s] + common_deps):
+                jobs.append([HIPCC] + HIP_FLAGS + ["-DCPMCU_TIMELINE", "-c", s, "-o", o])
+        else:
+            tl_objs.append(os.path.join(OBJ_DIR, src.replace(".hip", ".o")))
     with ThreadPoolExecutor(max_workers=min(8, max(1, len(jobs)))) as ex:
         for out in ex.map(_run, jobs):
             if verbose and out.strip():
                 print(out)
     if force or jobs or _stale(LIB_PATH, objs):
         _run([HIPCC, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", LIB_PATH] + objs)
+    if force or jobs or _stale(TIMELINE_LIB_PATH, tl_objs):
+        _run([HIPCC, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", TIMELINE_LIB_PATH] + tl_objs)
     # pybind11 module `C`: the reference's entry-point names over the C-ABI
     import pybind11
     mod = pybind_module_path()

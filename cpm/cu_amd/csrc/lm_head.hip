@@ -34,6 +34,7 @@
 
 #include "common.h"
 #include "internal.h"
+#include "timeline.h"
 #include "topk_keys.h"
 
 namespace cpmcu {
@@ -110,6 +111,12 @@ struct HeadFuseReport {
     unsigned int fused_rows;  // rows finished from the published candidates
 };
 __device__ HeadFuseReport g_head_fuse_report;
+
+// Timeline records of the streaming kernels (timeline.h): 0 start, 1 wave 0 out of the K loop, 2 full passes folded,
+// 3 last pass folded, 4 workgroup's partials / statistics out, 8..15 each wave out of the K loop; one-launch FR-Spec
+// form: 5 keys published, 6 stores acknowledged, 7 place known (note 12: place + 1), finishers: 9 all words seen,
+// 10 bound known, 11 candidates listed, 13 row written (note 14: candidates).
+CPMCU_TIMELINE_STORAGE(g_head_timeline)
 
 struct FuseParams {
     HeadFuseState* st;
@@ -714,6 +721,7 @@ __device__ __forceinline__ void fuse_finish_row(const HeadParams& p, const FuseP
     }
     if (late) s_timeout = 1;
     __syncthreads();
+    CPMCU_STAMP(g_head_timeline, blockIdx.x, 9);
     if (s_timeout) {
         // some workgroup's words never came (it was not resident within the wait): the row is not written; the host
         // reads the count at its next synchronisation and reports the call as failed
@@ -777,6 +785,7 @@ __device__ __forceinline__ void fuse_finish_row(const HeadParams& p, const FuseP
     }
     if (lane == 0) s_wave_kth[wave] = kth;
     __syncthreads();
+    CPMCU_STAMP(g_head_timeline, blockIdx.x, 10);
     uint32_t bound = 0;
 #pragma unroll
     for (int i = 1; i < kHeadWaves; ++i) bound = s_wave_kth[i] > bound ? s_wave_kth[i] : bound;
@@ -819,6 +828,7 @@ __device__ __forceinline__ void fuse_finish_row(const HeadParams& p, const FuseP
         }
     }
     __syncthreads();
+    CPMCU_STAMP(g_head_timeline, blockIdx.x, 11);
     const int C = s_ncand;
     if (!s_slow && C <= kFuseCap) {
         int32_t mapped = 0;
@@ -857,6 +867,8 @@ __device__ __forceinline__ void fuse_finish_row(const HeadParams& p, const FuseP
             fp.pos[o] = key_index(key);
             if (fp.ids) fp.ids[o] = mapped;
         }
+        CPMCU_STAMP(g_head_timeline, blockIdx.x, 13);
+        CPMCU_STAMP_VALUE(g_head_timeline, blockIdx.x, 14, C);
         if (tid == 0) {
             __hip_atomic_fetch_add(&g_head_fuse_report.fused_rows, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             st->gen[R] = g1;
@@ -982,6 +994,7 @@ __device__ __forceinline__ void head_gemm_stream_body(const HeadParams& p, const
     const int rotc = c % nch;  // workgroups start their K walk at different chunks (HBM channel spread)
     const E sc = (E)p.head_scale;
 
+    CPMCU_STAMP(g_head_timeline, blockIdx.x, 0);
     int32_t my_tok = 0;
     uint32_t my_gen = 0;
     if constexpr (FUSE) {
@@ -1118,6 +1131,10 @@ __device__ __forceinline__ void head_gemm_stream_body(const HeadParams& p, const
     };
     for (int q = 0; q + 1 < nch; ++q) chunk_body(q, std::true_type{});
     chunk_body(nch - 1, std::false_type{});
+    CPMCU_STAMP(g_head_timeline, blockIdx.x, 1);
+#ifdef CPMCU_TIMELINE
+    if (lane == 0 && blockIdx.x < 1024) g_head_timeline[blockIdx.x * 16 + 8 + wave] = wall_clock64();
+#endif
     unsigned long long ticket = 0;
     if constexpr (FUSE) {
         // this workgroup's place in the order of finishing (used at the very end; wave 7 has the least to do after the loop)
@@ -1131,6 +1148,7 @@ __device__ __forceinline__ void head_gemm_stream_body(const HeadParams& p, const
     };
 #pragma unroll
     for (int pl = 0; pl < FP; ++pl) epilogue(acc[pl], pl * kHeadWaves + wave);
+    CPMCU_STAMP(g_head_timeline, blockIdx.x, 2);
     if (p.rem_blocks > 0) {
         // The waves that shared a block of the last pass hold partial sums over their K slices: they meet in LDS
         // (the hidden buffers are free now) and the first wave of each group adds them up in wave order.
@@ -1171,8 +1189,10 @@ __device__ __forceinline__ void head_gemm_stream_body(const HeadParams& p, const
             }
         }
     }
+    CPMCU_STAMP(g_head_timeline, blockIdx.x, 3);
     if constexpr (!FUSE) {
         head_finish<NB>(p, ea, eb, red_a, red_b, tid, wave, lane, c);
+        CPMCU_STAMP(g_head_timeline, blockIdx.x, 4);
     } else {
         HeadFuseState* st = fp.st;
         // the workgroup's (max, sum exp) of every hidden row, as one tagged word
@@ -1185,6 +1205,7 @@ __device__ __forceinline__ void head_gemm_stream_body(const HeadParams& p, const
                                   (uint64_t)(__float_as_uint(b) | (wide ? 0x80000000u : 0u));
             fuse_store(&st->stats[row][c], word);
         });
+        CPMCU_STAMP(g_head_timeline, blockIdx.x, 4);
         // (head_finish_with has a barrier in it: every wave's keys are in LDS.)  Two hidden rows per wave, one per half
         // of its lanes: the threshold that leaves between fuse_publish_min(k) and 16 of the workgroup's keys of the
         // row, found from the top bit down (keys are unique, so the search ends at exactly that many at the latest).
@@ -1254,12 +1275,16 @@ __device__ __forceinline__ void head_gemm_stream_body(const HeadParams& p, const
         };
         if (p.rem_blocks > 0) select_rows(std::integral_constant<int, (FP + 1) * 4>{});
         else select_rows(std::integral_constant<int, FP * 4>{});
+        CPMCU_STAMP(g_head_timeline, blockIdx.x, 5);
         // every store of this workgroup acknowledged (the logits among them), then its mark; the ticket has long returned
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        CPMCU_STAMP(g_head_timeline, blockIdx.x, 6);
         if (tid == kHeadThreads - 64) s_ticket = (uint32_t)(ticket % (unsigned long long)G);
         __syncthreads();
         if (tid == 0) fuse_store(&st->done[c], (uint64_t)(s_gen[0] + 1));
         const int place = (int)s_ticket;
+        CPMCU_STAMP(g_head_timeline, blockIdx.x, 7);
+        CPMCU_STAMP_VALUE(g_head_timeline, blockIdx.x, 12, place + 1);
         if (place < p.n) fuse_finish_row<E>(p, fp, place, s_gen[place], s_gen[0]);
     }
 }
@@ -1816,3 +1841,5 @@ extern "C" int cpmcu_lm_head_argmax_static(const void* hidden, const void* w, in
     // point creates nothing
     return lm_head_argmax_on(hidden, w, w_layout, n, V, H, apply_scale, head_scale, logits, gt, part, (hipStream_t)stream);
 }
+
+CPMCU_TIMELINE_READER(cpmcu_timeline_read_head, cpmcu::g_head_timeline)

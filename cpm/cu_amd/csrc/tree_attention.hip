@@ -38,6 +38,7 @@
 //    land on the same XCD (workgroup id modulo 8) and share its L2.
 #include "common.h"
 #include "internal.h"
+#include "timeline.h"
 
 #include <map>
 #include <mutex>
@@ -82,6 +83,13 @@ struct AttnReport {
     unsigned int abandoned;
 };
 __device__ AttnReport g_attn_report;
+
+// Timeline records of the split kernel (timeline.h; kept in registers and stored at the end, since the kernel counts its
+// outstanding memory operations by hand): 0 start, 1 K loop entered, 2 K loop left, 3 KV groups merged, 4 partials
+// issued, 5 partials acknowledged, 6 every split of the unit has arrived, 7 end; notes: 8 iterations, 9 tiles, 10 split,
+// 11 M-tile; 12 / 13 second / third iteration entered, 14 / 15 last patch of landed tiles (appended rows, end of the
+// stream) begun / done.
+CPMCU_TIMELINE_STORAGE(g_attn_timeline)
 
 struct AttnParams {
     const f16* q;
@@ -330,6 +338,7 @@ __device__ __forceinline__ void tree_attn_split_body(const AttnParams& p) {
     __shared__ __attribute__((aligned(1024))) char ring[kStages * kStageBytes];
     __shared__ __attribute__((aligned(1024))) char vstage[kVStageRows * kHeadDim * 2];  // first appended V rows, row-major
     __shared__ uint64_t s_mask[kMaxTree * 2];                                            // the tree mask as handed in
+    __shared__ int s_append_page[3];  // pages of the (at most three: T <= 128) tiles that hold appended rows, as their requests found them
 
     // XCD-aware work mapping: the grid is (splits x KV heads, padded to a multiple of the XCD count) x M-tiles.
     // Workgroups are numbered x first and consecutive numbers go to consecutive XCDs, so x % 8 picks the XCD:
@@ -340,6 +349,18 @@ __device__ __forceinline__ void tree_attn_split_body(const AttnParams& p) {
                  "s"(p.mask), "s"(p.mask_words), "s"(p.mask_k_range), "s"(p.T), "s"(p.Hq), "s"(p.Hkv), "s"(p.group), "s"(p.group_shift),
                  "s"(p.hkv_shift), "s"(p.num_splits), "s"(p.num_mtiles), "s"(p.ntiles_max), "s"(p.table_pages), "s"(p.window_blocks),
                  "s"(p.max_kv_len));
+    CPMCU_CLOCK_VAR(tl_start);
+    CPMCU_CLOCK_VAR(tl_loop);
+    CPMCU_CLOCK_VAR(tl_loop_end);
+    CPMCU_CLOCK_VAR(tl_groups);
+    CPMCU_CLOCK_VAR(tl_stored);
+    CPMCU_CLOCK_VAR(tl_acked);
+    CPMCU_CLOCK_VAR(tl_go);
+    CPMCU_CLOCK_VAR(tl_it1);
+    CPMCU_CLOCK_VAR(tl_it2);
+    CPMCU_CLOCK_VAR(tl_fix0);
+    CPMCU_CLOCK_VAR(tl_fix1);
+    CPMCU_CLOCK(tl_start);
     const int sh = blockIdx.x;
     const int mt = blockIdx.y;
     if (sh >= p.num_splits * p.Hkv) return;
@@ -457,9 +478,11 @@ __device__ __forceinline__ void tree_attn_split_body(const AttnParams& p) {
     auto issue_tile_i = [&](int i) {  // the i-th tile of this workgroup's range, into its ring stage
         const int tile = t0 + i;
         const int page = page_of_tile(tile);
-        if (p.k_new != nullptr && (tile + 1) * kTileN > P)
+        if (p.k_new != nullptr && (tile + 1) * kTileN > P) {
+            // (the page is kept for the patch of the landed tile: a table load there would sit in front of its LDS reads)
+            if (tid == 0) s_append_page[min(max(tile - P / kTileN, 0), 2)] = page;
             issue_tile_append(p, g, tile, page, ring + (i % kStages) * kStageBytes, wave_u, lane, koff, voff, P, S);
-        else
+        } else
             issue_tile(p, g, tile, page, ring + (i % kStages) * kStageBytes, wave_u, koff, voff);
     };
     auto issue_iter = [&](int it) {
@@ -557,6 +580,7 @@ __device__ __forceinline__ void tree_attn_split_body(const AttnParams& p) {
             }
     }
 
+    CPMCU_CLOCK(tl_loop);
     for (int it = 0; it < niter; ++it) {
         // Wait for this iteration's tiles.  The prologue issued iterations 0..kDepth and iteration
         // j >= 1 issues iteration j + kDepth right after its barrier, so the tiles issued so far are
@@ -591,6 +615,9 @@ __device__ __forceinline__ void tree_attn_split_body(const AttnParams& p) {
         //  * the tile that holds position S-1 may extend past it: stale page contents there must not
         //    reach the MFMA (0 * NaN = NaN), so the V^T columns of tokens >= S are zeroed.  K needs
         //    nothing: the scores of those keys are replaced (not scaled) by -inf below.
+#ifdef CPMCU_TIMELINE
+        if (it == 1) tl_it1 = wall_clock64();
+#endif
         const int iter_end = (t0 + it * G) * kTileN + G * kTileN;
         const bool iter_needs_fix = iter_end > S || (p.k_new != nullptr && iter_end > P);
         if (iter_needs_fix) {
@@ -600,7 +627,8 @@ __device__ __forceinline__ void tree_attn_split_body(const AttnParams& p) {
                 if (ie >= n) continue;
                 char* st = ring + (ie % kStages) * kStageBytes;
                 const bool append = p.k_new != nullptr && ce + kTileN > P;
-                const int pg = append ? p.block_table[min((ce + kTileN - 1) / kPage, p.table_pages - 1)] : 0;  // a tile lies inside one page
+                // a tile lies inside one page; the id was left in LDS when the tile was requested (a barrier ago at least)
+                const int pg = !append ? 0 : __builtin_amdgcn_readfirstlane(s_append_page[min(max(t0 + ie - P / kTileN, 0), 2)]);
                 if (ROPE && append) {
                     // Fused rotary embedding of the appended K rows (src/model/rotary.cuh:23-33): the tile holds
                     // them as fetched from k_new; one thread per (key, 16-byte piece of the lower half) rotates
@@ -641,6 +669,7 @@ __device__ __forceinline__ void tree_attn_split_body(const AttnParams& p) {
                                 *reinterpret_cast<const f16x8*>(st + k_lds_off(key, piece));
                     }
                 }
+                CPMCU_CLOCK(tl_it2);
                 if (append || ce + kTileN > S) {
                     // V^T, one 16-byte piece (8 token slots of one dim) per thread, read-modify-write:
                     // slots of appended tokens take the value from the staged row-major copy (the
@@ -649,28 +678,57 @@ __device__ __forceinline__ void tree_attn_split_body(const AttnParams& p) {
                     // v_new; the choice is uniform, so the usual case issues no global load here.
                     auto patch_v = [&](auto all_staged_c) {
                         constexpr bool kAllStaged = decltype(all_staged_c)::value;
-                        for (int x = tid; x < kHeadDim * 8; x += kThreads) {
-                            const int d = x & (kHeadDim - 1), sg = x >> 7;
+                        // A wave works on one group of 8 token slots at a time, so which of them are appended rows, which lie
+                        // beyond the end and which staged row each takes its value from are scalar quantities: the per-slot
+                        // index arithmetic and the case distinctions stay off the vector pipe.
+                        static_assert(kThreads % kHeadDim == 0 && (kHeadDim * 8) % kThreads == 0, "whole waves per slot group");
+                        const int d = tid & (kHeadDim - 1);
+#pragma unroll
+                        for (int pass = 0; pass < (kHeadDim * 8) / kThreads; ++pass) {
+                            const int sg = __builtin_amdgcn_readfirstlane(tid / kHeadDim + pass * (kThreads / kHeadDim));
                             f16x8* pp = reinterpret_cast<f16x8*>(st + v_lds_off(d, sg));
                             f16x8 cur = *pp;
                             bool has_new = false;
                             // all eight staged values are read unconditionally (clamped index) and selected
                             // afterwards: conditional reads would each wait for their own LDS round trip
-                            f16 nv[8];
+                            uint16_t nv[8];
 #pragma unroll
                             for (int j = 0; j < 8; ++j) {
                                 const int r = min(max(ce + v_slot16(sg * 8 + j) - P, 0), kAllStaged ? p.T - 1 : kVStageRows - 1);
-                                nv[j] = reinterpret_cast<const f16*>(vstage)[r * kHeadDim + d];
+                                nv[j] = reinterpret_cast<const uint16_t*>(vstage)[r * kHeadDim + d];
                             }
+                            if constexpr (kAllStaged) {
+                                // The eight slots of a group are two runs of four consecutive token positions (v_slot16
+                                // swaps bits 2 and 3 of the slot number), so which of them take the staged value
+                                // ([P, S)), keep the pool's (below P, or below S when nothing is appended) or become
+                                // zero (from S on) are two bit ranges per run: a handful of scalar instructions and one
+                                // and-or per 64 bits, where a comparison chain per slot cost more than the tile's MFMAs.
+                                uint64_t w2[2] = {__builtin_bit_cast(uint4, cur).x | ((uint64_t)__builtin_bit_cast(uint4, cur).y << 32),
+                                                  __builtin_bit_cast(uint4, cur).z | ((uint64_t)__builtin_bit_cast(uint4, cur).w << 32)};
 #pragma unroll
-                            for (int j = 0; j < 8; ++j) {
-                                const int c = ce + v_slot16(sg * 8 + j);
-                                if (append && c >= P && c < S) {
-                                    if (kAllStaged || c - P < kVStageRows) cur[j] = nv[j];
-                                    else cur[j] = p.v_new[((size_t)(c - P) * p.Hkv + g) * kHeadDim + d];
-                                    has_new = true;
-                                } else if (c >= S) {
-                                    cur[j] = (f16)0.f;
+                                for (int h = 0; h < 2; ++h) {
+                                    const int c0 = ce + v_slot16(sg * 8 + 4 * h);
+                                    const int end = min(max(S - c0, 0), 4);
+                                    const int beg = append ? min(max(P - c0, 0), end) : end;
+                                    const uint64_t below_end = end >= 4 ? ~0ull : (1ull << (16 * end)) - 1ull;
+                                    const uint64_t below_beg = beg >= 4 ? ~0ull : (1ull << (16 * beg)) - 1ull;
+                                    const uint64_t staged = (uint64_t)nv[4 * h] | ((uint64_t)nv[4 * h + 1] << 16) | ((uint64_t)nv[4 * h + 2] << 32) |
+                                                            ((uint64_t)nv[4 * h + 3] << 48);
+                                    w2[h] = (staged & below_end & ~below_beg) | (w2[h] & below_beg);
+                                    has_new = has_new || end > beg;
+                                }
+                                cur = __builtin_bit_cast(f16x8, make_uint4((uint32_t)w2[0], (uint32_t)(w2[0] >> 32), (uint32_t)w2[1], (uint32_t)(w2[1] >> 32)));
+                            } else {
+#pragma unroll
+                                for (int j = 0; j < 8; ++j) {
+                                    const int c = ce + v_slot16(sg * 8 + j);
+                                    if (append && c >= P && c < S) {
+                                        if (c - P < kVStageRows) cur[j] = __builtin_bit_cast(f16, nv[j]);
+                                        else cur[j] = p.v_new[((size_t)(c - P) * p.Hkv + g) * kHeadDim + d];
+                                        has_new = true;
+                                    } else if (c >= S) {
+                                        cur[j] = (f16)0.f;
+                                    }
                                 }
                             }
                             *pp = cur;
@@ -682,7 +740,9 @@ __device__ __forceinline__ void tree_attn_split_body(const AttnParams& p) {
                     else patch_v(std::false_type{});
                 }
             }
+            CPMCU_CLOCK(tl_fix0);
             __syncthreads();
+            CPMCU_CLOCK(tl_fix1);
         }
         if (i < n && wave_has_rows) {
             // ---- S^T = K.Q^T : two 32-key blocks.  All 16 operand reads are issued before the first
@@ -798,6 +858,7 @@ __device__ __forceinline__ void tree_attn_split_body(const AttnParams& p) {
         }
     }
 
+    CPMCU_CLOCK(tl_loop_end);
     // ---- the two KV groups meet through LDS ----
     // Each wave keeps half of the output dims of its rows (group 0: d < 64, group 1: d >= 64) and hands the other half
     // to the wave of the other group with the same rows, so that the exchange, the merge and the stores behind it are
@@ -848,6 +909,7 @@ __device__ __forceinline__ void tree_attn_split_body(const AttnParams& p) {
         m_ref = m_new;
     }
 
+    CPMCU_CLOCK(tl_groups);
     // oacc[db][r] is O[query qcol][d = db*32 + 8*(r/4) + 4*hf + r%4], unnormalised; with two KV groups a wave now holds
     // the d blocks [2 * grp, 2 * grp + 2) of its rows.
     const float l_tot = l_run + __shfl_xor(l_run, 32);
@@ -909,8 +971,10 @@ __device__ __forceinline__ void tree_attn_split_body(const AttnParams& p) {
         // the abandoned shares after its own, so the output is complete either way.
         __shared__ int s_merge_go, s_merge_last;
         __shared__ uint32_t s_merge_abandoned;
+        CPMCU_CLOCK(tl_stored);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
+        CPMCU_CLOCK(tl_acked);
         uint32_t* const unit_abandoned = unit_ctr + 1;  // one bit per share; zero between launches (a mark that was made just
                                                         // behind the last arrival's collection is taken back by its maker)
         if (tid == 0) {
@@ -951,6 +1015,7 @@ __device__ __forceinline__ void tree_attn_split_body(const AttnParams& p) {
             s_merge_last = last;
         }
         __syncthreads();
+        CPMCU_CLOCK(tl_go);
         if (!s_merge_go) return;
         const bool last = s_merge_last != 0;
         // the last one collects the abandoned shares while it merges its own
@@ -967,6 +1032,27 @@ __device__ __forceinline__ void tree_attn_split_body(const AttnParams& p) {
             __syncthreads();
             for (uint32_t m = s_merge_abandoned; m != 0; m &= m - 1) merge_share(__builtin_ctz(m));
         }
+#ifdef CPMCU_TIMELINE
+        {
+            const int wg = blockIdx.y * gridDim.x + blockIdx.x;
+            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 0, tl_start);
+            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 1, tl_loop);
+            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 2, tl_loop_end);
+            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 3, tl_groups);
+            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 4, tl_stored);
+            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 5, tl_acked);
+            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 6, tl_go);
+            CPMCU_STAMP(g_attn_timeline, wg, 7);
+            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 8, niter);
+            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 9, n);
+            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 10, split);
+            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 11, mt);
+            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 12, tl_it1);
+            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 13, tl_it2);
+            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 14, tl_fix0);
+            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 15, tl_fix1);
+        }
+#endif
     }
 }
 
@@ -1437,3 +1523,5 @@ extern "C" int cpmcu_rope_apply(const float* cos_sin, int T, int Hq, int Hkv, vo
     CPMCU_LAUNCH_CHECK();
     return CPMCU_OK;
 }
+
+CPMCU_TIMELINE_READER(cpmcu_timeline_read_attention, cpmcu::g_attn_timeline)
