@@ -66,7 +66,8 @@ def attention(L, torch, prefixes):
         _read(L, "attention", 1024)  # clears
         ops.tree_attention(q, cache, 0, kv_len, pad, mask, out=out, k_new=kn, v_new=vn)
         d = _read(L, "attention", 1024)
-        d = d[d[:, 0] > 0]
+        buf_mask = d[:, 0] > 0
+        d = d[buf_mask]
         t0 = d[:, 0].min()
         rel = (d[:, :8] - t0) / 100.0
         kernels, splits, groups, wgs = ops.attention_plan(T, Hq, Hkv, pad)
@@ -78,6 +79,8 @@ def attention(L, torch, prefixes):
         for nt in np.unique(tiles):
             r = rel[tiles == nt]
             print("  workgroups with %d tiles (%d): loop left %.2f, arrived %.2f, end %.2f (medians)" % (nt, len(r), np.median(r[:, 2]), np.median(r[:, 6]), np.median(r[:, 7])))
+        wg = np.nonzero(buf_mask)[0]
+        print("  K loop left by XCD (workgroup number mod 8), medians: " + " ".join("%.1f" % np.median(rel[wg % 8 == x, 2]) for x in range(8)))
         last = d[d[:, 10] == d[:, 10].max()]  # the last split: the appended rows and the end of the stream
         rl = (last - t0) / 100.0
         print("  last split (%d workgroups, %s tiles): loop entered %.2f, second iteration %.2f, patch begun %.2f, V patch begun %.2f, patch done %.2f, loop left %.2f (medians; patch of the M-tile-0 workgroups done %.2f)" %
