@@ -26,6 +26,19 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(raw, name), "libcpmcu_amd.so does not export %s" % name
 
 
+def test_timeline_library_is_the_product_plus_its_readers():
+    """The build with the in-kernel stamps (csrc/timeline.h) exports everything the product library does, and the two
+    functions that hand the records over; the product library has neither."""
+    from cpm.cu_amd import build, lib
+    tl = ctypes.CDLL(build.TIMELINE_LIB_PATH)
+    for name in declared_symbols():
+        assert hasattr(tl, name), "libcpmcu_amd_timeline.so does not export %s" % name
+    product = ctypes.CDLL(lib.LIB_PATH)
+    for name in ("cpmcu_timeline_read_attention", "cpmcu_timeline_read_head"):
+        assert hasattr(tl, name)
+        assert not hasattr(product, name)
+
+
 def test_ctypes_table_matches_header():
     from cpm.cu_amd import lib
     assert sorted(lib.SIGNATURES) == declared_symbols()
