@@ -40,15 +40,14 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 # names the library reports for the dispatch taken: a different instantiation finds no entry and reports null.
 MEASURED_TRAFFIC = {
     "source": "profiles/verify_step_hbm_traffic.md, profiles/tree_attention_long_context_traffic.md",
-    # the library the counters were read on (git rev-parse --short HEAD of that run; the attention kernel, and with it the
-    # long-context figures below, has not changed since 8907f19)
-    "measured_at_commit": "8068df6",
+    # the library the counters were read on (git rev-parse --short HEAD of that run, all figures)
+    "measured_at_commit": "56e9314",
     "kib_per_launch": {
-        "tree_attn_split_kernel<2,false>": 15174 + 9463,  # the merge of the split partials runs inside the launch
+        "tree_attn_split_kernel<2,false>": 15182 + 9463,  # the merge of the split partials runs inside the launch
         "head_gemm_stream_kernel<4,2,256>": 591978 + 128,
     },
     # the attention launch at the longer contexts (32 splits of 256-row workgroups), by prefix length
-    "attention_kib_per_launch_by_context": {"32768": 52479 + 17894, "131072": 150801 + 17894},
+    "attention_kib_per_launch_by_context": {"32768": 52483 + 17894, "131072": 150803 + 17894},
 }
 
 
