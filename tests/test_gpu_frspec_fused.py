@@ -253,3 +253,37 @@ def test_a_wait_that_runs_out_is_reported(gpu, orc, set_option):
     again = ops.frspec_head_topk(to_dev(torch, hid), d_w, d_remap, k)
     lib.get().synchronize()
     _assert_same({key: to_np(v) for key, v in again.items()}, good, "after the wait limit was restored")
+
+
+def test_randomised_sweep(gpu, orc, set_option):
+    """80 random shapes and data sets (1-16 rows, k 1-16, vocabularies of one and two passes with and without a last
+    pass, weights from ordinary to flat to constant, a third of the rows duplicated): nothing differs from the
+    two-launch form, whichever way a row was finished."""
+    torch = gpu
+    from cpm.cu_amd import lib, ops
+    rng = np.random.default_rng(2024)
+    H = 512
+    weights = {}
+    lib.get().synchronize()
+    before = _rows_seen(lib)
+    rows = 0
+    for it in range(80):
+        V = int(rng.choice([4096, 8192, 16384, 32768, 32768, 37568, 50000, 65536]))
+        n, k = int(rng.integers(1, 17)), int(rng.integers(1, 17))
+        std = float(rng.choice([0.02, 0.02, 0.002, 0.0003, 0.0]))
+        if (V, std) not in weights:
+            if len(weights) > 5:
+                weights.clear()
+            w = synth.normal_f16((V, H), it, 2, std=std) if std > 0 else np.zeros((V, H), np.float16)
+            if rng.random() < 0.3:
+                w[rng.integers(1, V, size=V // 3)] = w[0]
+            weights[(V, std)] = ops.tile_head_weight(to_dev(torch, w))
+        hid = (synth.normal_f16((n, H), it, 1).astype(np.float32) * float(rng.choice([1.0, 0.1, 4.0]))).astype(np.float16)
+        remap = rng.permutation(V + 1000)[:V].astype(np.int32)
+        one, two = _both_forms(torch, set_option, hid, weights[(V, std)], to_dev(torch, remap), k)
+        _assert_same(one, two, "case %d: V=%d n=%d k=%d std=%g" % (it, V, n, k, std))
+        rows += n
+    lib.get().synchronize()
+    after = _rows_seen(lib)
+    assert after[2] == before[2]
+    assert after[0] - before[0] > 0 and after[1] - before[1] > 0, "both ways of finishing a row are expected in the sweep"
