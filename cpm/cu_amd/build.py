@@ -21,7 +21,7 @@ HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 ARCH = "gfx950"
 
 HIP_SOURCES = ["runtime.hip", "tree_attention.hip", "lm_head.hip", "topk.hip", "tree_accept.hip", "draft_tree.hip"]
-TIMELINE_SOURCES = ["tree_attention.hip", "lm_head.hip"]  # kernels with optional wall-clock stamps (csrc/timeline.h)
+TIMELINE_SOURCES = ["tree_attention.hip", "lm_head.hip", "topk.hip"]  # kernels with optional wall-clock stamps (csrc/timeline.h)
 TIMELINE_LIB_PATH = os.path.join(HERE, "libcpmcu_amd_timeline.so")  # loaded only by `python -m cpm.cu_amd.timeline`
 HEADERS = sorted(f for f in os.listdir(CSRC) if f.endswith(".h"))
 

@@ -17,10 +17,15 @@
 // reduced from the GEMM's per-workgroup partials, and rank that.
 #include "common.h"
 #include "internal.h"
+#include "timeline.h"
 #include "topk_keys.h"
 
 namespace cpmcu {
 namespace {
+
+// Timeline records of the row kernel (timeline.h): 0 start, 1 the row is in registers as ordered images, 2 bound and row
+// statistics known, 3 candidate lanes handed to LDS, 4 candidates extracted, 5 ranked, 6 outputs written.
+CPMCU_TIMELINE_STORAGE(g_topk_timeline)
 
 struct TopkParams {
     const uint16_t* x;  // [n][dim] fp16 bits
@@ -177,6 +182,7 @@ __device__ __forceinline__ void topk_row_body(const TopkParams& p) {
     __shared__ int ncand, nlanes;
     __shared__ uint4 lanebuf[kRowPieces][kRowLaneCap];  // piece-major: neighbouring slots are neighbouring 16 bytes
     __shared__ int lane_owner[kRowLaneCap];
+    CPMCU_STAMP(g_topk_timeline, blockIdx.x, 0);
     const int row = blockIdx.x;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int npieces = p.dim >> 3;
@@ -222,6 +228,10 @@ __device__ __forceinline__ void topk_row_body(const TopkParams& p) {
         }
     }
     const uint32_t lmax = lmax2[0] > lmax2[1] ? lmax2[0] : lmax2[1];
+#ifdef CPMCU_TIMELINE
+    asm volatile("" ::"v"(lmax));
+#endif
+    CPMCU_STAMP(g_topk_timeline, blockIdx.x, 1);
     // k-th largest of this wave's lane maxima, rounded down to a multiple of 2^kRowBoundDrop (0 when
     // fewer than k lanes hold anything): a slightly lower bound is as valid and costs fewer steps
     // (with fused statistics wave 0 reduces those meanwhile and contributes no bound: any subset of
@@ -265,6 +275,7 @@ __device__ __forceinline__ void topk_row_body(const TopkParams& p) {
         }
     }
     __syncthreads();
+    CPMCU_STAMP(g_topk_timeline, blockIdx.x, 2);
     uint32_t bound = wave_kth[0];
 #pragma unroll
     for (int w = 1; w < kRowWaves; ++w) bound = wave_kth[w] > bound ? wave_kth[w] : bound;
@@ -295,6 +306,7 @@ __device__ __forceinline__ void topk_row_body(const TopkParams& p) {
         }
     }
     __syncthreads();
+    CPMCU_STAMP(g_topk_timeline, blockIdx.x, 3);
     const int NT = nlanes;
     const bool compact = bounded && NT <= kRowLaneCap;
     // ... where a few waves take them over with most of their lanes busy: bit mask of the
@@ -344,6 +356,7 @@ __device__ __forceinline__ void topk_row_body(const TopkParams& p) {
         }
     }
     __syncthreads();
+    CPMCU_STAMP(g_topk_timeline, blockIdx.x, 4);
     const int C = ncand;
     if (compact && C <= kRowCap) {
         int shift = 6;
@@ -368,6 +381,7 @@ __device__ __forceinline__ void topk_row_body(const TopkParams& p) {
             if (r) atomicAdd(&rank[i], r);
         }
         __syncthreads();
+        CPMCU_STAMP(g_topk_timeline, blockIdx.x, 5);
         if (tid < C && rank[tid] < p.top) {
             const uint64_t key = cand[tid];
             const int idx = key_index(key);
@@ -376,6 +390,7 @@ __device__ __forceinline__ void topk_row_body(const TopkParams& p) {
             p.pos[o] = idx;
             if (p.ids) p.ids[o] = mapped;
         }
+        CPMCU_STAMP(g_topk_timeline, blockIdx.x, 6);
         return;
     }
     uint64_t prev = ~0ull;
@@ -601,3 +616,5 @@ extern "C" int cpmcu_head_release_workspace(const void* workspace) {
     head_fuse_release_workspace(workspace);
     return CPMCU_OK;
 }
+
+CPMCU_TIMELINE_READER(cpmcu_timeline_read_topk, cpmcu::g_topk_timeline)

@@ -23,7 +23,7 @@ def _load():
         raise ImportError("%s is missing: run `python -m cpm.cu_amd.build`" % build.TIMELINE_LIB_PATH)
     libmod.LIB_PATH = build.TIMELINE_LIB_PATH  # before the first lib.get()
     L = libmod.get()
-    for name in ("cpmcu_timeline_read_head", "cpmcu_timeline_read_attention"):
+    for name in ("cpmcu_timeline_read_head", "cpmcu_timeline_read_attention", "cpmcu_timeline_read_topk"):
         getattr(L.raw, name).argtypes = [ctypes.c_void_p]
         getattr(L.raw, name).restype = ctypes.c_int
     return L
@@ -143,6 +143,7 @@ def frspec(L, torch):
         print("FR-Spec head %d x %d, %d rows, top-%d: %s, %.2f us per call (eager, rotated copies, stamps compiled in)" %
               (V, H, n, k, ops.frspec_head_plan(n, ws[0], k), e0.elapsed_time(e1) / (20 * copies) * 1e3))
         _read(L, "head", 1024)
+        _read(L, "topk", 16)
         ops.frspec_head_topk(hid, ws[0], remap, k)
         d, t0 = _head_records(L, 256)
         rel = (d - t0) / 100.0
@@ -161,6 +162,14 @@ def frspec(L, torch):
             print("  last keys published %.2f, last row written %.2f" % (rel[:, 5].max(), ((fin[:, 13] - t0) / 100.0).max()))
         else:
             print(_spread("every wave out of the K loop", waves))
+            # the row kernel that follows (records of its own clock origin: its first workgroup's start)
+            tk = _read(L, "topk", n)
+            gemm_end = rel[:, 4].max()
+            tr = (tk[:, :7] - tk[:, 0].min()) / 100.0
+            print("  topk_row_kernel<true> (%d workgroups of 1024 threads), from the start of its first workgroup, which comes %.2f us after the GEMM's last partials:" %
+                  (n, (tk[:, 0].min() - t0) / 100.0 - gemm_end))
+            for i, nm in enumerate(["start", "row in registers", "bound and statistics known", "candidate lanes in LDS", "candidates extracted", "ranked", "outputs written"]):
+                print(_spread(nm, tr[:, i]))
     libmod.get().set_option(b"frspec_fused", 0)
 
 

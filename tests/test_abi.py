@@ -34,7 +34,7 @@ def test_timeline_library_is_the_product_plus_its_readers():
     for name in declared_symbols():
         assert hasattr(tl, name), "libcpmcu_amd_timeline.so does not export %s" % name
     product = ctypes.CDLL(lib.LIB_PATH)
-    for name in ("cpmcu_timeline_read_attention", "cpmcu_timeline_read_head"):
+    for name in ("cpmcu_timeline_read_attention", "cpmcu_timeline_read_head", "cpmcu_timeline_read_topk"):
         assert hasattr(tl, name)
         assert not hasattr(product, name)
 
