@@ -138,6 +138,7 @@ def draft_ids_for_accept(tree, gt, accept_depth, vocab, seed, leaf=None):
         if i in on_path:
             tok = int(gt[p])
         else:
+            assert len(taken) + 1 < vocab, "node %d has more children than the vocabulary has distinct tokens" % p
             while True:
                 tok = int(g.integers(vocab))
                 if tok != int(gt[p]) and tok not in taken:

@@ -1,0 +1,144 @@
+"""Time-boxed random parity runs of every operator of the path against the CPU oracle, on cuda:0.
+
+    python tests/fuzz_parity.py [seconds (default 360)] [first seed (default 1000)]
+
+Not collected by pytest (the suites in test_gpu_*.py are the fixed, seeded cases); this draws fresh shapes and data for as
+long as it is given and applies the same checks through the tests' own helpers: tree attention in its three input modes
+(values to fp16 tolerance, appended cache rows bit for bit), the target head's arg-max, the FR-Spec head with log-softmax,
+top-k and id map-back, the stand-alone top-k (ties, -inf, wide ranges), acceptance / compaction / the one-launch tail, and
+the draft-tree construction (all bit-exact).  Shapes the C-ABI refuses by contract (a documented limit) are counted, not
+failures.  Exit status 1 and one line per mismatch (operator, seed, message) if anything differs.
+"""
+import os
+import sys
+import time
+import warnings
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, ROOT)
+sys.path.insert(0, os.path.join(ROOT, "tests"))
+
+import numpy as np  # noqa: E402
+
+
+def main(argv):
+    import torch
+    import oracle as orc
+    from cpm.cu_amd import lib, ops, synth
+    import test_gpu_accept as t_accept
+    import test_gpu_attention as t_attention
+    import test_gpu_draft_tree as t_draft
+    import test_gpu_heads as t_heads
+    from util import to_dev, to_np
+
+    budget = float(argv[0]) if len(argv) > 0 else 360.0
+    first_seed = int(argv[1]) if len(argv) > 1 else 1000
+    lib.get()  # raises if libcpmcu_amd.so is missing: nothing here runs without the HIP library
+    torch.cuda.set_device(0)
+    warnings.simplefilter("ignore")
+    fails = []
+
+    def run(name, fn, secs):
+        t0 = time.time()
+        n = refused = 0
+        while time.time() - t0 < secs:
+            seed = first_seed + n
+            try:
+                fn(seed)
+            except ValueError as e:  # CPMCU_ERR_INVALID_ARGUMENT: a shape outside a documented limit
+                if "limit" not in str(e) and "outside" not in str(e):
+                    raise
+                refused += 1
+            except AssertionError as e:
+                fails.append((name, seed, str(e)[:300]))
+                print("MISMATCH", name, seed, str(e)[:300], flush=True)
+            n += 1
+        print("%s: %d cases (%d refused by the API) in %.0f s, %d mismatches so far" % (name, n, refused, time.time() - t0, len(fails)), flush=True)
+
+    def attention(seed):
+        g = synth.rng(seed, 91)
+        edges_p = [0, 1, 63, 64, 65, 127, 128, 129, 255, 256, 257, 511, 512, 513, 1023, 1024, 1025, 2047, 2048, 2049]
+        edges_t = [1, 2, 3, 8, 15, 16, 17, 31, 32, 33, 60, 63, 64, 65, 100, 127, 128]
+        P = int(edges_p[g.integers(len(edges_p))]) if g.random() < 0.5 else int(g.integers(0, 5000))
+        T = int(edges_t[g.integers(len(edges_t))]) if g.random() < 0.6 else int(g.integers(1, 129))
+        mode = ["in_cache", "append", "append_rope"][int(g.integers(3))]
+        splits = [0, 0, 0, 1, 2, 3, 5, 7, 16][int(g.integers(9))]
+        slack = [0, 0, 1, 63, 64, 200, 1000][int(g.integers(7))]
+        t_attention.test_randomised_shape_sweep(torch, orc, P, T, mode, splits, slack, seed)
+
+    def target_head(seed):
+        g = synth.rng(seed, 92)
+        n = int(g.integers(1, 129))
+        V = int(g.integers(16, 40000))
+        H = int([512, 1024, 2048, 4096][g.integers(4)])
+        if H >= 2048:
+            V = min(V, 12000)
+        t_heads._argmax_check(torch, orc, n, V=V, H=H, seed=seed, scale=[None, 0.5, 1.7][int(g.integers(3))], tiled=bool(g.integers(2)))
+
+    def frspec_head(seed):
+        g = synth.rng(seed, 93)
+        n = int(g.integers(1, 17))
+        H = int([512, 1024][g.integers(2)])
+        Vs = int(g.integers(2, 4200)) * 8
+        V = Vs + int(g.integers(0, 5000))
+        t_heads._frspec_check(torch, orc, n, V, Vs, H, int(g.integers(1, 17)), seed, tiled=bool(g.integers(2)))
+
+    def topk(seed):
+        g = synth.rng(seed, 94)
+        n = int(g.integers(1, 6))
+        dim = int(g.integers(1, 40000))
+        top = int(g.integers(1, min(dim, 128) + 1))
+        kind = int(g.integers(4))
+        if kind == 0:
+            x = g.standard_normal((n, dim)).astype(np.float16)
+        elif kind == 1:
+            x = g.integers(-3, 3, size=(n, dim)).astype(np.float16)  # ties everywhere
+        elif kind == 2:
+            x = np.full((n, dim), -np.inf, np.float16)  # mostly -inf
+            idx = g.integers(0, dim, size=max(1, dim // 50))
+            x[:, idx] = g.standard_normal(len(idx)).astype(np.float16)
+        else:
+            x = (g.standard_normal((n, dim)) * np.exp(g.standard_normal((n, dim)) * 2)).astype(np.float16)
+        val, pos = ops.topk(to_dev(torch, x), top)
+        torch.cuda.synchronize()
+        v_ref, p_ref = orc.topk(x, top)
+        what = "n=%d dim=%d top=%d kind=%d" % (n, dim, top, kind)
+        assert np.array_equal(to_np(pos), p_ref), "top-k positions, " + what
+        assert np.array_equal(to_np(val).view(np.uint16), v_ref.view(np.uint16)), "top-k values, " + what
+
+    def tail(seed):
+        g = synth.rng(seed, 95)
+        T = int(g.integers(1, 129))
+        tree = synth.random_tree(T, seed, max_children=int(g.integers(1, 8)), max_depth=int(g.integers(1, 14)))
+        P = int(g.integers(0, 1200))
+        depth = int(g.integers(0, int(tree.depth.max()) + 1))
+        kind = int(g.integers(3))
+        if kind == 0:
+            t_accept._compact_case(torch, orc, tree, P, depth, layers=2, seed=seed, page_perm=bool(g.integers(2)))
+        elif kind == 1:
+            t_accept._tail_case(torch, orc, tree, P, depth, layers=2, seed=seed, H=512, V=int(g.integers(200, 5000)), from_partials=bool(g.integers(2)))
+        else:
+            t_accept._commit_case(torch, orc, tree, P, depth, layers=2, seed=seed)
+
+    def draft_tree(seed):
+        g = synth.rng(seed, 96)
+        k = int(g.integers(1, 17))
+        num_iter = min(int(g.integers(2, 9)), max(2, 64 // k))  # k * num_iter fits the 64-bit draft mask
+        T = int(g.integers(2, min(128, 1 + k * num_iter) + 1))
+        t_draft.test_draft_tree_equals_oracle(torch, orc, k, num_iter, T, seed, bool(g.integers(2)), bool(g.integers(2)))
+
+    share = budget / 6
+    run("tree attention", attention, share)
+    run("target head", target_head, share)
+    run("FR-Spec head", frspec_head, share)
+    run("top-k", topk, share)
+    run("accept / compaction / tail", tail, share)
+    run("draft tree", draft_tree, share)
+    print("mismatches: %d" % len(fails))
+    for f in fails:
+        print(f)
+    return 1 if fails else 0
+
+
+if __name__ == "__main__":
+    sys.exit(main(sys.argv[1:]))
