@@ -181,26 +181,24 @@ def test_pybind_module_drives_the_path_end_to_end(gpu, orc):
     C.shutdown()
 
 
-def test_library_graph_replays_equal_eager_steps(gpu, orc):
+def _graph_replays_equal_eager_steps(torch, orc, seed, T, P0, STEPS, LAYERS=3, V=3000, H=512, num_iter=6, topk=4, min_paddings=2):
     """cpmcu_verify_step on the library's own storage: the same sequence of steps enqueued eagerly and as replays of
     the library's HIP graphs (one per padded length, lengths and positions advancing on the device) must give the same
     accept lengths, ids, gathered hidden rows and caches, and both must match the oracle's acceptance on the device's
     own arg-max.  The second model instance reuses the process-global model after a shutdown."""
     from cpm.cu_amd import ops
     from cpm.cu_amd.model import PathModel
-    torch = gpu
-    V, H, LAYERS, T, P0, STEPS = 3000, 512, 3, 24, 1000, 10
-    tree = synth.random_tree(T, 3, max_children=3, max_depth=6)
+    tree = synth.random_tree(T, seed, max_children=3, max_depth=6)
     mask, parent = to_dev(torch, tree.mask), to_dev(torch, tree.parent)
-    w = synth.normal_f16((V, H), 3, 2, std=0.02)
+    w = synth.normal_f16((V, H), seed, 2, std=0.02)
     w_dev = ops.tile_head_weight(to_dev(torch, w))
-    rg = synth.rng(3, 8)
+    rg = synth.rng(seed, 8)
     inputs = []
     for s in range(STEPS):
-        x = dict(q=[to_dev(torch, synth.normal_f16((T, HQ, D), 3, 1000 + 10 * s + l)) for l in range(LAYERS)],
-                 k=[to_dev(torch, synth.normal_f16((T, HKV, D), 3, 2000 + 10 * s + l)) for l in range(LAYERS)],
-                 v=[to_dev(torch, synth.normal_f16((T, HKV, D), 3, 3000 + 10 * s + l)) for l in range(LAYERS)],
-                 hidden=to_dev(torch, synth.normal_f16((T, H), 3, 4000 + s)))
+        x = dict(q=[to_dev(torch, synth.normal_f16((T, HQ, D), seed, 1000 + 10 * s + l)) for l in range(LAYERS)],
+                 k=[to_dev(torch, synth.normal_f16((T, HKV, D), seed, 2000 + 10 * s + l)) for l in range(LAYERS)],
+                 v=[to_dev(torch, synth.normal_f16((T, HKV, D), seed, 3000 + 10 * s + l)) for l in range(LAYERS)],
+                 hidden=to_dev(torch, synth.normal_f16((T, H), seed, 4000 + s)))
         x["gt"] = to_np(ops.lm_head_argmax(x["hidden"], w_dev, head_scale=0.5))
         x["depth"] = int(rg.integers(0, int(tree.depth.max()) + 1))
         pred, leaf = synth.draft_ids_for_accept(tree, x["gt"], x["depth"], V, 300 + s)
@@ -210,13 +208,13 @@ def test_library_graph_replays_equal_eager_steps(gpu, orc):
     del w_dev
 
     def run(graph):
-        m = PathModel(V, LAYERS, H, HQ, HKV, memory_limit=0.01, scale_lmhead=0.5, tree_size=T, num_iter=6, topk=4)
+        m = PathModel(V, LAYERS, H, HQ, HKV, memory_limit=0.01, scale_lmhead=0.5, tree_size=T, num_iter=num_iter, topk=topk)
         try:
             m.load_head(w)
             cache = m.cache()
             for layer in range(LAYERS):
-                cache.write_logical(layer, 0, to_dev(torch, synth.normal_f16((P0, HKV, D), 3, 10 + layer)),
-                                    to_dev(torch, synth.normal_f16((P0, HKV, D), 3, 50 + layer)))
+                cache.write_logical(layer, 0, to_dev(torch, synth.normal_f16((P0, HKV, D), seed, 10 + layer)),
+                                    to_dev(torch, synth.normal_f16((P0, HKV, D), seed, 50 + layer)))
             f16 = dict(dtype=torch.float16, device="cuda")
             bq = [torch.zeros((T, HQ, D), **f16) for _ in range(LAYERS)]
             bk = [torch.zeros((T, HKV, D), **f16) for _ in range(LAYERS)]
@@ -258,12 +256,16 @@ def test_library_graph_replays_equal_eager_steps(gpu, orc):
 
     hist_e, kv_e, P_e, _ = run(False)
     hist_g, kv_g, P_g, npad = run(True)
-    assert P_e == P_g and npad >= 2, "the run should cross a padded length (%d seen)" % npad
+    assert P_e == P_g and npad >= min_paddings, "the run should cross a padded length (%d seen)" % npad
     for (a1, i1, o1), (a2, i2, o2) in zip(hist_e, hist_g):
         assert (a1, i1) == (a2, i2)
         assert np.array_equal(o1.view(np.uint16), o2.view(np.uint16))  # same launches, same split geometry: same bits
     for (k1, v1), (k2, v2) in zip(kv_e, kv_g):
         assert np.array_equal(k1.view(np.uint16), k2.view(np.uint16)) and np.array_equal(v1.view(np.uint16), v2.view(np.uint16))
+
+
+def test_library_graph_replays_equal_eager_steps(gpu, orc):
+    _graph_replays_equal_eager_steps(gpu, orc, seed=3, T=24, P0=1000, STEPS=10)
 
 
 def test_step_graph_cache_is_bounded(gpu, orc):
