@@ -7,7 +7,8 @@ long as it is given and applies the same checks through the tests' own helpers: 
 (values to fp16 tolerance, appended cache rows bit for bit), the target head's arg-max, the FR-Spec head with log-softmax,
 top-k and id map-back, the stand-alone top-k (ties, -inf, wide ranges), acceptance / compaction / the one-launch tail,
 the draft-tree construction (all bit-exact), sequences of model-level verify steps enqueued eagerly and replayed as the
-library's graphs, and a speculative loop on a toy target against plain greedy decoding.  Shapes the C-ABI refuses by contract (a documented limit) are counted, not
+library's graphs, a speculative loop on a toy target against plain greedy decoding, and the bfloat16 instantiations of the
+attention and the two heads.  Shapes the C-ABI refuses by contract (a documented limit) are counted, not
 failures.  Exit status 1 and one line per mismatch (operator, seed, message) if anything differs.
 """
 import os
@@ -28,6 +29,7 @@ def main(argv):
     from cpm.cu_amd import lib, ops, synth
     import test_gpu_accept as t_accept
     import test_gpu_attention as t_attention
+    import test_gpu_bf16 as t_bf16
     import test_gpu_draft_tree as t_draft
     import test_gpu_heads as t_heads
     import test_gpu_spec_loop as t_loop
@@ -142,9 +144,36 @@ def main(argv):
     def speculative_loop(seed):
         t_loop._speculative_loop(torch, orc, seed)
 
+    def bf16_operators(seed):
+        g = synth.rng(seed, 98)
+        L = lib.get()
+
+        def set_option(name, value):
+            L.set_option(name.encode(), int(value))
+        set_option("dtype", 1)
+        orc.set_dtype("bf16")
+        try:
+            kind = int(g.integers(3))
+            if kind == 0:
+                t_bf16.test_bf16_tree_attention_with_fused_append(torch, orc, None, set_option, int(g.integers(1, 3)), int(g.integers(0, 5000)),
+                                                                  int(g.integers(2, 61)), bool(g.integers(2)))
+            elif kind == 1:
+                H = int([512, 1024, 2048][g.integers(3)])
+                t_bf16.test_bf16_target_head_and_argmax(torch, orc, None, int(g.integers(1, 129)), int(g.integers(16, 12000)), H, bool(g.integers(2)),
+                                                        [None, 0.3125][int(g.integers(2))])
+            else:
+                Vs = int(g.integers(2, 2100)) * 8
+                t_bf16.test_bf16_frspec_head_topk(torch, orc, None, int(g.integers(1, 17)), Vs + int(g.integers(0, 3000)), Vs, int([512, 1024][g.integers(2)]),
+                                                  int(g.integers(1, 17)), bool(g.integers(2)))
+        finally:
+            orc.set_dtype("f16")
+            set_option("dtype", 0)
+            set_option("attn_kv_groups", 0)
+
     stages = [("attention", "tree attention", attention), ("head", "target head", target_head), ("frspec", "FR-Spec head", frspec_head),
               ("topk", "top-k", topk), ("tail", "accept / compaction / tail", tail), ("draft", "draft tree", draft_tree),
-              ("steps", "verify steps, eager and as graph replays", verify_steps), ("loop", "speculative loop against greedy decoding", speculative_loop)]
+              ("steps", "verify steps, eager and as graph replays", verify_steps), ("loop", "speculative loop against greedy decoding", speculative_loop),
+              ("bf16", "bfloat16: attention with fused append, target head, FR-Spec head", bf16_operators)]
     if len(argv) > 2:
         wanted = argv[2].split(",")
         unknown = [w for w in wanted if w not in [k for k, _, _ in stages]]
