@@ -8,7 +8,7 @@ long as it is given and applies the same checks through the tests' own helpers: 
 top-k and id map-back, the stand-alone top-k (ties, -inf, wide ranges), acceptance / compaction / the one-launch tail,
 the draft-tree construction (all bit-exact), sequences of model-level verify steps enqueued eagerly and replayed as the
 library's graphs, a speculative loop on a toy target against plain greedy decoding, and the bfloat16 instantiations of the
-attention and the two heads.  Shapes the C-ABI refuses by contract (a documented limit) are counted, not
+attention and the two heads; the FR-Spec head's one-launch form is held to the two-launch one.  Shapes the C-ABI refuses by contract (a documented limit) are counted, not
 failures.  Exit status 1 and one line per mismatch (operator, seed, message) if anything differs.
 """
 import os
@@ -31,6 +31,7 @@ def main(argv):
     import test_gpu_attention as t_attention
     import test_gpu_bf16 as t_bf16
     import test_gpu_draft_tree as t_draft
+    import test_gpu_frspec_fused as t_fused
     import test_gpu_heads as t_heads
     import test_gpu_spec_loop as t_loop
     import test_gpu_verify_step as t_step
@@ -45,9 +46,12 @@ def main(argv):
     fails = []
 
     def run(name, fn, secs):
-        t0 = time.time()
+        t0 = last = time.time()
         n = refused = 0
         while time.time() - t0 < secs:
+            if time.time() - last > 30:  # a sign of life for whoever watches the output
+                last = time.time()
+                print("  %s: %d cases so far" % (name, n), flush=True)
             seed = first_seed + n
             try:
                 fn(seed)
@@ -170,9 +174,33 @@ def main(argv):
             set_option("dtype", 0)
             set_option("attn_kv_groups", 0)
 
+    fused_weights = {}
+
+    def frspec_one_launch(seed):
+        # the one-launch form (option frspec_fused) against the two-launch form, which the "frspec" stage holds to the oracle
+        g = synth.rng(seed, 99)
+        H = 512
+        V = int([2048, 4096, 8192, 16384, 32768, 32768, 37568, 50000, 65536][g.integers(9)])
+        std = float([0.02, 0.02, 0.002, 0.0003, 0.0][g.integers(5)])
+        n, k = int(g.integers(1, 17)), int(g.integers(1, 17))
+        if (V, std) not in fused_weights:
+            if len(fused_weights) > 5:
+                fused_weights.clear()
+            w = synth.normal_f16((V, H), seed, 2, std=std) if std > 0 else np.zeros((V, H), np.float16)
+            if g.random() < 0.3:
+                w[g.integers(1, V, size=V // 3)] = w[0]
+            fused_weights[(V, std)] = ops.tile_head_weight(to_dev(torch, w))
+        hid = (synth.normal_f16((n, H), seed, 1).astype(np.float32) * float([1.0, 0.1, 4.0][g.integers(3)])).astype(np.float16)
+        remap = g.permutation(V + 1000)[:V].astype(np.int32)
+        one, two = t_fused._both_forms(torch, lambda name, v: lib.get().set_option(name.encode(), int(v)), hid, fused_weights[(V, std)],
+                                       to_dev(torch, remap), k)
+        t_fused._assert_same(one, two, "V=%d n=%d k=%d std=%g" % (V, n, k, std))
+        lib.get().synchronize()  # a wait that ran out would be an error here
+
     stages = [("attention", "tree attention", attention), ("head", "target head", target_head), ("frspec", "FR-Spec head", frspec_head),
               ("topk", "top-k", topk), ("tail", "accept / compaction / tail", tail), ("draft", "draft tree", draft_tree),
               ("steps", "verify steps, eager and as graph replays", verify_steps), ("loop", "speculative loop against greedy decoding", speculative_loop),
+              ("fused", "FR-Spec head in one launch against the two-launch form", frspec_one_launch),
               ("bf16", "bfloat16: attention with fused append, target head, FR-Spec head", bf16_operators)]
     if len(argv) > 2:
         wanted = argv[2].split(",")
@@ -183,6 +211,9 @@ def main(argv):
         stages = [st for st in stages if st[0] in wanted]
     for _, name, fn in stages:
         run(name, fn, budget / len(stages))
+    rows = t_fused._rows_seen(lib)
+    if any(rows):
+        print("one-launch FR-Spec rows: %d finished from the published keys, %d redone from the logits, %d waits ran out" % rows)
     print("mismatches: %d" % len(fails))
     for f in fails:
         print(f)
