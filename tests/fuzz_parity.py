@@ -76,7 +76,11 @@ def main(argv):
         mode = ["in_cache", "append", "append_rope"][int(g.integers(3))]
         splits = [0, 0, 0, 1, 2, 3, 5, 7, 16][int(g.integers(9))]
         slack = [0, 0, 1, 63, 64, 200, 1000][int(g.integers(7))]
-        t_attention.test_randomised_shape_sweep(torch, orc, P, T, mode, splits, slack, seed)
+        lib.get().set_option(b"attn_kv_groups", int(g.integers(3)))  # 0 = the library's choice
+        try:
+            t_attention.test_randomised_shape_sweep(torch, orc, P, T, mode, splits, slack, seed)
+        finally:
+            lib.get().set_option(b"attn_kv_groups", 0)
 
     def target_head(seed):
         g = synth.rng(seed, 92)
@@ -174,6 +178,34 @@ def main(argv):
             set_option("dtype", 0)
             set_option("attn_kv_groups", 0)
 
+    def windows(seed):
+        # the drafter's own layers: a mask over k*d columns, the block sliding window; and the window under a verify-sized tree
+        g = synth.rng(seed, 100)
+        kind = int(g.integers(3))
+        window = int([128, 256, 512, 1024, 2048, 4096][g.integers(6)])
+        if kind == 2:
+            t_attention.test_tree_block_window_with_rope(torch, orc, int(g.integers(0, 6000)), int(g.integers(1, 65)), window, bool(g.integers(2)))
+            return
+        k = int(g.integers(1, 17))
+        d = int(g.integers(1, min(8, 64 // k) + 1))
+        P0 = int(g.integers(0, 5000))
+        if kind == 0:
+            t_attention.test_draft_layer_mask_range(torch, orc, k, d, P0, seed)
+        else:
+            t_attention.test_draft_layer_block_window(torch, orc, k, d, P0, window, int([0, 0, 1, 2, 3, 5][g.integers(6)]), seed)
+
+    def merge_forms(seed):
+        # the merge inside the split launch against the separate combine launch: bit-identical outputs when the split count
+        # is the same (left to the library, the two forms may partition the keys differently: other roundings)
+        g = synth.rng(seed, 101)
+        L = lib.get()
+        try:
+            t_attention.test_merge_in_launch_equals_separate_merge(torch, lambda name, v: L.set_option(name.encode(), int(v)), int(g.integers(0, 9000)),
+                                                                   int(g.integers(1, 129)), int([1, 2, 3, 4, 5, 7, 8, 11, 16, 24, 32][g.integers(11)]),
+                                                                   bool(g.integers(2)), bool(g.integers(2)))
+        finally:
+            L.set_option(b"attn_merge_in_launch", 1)
+
     fused_weights = {}
 
     def frspec_one_launch(seed):
@@ -200,6 +232,8 @@ def main(argv):
     stages = [("attention", "tree attention", attention), ("head", "target head", target_head), ("frspec", "FR-Spec head", frspec_head),
               ("topk", "top-k", topk), ("tail", "accept / compaction / tail", tail), ("draft", "draft tree", draft_tree),
               ("steps", "verify steps, eager and as graph replays", verify_steps), ("loop", "speculative loop against greedy decoding", speculative_loop),
+              ("window", "drafter-layer attention: mask range, block window; window under a tree with rotary embedding", windows),
+              ("merge", "attention merged inside the launch against the combine launch", merge_forms),
               ("fused", "FR-Spec head in one launch against the two-launch form", frspec_one_launch),
               ("bf16", "bfloat16: attention with fused append, target head, FR-Spec head", bf16_operators)]
     if len(argv) > 2:
