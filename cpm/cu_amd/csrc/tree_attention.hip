@@ -147,70 +147,113 @@ __device__ inline To bits_as(const From& v) {
     return __builtin_bit_cast(To, v);
 }
 
-// Merge of the split partials of one 32-row block and one quad of output dims (one wave; lane = accumulator lane):
+// Merge of the split partials of one 32-row block and one quad of output dims (lane = accumulator lane):
 // M = max_s m_s, L = sum_s l_s 2^(m_s - M), O = sum_s l_s 2^(m_s - M) (O_s / l_s) / L -- the log-sum-exp merge of
-// src/flash_attn/src/flash_fwd_kernel.h:2392-2472 in base-2 form.  The statistics and the O partials of up to 16
-// splits are all requested before any is used, so a block pays one memory round trip, not one per split.
+// src/flash_attn/src/flash_fwd_kernel.h:2392-2472 in base-2 form -- in batches of up to 16 splits: the statistics and
+// the O partials of a batch are all requested before any is used (one memory round trip, not one per split) and summed
+// relative to the batch's own maximum; the batch sums are then folded into the running result in batch order.  One wave
+// can run the batches one after the other (combine_block: the split workgroups' own merge, and the merge launch for up
+// to 16 splits) or a wave each with one wave folding them (the merge launch beyond 16 splits): the same arithmetic in
+// the same order either way, so the two give the same bits.
 // DEV: the partials were written by other workgroups of this launch (device-scope loads).
 constexpr int kCombineBatch = 16;
-template <bool DEV, typename E>
-__device__ inline void combine_block(const AttnParams& p, int g, int rb, int quad, int lane) {
+struct CombineSum {
+    float M, L;
+    f32x4 acc;
+};
+template <typename E>
+struct CombineWhere {
+    const float2* ml;
+    const typename Elem<E>::x4* op;
+    size_t ml_stride, o_stride;
+    int node, head, d0;
+    bool valid;
+};
+template <typename E>
+__device__ inline CombineWhere<E> combine_where(const AttnParams& p, int g, int rb, int quad, int lane) {
     typedef typename Elem<E>::x4 X4;
+    CombineWhere<E> w;
     const int nrb = p.rows_pad / kRowsPerWave;  // 32-row blocks per kv head
     const int qcol = lane & 31, hf = lane >> 5;
     const int R = rb * kRowsPerWave + qcol;
-    if (R >= p.group * p.T) return;
-    const int node = p.group_shift >= 0 ? R >> p.group_shift : R / p.group;
-    const int head = g * p.group + (p.group_shift >= 0 ? R & (p.group - 1) : R % p.group);
-    const int d0 = (quad >> 2) * 32 + (quad & 3) * 8 + hf * 4;
-    const float2* ml = reinterpret_cast<const float2*>(p.ml_part) + (size_t)g * p.num_splits * p.rows_pad + R;
-    const X4* op = reinterpret_cast<const X4*>(p.o_part) +
-                      (((size_t)g * p.num_splits) * nrb + rb) * 16 * 64 + quad * 64 + lane;
-    const size_t ml_stride = (size_t)p.rows_pad;
-    const size_t o_stride = (size_t)nrb * 16 * 64;
-
-    float M = -INFINITY, L = 0.f;
-    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-    for (int s0 = 0; s0 < p.num_splits; s0 += kCombineBatch) {
-        float2 v[kCombineBatch];
-        X4 o[kCombineBatch];
+    w.valid = R < p.group * p.T;
+    w.node = p.group_shift >= 0 ? R >> p.group_shift : R / p.group;
+    w.head = g * p.group + (p.group_shift >= 0 ? R & (p.group - 1) : R % p.group);
+    w.d0 = (quad >> 2) * 32 + (quad & 3) * 8 + hf * 4;
+    w.ml = reinterpret_cast<const float2*>(p.ml_part) + (size_t)g * p.num_splits * p.rows_pad + R;
+    w.op = reinterpret_cast<const X4*>(p.o_part) + (((size_t)g * p.num_splits) * nrb + rb) * 16 * 64 + quad * 64 + lane;
+    w.ml_stride = (size_t)p.rows_pad;
+    w.o_stride = (size_t)nrb * 16 * 64;
+    return w;
+}
+// the sum over splits [s0, s0 + 16) relative to their own maximum; M = -inf, L = 0 when all of them are empty
+template <bool DEV, typename E>
+__device__ inline CombineSum combine_batch(const CombineWhere<E>& w, int s0, int num_splits) {
+    typedef typename Elem<E>::x4 X4;
+    float2 v[kCombineBatch];
+    X4 o[kCombineBatch];
 #pragma unroll
-        for (int u = 0; u < kCombineBatch; ++u) {
-            const int s = min(s0 + u, p.num_splits - 1);  // clamp: repeats are ignored below
-            if (DEV) {
-                const uint64_t mlw = load_dev64(&ml[s * ml_stride]);
-                v[u] = make_float2(__uint_as_float((uint32_t)mlw), __uint_as_float((uint32_t)(mlw >> 32)));
-                o[u] = bits_as<X4>(load_dev64(&op[s * o_stride]));
-            } else {
-                v[u] = ml[s * ml_stride];
-                o[u] = op[s * o_stride];
-            }
-        }
-        float Mb = M;
-#pragma unroll
-        for (int u = 0; u < kCombineBatch; ++u)
-            if (s0 + u < p.num_splits && v[u].y > 0.f) Mb = fmaxf(Mb, v[u].x);
-        if (Mb == -INFINITY) continue;  // nothing but empty splits so far
-        const float resc = __builtin_amdgcn_exp2f(M - Mb);  // 0 when M was -inf
-        L *= resc;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) acc[e] *= resc;
-        M = Mb;
-#pragma unroll
-        for (int u = 0; u < kCombineBatch; ++u) {
-            // an empty split (l == 0) has no meaningful O partial: select it away, never scale it
-            if (!(s0 + u < p.num_splits && v[u].y > 0.f)) continue;
-            const float w = __builtin_amdgcn_exp2f(v[u].x - M) * v[u].y;  // partials are stored normalised
-            L += w;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) acc[e] += w * (float)o[u][e];
+    for (int u = 0; u < kCombineBatch; ++u) {
+        const int s = min(s0 + u, num_splits - 1);  // clamp: repeats are ignored below
+        if (DEV) {
+            const uint64_t mlw = load_dev64(&w.ml[s * w.ml_stride]);
+            v[u] = make_float2(__uint_as_float((uint32_t)mlw), __uint_as_float((uint32_t)(mlw >> 32)));
+            o[u] = bits_as<X4>(load_dev64(&w.op[s * w.o_stride]));
+        } else {
+            v[u] = w.ml[s * w.ml_stride];
+            o[u] = w.op[s * w.o_stride];
         }
     }
-    const float inv = (L == 0.f || L != L) ? 1.f : 1.f / L;
+    CombineSum r;
+    r.M = -INFINITY;
+    r.L = 0.f;
+    r.acc = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int u = 0; u < kCombineBatch; ++u)
+        if (s0 + u < num_splits && v[u].y > 0.f) r.M = fmaxf(r.M, v[u].x);
+    if (r.M == -INFINITY) return r;
+#pragma unroll
+    for (int u = 0; u < kCombineBatch; ++u) {
+        // an empty split (l == 0) has no meaningful O partial: select it away, never scale it
+        if (!(s0 + u < num_splits && v[u].y > 0.f)) continue;
+        const float wt = __builtin_amdgcn_exp2f(v[u].x - r.M) * v[u].y;  // partials are stored normalised
+        r.L += wt;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) r.acc[e] += wt * (float)o[u][e];
+    }
+    return r;
+}
+// folds a batch sum into the running result (the first batch into an empty one exactly: scale 0 and scale 1); the
+// multiply-adds are spelled out so that every kernel that inlines this rounds alike
+__device__ inline void combine_fold(CombineSum& t, const CombineSum& b) {
+    if (b.M == -INFINITY) return;
+    const float Mn = fmaxf(t.M, b.M);
+    const float ra = __builtin_amdgcn_exp2f(t.M - Mn);  // 0 while the running result is empty
+    const float rb = __builtin_amdgcn_exp2f(b.M - Mn);
+    t.L = __builtin_fmaf(t.L, ra, b.L * rb);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) t.acc[e] = __builtin_fmaf(t.acc[e], ra, b.acc[e] * rb);
+    t.M = Mn;
+}
+template <typename E>
+__device__ inline void combine_store(const AttnParams& p, const CombineWhere<E>& w, const CombineSum& t) {
+    typedef typename Elem<E>::x4 X4;
+    const float inv = (t.L == 0.f || t.L != t.L) ? 1.f : 1.f / t.L;
     X4 o;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) o[e] = (E)(acc[e] * inv);
-    *reinterpret_cast<X4*>(p.out + ((size_t)node * p.Hq + head) * kHeadDim + d0) = o;
+    for (int e = 0; e < 4; ++e) o[e] = (E)(t.acc[e] * inv);
+    *reinterpret_cast<X4*>(p.out + ((size_t)w.node * p.Hq + w.head) * kHeadDim + w.d0) = o;
+}
+template <bool DEV, typename E>
+__device__ inline void combine_block(const AttnParams& p, int g, int rb, int quad, int lane) {
+    const CombineWhere<E> w = combine_where<E>(p, g, rb, quad, lane);
+    if (!w.valid) return;
+    CombineSum t;
+    t.M = -INFINITY;
+    t.L = 0.f;
+    t.acc = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < p.num_splits; s0 += kCombineBatch) combine_fold(t, combine_batch<DEV, E>(w, s0, p.num_splits));
+    combine_store<E>(p, w, t);
 }
 
 // One rotary pair: (a, b) -> (a cos - b sin, a sin + b cos), every product and sum rounded on its own
@@ -959,6 +1002,31 @@ __device__ __forceinline__ void tree_attn_split_body(const AttnParams& p) {
                 p.ml_part[prow * 2 + 1] = l_tot;
             }
         }
+#ifdef CPMCU_TIMELINE
+        // the records of this workgroup (the stamps sit in registers until here; see timeline.h); records 4..7 stay zero
+        // when the merge is a launch of its own
+        const auto tl_record = [&]() {
+            const int wg = blockIdx.y * gridDim.x + blockIdx.x;
+            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 0, tl_start);
+            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 1, tl_loop);
+            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 2, tl_loop_end);
+            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 3, tl_groups);
+            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 4, tl_stored);
+            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 5, tl_acked);
+            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 6, tl_go);
+            if (unit_ctr != nullptr) CPMCU_STAMP(g_attn_timeline, wg, 7);
+            else CPMCU_STAMP(g_attn_timeline, wg, 4);  // partials issued; the launch ends with them
+            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 8, niter);
+            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 9, n);
+            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 10, split);
+            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 11, mt);
+            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 12, tl_it1);
+            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 13, tl_it2);
+            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 14, tl_fix0);
+            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 15, tl_fix1);
+        };
+        if (unit_ctr == nullptr) tl_record();
+#endif
         if (unit_ctr == nullptr) return;
         // ---- merge inside the launch ----
         // Every workgroup of the unit (same KV head and M-tile, one per split) announces its partials once they
@@ -1033,25 +1101,7 @@ __device__ __forceinline__ void tree_attn_split_body(const AttnParams& p) {
             for (uint32_t m = s_merge_abandoned; m != 0; m &= m - 1) merge_share(__builtin_ctz(m));
         }
 #ifdef CPMCU_TIMELINE
-        {
-            const int wg = blockIdx.y * gridDim.x + blockIdx.x;
-            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 0, tl_start);
-            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 1, tl_loop);
-            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 2, tl_loop_end);
-            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 3, tl_groups);
-            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 4, tl_stored);
-            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 5, tl_acked);
-            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 6, tl_go);
-            CPMCU_STAMP(g_attn_timeline, wg, 7);
-            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 8, niter);
-            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 9, n);
-            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 10, split);
-            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 11, mt);
-            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 12, tl_it1);
-            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 13, tl_it2);
-            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 14, tl_fix0);
-            CPMCU_STAMP_VALUE(g_attn_timeline, wg, 15, tl_fix1);
-        }
+        tl_record();
 #endif
     }
 }
@@ -1079,6 +1129,50 @@ __device__ __forceinline__ void tree_attn_combine_body(const AttnParams& p) {
 __global__ __launch_bounds__(256) void tree_attn_combine_kernel(AttnParams p) { tree_attn_combine_body<f16>(p); }
 __global__ __launch_bounds__(256) void tree_attn_combine_bf16_kernel(AttnParams p) { tree_attn_combine_body<bf16>(p); }
 
+// The same beyond 16 splits: one workgroup per (kv head, 32-row block, quad) with a wave per batch of 16 splits -- all
+// batches in one memory round trip instead of one after the other (128 splits: eight) -- and wave 0 folding the batch
+// sums in batch order.
+constexpr int kCombineWideWaves = kMaxSplits / kCombineBatch;
+template <typename E>
+__device__ __forceinline__ void tree_attn_combine_wide_body(const AttnParams& p) {
+    __shared__ float s_sum[kCombineWideWaves][6][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int quad = blockIdx.x & 15;
+    const int nrb = p.rows_pad / kRowsPerWave;
+    const int grb = blockIdx.x >> 4;
+    const CombineWhere<E> w = combine_where<E>(p, grb / nrb, grb % nrb, quad, lane);
+    const int nb = (p.num_splits + kCombineBatch - 1) / kCombineBatch;
+    CombineSum mine;
+    mine.M = -INFINITY;
+    mine.L = 0.f;
+    mine.acc = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (w.valid && wave < nb) mine = combine_batch<false, E>(w, wave * kCombineBatch, p.num_splits);
+    if (wave != 0) {
+        s_sum[wave][0][lane] = mine.M;
+        s_sum[wave][1][lane] = mine.L;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) s_sum[wave][2 + e][lane] = mine.acc[e];
+    }
+    __syncthreads();
+    if (wave != 0 || !w.valid) return;
+    CombineSum t;
+    t.M = -INFINITY;
+    t.L = 0.f;
+    t.acc = f32x4{0.f, 0.f, 0.f, 0.f};
+    combine_fold(t, mine);
+    for (int b = 1; b < nb; ++b) {
+        CombineSum o;
+        o.M = s_sum[b][0][lane];
+        o.L = s_sum[b][1][lane];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) o.acc[e] = s_sum[b][2 + e][lane];
+        combine_fold(t, o);
+    }
+    combine_store<E>(p, w, t);
+}
+__global__ __launch_bounds__(64 * kCombineWideWaves) void tree_attn_combine_wide_kernel(AttnParams p) { tree_attn_combine_wide_body<f16>(p); }
+__global__ __launch_bounds__(64 * kCombineWideWaves) void tree_attn_combine_wide_bf16_kernel(AttnParams p) { tree_attn_combine_wide_body<bf16>(p); }
+
 int device_cu_count() {
     static int cus[64] = {0};
     int dev = 0;
@@ -1094,46 +1188,66 @@ int device_cu_count() {
 int choose_splits(int T, int group, int Hkv, int max_kv_len, int G) {
     const int num_mtiles = ceil_div(group * T, rows_per_wg(G));
     const int ntiles = ceil_div(max_kv_len, kTileN);
-    // One workgroup per CU.
+    // One workgroup per CU.  The grid is (splits x KV heads, padded to a multiple of the XCD count) x M-tiles, and the padding
+    // counts: 42 splits of 2 heads on 3 M-tiles are 88 x 3 = 264 workgroups -- too many for the launch to merge itself.
     const int cus = device_cu_count() > 0 ? device_cu_count() : 256;
-    int splits = cus / (num_mtiles * Hkv);
+    int splits = (cus / num_mtiles / kXcds * kXcds) / Hkv;
     if (splits < 1) splits = 1;
     const bool merge = options().attn_merge_in_launch != 0;
-    // One or two row units (plain decode, trees of up to 32 nodes) could take 64 or 128 splits; up to about 28K context
-    // they do better on at most 32, which the launch can merge itself: 16 while a split still gets about four tiles,
-    // 32 beyond.  One query, us per call, 16 / 32 splits merged in the launch against the split count below with its
-    // second launch: 13.3 / 13.8 vs 17.5 at 4K, 17.3 / 15.1 vs 20.9 at 8K, 24.9 / 18.9 vs 21.8 at 16K, 32.8 / 22.8 vs 24.0
-    // at 24K, - / 27.2 vs 25.9 at 32K.
-    constexpr int kShortContextTiles = 448;
+    // Between 33 and 63 splits (three M-tiles) a second launch would merge what 32 splits merge in the launch.  24-node tree,
+    // us per layer, 42 splits + combine launch against 32 splits: 43.5 / 26.8 at 32K, 55.4 / 34.5 at 48K, 67.5 / 41.9 at
+    // 64K, 119 / 79.5 at 128K.
+    if (merge && splits > kMergeMaxSplits && splits < 2 * kMergeMaxSplits) splits = kMergeMaxSplits;
+    // One or two M-tiles (plain decode, trees of up to 16 nodes) could take 64 or 128 splits; up to about 10K context they
+    // do better on at most 32, which the launch can merge itself: 16 while a split still gets about four tiles, 32 beyond.
+    // One query, us per layer, 32 splits merged in the launch against 64 with the merge launch (a wave per batch of 16
+    // splits): 12.5 / 14.2 at 4K, 14.3 / 14.4 at 8K, 16.2 / 13.9 at 12K, 18.0 / 15.1 at 16K, 21.6 / 17.1 at 24K; 16 nodes:
+    // 15.3 / 15.9 at 8K, 17.1 / 17.4 at 12K, 19.0 / 17.7 at 16K.
+    constexpr int kShortContextTiles = 160;
     if (merge && splits > kMergeMaxSplits && ntiles <= kShortContextTiles) splits = std::min(kMergeMaxSplits, std::max(16, ntiles / 4));
     // Every split gets at least one tile -- one per KV group when a second launch merges: a launch that merges itself does
     // better on more, shorter splits at short contexts (60-node tree at 512 tokens: 12.7 us on 10 splits, 16.2 on 4).
     const int tile_cap = merge && splits <= kMergeMaxSplits ? ntiles : ntiles / G;
     if (splits > tile_cap) splits = tile_cap > 0 ? tile_cap : 1;
-    // More than 64 splits (one or two row units: plain decode, trees of up to 8 nodes) pay for their partials
-    // and per-workgroup latencies only when every KV group still gets a run of 8 tiles: with one query,
-    // 128 against 64 splits take 50.7 vs 55.0 us per layer at 128K context, but 38.1 vs 34.8 at 64K and
-    // 30.7 vs 22.6 at 16K.
-    if (splits > 64) splits = std::max(64, std::min(splits, ntiles / (G * 8)));
+    // More than 64 splits (one M-tile: plain decode, trees of up to 8 nodes) pay for their partials and per-workgroup
+    // latencies once every KV group still gets a run of about 3 tiles: one query, 128 against 64 splits, us per layer:
+    // 18.6 / 19.0 at 32K, 21.3 / 23.2 at 48K, 23.6 / 27.1 at 64K, 36.4 / 47.5 at 128K (15.8 / 15.1 at 16K).
+    if (splits > 64) splits = std::max(64, std::min(splits, ntiles / (G * 3)));
     if (splits > kMaxSplits) splits = kMaxSplits;
     return splits;
 }
 
-// KV groups per workgroup.  The 256-row shape pays off once every workgroup of a full-GPU launch has
-// a long enough run of tiles to amortise its larger split count (twice the partials to merge), and
-// only if its (KV head, M-tile) units times the split limit can fill the GPU at all: it is taken
-// when there are at least 4 such units and at least 16 tiles per workgroup.  Measured, us per layer,
-// 256-row shape vs two-group shape:  60-node tree (8 units): 32.8 / 31.1 at 16K, 50 / 50 at 32K,
-// 67.7 / 71.2 at 48K, 156 / 170 at 128K;  128-node tree (16 units): 30.3 / 29.5 at 4K, 56.1 / 59.3 at
-// 16K, 301 / 326 at 128K;  16 nodes or one (2 units): 74.8 / 62.4 and 73.2 / 55.0 at 128K.
+// KV groups per workgroup.  Per workgroup the 256-row shape runs ntiles / s1 tiles and the two-group shape
+// ntiles / (2 s2) iterations of two tiles each, about 1.1-1.2 times as long at long contexts (every tile is fetched
+// by twice as many M-tiles), where s1 and s2 are the split counts that fill the CUs with either shape:
+//   * s1 beyond what a launch merges itself (one or two 256-row M-tiles, trees of up to 32 nodes; three, up to 48
+//     nodes, where the two-group shape has 1.25-1.5 times the splits per tile): two groups.  us per layer, 256-row
+//     shape / two groups: 24 nodes 34.6 / 26.9 at 32K, 49.0 / 42.3 at 64K, 82 / 81 at 128K; 40 nodes 40.3 / 33.3 at
+//     32K, 67.6 / 56.6 at 64K, 124.5 / 105.7 at 128K; 48 nodes 68.2 / 64.6 at 64K, 127.7 / 122.3 at 128K; 16 nodes or
+//     one 74.8 / 62.4 and 73.2 / 55.0 at 128K;
+//   * 2 s2 well below s1 (81 to 96 nodes: 8 splits against 20): the 256-row shape from 8K on (96 nodes: 28.7 / 30.8
+//     at 8K, 40.0 / 45.9 at 16K, 64.6 / 78.2 at 32K; 21.3 / 19.0 at 2K);
+//   * 2 s2 = s1 otherwise: the 256-row shape once every workgroup has a run of at least 16 tiles to amortise its larger
+//     split count (twice the partials to merge).  60-node tree (8 units): 30.2 / 27.8 at 16K, 44 / 43 at 32K,
+//     75.2 / 77.6 at 64K, 146-152 / 158 at 128K; 128-node tree (16 units): 26.5 / 24.7 at 4K, 49.1 / 49.5 at 16K,
+//     82 / 86.5 at 32K, 282 / 300 at 128K; 72 nodes 33.7 / 33.7 at 16K, 53.4 / 55.1 at 32K.
 // The option attn_kv_groups (cpmcu_set_option; CPMCU_ATTN_KV_GROUPS=1|2 in the environment at load) overrides the
 // choice: tests exercise both shapes.
 constexpr int kLongRunTiles = 16;
+int splits_that_fill(int T, int group, int Hkv, int G) {
+    const int cus = device_cu_count() > 0 ? device_cu_count() : 256;
+    const int s = (cus / ceil_div(group * T, rows_per_wg(G)) / kXcds * kXcds) / Hkv;
+    return s < 1 ? 1 : s;
+}
 int choose_groups(int T, int group, int Hkv, int max_kv_len) {
     if (options().attn_kv_groups != 0) return options().attn_kv_groups;
     const int units = ceil_div(group * T, rows_per_wg(1)) * Hkv;
     const int ntiles = ceil_div(max_kv_len, kTileN);
-    return units >= 4 && (long long)ntiles * units >= (long long)kLongRunTiles * 256 ? 1 : 2;
+    const int s1 = splits_that_fill(T, group, Hkv, 1), s2 = splits_that_fill(T, group, Hkv, 2);
+    if (units < 4 || s1 > kMergeMaxSplits) return 2;
+    if (40 * s2 >= 23 * s1) return 2;                       // 2 s2 / s1 >= 1.15
+    if (40 * s2 <= 17 * s1) return ntiles >= 128 ? 1 : 2;   // 2 s2 / s1 <= 0.85
+    return (long long)ntiles * units >= (long long)kLongRunTiles * 256 ? 1 : 2;
 }
 
 // Shape of one attention launch: which kernel shape, how many KV splits and M-tiles.
@@ -1231,7 +1345,7 @@ extern "C" int cpmcu_tree_attention_plan(int T, int Hq, int Hkv, int max_kv_len,
     const LaunchPlan pl = plan_launch(T, Hq / Hkv, Hkv, max_kv_len, block_window_size, num_splits_override);
     if (kernel_names && kernel_names_bytes > 0)
         snprintf(kernel_names, kernel_names_bytes, "tree_attn_split_kernel<%d,%s>%s", pl.kv_groups, with_rope ? "true" : "false",
-                 pl.num_splits > 1 && !pl.merge_in_launch ? "+tree_attn_combine_kernel" : "");
+                 pl.num_splits <= 1 || pl.merge_in_launch ? "" : pl.num_splits > kCombineBatch ? "+tree_attn_combine_wide_kernel" : "+tree_attn_combine_kernel");
     if (num_splits) *num_splits = pl.num_splits;
     if (kv_groups) *kv_groups = pl.kv_groups;
     if (num_workgroups) *num_workgroups = kXcds * ceil_div(pl.num_splits * Hkv, kXcds) * pl.num_mtiles;
@@ -1429,9 +1543,16 @@ static int tree_attention_impl(const void* q, void* k_pool, void* v_pool,
     }
     CPMCU_LAUNCH_CHECK();
     if (p.num_splits > 1 && p.merge_ctr == nullptr) {
-        const int threads_total = Hkv * (p.rows_pad / kRowsPerWave) * 16 * 64;
-        if (is_bf16) hipLaunchKernelGGL(tree_attn_combine_bf16_kernel, dim3(ceil_div(threads_total, 256)), dim3(256), 0, st, p);
-        else hipLaunchKernelGGL(tree_attn_combine_kernel, dim3(ceil_div(threads_total, 256)), dim3(256), 0, st, p);
+        const int waves_total = Hkv * (p.rows_pad / kRowsPerWave) * 16;  // one per (kv head, 32-row block, quad)
+        if (p.num_splits > kCombineBatch) {
+            const dim3 block(64 * ceil_div(p.num_splits, kCombineBatch));
+            if (is_bf16) hipLaunchKernelGGL(tree_attn_combine_wide_bf16_kernel, dim3(waves_total), block, 0, st, p);
+            else hipLaunchKernelGGL(tree_attn_combine_wide_kernel, dim3(waves_total), block, 0, st, p);
+        } else if (is_bf16) {
+            hipLaunchKernelGGL(tree_attn_combine_bf16_kernel, dim3(ceil_div(waves_total * 64, 256)), dim3(256), 0, st, p);
+        } else {
+            hipLaunchKernelGGL(tree_attn_combine_kernel, dim3(ceil_div(waves_total * 64, 256)), dim3(256), 0, st, p);
+        }
         CPMCU_LAUNCH_CHECK();
     }
     return CPMCU_OK;

@@ -1,6 +1,6 @@
 """Where the time of a launch goes, from wall-clock stamps taken inside the kernels.
 
-    python -m cpm.cu_amd.timeline attention [P ...]     tree attention, 60-node tree, prefix lengths P (default 4096)
+    python -m cpm.cu_amd.timeline attention [P ...] [--rows T]   tree attention, T-node tree (default 60), prefix lengths P (default 4096)
     python -m cpm.cu_amd.timeline head [n ...]          target head 73448 x 4096, n hidden rows (default 60 16)
     python -m cpm.cu_amd.timeline frspec                FR-Spec head 32768 x 4096, 10 rows: two launches and one launch
 
@@ -41,12 +41,13 @@ def _spread(name, x):
     return "  %-34s min %6.2f  median %6.2f  p90 %6.2f  max %6.2f" % (name, x.min(), np.median(x), np.percentile(x, 90), x.max())
 
 
-def attention(L, torch, prefixes):
+def attention(L, torch, prefixes, T=60):
     from . import ops, synth
     from .kvcache import PagedKVCache
-    T, Hq, Hkv, D, NL = 60, 32, 2, 128, 8
-    tree = synth.eagle_tree(6, 10, T, 0)
-    mask = torch.from_numpy(tree.mask.view(np.int64)).cuda()
+    Hq, Hkv, D, NL = 32, 2, 128, 8
+    mask = None  # one row, or a chain beyond 64 rows
+    if 1 < T <= 64:
+        mask = torch.from_numpy(synth.eagle_tree(6, 10, T, 0).mask.view(np.int64)).cuda()
     for P in prefixes:
         S = P + T
         cache = PagedKVCache(NL, Hkv, (S + 255) // 256 + 1)
@@ -74,11 +75,17 @@ def attention(L, torch, prefixes):
         print("tree attention, %d-token prefix + %d-node tree: %s, %d splits, %d workgroups recorded" % (P, T, kernels, splits, len(d)))
         for i, name in enumerate(["start", "K loop entered", "K loop left", "KV groups merged", "partials issued", "partials acknowledged",
                                   "all splits of the unit arrived", "end (own share merged, output stored)"]):
+            if i >= 5 and not d[:, i].any():
+                continue  # the merge is a launch of its own: the split launch ends with its partials
             print(_spread(name, rel[:, i]))
         tiles = d[:, 9]
+        merged = d[:, 7].any()
         for nt in np.unique(tiles):
             r = rel[tiles == nt]
-            print("  workgroups with %d tiles (%d): loop left %.2f, arrived %.2f, end %.2f (medians)" % (nt, len(r), np.median(r[:, 2]), np.median(r[:, 6]), np.median(r[:, 7])))
+            if merged:
+                print("  workgroups with %d tiles (%d): loop left %.2f, arrived %.2f, end %.2f (medians)" % (nt, len(r), np.median(r[:, 2]), np.median(r[:, 6]), np.median(r[:, 7])))
+            else:
+                print("  workgroups with %d tiles (%d): loop left %.2f, partials issued %.2f (medians)" % (nt, len(r), np.median(r[:, 2]), np.median(r[:, 4])))
         wg = np.nonzero(buf_mask)[0]
         print("  K loop left by XCD (workgroup number mod 8), medians: " + " ".join("%.1f" % np.median(rel[wg % 8 == x, 2]) for x in range(8)))
         last = d[d[:, 10] == d[:, 10].max()]  # the last split: the appended rows and the end of the stream
@@ -181,7 +188,12 @@ def main(argv):
     L = _load()
     torch.cuda.set_device(0)
     if argv[0] == "attention":
-        attention(L, torch, [int(x) for x in argv[1:]] or [4096])
+        rest, T = argv[1:], 60
+        if "--rows" in rest:
+            i = rest.index("--rows")
+            T = int(rest[i + 1])
+            rest = rest[:i] + rest[i + 2:]
+        attention(L, torch, [int(x) for x in rest] or [4096], T)
     elif argv[0] == "head":
         head(L, torch, [int(x) for x in argv[1:]] or [60, 16])
     else:

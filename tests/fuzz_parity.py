@@ -74,7 +74,7 @@ def main(argv):
         P = int(edges_p[g.integers(len(edges_p))]) if g.random() < 0.5 else int(g.integers(0, 5000))
         T = int(edges_t[g.integers(len(edges_t))]) if g.random() < 0.6 else int(g.integers(1, 129))
         mode = ["in_cache", "append", "append_rope"][int(g.integers(3))]
-        splits = [0, 0, 0, 1, 2, 3, 5, 7, 16][int(g.integers(9))]
+        splits = [0, 0, 0, 1, 2, 3, 5, 7, 16, 17, 24, 32, 33, 64, 100, 128][int(g.integers(16))]
         slack = [0, 0, 1, 63, 64, 200, 1000][int(g.integers(7))]
         lib.get().set_option(b"attn_kv_groups", int(g.integers(3)))  # 0 = the library's choice
         try:
