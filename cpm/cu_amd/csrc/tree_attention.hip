@@ -147,16 +147,76 @@ __device__ inline To bits_as(const From& v) {
     return __builtin_bit_cast(To, v);
 }
 
-// Merge of the split partials of one 32-row block and one quad of output dims (lane = accumulator lane):
+// Merge of the split partials of one 32-row block and one quad of output dims (one wave; lane = accumulator lane):
 // M = max_s m_s, L = sum_s l_s 2^(m_s - M), O = sum_s l_s 2^(m_s - M) (O_s / l_s) / L -- the log-sum-exp merge of
-// src/flash_attn/src/flash_fwd_kernel.h:2392-2472 in base-2 form -- in batches of up to 16 splits: the statistics and
-// the O partials of a batch are all requested before any is used (one memory round trip, not one per split) and summed
-// relative to the batch's own maximum; the batch sums are then folded into the running result in batch order.  One wave
-// can run the batches one after the other (combine_block: the split workgroups' own merge, and the merge launch for up
-// to 16 splits) or a wave each with one wave folding them (the merge launch beyond 16 splits): the same arithmetic in
-// the same order either way, so the two give the same bits.
+// src/flash_attn/src/flash_fwd_kernel.h:2392-2472 in base-2 form.  The statistics and the O partials of up to 16
+// splits are all requested before any is used, so a block pays one memory round trip, not one per split.
 // DEV: the partials were written by other workgroups of this launch (device-scope loads).
 constexpr int kCombineBatch = 16;
+template <bool DEV, typename E>
+__device__ inline void combine_block(const AttnParams& p, int g, int rb, int quad, int lane) {
+    typedef typename Elem<E>::x4 X4;
+    const int nrb = p.rows_pad / kRowsPerWave;  // 32-row blocks per kv head
+    const int qcol = lane & 31, hf = lane >> 5;
+    const int R = rb * kRowsPerWave + qcol;
+    if (R >= p.group * p.T) return;
+    const int node = p.group_shift >= 0 ? R >> p.group_shift : R / p.group;
+    const int head = g * p.group + (p.group_shift >= 0 ? R & (p.group - 1) : R % p.group);
+    const int d0 = (quad >> 2) * 32 + (quad & 3) * 8 + hf * 4;
+    const float2* ml = reinterpret_cast<const float2*>(p.ml_part) + (size_t)g * p.num_splits * p.rows_pad + R;
+    const X4* op = reinterpret_cast<const X4*>(p.o_part) +
+                      (((size_t)g * p.num_splits) * nrb + rb) * 16 * 64 + quad * 64 + lane;
+    const size_t ml_stride = (size_t)p.rows_pad;
+    const size_t o_stride = (size_t)nrb * 16 * 64;
+
+    float M = -INFINITY, L = 0.f;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < p.num_splits; s0 += kCombineBatch) {
+        float2 v[kCombineBatch];
+        X4 o[kCombineBatch];
+#pragma unroll
+        for (int u = 0; u < kCombineBatch; ++u) {
+            const int s = min(s0 + u, p.num_splits - 1);  // clamp: repeats are ignored below
+            if (DEV) {
+                const uint64_t mlw = load_dev64(&ml[s * ml_stride]);
+                v[u] = make_float2(__uint_as_float((uint32_t)mlw), __uint_as_float((uint32_t)(mlw >> 32)));
+                o[u] = bits_as<X4>(load_dev64(&op[s * o_stride]));
+            } else {
+                v[u] = ml[s * ml_stride];
+                o[u] = op[s * o_stride];
+            }
+        }
+        float Mb = M;
+#pragma unroll
+        for (int u = 0; u < kCombineBatch; ++u)
+            if (s0 + u < p.num_splits && v[u].y > 0.f) Mb = fmaxf(Mb, v[u].x);
+        if (Mb == -INFINITY) continue;  // nothing but empty splits so far
+        const float resc = __builtin_amdgcn_exp2f(M - Mb);  // 0 when M was -inf
+        L *= resc;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] *= resc;
+        M = Mb;
+#pragma unroll
+        for (int u = 0; u < kCombineBatch; ++u) {
+            // an empty split (l == 0) has no meaningful O partial: select it away, never scale it
+            if (!(s0 + u < p.num_splits && v[u].y > 0.f)) continue;
+            const float w = __builtin_amdgcn_exp2f(v[u].x - M) * v[u].y;  // partials are stored normalised
+            L += w;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) acc[e] += w * (float)o[u][e];
+        }
+    }
+    const float inv = (L == 0.f || L != L) ? 1.f : 1.f / L;
+    X4 o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) o[e] = (E)(acc[e] * inv);
+    *reinterpret_cast<X4*>(p.out + ((size_t)node * p.Hq + head) * kHeadDim + d0) = o;
+}
+
+// The same merge for more splits than a launch merges itself (more than kMergeMaxSplits: plain decode and small trees at long
+// contexts), where combine_block's one batch after the other would be up to eight memory round trips: every batch of 16 is
+// summed relative to its own maximum by a wave of its own, and one wave folds the batch sums in batch order.  (Another
+// order of additions than combine_block's running sum: the two agree to rounding, not to the bit -- no launch has both.)
 struct CombineSum {
     float M, L;
     f32x4 acc;
@@ -223,8 +283,7 @@ __device__ inline CombineSum combine_batch(const CombineWhere<E>& w, int s0, int
     }
     return r;
 }
-// folds a batch sum into the running result (the first batch into an empty one exactly: scale 0 and scale 1); the
-// multiply-adds are spelled out so that every kernel that inlines this rounds alike
+// folds a batch sum into the running result (the first batch into an empty one exactly: scale 0 and scale 1)
 __device__ inline void combine_fold(CombineSum& t, const CombineSum& b) {
     if (b.M == -INFINITY) return;
     const float Mn = fmaxf(t.M, b.M);
@@ -243,17 +302,6 @@ __device__ inline void combine_store(const AttnParams& p, const CombineWhere<E>&
 #pragma unroll
     for (int e = 0; e < 4; ++e) o[e] = (E)(t.acc[e] * inv);
     *reinterpret_cast<X4*>(p.out + ((size_t)w.node * p.Hq + w.head) * kHeadDim + w.d0) = o;
-}
-template <bool DEV, typename E>
-__device__ inline void combine_block(const AttnParams& p, int g, int rb, int quad, int lane) {
-    const CombineWhere<E> w = combine_where<E>(p, g, rb, quad, lane);
-    if (!w.valid) return;
-    CombineSum t;
-    t.M = -INFINITY;
-    t.L = 0.f;
-    t.acc = f32x4{0.f, 0.f, 0.f, 0.f};
-    for (int s0 = 0; s0 < p.num_splits; s0 += kCombineBatch) combine_fold(t, combine_batch<DEV, E>(w, s0, p.num_splits));
-    combine_store<E>(p, w, t);
 }
 
 // One rotary pair: (a, b) -> (a cos - b sin, a sin + b cos), every product and sum rounded on its own
@@ -1129,7 +1177,7 @@ __device__ __forceinline__ void tree_attn_combine_body(const AttnParams& p) {
 __global__ __launch_bounds__(256) void tree_attn_combine_kernel(AttnParams p) { tree_attn_combine_body<f16>(p); }
 __global__ __launch_bounds__(256) void tree_attn_combine_bf16_kernel(AttnParams p) { tree_attn_combine_body<bf16>(p); }
 
-// The same beyond 16 splits: one workgroup per (kv head, 32-row block, quad) with a wave per batch of 16 splits -- all
+// Beyond kMergeMaxSplits splits: one workgroup per (kv head, 32-row block, quad) with a wave per batch of 16 splits -- all
 // batches in one memory round trip instead of one after the other (128 splits: eight) -- and wave 0 folding the batch
 // sums in batch order.
 constexpr int kCombineWideWaves = kMaxSplits / kCombineBatch;
@@ -1345,7 +1393,7 @@ extern "C" int cpmcu_tree_attention_plan(int T, int Hq, int Hkv, int max_kv_len,
     const LaunchPlan pl = plan_launch(T, Hq / Hkv, Hkv, max_kv_len, block_window_size, num_splits_override);
     if (kernel_names && kernel_names_bytes > 0)
         snprintf(kernel_names, kernel_names_bytes, "tree_attn_split_kernel<%d,%s>%s", pl.kv_groups, with_rope ? "true" : "false",
-                 pl.num_splits <= 1 || pl.merge_in_launch ? "" : pl.num_splits > kCombineBatch ? "+tree_attn_combine_wide_kernel" : "+tree_attn_combine_kernel");
+                 pl.num_splits <= 1 || pl.merge_in_launch ? "" : pl.num_splits > kMergeMaxSplits ? "+tree_attn_combine_wide_kernel" : "+tree_attn_combine_kernel");
     if (num_splits) *num_splits = pl.num_splits;
     if (kv_groups) *kv_groups = pl.kv_groups;
     if (num_workgroups) *num_workgroups = kXcds * ceil_div(pl.num_splits * Hkv, kXcds) * pl.num_mtiles;
@@ -1544,7 +1592,7 @@ static int tree_attention_impl(const void* q, void* k_pool, void* v_pool,
     CPMCU_LAUNCH_CHECK();
     if (p.num_splits > 1 && p.merge_ctr == nullptr) {
         const int waves_total = Hkv * (p.rows_pad / kRowsPerWave) * 16;  // one per (kv head, 32-row block, quad)
-        if (p.num_splits > kCombineBatch) {
+        if (p.num_splits > kMergeMaxSplits) {
             const dim3 block(64 * ceil_div(p.num_splits, kCombineBatch));
             if (is_bf16) hipLaunchKernelGGL(tree_attn_combine_wide_bf16_kernel, dim3(waves_total), block, 0, st, p);
             else hipLaunchKernelGGL(tree_attn_combine_wide_kernel, dim3(waves_total), block, 0, st, p);

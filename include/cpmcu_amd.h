@@ -342,7 +342,7 @@ int cpmcu_tree_attention_release_workspace(const void* workspace);
 
 /* No reference counterpart: which kernels a cpmcu_tree_attention* call of this shape launches, without
  * launching -- for reports that must name the instantiation actually taken.  kernel_names receives e.g.
- * "tree_attn_split_kernel<2,false>+tree_attn_combine_kernel" (beyond 16 splits: "+tree_attn_combine_wide_kernel"); the
+ * "tree_attn_split_kernel<2,false>+tree_attn_combine_kernel" (beyond 32 splits: "+tree_attn_combine_wide_kernel"); the
  * outputs may each be NULL. */
 int cpmcu_tree_attention_plan(int T, int Hq, int Hkv, int max_kv_len, int with_rope, int block_window_size,
                               int num_splits_override, char* kernel_names, size_t kernel_names_bytes, int* num_splits,
