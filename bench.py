@@ -41,13 +41,13 @@ MFMA_F16_PEAK_TFLOPS = 2500.0
 MEASURED_TRAFFIC = {
     "source": "profiles/verify_step_hbm_traffic.md, profiles/tree_attention_long_context_traffic.md",
     # the library the counters were read on (git rev-parse --short HEAD of that run, all figures)
-    "measured_at_commit": "56e9314",
+    "measured_at_commit": "5ad0aba",
     "kib_per_launch": {
-        "tree_attn_split_kernel<2,false>": 15182 + 9463,  # the merge of the split partials runs inside the launch
+        "tree_attn_split_kernel<2,false>": 15185 + 9463,  # the merge of the split partials runs inside the launch
         "head_gemm_stream_kernel<4,2,256>": 591978 + 128,
     },
     # the attention launch at the longer contexts (32 splits of 256-row workgroups), by prefix length
-    "attention_kib_per_launch_by_context": {"32768": 52483 + 17894, "131072": 150803 + 17894},
+    "attention_kib_per_launch_by_context": {"32768": 52487 + 17894, "131072": 150806 + 17894},
 }
 
 
