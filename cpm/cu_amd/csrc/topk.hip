@@ -30,6 +30,7 @@ CPMCU_TIMELINE_STORAGE(g_topk_timeline)
 struct TopkParams {
     const uint16_t* x;  // [n][dim] fp16 bits
     int n, dim, top, nchunks;
+    int slice_len;      // row kernel: elements per workgroup when a row is cut into slices (0: the whole row)
     uint64_t* cand;     // [n][nchunks][top]
     uint16_t* val;      // [n][top]
     int32_t* pos;
@@ -185,8 +186,14 @@ __device__ __forceinline__ void topk_row_body(const TopkParams& p) {
     CPMCU_STAMP(g_topk_timeline, blockIdx.x, 0);
     const int row = blockIdx.x;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const int npieces = p.dim >> 3;
-    const uint4* xr = (const uint4*)(p.x + (size_t)row * p.dim);
+    // a row longer than kRowMaxDim is cut into slices, one workgroup each: this one ranks elements [slice_base, slice_base + len) and
+    // leaves its k best as keys for the merge launch instead of writing the outputs
+    const bool sliced = p.slice_len != 0;
+    const int slice_base = sliced ? blockIdx.y * p.slice_len : 0;
+    const int npieces = (sliced ? min(p.slice_len, p.dim - slice_base) : p.dim) >> 3;
+    const uint4* xr = (const uint4*)(p.x + (size_t)row * p.dim + slice_base);
+    uint64_t* slice_out = sliced ? p.cand + ((size_t)row * gridDim.y + blockIdx.y) * p.top : nullptr;
+    if (sliced && tid < p.top) slice_out[tid] = 0;  // slots this slice cannot fill stay empty (overwritten behind a barrier)
     // slots beyond the row read as 0xFFFF, whose raw image is 0: below every bound that is used
     uint4 raw[kRowPieces];
 #pragma unroll
@@ -268,7 +275,7 @@ __device__ __forceinline__ void topk_row_body(const TopkParams& p) {
             const float l = __logf(b);
             row_m_lse[0] = wm;
             row_m_lse[1] = l;
-            if (p.row_stats) {
+            if (p.row_stats && slice_base == 0) {
                 p.row_stats[row * 2 + 0] = wm;
                 p.row_stats[row * 2 + 1] = l;
             }
@@ -350,7 +357,7 @@ __device__ __forceinline__ void topk_row_body(const TopkParams& p) {
                 em &= em - 1;
                 const int e = 2 * (t & 15) + (t >> 4);  // element of the owner thread
                 const uint32_t o = ((const uint16_t*)&lanebuf[e >> 3][s])[e & 7];
-                if (slot < kRowCap) cand[slot] = key_from_image(o, ((e >> 3) * kRowThreads + owner) * 8 + (e & 7));
+                if (slot < kRowCap) cand[slot] = key_from_image(o, slice_base + ((e >> 3) * kRowThreads + owner) * 8 + (e & 7));
                 ++slot;
             }
         }
@@ -365,7 +372,7 @@ __device__ __forceinline__ void topk_row_body(const TopkParams& p) {
         const int part = tid >> shift, nparts = kRowThreads >> shift;
         // the mapped id of candidate tid is fetched now and used after the ranking
         int32_t mapped = 0;
-        if (tid < C && p.ids) mapped = p.remap ? p.remap[key_index(cand[tid])] : key_index(cand[tid]);
+        if (tid < C && p.ids && !sliced) mapped = p.remap ? p.remap[key_index(cand[tid])] : key_index(cand[tid]);
         if (i < C) {
             // slots from C on hold key 0, so whole groups of eight can be compared
             const uint64_t my = cand[i];
@@ -384,11 +391,15 @@ __device__ __forceinline__ void topk_row_body(const TopkParams& p) {
         CPMCU_STAMP(g_topk_timeline, blockIdx.x, 5);
         if (tid < C && rank[tid] < p.top) {
             const uint64_t key = cand[tid];
-            const int idx = key_index(key);
-            const size_t o = (size_t)row * p.top + rank[tid];
-            p.val[o] = LOGSOFTMAX ? key_bits(key) : p.x[(size_t)row * p.dim + idx];
-            p.pos[o] = idx;
-            if (p.ids) p.ids[o] = mapped;
+            if (sliced) {
+                slice_out[rank[tid]] = key;
+            } else {
+                const int idx = key_index(key);
+                const size_t o = (size_t)row * p.top + rank[tid];
+                p.val[o] = LOGSOFTMAX ? key_bits(key) : p.x[(size_t)row * p.dim + idx];
+                p.pos[o] = idx;
+                if (p.ids) p.ids[o] = mapped;
+            }
         }
         CPMCU_STAMP(g_topk_timeline, blockIdx.x, 6);
         return;
@@ -402,7 +413,7 @@ __device__ __forceinline__ void topk_row_body(const TopkParams& p) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const uint32_t o = (img[j * 4 + (e >> 1)] >> ((e & 1) * 16)) & 0xFFFFu;
-                const uint64_t key = pv ? key_from_image(o, (j * kRowThreads + tid) * 8 + e) : 0ull;
+                const uint64_t key = pv ? key_from_image(o, slice_base + (j * kRowThreads + tid) * 8 + e) : 0ull;
                 if (key < prev && key > mine) mine = key;
             }
         }
@@ -413,9 +424,32 @@ __device__ __forceinline__ void topk_row_body(const TopkParams& p) {
         uint64_t best = wb[0];
 #pragma unroll
         for (int w = 1; w < kRowWaves; ++w) best = wb[w] > best ? wb[w] : best;
-        if (tid == 0) emit_final<LOGSOFTMAX>(p, row, round, best);
+        if (tid == 0) {
+            if (sliced) slice_out[round] = best;
+            else emit_final<LOGSOFTMAX>(p, row, round, best);
+        }
         prev = best;
         if (best == 0) break;
+    }
+}
+
+// The slices' k best keys of a row (at most kSliceMergeCap of them, empty slots are 0) ranked by counting: one workgroup per
+// row, the count of larger keys is the output slot.
+constexpr int kSliceMergeCap = 1024;
+template <bool LOGSOFTMAX>
+__global__ __launch_bounds__(kTopkThreads) void topk_slice_merge_kernel(TopkParams p) {
+    __shared__ uint64_t keys[kSliceMergeCap];
+    const int row = blockIdx.x;
+    const int ncand = p.nchunks * p.top;
+    const uint64_t* in = p.cand + (size_t)row * ncand;
+    for (int i = threadIdx.x; i < ncand; i += kTopkThreads) keys[i] = in[i];
+    __syncthreads();
+    for (int i = threadIdx.x; i < ncand; i += kTopkThreads) {
+        const uint64_t my = keys[i];
+        if (my == 0) continue;
+        int r = 0;
+        for (int j = 0; j < ncand; ++j) r += keys[j] > my ? 1 : 0;
+        if (r < p.top) emit_final<LOGSOFTMAX>(p, row, r, my);
     }
 }
 
@@ -487,6 +521,7 @@ int launch_topk(const void* x, int n, int dim, int top, void* val, int32_t* pos,
     p.dim = dim;
     p.top = top;
     p.nchunks = ceil_div(dim, kChunk);
+    p.slice_len = 0;
     p.cand = (uint64_t*)workspace;
     p.val = (uint16_t*)val;
     p.pos = pos;
@@ -502,6 +537,22 @@ int launch_topk(const void* x, int n, int dim, int top, void* val, int32_t* pos,
         if (stats && options().dtype == 1) hipLaunchKernelGGL(topk_row_bf16_kernel, dim3(n), dim3(kRowThreads), 0, st, p);
         else if (stats) hipLaunchKernelGGL(topk_row_kernel<true>, dim3(n), dim3(kRowThreads), 0, st, p);
         else hipLaunchKernelGGL(topk_row_kernel<false>, dim3(n), dim3(kRowThreads), 0, st, p);
+        CPMCU_LAUNCH_CHECK();
+        return CPMCU_OK;
+    }
+    // longer rows in slices of at most kRowMaxDim elements: the row kernel on every slice, and a merge of the slices' k best
+    const int nslices = ceil_div(dim, kRowMaxDim);
+    if (dim % 8 == 0 && top <= kRowMaxTop && ((uintptr_t)x & 15) == 0 && nslices * top <= kSliceMergeCap && workspace &&
+        workspace_bytes >= (size_t)n * nslices * top * sizeof(uint64_t)) {
+        p.slice_len = (ceil_div(dim, nslices) + 7) / 8 * 8;
+        p.nchunks = nslices;
+        const dim3 grid(n, nslices);
+        if (stats && options().dtype == 1) hipLaunchKernelGGL(topk_row_bf16_kernel, grid, dim3(kRowThreads), 0, st, p);
+        else if (stats) hipLaunchKernelGGL(topk_row_kernel<true>, grid, dim3(kRowThreads), 0, st, p);
+        else hipLaunchKernelGGL(topk_row_kernel<false>, grid, dim3(kRowThreads), 0, st, p);
+        CPMCU_LAUNCH_CHECK();
+        if (stats) hipLaunchKernelGGL(topk_slice_merge_kernel<true>, dim3(n), dim3(kTopkThreads), 0, st, p);
+        else hipLaunchKernelGGL(topk_slice_merge_kernel<false>, dim3(n), dim3(kTopkThreads), 0, st, p);
         CPMCU_LAUNCH_CHECK();
         return CPMCU_OK;
     }

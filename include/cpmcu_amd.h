@@ -427,9 +427,8 @@ int cpmcu_frspec_head_topk(const void* hidden, const void* w, int w_layout, cons
  * or two full passes of 16-row blocks over the GPU -- the FR-Spec vocabulary of 32768 is one) and one of the library's 8
  * publication states per device is free for (workspace, grid size): every GEMM workgroup publishes its k..16 best
  * (value, index, token id) per hidden row as tagged 64-bit words, and the first n workgroups to finish rank one row
- * each.  Same outputs, bit for bit, as the two-launch form (cpmcu_set_option("frspec_fused", 0)) for V <= 32768; beyond
- * that the two forms add the row statistics up in different orders, ln(sum exp) may differ in its last bit, and each is
- * exact on its own statistics.  Logits are complete when the launch ends.  A state stays with its (workspace, grid) until cpmcu_head_release_workspace; calls that
+ * each.  Same outputs, bit for bit, as the two-launch form (cpmcu_set_option("frspec_fused", 0)); logits are complete
+ * when the launch ends.  A state stays with its (workspace, grid) until cpmcu_head_release_workspace; calls that
  * overlap on one GPU must use different workspaces, as before.  A finisher waits at most frspec_wait_us (option,
  * default 50000) for the other workgroups of its launch to become resident; if that runs out its row holds index -1,
  * the next synchronising call of the library returns CPMCU_ERR_RUNTIME, and the device goes back to two launches.

@@ -102,7 +102,7 @@ def main(argv):
     def topk(seed):
         g = synth.rng(seed, 94)
         n = int(g.integers(1, 6))
-        dim = int(g.integers(1, 40000))
+        dim = int(g.integers(1, 40000)) if g.random() < 0.7 else int(g.integers(4096, 17000)) * 8  # the latter: slices of the row kernel
         top = int(g.integers(1, min(dim, 128) + 1))
         kind = int(g.integers(4))
         if kind == 0:
