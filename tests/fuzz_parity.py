@@ -82,6 +82,12 @@ def main(argv):
         finally:
             lib.get().set_option(b"attn_kv_groups", 0)
 
+    def head_counts(seed):
+        g = synth.rng(seed, 102)
+        HKV = int([1, 1, 2, 3, 4, 8, 16, 32][g.integers(8)])
+        HQ = HKV * int([1, 1, 2, 3, 4, 5, 8, 16][g.integers(8)])
+        t_attention._heads_case(torch, orc, HQ, HKV, int(g.integers(0, 4000)), int(g.integers(1, 129)), ["in_cache", "append", "append_rope"][int(g.integers(3))], seed)
+
     def target_head(seed):
         g = synth.rng(seed, 92)
         n = int(g.integers(1, 129))
@@ -229,7 +235,7 @@ def main(argv):
         t_fused._assert_same(one, two, "V=%d n=%d k=%d std=%g" % (V, n, k, std))
         lib.get().synchronize()  # a wait that ran out would be an error here
 
-    stages = [("attention", "tree attention", attention), ("head", "target head", target_head), ("frspec", "FR-Spec head", frspec_head),
+    stages = [("attention", "tree attention", attention), ("heads", "tree attention with other query / KV head counts", head_counts), ("head", "target head", target_head), ("frspec", "FR-Spec head", frspec_head),
               ("topk", "top-k", topk), ("tail", "accept / compaction / tail", tail), ("draft", "draft tree", draft_tree),
               ("steps", "verify steps, eager and as graph replays", verify_steps), ("loop", "speculative loop against greedy decoding", speculative_loop),
               ("window", "drafter-layer attention: mask range, block window; window under a tree with rotary embedding", windows),

@@ -405,6 +405,51 @@ def test_randomised_shape_sweep(gpu, orc, P, T, mode, splits, slack, seed):
         assert np.array_equal(to_np(vc).view(np.uint16), v.view(np.uint16))
 
 
+def _heads_case(torch, orc, HQ_, HKV_, P, T, mode, seed):
+    """One attention call with HQ_ query heads on HKV_ KV heads (any ratio) against the oracle; appended rows bit for bit."""
+    from cpm.cu_amd import ops
+    from cpm.cu_amd.kvcache import PagedKVCache
+    tree = synth.random_tree(T, seed, max_children=5, max_depth=10)
+    S = P + T
+    npages = (S + 255) // 256 + 1
+    table = synth.rng(seed, 4).permutation(npages).astype(np.int32)
+    q = synth.normal_f16((T, HQ_, D), seed, 1)
+    k = synth.normal_f16((S, HKV_, D), seed, 2)
+    v = synth.normal_f16((S, HKV_, D), seed, 3)
+    cache = PagedKVCache(1, HKV_, npages, block_table=table, fill=float("nan"))
+    kv_len = torch.tensor([S], dtype=torch.int32, device="cuda")
+    mask = to_dev(torch, tree.mask)
+    q_ref, k_ref = q, k
+    if mode == "in_cache":
+        cache.write_logical(0, 0, to_dev(torch, k), to_dev(torch, v))
+        out = ops.tree_attention(to_dev(torch, q), cache, 0, kv_len, S, mask)
+    else:
+        if P:
+            cache.write_logical(0, 0, to_dev(torch, k[:P]), to_dev(torch, v[:P]))
+        rope = None
+        if mode == "append_rope":
+            inv_freq = (10000.0 ** (-np.arange(D // 2, dtype=np.float64) / (D // 2))).astype(np.float32)
+            rope = ops.rope_table(to_dev(torch, tree.positions(P)), to_dev(torch, inv_freq))
+            q_ref, k_rot = orc.rope(q, k[P:], table=to_np(rope))
+            k_ref = np.concatenate([k[:P], k_rot], 0)
+        out = ops.tree_attention(to_dev(torch, q), cache, 0, kv_len, S, mask, k_new=to_dev(torch, k[P:]), v_new=to_dev(torch, v[P:]), rope=rope)
+    torch.cuda.synchronize()
+    ref = orc.tree_attention(q_ref, k_ref, v, tree.mask, P)
+    assert_close_f16(to_np(out), ref, "Hq=%d Hkv=%d P=%d T=%d %s" % (HQ_, HKV_, P, T, mode))
+    if mode != "in_cache":
+        kc, vc = cache.read_logical(0, 0, S)
+        assert np.array_equal(to_np(kc).view(np.uint16), k_ref.view(np.uint16))
+        assert np.array_equal(to_np(vc).view(np.uint16), v.view(np.uint16))
+
+
+@pytest.mark.parametrize("HQ_,HKV_", [(32, 8), (32, 32), (8, 1), (40, 8), (48, 16), (6, 2), (1, 1)])
+@pytest.mark.parametrize("P,T,mode", [(1000, 16, "append"), (4096, 60, "append"), (300, 60, "in_cache"), (2049, 128, "append_rope"), (64, 1, "append")])
+def test_other_head_counts(gpu, orc, HQ_, HKV_, P, T, mode):
+    """Query / KV head counts other than the 32 / 2 of the configurations: 4, 1, 8, 5 (not a power of two), 3 and 1 query heads per
+    KV head, one KV head and thirty-two -- the packing of rows into waves, the split counts and the merge all depend on them."""
+    _heads_case(gpu, orc, HQ_, HKV_, P, T, mode, HQ_ * 1000 + P)
+
+
 @pytest.mark.parametrize("P,T,splits,fused_append,rope", [
     (4096, 60, 0, True, False),    # the verify step's shape: 16 splits (two groups) / 32 splits (one group), 256 workgroups
     (4096, 60, 0, True, True),
