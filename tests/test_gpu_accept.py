@@ -291,6 +291,20 @@ def test_verify_tail_finishes_the_head_partials(gpu, orc, T, num_iter, topk):
     _tail_case(gpu, orc, tree, 513, min(2, int(tree.depth.max())), layers=2, seed=T, H=512, V=40000, from_partials=True)
 
 
+@pytest.mark.parametrize("hkv", [1, 8, 32])
+def test_compaction_and_tail_with_other_kv_head_counts(gpu, orc, monkeypatch, hkv):
+    """Compaction, the one-launch tail and the commit on caches of 1, 8 and 32 KV heads (the configurations have 2)."""
+    import sys
+    monkeypatch.setattr(sys.modules[__name__], "HKV", hkv)
+    for seed in range(3):
+        g = synth.rng(seed, 5)
+        tree = synth.random_tree(int(g.integers(2, 65)), seed, max_children=4, max_depth=8)
+        depth = int(g.integers(0, int(tree.depth.max()) + 1))
+        _compact_case(gpu, orc, tree, int(g.integers(0, 900)), depth, layers=2, seed=seed)
+        _tail_case(gpu, orc, tree, int(g.integers(0, 900)), depth, layers=2, seed=seed, H=512, V=3000, from_partials=bool(seed & 1))
+        _commit_case(gpu, orc, tree, int(g.integers(0, 900)), depth, layers=2, seed=seed)
+
+
 def test_verify_tail_random_trees_duplicate_siblings(gpu, orc):
     """Tiny vocabulary: accidental matches and duplicate sibling tokens, so the tournament's tie rule decides."""
     from cpm.cu_amd import ops

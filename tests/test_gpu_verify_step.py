@@ -268,6 +268,16 @@ def test_library_graph_replays_equal_eager_steps(gpu, orc):
     _graph_replays_equal_eager_steps(gpu, orc, seed=3, T=24, P0=1000, STEPS=10)
 
 
+@pytest.mark.parametrize("hq,hkv", [(32, 8), (8, 1), (40, 8)])
+def test_model_level_steps_with_other_head_counts(gpu, orc, monkeypatch, hq, hkv):
+    """The same sequence of steps on models with 4, 8 and 5 query heads per KV head (the configurations all have 16)."""
+    import sys
+    me = sys.modules[__name__]
+    monkeypatch.setattr(me, "HQ", hq)
+    monkeypatch.setattr(me, "HKV", hkv)
+    _graph_replays_equal_eager_steps(gpu, orc, seed=hq, T=20 + hkv, P0=700, STEPS=6, LAYERS=2, num_iter=8, topk=8, min_paddings=1)
+
+
 def test_step_graph_cache_is_bounded(gpu, orc):
     """A caller whose buffers are not static makes cpmcu_verify_step capture a graph per set of addresses: the library keeps
     the 16 used most recently and frees the rest.  40 sets of addresses, revisited in a different order, give the results of
