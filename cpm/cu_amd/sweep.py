@@ -1,0 +1,141 @@
+"""Timings of the operators over ranges of shapes, with the kernels the library picks for each: looks for cliffs in the launch plans.
+
+    python -m cpm.cu_amd.sweep attention [--groups]   tree attention, prefix 256..131072 x tree rows 1..128 (us per layer);
+                                                      --groups: the automatic choice beside both kernel shapes forced
+    python -m cpm.cu_amd.sweep head                   target head (arg-max), rows 1..128 x vocabulary 8K..152K x hidden 2048/4096/8192
+    python -m cpm.cu_amd.sweep frspec                 FR-Spec head + log-softmax + top-k + id map-back, vocabulary 8K..73448 x rows x k
+
+Eager launches on cuda:0, random fp16 data, event-timed; attention rotates over several layers' K/V pools and the heads over
+copies of the weight matrix, so that no pass is served from the last-level cache.  Fractions are of 8 TB/s (heads) and TFLOP/s
+are 4 * Hq * T * D * S per layer (attention).
+"""
+import sys
+
+import numpy as np
+
+
+def _time(torch, fn, reps):
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / reps * 1e3
+
+
+def attention(torch, with_groups):
+    from . import lib, ops, synth
+    from .kvcache import PagedKVCache
+    Hq, Hkv, D = 32, 2, 128
+    L = lib.get()
+    prefixes = [256, 1024, 2048, 4096, 8192, 16384, 32768, 65536, 131072]
+    rows = [1, 8, 16, 24, 32, 40, 48, 60, 64, 96, 128]
+    print("tree attention, %d query / %d KV heads: us per layer (kernel shape <G>, KV splits, +c: merge launch)" % (Hq, Hkv))
+    print("%8s" % "P \\ T" + "".join("%22d" % t for t in rows))
+    for P in prefixes:
+        line = "%8d" % P
+        for T in rows:
+            mask = None
+            if 1 < T <= 64:
+                mask = torch.from_numpy(synth.eagle_tree(6, 10, T, 0).mask.view(np.int64)).cuda()
+            S = P + T
+            nl = 6 if P <= 32768 else 3
+            cache = PagedKVCache(nl, Hkv, (S + 255) // 256 + 1)
+            for l in range(nl):
+                cache.k[l].normal_()
+                cache.v[l].normal_()
+            q = torch.randn(T, Hq, D, device="cuda").half()
+            kn = torch.randn(T, Hkv, D, device="cuda").half()
+            vn = torch.randn(T, Hkv, D, device="cuda").half()
+            kv_len = torch.tensor([S], dtype=torch.int32, device="cuda")
+            out = torch.empty_like(q)
+            pad = (S + 127) // 128 * 128
+
+            def run():
+                for l in range(nl):
+                    ops.tree_attention(q, cache, l, kv_len, pad, mask, out=out, k_new=kn, v_new=vn)
+            cell = []
+            for G in ((0, 1, 2) if with_groups else (0,)):
+                L.set_option(b"attn_kv_groups", G)
+                for _ in range(3):
+                    run()
+                torch.cuda.synchronize()
+                us = _time(torch, run, 12 if P <= 32768 else 6) / nl
+                kernels, splits, groups, _ = ops.attention_plan(T, Hq, Hkv, pad)
+                cell.append("%.1f <%d> s%d%s" % (us, groups, splits, "+c" if "combine" in kernels else ""))
+            L.set_option(b"attn_kv_groups", 0)
+            line += "%22s" % cell[0] if not with_groups else "  [" + " | ".join(cell) + "]"
+            del cache
+        print(line, flush=True)
+
+
+def head(torch):
+    from . import ops
+    rows = [1, 16, 17, 32, 33, 60, 64, 100, 128]
+    for H in (2048, 4096, 8192):
+        print("target head, hidden size %d: fraction of 8 TB/s (kernel)" % H)
+        print("%8s" % "V \\ n" + "".join("%20d" % n for n in rows))
+        for V in (8192, 16384, 32768, 50000, 73448, 100000, 131072, 151936):
+            w = (torch.randn(V, H, device="cuda") * 0.02).half()
+            copies = [ops.tile_head_weight(w) for _ in range(2 if V * H * 2 < 1.5e9 else 1)]
+            del w
+            line = "%8d" % V
+            for n in rows:
+                hid = torch.randn(n, H, device="cuda").half()
+                name = ops.head_plan(n, copies[0])[0].replace("head_gemm_", "").replace("stream_kernel", "S").replace("chunked_kernel", "C")
+
+                def run():
+                    for c in copies:
+                        ops.lm_head_argmax(hid, c)
+                for _ in range(3):
+                    run()
+                torch.cuda.synchronize()
+                us = _time(torch, run, 10) / len(copies)
+                line += "%20s" % ("%.2f %s" % (V * H * 2 / us * 1e-3 / 8000, name))
+            print(line, flush=True)
+            del copies
+
+
+def frspec(torch):
+    from . import ops
+    H = 4096
+    print("FR-Spec head + log-softmax + top-k + id map-back, hidden size %d: us per call, fraction of 8 TB/s" % H)
+    for Vs in (8192, 16384, 32768, 40960, 49152, 65536, 73448):
+        w = (torch.randn(Vs, H, device="cuda") * 0.02).half()
+        copies = [ops.tile_head_weight(w) for _ in range(3)]
+        remap = torch.arange(Vs, dtype=torch.int32, device="cuda")
+        del w
+        for n, k in ((1, 10), (10, 1), (10, 10), (16, 16)):
+            hid = torch.randn(n, H, device="cuda").half()
+
+            def run():
+                for c in copies:
+                    ops.frspec_head_topk(hid, c, remap, k)
+            for _ in range(3):
+                run()
+            torch.cuda.synchronize()
+            us = _time(torch, run, 10) / 3
+            print("  V' = %6d  rows %2d  k %2d   %6.1f us  %.2f   %s" % (Vs, n, k, us, Vs * H * 2 / us * 1e-3 / 8000, ops.frspec_head_plan(n, copies[0], k)), flush=True)
+        del copies
+
+
+def main(argv):
+    if not argv or argv[0] not in ("attention", "head", "frspec"):
+        print(__doc__)
+        return 2
+    import torch
+    from . import lib
+    lib.get()  # raises if libcpmcu_amd.so is missing
+    torch.cuda.set_device(0)
+    if argv[0] == "attention":
+        attention(torch, "--groups" in argv[1:])
+    elif argv[0] == "head":
+        head(torch)
+    else:
+        frspec(torch)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main(sys.argv[1:]))
