@@ -345,6 +345,37 @@ def test_128k_context_closed_form_and_split_invariance(gpu):
         assert_close_f16(o, outs[0], "split invariance at 128K", atol=4e-3, rtol=4e-3)
 
 
+def test_one_million_token_context_closed_form(gpu):
+    """A million-token prefix (not a multiple of anything) on a permuted page table: with identical K rows every visible key
+    weighs the same, so a row's output is the mean of its visible V rows (fp64 running sums in numpy) -- nothing in the index
+    arithmetic (page offsets beyond 2^32 bytes, split ranges, the merge of 32 splits) may lose a key on the way."""
+    from cpm.cu_amd import ops
+    from cpm.cu_amd.kvcache import PagedKVCache
+    torch = gpu
+    P, T = 1000003, 60
+    S = P + T
+    tree = synth.eagle_tree(6, 10, T, seed=2)
+    npages = (S + 255) // 256 + 1
+    table = synth.rng(5, 4).permutation(npages).astype(np.int32)
+    q = synth.normal_f16((T, HQ, D), 70, 1)
+    v = synth.rng(70, 3).standard_normal((S, HKV, D), dtype=np.float32).astype(np.float16)
+    k_row = synth.normal_f16((1, HKV, D), 70, 2)
+    cache = PagedKVCache(1, HKV, npages, block_table=table, fill=float("nan"))
+    step = 1 << 18
+    for a in range(0, S, step):
+        b = min(S, a + step)
+        cache.write_logical(0, a, to_dev(torch, np.ascontiguousarray(np.broadcast_to(k_row, (b - a, HKV, D)))), to_dev(torch, v[a:b]))
+    kv_len = torch.tensor([S], dtype=torch.int32, device="cuda")
+    out = to_np(ops.tree_attention(to_dev(torch, q), cache, 0, kv_len, S, to_dev(torch, tree.mask))).astype(np.float64)
+    v64 = v.astype(np.float64)
+    prefix_sum = v64[:P].sum(0)
+    for i in range(T):
+        anc = [j for j in range(T) if (int(tree.mask[i, j >> 6]) >> (j & 63)) & 1]
+        mean = (prefix_sum + v64[P + np.array(anc)].sum(0)) / (P + len(anc))
+        for h in range(HQ):
+            assert np.abs(out[i, h] - mean[h // (HQ // HKV)]).max() < 2e-5, (i, h)  # outputs are O(3e-3) at this length
+
+
 def _sweep_configs():
     """Seeded random (P, T, mode, splits, slack) tuples, biased to tile (64), page (256) and wave-row (2, 16 nodes)
     boundaries; slack = how far the host-side bound on the KV length exceeds the true length."""
