@@ -497,6 +497,9 @@ _STREAM_SHAPES = [
     (7, 140000, 512, None),       # <1,4,256>, 2
     (40, 65536, 512, None),       # <4,2,256>, no last pass
     (24, 65536 + 16 * 2047, 1024, None),  # <2,2,256>, 1: all but one wave slot of the last pass filled
+    (128, 100000, 512, None),     # <8,1,128> on twice as many workgroups as CUs (three full passes would not fit the accumulators)
+    (100, 151936, 512, 0.3125),   # <8,2,128> likewise
+    (65, 220000, 512, None),      # <8,2,128> on three times as many
 ]
 
 
