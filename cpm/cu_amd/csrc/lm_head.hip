@@ -1442,12 +1442,14 @@ int plan_head_gemm(const void* hidden, const void* w, int w_layout, int n, int V
     const int nrb = ceil_div(V, 16);
     int G = num_cus();
     if (G * kHeadWaves > nrb) G = ceil_div(nrb, kHeadWaves);
-    // 65 to 128 hidden rows: the streaming kernel has accumulators for two full passes (three or four spill), so a vocabulary
-    // of more passes than that gets a multiple of the CU count in workgroups -- they run one after the other on a CU, each
-    // with at most two full passes, the stream does not stop between them -- instead of the K-chunked kernel (128 rows
-    // x 151936 x 4096: 0.75 against 0.53 of HBM peak).
-    if (NB == 8 && p.w_tiled && options().head_stream_kernel && H % 128 == 0 && nrb / (G * kHeadWaves) > 2) {
-        const int m = nrb / (G * kHeadWaves * 3) + 1;
+    // The streaming kernel has accumulators for four full passes per wave (two for 65 to 128 hidden rows: three or four
+    // spill), so a vocabulary of more passes than that gets a multiple of the CU count in workgroups -- they run one after
+    // the other on a CU, the stream does not stop between them -- instead of the K-chunked kernel (128 rows x 151936 x 4096:
+    // 0.75 against 0.53 of HBM peak; 60 rows x 200000 x 4096: 0.82 against 0.76; 1 to 60 rows x 262144 x 4096: 0.81 against
+    // 0.81 to 0.83).
+    const int stream_passes = NB == 8 ? 2 : 4;
+    if (p.w_tiled && options().head_stream_kernel && H % (NB == 8 ? 128 : 256) == 0 && nrb / (G * kHeadWaves) > stream_passes) {
+        const int m = nrb / (G * kHeadWaves * (stream_passes + 1)) + 1;
         if (G * m <= head_max_grid()) G *= m;
     }
     p.npasses = ceil_div(nrb, G * kHeadWaves);

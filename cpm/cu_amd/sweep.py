@@ -2,7 +2,7 @@
 
     python -m cpm.cu_amd.sweep attention [--groups]   tree attention, prefix 256..131072 x tree rows 1..128 (us per layer);
                                                       --groups: the automatic choice beside both kernel shapes forced
-    python -m cpm.cu_amd.sweep head                   target head (arg-max), rows 1..128 x vocabulary 8K..152K x hidden 2048/4096/8192
+    python -m cpm.cu_amd.sweep head                   target head (arg-max), rows 1..128 x vocabulary 8K..256K x hidden 2048/4096/8192
     python -m cpm.cu_amd.sweep frspec                 FR-Spec head + log-softmax + top-k + id map-back, vocabulary 8K..73448 x rows x k
 
 Eager launches on cuda:0, random fp16 data, event-timed; attention rotates over several layers' K/V pools and the heads over
@@ -76,7 +76,7 @@ def head(torch):
     for H in (2048, 4096, 8192):
         print("target head, hidden size %d: fraction of 8 TB/s (kernel)" % H)
         print("%8s" % "V \\ n" + "".join("%20d" % n for n in rows))
-        for V in (8192, 16384, 32768, 50000, 73448, 100000, 131072, 151936):
+        for V in (8192, 16384, 32768, 50000, 73448, 100000, 131072, 151936, 200000, 262144):
             w = (torch.randn(V, H, device="cuda") * 0.02).half()
             copies = [ops.tile_head_weight(w) for _ in range(2 if V * H * 2 < 1.5e9 else 1)]
             del w

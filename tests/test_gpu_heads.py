@@ -125,10 +125,10 @@ def test_frspec_tiled_chunk_rotation_shapes(gpu, orc):
 
 
 @pytest.mark.parametrize("n,V,Vs,H,k", [(10, 73448, 32768 + 16 * 300, 1024, 10), (16, 60000, 50000, 512, 10), (3, 73448, 70000, 512, 32),
-                                        (12, 50000, 36000, 512, 5)])
+                                        (12, 50000, 36000, 512, 5), (10, 200000, 180000, 512, 10)])
 def test_frspec_streaming_kernel_with_a_shared_last_pass(gpu, orc, n, V, Vs, H, k):
     """Sub-vocabularies that are not a whole number of passes: the streaming GEMM with its statistics epilogue, the
-    last pass shared by 4, 1, 4 (behind two full passes) and 8 waves."""
+    last pass shared by 4, 1, 4 (behind two full passes) and 8 waves; 180000 rows: twice as many workgroups as CUs."""
     from cpm.cu_amd import ops
     assert "head_gemm_stream_kernel" in ops.head_plan(n, ops.tile_head_weight(to_dev(gpu, np.zeros((Vs, H), np.float16))))[0]
     _frspec_check(gpu, orc, n=n, V=V, Vs=Vs, H=H, k=k, seed=Vs % 97, tiled=True)
@@ -500,6 +500,9 @@ _STREAM_SHAPES = [
     (128, 100000, 512, None),     # <8,1,128> on twice as many workgroups as CUs (three full passes would not fit the accumulators)
     (100, 151936, 512, 0.3125),   # <8,2,128> likewise
     (65, 220000, 512, None),      # <8,2,128> on three times as many
+    (16, 200000, 512, None),      # <1,3,256> on twice as many (six passes over the CUs' wave slots)
+    (40, 262144, 512, 2.0),       # <4,4,128> on twice as many, no last pass
+    (20, 400000, 512, None),      # <2,4,128> on three times as many
 ]
 
 
