@@ -21,8 +21,9 @@
 //   * the hidden rows are the B operand, staged in LDS: resident for the whole K range with up
 //     to 16 rows on the row-major path (head_gemm_kernel), otherwise walked in K chunks that are
 //     brought in by direct-to-LDS loads, double buffered, in the OUTER loop, with one accumulator
-//     set per row block of a sweep (head_gemm_chunked_kernel); tiled weights of one to four full passes run
-//     head_gemm_stream_kernel, which keeps the W stream in a register ring refilled fragment by fragment;
+//     set per row block of a sweep (head_gemm_chunked_kernel); tiled weights of at least one full pass run
+//     head_gemm_stream_kernel, which keeps the W stream in a register ring refilled fragment by fragment
+//     (one to four full passes per wave; more workgroups than CUs for larger vocabularies);
 //   * when the row blocks do not divide evenly over the wave slots, the blocks of the partly
 //     filled last pass are dealt round-robin to the workgroups and several waves share each of
 //     them, every one taking a subset of the K chunks; their partial sums meet in LDS.

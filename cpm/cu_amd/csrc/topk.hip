@@ -151,7 +151,9 @@ __global__ __launch_bounds__(kTopkThreads) void topk_merge_kernel(TopkParams p) 
 //   1. a lower bound of the k-th largest value: every wave takes the k-th largest of its 64
 //      per-lane maxima (bisection over the 16 bits with ballots, no barrier); the largest of the 16
 //      wave results has at least k elements at or above it, and on anything but tie-heavy data only
-//      a few hundred;
+//      a few hundred.  Beyond k = 16 that bound sinks towards the smallest lane maximum, so the waves whose 64 lanes all
+//      hold elements also take their ceil(k / waves)-th largest lane maximum each: the smallest of those has k lanes at
+//      or above it as well, and the higher of the two bounds is used (k up to 128);
 //   2. fused log-softmax: ranking is on f16((z - max) - ln sum), a monotone map of z that merges
 //      neighbours, so the bound moves down by four ulps of the mapped bound -- every z that can map
 //      to the same fp16 value or above stays a candidate -- and only candidates are mapped;
@@ -168,7 +170,7 @@ constexpr int kRowCap = kRowThreads;                   // candidate keys held in
 constexpr int kRowBoundDrop = 4;                       // low bits of the bound that are not searched
 constexpr int kRowDenseWaves = 8;                      // waves that extract the candidates
 constexpr int kRowLaneCap = 512;                       // threads with candidates whose registers LDS can take
-constexpr int kRowMaxTop = 64;                         // the wave-level bound needs k <= 64 lanes
+constexpr int kRowMaxTop = 128;                        // output slots are ranks below k <= kRowCap; beyond 64 see row_kernel_ranks()
 
 typedef int16_t s16x2 __attribute__((ext_vector_type(2)));
 typedef uint16_t u16x2 __attribute__((ext_vector_type(2)));
@@ -179,7 +181,7 @@ __device__ __forceinline__ void topk_row_body(const TopkParams& p) {
     __shared__ int rank[kRowCap];
     __shared__ uint64_t wave_best[2][kRowWaves];
     __shared__ float row_m_lse[2];
-    __shared__ uint32_t wave_kth[kRowWaves];
+    __shared__ uint32_t wave_kth[kRowWaves], wave_few[kRowWaves];
     __shared__ int ncand, nlanes;
     __shared__ uint4 lanebuf[kRowPieces][kRowLaneCap];  // piece-major: neighbouring slots are neighbouring 16 bytes
     __shared__ int lane_owner[kRowLaneCap];
@@ -244,10 +246,23 @@ __device__ __forceinline__ void topk_row_body(const TopkParams& p) {
     // (with fused statistics wave 0 reduces those meanwhile and contributes no bound: any subset of
     // the waves gives a valid one)
     uint32_t kth = 0;
+    // k > 16: the full waves share k between them (wave 0 is busy with the statistics when those are fused)
+    const int first_wave = LOGSOFTMAX ? 1 : 0;
+    const int full_waves = min(kRowWaves, npieces >> 6);
+    const bool spread = p.top > 16 && full_waves - first_wave >= 2;
     if (!(LOGSOFTMAX && wave == 0)) {
         for (int bit = 15; bit >= kRowBoundDrop; --bit) {
             const uint32_t c = kth | (1u << bit);
             if (__popcll(__ballot(lmax >= c)) >= p.top) kth = c;
+        }
+        if (spread && wave < full_waves) {
+            const int few = (p.top + full_waves - first_wave - 1) / (full_waves - first_wave);
+            uint32_t kf = 0;
+            for (int bit = 15; bit >= kRowBoundDrop; --bit) {
+                const uint32_t c = kf | (1u << bit);
+                if (__popcll(__ballot(lmax >= c)) >= few) kf = c;
+            }
+            if (lane == 0) wave_few[wave] = kf;
         }
     }
     if (lane == 0) wave_kth[wave] = kth;
@@ -286,6 +301,13 @@ __device__ __forceinline__ void topk_row_body(const TopkParams& p) {
     uint32_t bound = wave_kth[0];
 #pragma unroll
     for (int w = 1; w < kRowWaves; ++w) bound = wave_kth[w] > bound ? wave_kth[w] : bound;
+    if (spread) {
+        uint32_t least = ~0u;
+#pragma unroll
+        for (int w = 0; w < kRowWaves; ++w)
+            if (w >= first_wave && w < full_waves) least = wave_few[w] < least ? wave_few[w] : least;
+        bound = least > bound ? least : bound;
+    }
     uint32_t lo = bound > 0 ? bound - 1 : 0;  // candidates: raw image >= lo
     float m = 0.f, lse = 0.f;
     if (LOGSOFTMAX) {
@@ -293,6 +315,9 @@ __device__ __forceinline__ void topk_row_body(const TopkParams& p) {
         lse = row_m_lse[1];
         if (bound > 0) lo = mapped_lower_image<E>(bound, m, lse);
     }
+    // a row that fits the candidate buffer needs no bound: every element whose image is not 0 is a candidate (image 0 is
+    // the NaN 0xFFFF, which also pads the registers beyond the row; a row that holds one goes the way of the k rounds below)
+    if (lo == 0 && !sliced && p.dim <= kRowCap) lo = 1;
 
     const auto key_from_image = [&](uint32_t o, int idx) -> uint64_t {
         uint16_t bits = (uint16_t)((o & 0x8000u) ? (o ^ 0x8000u) : (o ^ 0xFFFFu));
@@ -365,7 +390,7 @@ __device__ __forceinline__ void topk_row_body(const TopkParams& p) {
     __syncthreads();
     CPMCU_STAMP(g_topk_timeline, blockIdx.x, 4);
     const int C = ncand;
-    if (compact && C <= kRowCap) {
+    if (compact && C <= kRowCap && C >= p.top) {
         int shift = 6;
         while ((1 << shift) < C) ++shift;
         const int i = tid & ((1 << shift) - 1);
@@ -512,6 +537,14 @@ __global__ __launch_bounds__(256) void gather_rows_kernel(const f16x8* src, cons
 
 }  // namespace
 
+// Whether the row kernel finds a bound for the k-th largest of a row of `dim` elements (else it would fall to its k rounds):
+// up to 64 any wave's lanes do; beyond, the waves that are full of elements share k, at most 64 lanes' worth each.
+static bool row_kernel_ranks(int dim, int top, bool fused_stats) {
+    if (top <= 64 || dim <= kRowCap) return top <= kRowMaxTop;
+    const int sharing = std::min(kRowWaves, dim / 8 / 64) - (fused_stats ? 1 : 0);
+    return top <= kRowMaxTop && sharing >= 2 && sharing * 64 >= top;
+}
+
 int launch_topk(const void* x, int n, int dim, int top, void* val, int32_t* pos, int32_t* ids,
                 const int32_t* token_id_remap, const TopkStatsSource* stats, void* workspace,
                 size_t workspace_bytes, hipStream_t st) {
@@ -533,7 +566,7 @@ int launch_topk(const void* x, int n, int dim, int top, void* val, int32_t* pos,
     p.stride = stats ? stats->stride : 0;
     p.row_stats = stats ? stats->row_stats : nullptr;
     // rows that fit one workgroup's registers: one launch, no candidate buffer
-    if (dim <= kRowMaxDim && dim % 8 == 0 && top <= kRowMaxTop && ((uintptr_t)x & 15) == 0) {
+    if (dim <= kRowMaxDim && dim % 8 == 0 && row_kernel_ranks(dim, top, stats != nullptr) && ((uintptr_t)x & 15) == 0) {
         if (stats && options().dtype == 1) hipLaunchKernelGGL(topk_row_bf16_kernel, dim3(n), dim3(kRowThreads), 0, st, p);
         else if (stats) hipLaunchKernelGGL(topk_row_kernel<true>, dim3(n), dim3(kRowThreads), 0, st, p);
         else hipLaunchKernelGGL(topk_row_kernel<false>, dim3(n), dim3(kRowThreads), 0, st, p);

@@ -4,6 +4,7 @@
                                                       --groups: the automatic choice beside both kernel shapes forced
     python -m cpm.cu_amd.sweep head                   target head (arg-max), rows 1..128 x vocabulary 8K..256K x hidden 2048/4096/8192
     python -m cpm.cu_amd.sweep frspec                 FR-Spec head + log-softmax + top-k + id map-back, vocabulary 8K..73448 x rows x k
+    python -m cpm.cu_amd.sweep topk                   top-k of fp16 rows, row length 64..152K x rows 1..60 x k 1..128
 
 Eager launches on cuda:0, random fp16 data, event-timed; attention rotates over several layers' K/V pools and the heads over
 copies of the weight matrix, so that no pass is served from the last-level cache.  Fractions are of 8 TB/s (heads) and TFLOP/s
@@ -120,8 +121,36 @@ def frspec(torch):
         del copies
 
 
+def topk(torch):
+    from . import ops
+    tops = [1, 10, 16, 32, 64, 128]
+    for n in (1, 10, 60):
+        print("top-k of %d fp16 rows: us per call (k across, row length down)" % n)
+        print("%8s" % "dim \\ k" + "".join("%9d" % k for k in tops))
+        for dim in (64, 640, 1000, 4096, 8192, 16384, 32768, 32776, 65536, 73448, 151936):
+            xs = [torch.randn(n, dim, device="cuda").half() for _ in range(4)]
+            line = "%8d" % dim
+            for k in tops:
+                if k > dim:
+                    line += "%9s" % "-"
+                    continue
+
+                def run():
+                    for x in xs:
+                        ops.topk(x, k)
+                try:
+                    for _ in range(3):
+                        run()
+                except ValueError:  # a shape the operator refuses
+                    line += "%9s" % "refused"
+                    continue
+                torch.cuda.synchronize()
+                line += "%9.1f" % (_time(torch, run, 10) / len(xs))
+            print(line, flush=True)
+
+
 def main(argv):
-    if not argv or argv[0] not in ("attention", "head", "frspec"):
+    if not argv or argv[0] not in ("attention", "head", "frspec", "topk"):
         print(__doc__)
         return 2
     import torch
@@ -132,6 +161,8 @@ def main(argv):
         attention(torch, "--groups" in argv[1:])
     elif argv[0] == "head":
         head(torch)
+    elif argv[0] == "topk":
+        topk(torch)
     else:
         frspec(torch)
     return 0

@@ -82,9 +82,10 @@ const char* cpmcu_version(void);
  *                           shape of the tree-attention kernel (CPMCU_ATTN_KV_GROUPS=1|2);
  *   "head_share_last_pass"  1 = the waves of a workgroup share the row blocks of a partly filled last pass
  *                           of the head GEMM (default), 0 = plain mapping (CPMCU_HEAD_NO_SHARE set);
- *   "head_stream_kernel"    1 = tiled head weights whose row blocks make one to four full passes over the GPU's
- *                           wave slots run the streaming GEMM kernel (default), 0 = always the K-chunked kernel
- *                           (CPMCU_HEAD_NO_STREAM set);
+ *   "head_stream_kernel"    1 = tiled head weights whose row blocks make at least one full pass over the GPU's
+ *                           wave slots run the streaming GEMM kernel, on a multiple of the CU count in workgroups
+ *                           (up to 1024) beyond four passes (two for 65 to 128 hidden rows) (default), 0 = always
+ *                           the K-chunked kernel (CPMCU_HEAD_NO_STREAM set);
  *   "attn_merge_in_launch"  1 = the workgroups of a split tree-attention launch merge their own partials when the
  *                           launch fits the GPU's CUs and has at most 32 splits (default), 0 = always the separate
  *                           merge launch (CPMCU_ATTN_SEPARATE_MERGE set);

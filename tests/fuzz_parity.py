@@ -95,6 +95,8 @@ def main(argv):
         H = int([512, 1024, 2048, 4096][g.integers(4)])
         if H >= 2048:
             V = min(V, 12000)
+        elif g.random() < 0.2:  # one to twelve passes over the CUs' wave slots: the streaming kernel's shapes and grids
+            V, H = int(g.integers(33000, 420000)), 512
         t_heads._argmax_check(torch, orc, n, V=V, H=H, seed=seed, scale=[None, 0.5, 1.7][int(g.integers(3))], tiled=bool(g.integers(2)))
 
     def frspec_head(seed):

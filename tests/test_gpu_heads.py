@@ -508,7 +508,7 @@ _STREAM_SHAPES = [
 
 @pytest.mark.parametrize("n,V,H,scale", _STREAM_SHAPES)
 def test_streaming_head_kernel_equals_chunked_kernel(gpu, orc, set_option, n, V, H, scale):
-    """Tiled weights with one to four full passes run the streaming kernel (register ring refilled fragment by
+    """Tiled weights of at least one full pass run the streaming kernel (register ring refilled fragment by
     fragment, last pass shared by K slices).  Every (row blocks, full passes) shape it is built for, with 1, 2,
     4 and 8 waves per last-pass block and without a last pass: same logits as the K-chunked kernel up to the
     fp32 summation order, both within tolerance of the oracle, arg-max exact on each kernel's own logits."""
