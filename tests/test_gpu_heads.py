@@ -329,7 +329,12 @@ def test_target_head_c5_full_size(gpu, orc):
 
 
 @pytest.mark.parametrize("n,dim,top", [(1, 100, 10), (1, 510, 59), (10, 32768, 10), (3, 5000, 32), (2, 2048, 1),
-                                        (2, 2049, 128), (4, 73448, 10), (1, 7, 7)])
+                                        (2, 2049, 128), (4, 73448, 10), (1, 7, 7),
+                                        # the row kernel's bounds: no bound (up to 1024 elements, also k = the whole row), k shared by
+                                        # 2, 3, 4, 8 and 16 full waves, every lane of two waves needed, slices with k beyond 64
+                                        (1, 64, 10), (3, 64, 64), (2, 1000, 128), (2, 1024, 17), (1, 1032, 128), (2, 1032, 100),
+                                        (2, 1536, 128), (2, 2048, 128), (3, 4096, 64), (2, 4096, 17), (3, 32768, 64), (2, 32768, 128),
+                                        (2, 20000, 33), (2, 73448, 100), (2, 151936, 128), (2, 32776, 128)])
 def test_topk_matches_oracle(gpu, orc, n, dim, top):
     from cpm.cu_amd import ops
     torch = gpu
@@ -359,7 +364,8 @@ def test_topk_heavy_ties_and_neg_inf(gpu, orc):
     assert np.array_equal(p_ref[0], np.arange(32))
 
 
-@pytest.mark.parametrize("case", ["two_values", "mostly_neg_inf", "descending", "ascending", "wide_range", "k64", "tiny_rows"])
+@pytest.mark.parametrize("case", ["two_values", "mostly_neg_inf", "descending", "ascending", "wide_range", "k64", "tiny_rows",
+                                  "k128_descending", "k64_one_wave_neg_inf", "k100_two_values", "k40_few_finite"])
 def test_topk_row_kernel_shapes_of_data(gpu, orc, case):
     """Inputs chosen against the one-launch row kernel's bound / candidate / fallback logic."""
     from cpm.cu_amd import ops
@@ -387,6 +393,25 @@ def test_topk_row_kernel_shapes_of_data(gpu, orc, case):
     elif case == "k64":
         x = g.standard_normal((3, 32768)).astype(np.float16)
         top = 64
+    elif case == "k128_descending":
+        x = np.tile(np.linspace(8, -8, 32768, dtype=np.float32).astype(np.float16), (2, 1))   # the waves' shares of k are far apart
+        x[1] = x[1, ::-1]
+        top = 128
+    elif case == "k64_one_wave_neg_inf":
+        x = g.standard_normal((3, 16384)).astype(np.float16)
+        x[0, 8 * 64 * 3:8 * 64 * 4] = -np.inf                              # first piece of wave 3: that wave's share has no finite bound
+        x[1].reshape(2, 16, 64, 8)[:, 5] = -np.inf                         # everything wave 5 holds (piece, wave, lane, element)
+        x[2].reshape(2, 16, 64, 8)[:, 1:] = -np.inf                        # only wave 0 holds finite values
+        top = 64
+    elif case == "k100_two_values":
+        x = g.integers(0, 2, size=(3, 8192)).astype(np.float16)
+        x[1, 50:] = 0                                                      # fewer ones than k: the bound is the tie value
+        top = 100
+    elif case == "k40_few_finite":
+        x = np.full((2, 4096), -np.inf, np.float16)
+        x[0, ::128] = g.standard_normal(32).astype(np.float16)             # 32 finite values for k = 40
+        x[1, 7::64] = g.standard_normal(64).astype(np.float16)
+        top = 40
     else:
         x = g.standard_normal((6, 64)).astype(np.float16)                  # one wave holds everything
         top = 8
