@@ -1,7 +1,9 @@
 """Timings of the operators over ranges of shapes, with the kernels the library picks for each: looks for cliffs in the launch plans.
 
-    python -m cpm.cu_amd.sweep attention [--groups]   tree attention, prefix 256..131072 x tree rows 1..128 (us per layer);
-                                                      --groups: the automatic choice beside both kernel shapes forced
+    python -m cpm.cu_amd.sweep attention [--groups] [--heads Hq,Hkv]
+                                                      tree attention, prefix 256..131072 x tree rows 1..128 (us per layer);
+                                                      --groups: the automatic choice beside both kernel shapes forced;
+                                                      --heads: query / KV head counts other than 32,2
     python -m cpm.cu_amd.sweep head                   target head (arg-max), rows 1..128 x vocabulary 8K..256K x hidden 2048/4096/8192
     python -m cpm.cu_amd.sweep frspec                 FR-Spec head + log-softmax + top-k + id map-back, vocabulary 8K..73448 x rows x k
     python -m cpm.cu_amd.sweep topk                   top-k of fp16 rows, row length 64..152K x rows 1..60 x k 1..128
@@ -25,10 +27,10 @@ def _time(torch, fn, reps):
     return e0.elapsed_time(e1) / reps * 1e3
 
 
-def attention(torch, with_groups):
+def attention(torch, with_groups, Hq=32, Hkv=2):
     from . import lib, ops, synth
     from .kvcache import PagedKVCache
-    Hq, Hkv, D = 32, 2, 128
+    D = 128
     L = lib.get()
     prefixes = [256, 1024, 2048, 4096, 8192, 16384, 32768, 65536, 131072]
     rows = [1, 8, 16, 24, 32, 40, 48, 60, 64, 96, 128]
@@ -158,7 +160,8 @@ def main(argv):
     lib.get()  # raises if libcpmcu_amd.so is missing
     torch.cuda.set_device(0)
     if argv[0] == "attention":
-        attention(torch, "--groups" in argv[1:])
+        heads = argv[argv.index("--heads") + 1].split(",") if "--heads" in argv else (32, 2)
+        attention(torch, "--groups" in argv[1:], int(heads[0]), int(heads[1]))
     elif argv[0] == "head":
         head(torch)
     elif argv[0] == "topk":

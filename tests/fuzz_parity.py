@@ -105,7 +105,7 @@ def main(argv):
         H = int([512, 1024][g.integers(2)])
         Vs = int(g.integers(2, 4200)) * 8
         V = Vs + int(g.integers(0, 5000))
-        t_heads._frspec_check(torch, orc, n, V, Vs, H, int(g.integers(1, 17)), seed, tiled=bool(g.integers(2)))
+        t_heads._frspec_check(torch, orc, n, V, Vs, H, int(g.integers(1, 33)), seed, tiled=bool(g.integers(2)))
 
     def topk(seed):
         g = synth.rng(seed, 94)
@@ -180,7 +180,7 @@ def main(argv):
             else:
                 Vs = int(g.integers(2, 2100)) * 8
                 t_bf16.test_bf16_frspec_head_topk(torch, orc, None, int(g.integers(1, 17)), Vs + int(g.integers(0, 3000)), Vs, int([512, 1024][g.integers(2)]),
-                                                  int(g.integers(1, 17)), bool(g.integers(2)))
+                                                  int(g.integers(1, 33)), bool(g.integers(2)))
         finally:
             orc.set_dtype("f16")
             set_option("dtype", 0)

@@ -109,7 +109,9 @@ def test_bf16_target_head_full_size(gpu, orc, bf16):
 
 
 @pytest.mark.parametrize("n,V,Vs,H,k,tiled", [(10, 6000, 4096, 512, 10, False), (16, 9000, 4096 + 40, 2048, 10, True), (1, 3000, 2048, 1024, 10, False),
-                                               (10, 73448, 32768, 4096, 10, True)])
+                                               (10, 73448, 32768, 4096, 10, True),
+                                               # k beyond 16: the top-k bound is shared between the waves
+                                               (7, 40000, 32768, 512, 32, True), (4, 9000, 8192, 512, 20, False), (3, 50000, 40960, 512, 24, True)])
 def test_bf16_frspec_head_topk(gpu, orc, bf16, n, V, Vs, H, k, tiled):
     """The FR-Spec head in bfloat16: logits within tolerance, and the ranking of the rounded log-probabilities bit-exact
     when the oracle ranks the device's own logits and row statistics (bfloat16 keeps 8 bits: far more ties than fp16)."""
