@@ -31,6 +31,7 @@ struct TopkParams {
     const uint16_t* x;  // [n][dim] fp16 bits
     int n, dim, top, nchunks;
     int slice_len;      // row kernel: elements per workgroup when a row is cut into slices (0: the whole row)
+    int ragged;         // row kernel: rows are not whole 16-byte pieces (dim not a multiple of 8, or x not 16-byte aligned)
     uint64_t* cand;     // [n][nchunks][top]
     uint16_t* val;      // [n][top]
     int32_t* pos;
@@ -192,16 +193,34 @@ __device__ __forceinline__ void topk_row_body(const TopkParams& p) {
     // leaves its k best as keys for the merge launch instead of writing the outputs
     const bool sliced = p.slice_len != 0;
     const int slice_base = sliced ? blockIdx.y * p.slice_len : 0;
-    const int npieces = (sliced ? min(p.slice_len, p.dim - slice_base) : p.dim) >> 3;
+    const int len = sliced ? min(p.slice_len, p.dim - slice_base) : p.dim;
+    const int npieces = (len + 7) >> 3;
     const uint4* xr = (const uint4*)(p.x + (size_t)row * p.dim + slice_base);
     uint64_t* slice_out = sliced ? p.cand + ((size_t)row * gridDim.y + blockIdx.y) * p.top : nullptr;
     if (sliced && tid < p.top) slice_out[tid] = 0;  // slots this slice cannot fill stay empty (overwritten behind a barrier)
     // slots beyond the row read as 0xFFFF, whose raw image is 0: below every bound that is used
     uint4 raw[kRowPieces];
+    if (!p.ragged) {
 #pragma unroll
-    for (int j = 0; j < kRowPieces; ++j) {
-        const int pc = j * kRowThreads + tid;
-        raw[j] = pc < npieces ? xr[pc] : make_uint4(~0u, ~0u, ~0u, ~0u);
+        for (int j = 0; j < kRowPieces; ++j) {
+            const int pc = j * kRowThreads + tid;
+            raw[j] = pc < npieces ? xr[pc] : make_uint4(~0u, ~0u, ~0u, ~0u);
+        }
+    } else {
+        // rows that do not start on 16 bytes or do not end on a whole piece: element by element
+        const uint16_t* xe = (const uint16_t*)xr;
+#pragma unroll
+        for (int j = 0; j < kRowPieces; ++j) {
+            const int e0 = (j * kRowThreads + tid) * 8;
+            uint32_t w4[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const uint32_t a = e0 + 2 * q < len ? xe[e0 + 2 * q] : 0xFFFFu;
+                const uint32_t b = e0 + 2 * q + 1 < len ? xe[e0 + 2 * q + 1] : 0xFFFFu;
+                w4[q] = a | (b << 16);
+            }
+            raw[j] = make_uint4(w4[0], w4[1], w4[2], w4[3]);
+        }
     }
     if (tid == 0) {
         ncand = 0;
@@ -439,11 +458,11 @@ __device__ __forceinline__ void topk_row_body(const TopkParams& p) {
         uint64_t mine = 0;
 #pragma unroll
         for (int j = 0; j < kRowPieces; ++j) {
-            const bool pv = j * kRowThreads + tid < npieces;
+            const int e0 = (j * kRowThreads + tid) * 8;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 const uint32_t o = (img[j * 4 + (e >> 1)] >> ((e & 1) * 16)) & 0xFFFFu;
-                const uint64_t key = pv ? key_from_image(o, slice_base + (j * kRowThreads + tid) * 8 + e) : 0ull;
+                const uint64_t key = e0 + e < len ? key_from_image(o, slice_base + e0 + e) : 0ull;
                 if (key < prev && key > mine) mine = key;
             }
         }
@@ -560,6 +579,7 @@ int launch_topk(const void* x, int n, int dim, int top, void* val, int32_t* pos,
     p.top = top;
     p.nchunks = ceil_div(dim, kChunk);
     p.slice_len = 0;
+    p.ragged = dim % 8 != 0 || ((uintptr_t)x & 15) != 0;
     p.cand = (uint64_t*)workspace;
     p.val = (uint16_t*)val;
     p.pos = pos;
@@ -571,7 +591,7 @@ int launch_topk(const void* x, int n, int dim, int top, void* val, int32_t* pos,
     p.stride = stats ? stats->stride : 0;
     p.row_stats = stats ? stats->row_stats : nullptr;
     // rows that fit one workgroup's registers: one launch, no candidate buffer
-    if (dim <= kRowMaxDim && dim % 8 == 0 && row_kernel_ranks(dim, top, stats != nullptr) && ((uintptr_t)x & 15) == 0) {
+    if (dim <= kRowMaxDim && row_kernel_ranks(dim, top, stats != nullptr)) {
         if (stats && options().dtype == 1) hipLaunchKernelGGL(topk_row_bf16_kernel, dim3(n), dim3(kRowThreads), 0, st, p);
         else if (stats) hipLaunchKernelGGL(topk_row_kernel<true>, dim3(n), dim3(kRowThreads), 0, st, p);
         else hipLaunchKernelGGL(topk_row_kernel<false>, dim3(n), dim3(kRowThreads), 0, st, p);
@@ -580,7 +600,7 @@ int launch_topk(const void* x, int n, int dim, int top, void* val, int32_t* pos,
     }
     // longer rows in slices of at most kRowMaxDim elements: the row kernel on every slice, and a merge of the slices' k best
     const int nslices = ceil_div(dim, kRowMaxDim);
-    if (dim % 8 == 0 && top <= kRowMaxTop && ((uintptr_t)x & 15) == 0 && nslices * top <= kSliceMergeCap && workspace &&
+    if (top <= kRowMaxTop && nslices * top <= kSliceMergeCap && workspace &&
         workspace_bytes >= (size_t)n * nslices * top * sizeof(uint64_t)) {
         p.slice_len = (ceil_div(dim, nslices) + 7) / 8 * 8;
         p.nchunks = nslices;

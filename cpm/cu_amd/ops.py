@@ -210,9 +210,8 @@ def frspec_head_plan(n, w, k):
     if _lib().raw.cpmcu_frspec_head_mode(ctypes.c_void_p(ws.data_ptr()), layout, n, V, H, k) == 1:
         nb, fp, kc = gemm[gemm.index("<") + 1:-1].split(",")
         return "frspec_head_topk_kernel<%s,%s>" % (fp, kc)
-    if V % 8 == 0 and k <= 64:  # the row kernel: on the whole row up to 32768 elements, on slices of it beyond
-        return gemm + ("+topk_row_kernel<true>" if V <= 32768 else "+topk_row_kernel<true>+topk_slice_merge_kernel<true>")
-    return gemm + "+topk_chunk_kernel<true>+topk_merge_kernel<true>"
+    # the row kernel: on the whole row up to 32768 elements, on slices of it beyond
+    return gemm + ("+topk_row_kernel<true>" if V <= 32768 else "+topk_row_kernel<true>+topk_slice_merge_kernel<true>")
 
 
 def lm_head_argmax(hidden, w, head_scale=None, want_logits=False, gt=None):

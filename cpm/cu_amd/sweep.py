@@ -129,7 +129,7 @@ def topk(torch):
     for n in (1, 10, 60):
         print("top-k of %d fp16 rows: us per call (k across, row length down)" % n)
         print("%8s" % "dim \\ k" + "".join("%9d" % k for k in tops))
-        for dim in (64, 640, 1000, 4096, 8192, 16384, 32768, 32776, 65536, 73448, 151936):
+        for dim in (64, 510, 640, 1000, 4096, 8192, 16384, 32001, 32768, 32776, 65536, 73448, 151643, 151936):
             xs = [torch.randn(n, dim, device="cuda").half() for _ in range(4)]
             line = "%8d" % dim
             for k in tops:

@@ -103,7 +103,7 @@ def main(argv):
         g = synth.rng(seed, 93)
         n = int(g.integers(1, 17))
         H = int([512, 1024][g.integers(2)])
-        Vs = int(g.integers(2, 4200)) * 8
+        Vs = int(g.integers(2, 4200)) * 8 - (int(g.integers(8)) if g.random() < 0.3 else 0)
         V = Vs + int(g.integers(0, 5000))
         t_heads._frspec_check(torch, orc, n, V, Vs, H, int(g.integers(1, 33)), seed, tiled=bool(g.integers(2)))
 

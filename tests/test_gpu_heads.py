@@ -125,12 +125,15 @@ def test_frspec_tiled_chunk_rotation_shapes(gpu, orc):
 
 
 @pytest.mark.parametrize("n,V,Vs,H,k", [(10, 73448, 32768 + 16 * 300, 1024, 10), (16, 60000, 50000, 512, 10), (3, 73448, 70000, 512, 32),
-                                        (12, 50000, 36000, 512, 5), (10, 200000, 180000, 512, 10)])
+                                        (12, 50000, 36000, 512, 5), (10, 200000, 180000, 512, 10),
+                                        # sub-vocabularies whose rows of logits are not whole 16-byte pieces
+                                        (5, 9000, 4099, 512, 10), (3, 40000, 33001, 512, 7), (16, 70000, 65537, 512, 16)])
 def test_frspec_streaming_kernel_with_a_shared_last_pass(gpu, orc, n, V, Vs, H, k):
     """Sub-vocabularies that are not a whole number of passes: the streaming GEMM with its statistics epilogue, the
     last pass shared by 4, 1, 4 (behind two full passes) and 8 waves; 180000 rows: twice as many workgroups as CUs."""
     from cpm.cu_amd import ops
-    assert "head_gemm_stream_kernel" in ops.head_plan(n, ops.tile_head_weight(to_dev(gpu, np.zeros((Vs, H), np.float16))))[0]
+    if Vs >= 32768:
+        assert "head_gemm_stream_kernel" in ops.head_plan(n, ops.tile_head_weight(to_dev(gpu, np.zeros((Vs, H), np.float16))))[0]
     _frspec_check(gpu, orc, n=n, V=V, Vs=Vs, H=H, k=k, seed=Vs % 97, tiled=True)
 
 
@@ -334,13 +337,33 @@ def test_target_head_c5_full_size(gpu, orc):
                                         # 2, 3, 4, 8 and 16 full waves, every lane of two waves needed, slices with k beyond 64
                                         (1, 64, 10), (3, 64, 64), (2, 1000, 128), (2, 1024, 17), (1, 1032, 128), (2, 1032, 100),
                                         (2, 1536, 128), (2, 2048, 128), (3, 4096, 64), (2, 4096, 17), (3, 32768, 64), (2, 32768, 128),
-                                        (2, 20000, 33), (2, 73448, 100), (2, 151936, 128), (2, 32776, 128)])
+                                        (2, 20000, 33), (2, 73448, 100), (2, 151936, 128), (2, 32776, 128),
+                                        # rows that are not whole 16-byte pieces (every row but the first starts off 16 bytes)
+                                        (3, 510, 59), (4, 100, 10), (3, 1001, 128), (3, 4099, 59), (4, 32001, 59), (3, 32767, 10),
+                                        (2, 50257, 64), (2, 151643, 59), (2, 65537, 128), (5, 9, 9), (3, 1025, 100)])
 def test_topk_matches_oracle(gpu, orc, n, dim, top):
     from cpm.cu_amd import ops
     torch = gpu
     g = synth.rng(dim, top)
     x = g.standard_normal((n, dim)).astype(np.float16)
     val, pos = ops.topk(to_dev(torch, x), top)
+    torch.cuda.synchronize()
+    v_ref, p_ref = orc.topk(x, top)
+    assert np.array_equal(to_np(pos), p_ref)
+    assert np.array_equal(to_np(val).view(np.uint16), v_ref.view(np.uint16))
+
+
+@pytest.mark.parametrize("n,dim,top,off", [(3, 512, 59, 1), (2, 32768, 10, 3), (2, 40960, 64, 5), (4, 104, 10, 7), (2, 8200, 128, 2)])
+def test_topk_of_rows_that_start_off_16_bytes(gpu, orc, n, dim, top, off):
+    """The input begins `off` elements into an aligned buffer: the row kernel reads such rows element by element."""
+    from cpm.cu_amd import ops
+    torch = gpu
+    x = synth.rng(dim, off).standard_normal((n, dim)).astype(np.float16)
+    buf = torch.zeros(n * dim + 8, dtype=torch.float16, device="cuda")
+    d_x = buf[off:off + n * dim].view(n, dim)
+    d_x.copy_(to_dev(torch, x))
+    assert d_x.data_ptr() % 16 != 0
+    val, pos = ops.topk(d_x, top)
     torch.cuda.synchronize()
     v_ref, p_ref = orc.topk(x, top)
     assert np.array_equal(to_np(pos), p_ref)
