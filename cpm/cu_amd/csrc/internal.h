@@ -16,6 +16,7 @@ struct Options {
     int attn_merge_wait_us = 2000; // longest wait of a workgroup for the others of its merge before it abandons its share
     int frspec_fused = 0;          // 1: the FR-Spec head with its top-k as one launch where the shape allows (measured no faster: off)
     int frspec_wait_us = 50000;    // longest wait of a finisher of the fused FR-Spec launch for the other workgroups' words
+    int topk_row_kernel = 1;       // 0: top-k by k rounds per chunk of 2048 elements and a merge launch (tests compare the two)
 };
 Options& options();
 

@@ -240,6 +240,9 @@ extern "C" int cpmcu_set_option(const char* name, int value) {
         CPMCU_CHECK_ARG(value == 0 || value == 1, "set_option: frspec_fused=%d must be 0 or 1", value);
         options().frspec_fused = value;
         if (value) head_fuse_reenable();  // also after a wait that ran out
+    } else if (nm == "topk_row_kernel") {
+        CPMCU_CHECK_ARG(value == 0 || value == 1, "set_option: topk_row_kernel=%d must be 0 or 1", value);
+        options().topk_row_kernel = value;
     } else if (nm == "frspec_wait_us") {
         CPMCU_CHECK_ARG(value >= 0 && value <= 1000000, "set_option: frspec_wait_us=%d outside [0, 1000000]", value);
         options().frspec_wait_us = value;
@@ -793,7 +796,7 @@ uint64_t step_signature(const Model& m, const StepArgs& a) {
         mix(v);
     // the options decide which kernels a capture records: a graph captured under other settings is another graph
     const Options& o = options();
-    for (int v : {o.dtype, o.attn_kv_groups, o.head_share_last_pass, o.head_stream_kernel, o.attn_merge_in_launch, o.attn_merge_wait_us, o.frspec_fused, o.frspec_wait_us}) mix((uint64_t)(uint32_t)v);
+    for (int v : {o.dtype, o.attn_kv_groups, o.head_share_last_pass, o.head_stream_kernel, o.attn_merge_in_launch, o.attn_merge_wait_us, o.frspec_fused, o.frspec_wait_us, o.topk_row_kernel}) mix((uint64_t)(uint32_t)v);
     return h;
 }
 

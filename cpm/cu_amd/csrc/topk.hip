@@ -591,7 +591,8 @@ int launch_topk(const void* x, int n, int dim, int top, void* val, int32_t* pos,
     p.stride = stats ? stats->stride : 0;
     p.row_stats = stats ? stats->row_stats : nullptr;
     // rows that fit one workgroup's registers: one launch, no candidate buffer
-    if (dim <= kRowMaxDim && row_kernel_ranks(dim, top, stats != nullptr)) {
+    const bool row_kernel = options().topk_row_kernel != 0;
+    if (row_kernel && dim <= kRowMaxDim && row_kernel_ranks(dim, top, stats != nullptr)) {
         if (stats && options().dtype == 1) hipLaunchKernelGGL(topk_row_bf16_kernel, dim3(n), dim3(kRowThreads), 0, st, p);
         else if (stats) hipLaunchKernelGGL(topk_row_kernel<true>, dim3(n), dim3(kRowThreads), 0, st, p);
         else hipLaunchKernelGGL(topk_row_kernel<false>, dim3(n), dim3(kRowThreads), 0, st, p);
@@ -600,7 +601,7 @@ int launch_topk(const void* x, int n, int dim, int top, void* val, int32_t* pos,
     }
     // longer rows in slices of at most kRowMaxDim elements: the row kernel on every slice, and a merge of the slices' k best
     const int nslices = ceil_div(dim, kRowMaxDim);
-    if (top <= kRowMaxTop && nslices * top <= kSliceMergeCap && workspace &&
+    if (row_kernel && top <= kRowMaxTop && nslices * top <= kSliceMergeCap && workspace &&
         workspace_bytes >= (size_t)n * nslices * top * sizeof(uint64_t)) {
         p.slice_len = (ceil_div(dim, nslices) + 7) / 8 * 8;
         p.nchunks = nslices;

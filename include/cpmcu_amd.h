@@ -90,7 +90,11 @@ const char* cpmcu_version(void);
  *                           launch fits the GPU's CUs and has at most 32 splits (default), 0 = always the separate
  *                           merge launch (CPMCU_ATTN_SEPARATE_MERGE set);
  *   "attn_merge_wait_us"    longest time a workgroup of such a launch waits for the others of its merge before it
- *                           leaves its share to the last one to arrive (default 2000; 0 = never wait). */
+ *                           leaves its share to the last one to arrive (default 2000; 0 = never wait);
+ *   "topk_row_kernel"       1 = top-k by the one-launch row kernel (rows of more than 32768 elements in slices and a
+ *                           merge of the slices' k best) (default), 0 = k rounds of a maximum search per chunk of 2048
+ *                           elements and a merge launch, for chunks x k up to 2048: the same results, bit for bit,
+ *                           from independent code. */
 int cpmcu_set_option(const char* name, int value);
 
 /* ------------------------------------------------------------------------- */

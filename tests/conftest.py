@@ -36,7 +36,7 @@ def set_option():
     """Sets kernel-shape options of the library for one test and restores the defaults afterwards."""
     from cpm.cu_amd import lib
     defaults = {"dtype": 0, "attn_kv_groups": 0, "head_share_last_pass": 1, "head_stream_kernel": 1, "attn_merge_in_launch": 1, "attn_merge_wait_us": 2000,
-                "frspec_fused": 0, "frspec_wait_us": 50000}
+                "frspec_fused": 0, "frspec_wait_us": 50000, "topk_row_kernel": 1}
     touched = []
 
     def setter(name, value):

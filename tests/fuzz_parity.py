@@ -123,10 +123,17 @@ def main(argv):
             x[:, idx] = g.standard_normal(len(idx)).astype(np.float16)
         else:
             x = (g.standard_normal((n, dim)) * np.exp(g.standard_normal((n, dim)) * 2)).astype(np.float16)
-        val, pos = ops.topk(to_dev(torch, x), top)
-        torch.cuda.synchronize()
+        chunk_form = g.random() < 0.1 and -(-dim // 2048) * top <= 2048  # one case in ten: the chunk + merge form
+        if chunk_form:
+            lib.get().set_option(b"topk_row_kernel", 0)
+        try:
+            val, pos = ops.topk(to_dev(torch, x), top)
+            torch.cuda.synchronize()
+        finally:
+            if chunk_form:
+                lib.get().set_option(b"topk_row_kernel", 1)
         v_ref, p_ref = orc.topk(x, top)
-        what = "n=%d dim=%d top=%d kind=%d" % (n, dim, top, kind)
+        what = "n=%d dim=%d top=%d kind=%d chunk_form=%d" % (n, dim, top, kind, chunk_form)
         assert np.array_equal(to_np(pos), p_ref), "top-k positions, " + what
         assert np.array_equal(to_np(val).view(np.uint16), v_ref.view(np.uint16)), "top-k values, " + what
 

@@ -370,6 +370,42 @@ def test_topk_of_rows_that_start_off_16_bytes(gpu, orc, n, dim, top, off):
     assert np.array_equal(to_np(val).view(np.uint16), v_ref.view(np.uint16))
 
 
+@pytest.mark.parametrize("n,dim,top,kind", [(3, 510, 59, "normal"), (10, 32768, 10, "normal"), (2, 32768, 64, "ties"), (4, 5000, 32, "ties"),
+                                            (2, 73448, 25, "normal"), (3, 20000, 100, "normal"), (2, 32001, 63, "ties"), (5, 64, 64, "normal"),
+                                            (2, 16384, 40, "neg_inf")])
+def test_topk_row_kernel_equals_chunk_and_merge_form(gpu, orc, set_option, n, dim, top, kind):
+    """The library's two top-k implementations (option topk_row_kernel): the one-launch row kernel, which bounds, extracts
+    and ranks by counting, and k rounds of a maximum search per 2048-element chunk followed by a merge launch -- the same
+    positions and value bits from both, and from the oracle."""
+    from cpm.cu_amd import ops
+    torch = gpu
+    g = synth.rng(dim, top + 1)
+    if kind == "ties":
+        x = (g.integers(-3, 4, size=(n, dim)) * 0.5).astype(np.float16)
+    else:
+        x = g.standard_normal((n, dim)).astype(np.float16)
+    if kind == "neg_inf":
+        x[:, g.random(dim) < 0.97] = -np.inf
+    d_x = to_dev(torch, x)
+    got = []
+    for form in (1, 0):
+        set_option("topk_row_kernel", form)
+        val, pos = ops.topk(d_x, top)
+        torch.cuda.synchronize()
+        got.append((to_np(val).view(np.uint16).copy(), to_np(pos).copy()))
+    assert np.array_equal(got[0][0], got[1][0]) and np.array_equal(got[0][1], got[1][1])
+    v_ref, p_ref = orc.topk(x, top)
+    assert np.array_equal(got[0][1], p_ref) and np.array_equal(got[0][0], v_ref.view(np.uint16))
+
+
+def test_frspec_head_with_the_chunk_and_merge_top_k(gpu, orc, set_option):
+    """The FR-Spec head with the fused log-softmax statistics ranked by the chunk + merge form instead of the row kernel."""
+    set_option("topk_row_kernel", 0)
+    _frspec_check(gpu, orc, n=10, V=9000, Vs=4096, H=512, k=10, seed=31, tiled=True)
+    _frspec_check(gpu, orc, n=3, V=70000, Vs=65536, H=512, k=16, seed=32, tiled=True)
+    _frspec_check(gpu, orc, n=5, V=9000, Vs=4099, H=512, k=32, seed=33, tiled=False)
+
+
 def test_topk_heavy_ties_and_neg_inf(gpu, orc):
     from cpm.cu_amd import ops
     torch = gpu
