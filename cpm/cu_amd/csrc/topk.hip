@@ -506,16 +506,42 @@ template <bool LOGSOFTMAX>
 __global__ __launch_bounds__(kRowThreads) void topk_row_kernel(TopkParams p) { topk_row_body<LOGSOFTMAX, f16>(p); }
 __global__ __launch_bounds__(kRowThreads) void topk_row_bf16_kernel(TopkParams p) { topk_row_body<true, bf16>(p); }
 
-// log_softmax in place (src/model/eagle.cuh:29-89): one workgroup per row.
+// log_softmax in place (src/model/eagle.cuh:29-89): one workgroup per row.  The row is walked in 16-byte pieces from its
+// first 16-byte boundary on; the first four pieces of every thread stay in registers between the three passes (maximum, sum,
+// write), so a row of up to 32768 elements is read once; the up to seven elements in front of the first piece and behind
+// the last go one to a thread.
 template <typename E>
 __device__ __forceinline__ void log_softmax_body(uint16_t* x, int dim, float* row_stats) {
     __shared__ float red[16];
+    constexpr int kKeep = 4;
     const int row = blockIdx.x;
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63;
     uint16_t* xr = x + (size_t)row * dim;
-    float m = -INFINITY;
-    for (int i = tid; i < dim; i += 1024) m = fmaxf(m, Elem<E>::from_bits(xr[i]));
+    const int head = min(dim, (int)(((16 - ((uintptr_t)xr & 15)) & 15) >> 1));
+    const int npieces = (dim - head) >> 3;
+    const int tail0 = head + npieces * 8, ntail = dim - tail0;
+    uint4* xp = (uint4*)(xr + head);
+    const int single = tid < head ? tid : tid < head + ntail ? tail0 + (tid - head) : -1;  // this thread's element outside the pieces
+    const float single_v = single >= 0 ? Elem<E>::from_bits(xr[single]) : -INFINITY;
+    const uint32_t ninf2 = Elem<E>::to_bits(-INFINITY) * 0x10001u;
+    uint4 keep[kKeep];
+#pragma unroll
+    for (int j = 0; j < kKeep; ++j) {
+        const int pc = j * 1024 + tid;
+        keep[j] = pc < npieces ? xp[pc] : make_uint4(ninf2, ninf2, ninf2, ninf2);
+    }
+    const auto lo = [](uint32_t w) { return Elem<E>::from_bits((uint16_t)(w & 0xFFFFu)); };
+    const auto hi = [](uint32_t w) { return Elem<E>::from_bits((uint16_t)(w >> 16)); };
+    const auto piece_max = [&](const uint4& v, float a) {
+        a = fmaxf(fmaxf(a, lo(v.x)), fmaxf(hi(v.x), lo(v.y)));
+        a = fmaxf(fmaxf(a, hi(v.y)), fmaxf(lo(v.z), hi(v.z)));
+        return fmaxf(a, fmaxf(lo(v.w), hi(v.w)));
+    };
+    float m = single_v;
+#pragma unroll
+    for (int j = 0; j < kKeep; ++j) m = piece_max(keep[j], m);
+    for (int pc = kKeep * 1024 + tid; pc < npieces; pc += 1024) m = piece_max(xp[pc], m);
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
     if (lane == 0) red[wave] = m;
@@ -524,8 +550,17 @@ __device__ __forceinline__ void log_softmax_body(uint16_t* x, int dim, float* ro
 #pragma unroll
     for (int w = 1; w < 16; ++w) m = fmaxf(m, red[w]);
     __syncthreads();
-    float s = 0.f;
-    for (int i = tid; i < dim; i += 1024) s += expf(Elem<E>::from_bits(xr[i]) - m);
+    const auto piece_sum = [&](const uint4& v, float a) {
+        a += expf(lo(v.x) - m) + expf(hi(v.x) - m);
+        a += expf(lo(v.y) - m) + expf(hi(v.y) - m);
+        a += expf(lo(v.z) - m) + expf(hi(v.z) - m);
+        return a + (expf(lo(v.w) - m) + expf(hi(v.w) - m));
+    };
+    float s = single >= 0 ? expf(single_v - m) : 0.f;
+#pragma unroll
+    for (int j = 0; j < kKeep; ++j)
+        if (j * 1024 + tid < npieces) s = piece_sum(keep[j], s);
+    for (int pc = kKeep * 1024 + tid; pc < npieces; pc += 1024) s = piece_sum(xp[pc], s);
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) s += __shfl_xor(s, off);
     if (lane == 0) red[wave] = s;
@@ -534,9 +569,15 @@ __device__ __forceinline__ void log_softmax_body(uint16_t* x, int dim, float* ro
 #pragma unroll
     for (int w = 0; w < 16; ++w) s += red[w];
     const float lse = logf(s);
-    for (int i = tid; i < dim; i += 1024) {
-        xr[i] = Elem<E>::to_bits((Elem<E>::from_bits(xr[i]) - m) - lse);
-    }
+    const auto map2 = [&](uint32_t w) {
+        return (uint32_t)Elem<E>::to_bits((lo(w) - m) - lse) | ((uint32_t)Elem<E>::to_bits((hi(w) - m) - lse) << 16);  // src/model/eagle.cuh:87
+    };
+    const auto piece_map = [&](const uint4& v) { return make_uint4(map2(v.x), map2(v.y), map2(v.z), map2(v.w)); };
+#pragma unroll
+    for (int j = 0; j < kKeep; ++j)
+        if (j * 1024 + tid < npieces) xp[j * 1024 + tid] = piece_map(keep[j]);
+    for (int pc = kKeep * 1024 + tid; pc < npieces; pc += 1024) xp[pc] = piece_map(xp[pc]);
+    if (single >= 0) xr[single] = Elem<E>::to_bits((single_v - m) - lse);
     if (tid == 0 && row_stats) {
         row_stats[row * 2 + 0] = m;
         row_stats[row * 2 + 1] = lse;

@@ -137,10 +137,11 @@ def test_bf16_frspec_head_topk(gpu, orc, bf16, n, V, Vs, H, k, tiled):
     assert np.allclose(stats[:, 0], m_ref, atol=1e-6) and np.allclose(stats[:, 1], lse_ref, atol=1e-3)
 
 
-def test_bf16_log_softmax_and_raw_topk(gpu, orc, bf16):
+@pytest.mark.parametrize("n,dim", [(3, 32768), (2, 40001), (4, 510)])
+def test_bf16_log_softmax_and_raw_topk(gpu, orc, bf16, n, dim):
     torch = gpu
     from cpm.cu_amd import ops
-    x = orc.encode(synth.rng(5, 5).standard_normal((3, 32768)).astype(np.float32) * 1.3)
+    x = orc.encode(synth.rng(dim, 5).standard_normal((n, dim)).astype(np.float32) * 1.3)
     d = to_dev(torch, x)
     stats = to_np(ops.log_softmax_(d))
     torch.cuda.synchronize()

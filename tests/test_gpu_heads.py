@@ -481,11 +481,17 @@ def test_topk_row_kernel_shapes_of_data(gpu, orc, case):
     assert np.array_equal(to_np(val).view(np.uint16), v_ref.view(np.uint16))
 
 
-def test_log_softmax_operator(gpu, orc):
+@pytest.mark.parametrize("n,dim,off", [(3, 32768, 0), (1, 7, 0), (5, 510, 0), (2, 32768 + 8, 0), (3, 73448, 0), (2, 151643, 0), (4, 4096, 3),
+                                       (2, 40000, 5), (3, 33, 1), (16, 1000, 0)])
+def test_log_softmax_operator(gpu, orc, n, dim, off):
+    """Rows of whole 16-byte pieces, rows with single elements in front of and behind the pieces (odd lengths; a buffer that
+    starts `off` elements off 16 bytes), rows shorter than a piece, rows longer than the registers hold."""
     from cpm.cu_amd import ops
     torch = gpu
-    x = (synth.rng(5, 5).standard_normal((3, 32768)) * 1.3).astype(np.float16)
-    d = to_dev(torch, x)
+    x = (synth.rng(dim, 5 + off).standard_normal((n, dim)) * 1.3).astype(np.float16)
+    buf = torch.zeros(n * dim + 8, dtype=torch.float16, device="cuda")
+    d = buf[off:off + n * dim].view(n, dim)
+    d.copy_(to_dev(torch, x))
     stats = to_np(ops.log_softmax_(d))
     torch.cuda.synchronize()
     lp_ref, m_ref, lse_ref = orc.log_softmax(x)
@@ -494,6 +500,7 @@ def test_log_softmax_operator(gpu, orc):
     staged = orc.log_softmax_apply(x, stats[:, 0], stats[:, 1])
     assert np.array_equal(to_np(d).view(np.uint16), staged.view(np.uint16))
     assert_close_f16(to_np(d), lp_ref, "log_softmax", atol=2e-2, rtol=1e-2)
+    assert not to_np(buf[:off]).any() and not to_np(buf[off + n * dim:]).any()  # nothing written outside the rows
 
 
 @pytest.mark.parametrize("n,V,H", [(60, 1000 + 7, 512), (10, 4096, 1024), (24, 530, 2048), (128, 2000, 512), (1, 16, 512)])
