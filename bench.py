@@ -372,6 +372,15 @@ def main():
         print("bench.py: this path is measured on one GPU; --gpus %d is not supported (nothing in it is sharded)" % args.gpus,
               file=sys.stderr)
         sys.exit(2)
+    from cpm.cu_amd import synth
+    if args.workload not in synth.CONFIGS:
+        sys.exit("bench.py: unknown workload %s (one of %s)" % (args.workload, ", ".join(synth.CONFIGS)))
+    if synth.CONFIGS[args.workload]["T"] > 64:
+        # cpmcu_verify_step mirrors the reference's model-level call, whose trees have at most 64 nodes
+        # (src/model/minicpm4/minicpm4_eagle.cuh:69); wider trees go through the operator-level entry points
+        sys.exit("bench.py: %s has a %d-node tree; this bench times the model-level step, which takes up to 64 nodes -- the wide-tree "
+                 "step is run and checked operator by operator in tests/test_gpu_verify_step.py::test_c5_wide_tree_step_32_layers_every_depth"
+                 % (args.workload, synth.CONFIGS[args.workload]["T"]))
     import numpy as np
     import torch
     from cpm.cu_amd import lib, ops, synth
@@ -615,7 +624,7 @@ def main():
         dcache = model.cache(block_table=main_run["tables"][0], num_layers=L + 1)  # layer L: the drafter's own cache
         dcache.k[L][: main_run["npages"]].copy_(dcache.k[0][: main_run["npages"]])
         dcache.v[L][: main_run["npages"]].copy_(dcache.v[0][: main_run["npages"]])
-        hid1 = bufs.hidden[:1].contiguous()
+        hid1, hid_k = bufs.hidden[:1].contiguous(), bufs.hidden[:k_it].contiguous()  # k hidden rows per round after the first
         qd, kd, vd = bufs.q[0][:k_it].contiguous(), bufs.k_new[0][:k_it].contiguous(), bufs.v_new[0][:k_it].contiguous()
         d_len = [torch.tensor([P + k_it * d], dtype=torch.int32, device="cuda") for d in range(n_it)]
         d_out = torch.empty_like(qd)
@@ -627,7 +636,7 @@ def main():
             for d in range(1, n_it):
                 ops.tree_attention(qd, dcache, L, d_len[d], padded, dtree.draft_mask, out=d_out, k_new=kd, v_new=vd,
                                    mask_k_range=k_it * d, block_window_size=1024)
-                r = ops.frspec_head_topk(hid10, w_subs[d % FR_SETS], remap, k_it)
+                r = ops.frspec_head_topk(hid_k, w_subs[d % FR_SETS], remap, k_it)
                 dtree.extend(d, r["val"], r["pos"])
             dtree.finish(T, clen, tree_draft_ids=tree_ids)
         ms_draft_cold = timed_torch(torch, draft_path, reps, 2)
@@ -648,7 +657,7 @@ def main():
             model.draft_round(0, hid1, next_ids, None, dmask)
             for d in range(1, n_it):
                 model.draft_attention(0, k_it, padded, qd, kd, vd, d_len[d], dmask, k_it * d, d_out)
-                model.draft_round(d, hid10, next_ids, prows, dmask)
+                model.draft_round(d, hid_k, next_ids, prows, dmask)
             model.draft_finish(tree_ids, t_pos, clen, t_mask, t_par)
         gid = model.capture(draft_model_level)
         lib_stream = model.stream()
