@@ -90,8 +90,9 @@ def attention(L, torch, prefixes, T=60):
         print("  K loop left by XCD (workgroup number mod 8), medians: " + " ".join("%.1f" % np.median(rel[wg % 8 == x, 2]) for x in range(8)))
         last = d[d[:, 10] == d[:, 10].max()]  # the last split: the appended rows and the end of the stream
         rl = (last - t0) / 100.0
-        print("  last split (%d workgroups, %s tiles): loop entered %.2f, second iteration %.2f, patch begun %.2f, V patch begun %.2f, patch done %.2f, loop left %.2f (medians; patch of the M-tile-0 workgroups done %.2f)" %
-              (len(last), "/".join(str(x) for x in np.unique(last[:, 9])), np.median(rl[:, 1]), np.median(rl[:, 12]), np.median(rl[:, 14]), np.median(rl[:, 13]), np.median(rl[:, 15]), np.median(rl[:, 2]),
+        second = "%.2f" % np.median(rl[:, 12]) if (last[:, 12] != 0).all() else "none"  # a split of one or two tiles has no second iteration: no stamp
+        print("  last split (%d workgroups, %s tiles): loop entered %.2f, second iteration %s, patch begun %.2f, V patch begun %.2f, patch done %.2f, loop left %.2f (medians; patch of the M-tile-0 workgroups done %.2f)" %
+              (len(last), "/".join(str(x) for x in np.unique(last[:, 9])), np.median(rl[:, 1]), second, np.median(rl[:, 14]), np.median(rl[:, 13]), np.median(rl[:, 15]), np.median(rl[:, 2]),
                np.median(rl[last[:, 11] == 0][:, 15])))
         del cache
 
