@@ -338,19 +338,27 @@ def test_step_graph_cache_is_bounded(gpu, orc):
         m.close()
 
 
-def test_model_level_draft_rounds(gpu, orc):
+@pytest.mark.parametrize("frspec", [True, False])
+def test_model_level_draft_rounds(gpu, orc, frspec):
     """cpmcu_draft_round / cpmcu_draft_finish (the drafter's state owned by the library, driven through the pybind module)
     against (1) the operator-level chain on an independently built sub-matrix, bit for bit, and (2) the oracle's tree
-    bookkeeping fed with the device's per-round top-k, which pins ids, positions, masks and parents of the final tree."""
+    bookkeeping fed with the device's per-round top-k, which pins ids, positions, masks and parents of the final tree.
+    Once as the FR-Spec drafter of MiniCPM4 (init_minicpm4_eagle_model: a frequency-ranked sub-vocabulary and its id table),
+    once as the plain EAGLE drafter (init_eagle_model, src/entry.cu: the head on the whole vocabulary, no id table)."""
     from cpm.cu_amd import C, ops
     torch = gpu
     V, Vs, H, T, K, N, P = 5000, 2048, 512, 60, 10, 6, 777
     w = synth.normal_f16((V, H), 41, 2, std=0.05)
-    remap = synth.frspec_remap(V, Vs, 41)
     C.init_base_model(0.01, V, 1, H, 1024, HQ, HKV, D, 1e-5, 0, 2048, 1.0, 1.0, 1.0)
-    C.init_minicpm4_eagle_model(1, N, K, T, 0, False, 128, 1024, Vs, 1.0, True, True)
+    if frspec:
+        remap = synth.frspec_remap(V, Vs, 41)
+        C.init_minicpm4_eagle_model(1, N, K, T, 0, False, 128, 1024, Vs, 1.0, True, True)
+    else:
+        remap = np.arange(V, dtype=np.int32)
+        C.init_eagle_model(1, N, K, T, 0)
     C.init_storage()
-    C.load_model("eagle.token_id_remap", remap.ctypes.data)
+    if frspec:
+        C.load_model("eagle.token_id_remap", remap.ctypes.data)
     C.load_model("lm_head.weight", w.ctypes.data)
     try:
         hid = [to_dev(torch, synth.normal_f16((1 if d == 0 else K, H), 41, 100 + d)) for d in range(N)]
