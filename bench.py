@@ -375,12 +375,6 @@ def main():
     from cpm.cu_amd import synth
     if args.workload not in synth.CONFIGS:
         sys.exit("bench.py: unknown workload %s (one of %s)" % (args.workload, ", ".join(synth.CONFIGS)))
-    if synth.CONFIGS[args.workload]["T"] > 64:
-        # cpmcu_verify_step mirrors the reference's model-level call, whose trees have at most 64 nodes
-        # (src/model/minicpm4/minicpm4_eagle.cuh:69); wider trees go through the operator-level entry points
-        sys.exit("bench.py: %s has a %d-node tree; this bench times the model-level step, which takes up to 64 nodes -- the wide-tree "
-                 "step is run and checked operator by operator in tests/test_gpu_verify_step.py::test_c5_wide_tree_step_32_layers_every_depth"
-                 % (args.workload, synth.CONFIGS[args.workload]["T"]))
     import numpy as np
     import torch
     from cpm.cu_amd import lib, ops, synth
@@ -421,8 +415,11 @@ def main():
     w_dev = (torch.randn(V, H, device="cuda", dtype=torch.float32, generator=gen) * 0.02).to(torch.float16)
     w_host = w_dev.cpu().numpy()
     remap_np = synth.frspec_remap(V, shp["frspec_vocab"], 0)
+    # the drafter's masks have 64 bits, as the reference's: top-k x rounds <= 64 columns, trees of up to 64 nodes.  A wider tree
+    # (config 5) is synthetic on the verify side, and the draft side is timed with as many rounds of its top-k as fit.
+    draft_rounds = min(cfg["num_iter"], 64 // cfg["topk"])
     model = PathModel(V, L, H, Hq, Hkv, memory_limit=memory_limit, scale_lmhead=1.0, frspec_vocab=shp["frspec_vocab"], tree_size=T,
-                      num_iter=cfg["num_iter"], topk=cfg["topk"], draft_layers=1, eagle_window=1024)
+                      num_iter=draft_rounds, topk=cfg["topk"], draft_layers=1, eagle_window=1024)
     assert model.num_pages >= pages_needed, (model.num_pages, pages_needed)
     model.load_head(w_host, remap_np)
     bufs = StepBuffers(torch, L, T, Hq, Hkv, D, H, gen)
@@ -619,7 +616,8 @@ def main():
         # bookkeeping kernel; the final top-59 + tree build at the end.  The dense parts of the drafter layer (fc,
         # projections, FFN) are not on the path and are not run; the head reads a different copy of its matrix every
         # round, as it would after their weights.
-        k_it, n_it = cfg["topk"], cfg["num_iter"]
+        k_it, n_it = cfg["topk"], draft_rounds
+        Td = min(T, 64)  # src/model/minicpm4/minicpm4_eagle.cuh:69
         dtree = ops.DraftTree(k_it, n_it, remap)
         dcache = model.cache(block_table=main_run["tables"][0], num_layers=L + 1)  # layer L: the drafter's own cache
         dcache.k[L][: main_run["npages"]].copy_(dcache.k[0][: main_run["npages"]])
@@ -628,7 +626,7 @@ def main():
         qd, kd, vd = bufs.q[0][:k_it].contiguous(), bufs.k_new[0][:k_it].contiguous(), bufs.v_new[0][:k_it].contiguous()
         d_len = [torch.tensor([P + k_it * d], dtype=torch.int32, device="cuda") for d in range(n_it)]
         d_out = torch.empty_like(qd)
-        tree_ids = torch.full((T,), -1, dtype=torch.int32, device="cuda")
+        tree_ids = torch.full((Td,), -1, dtype=torch.int32, device="cuda")
 
         def draft_path():
             r = ops.frspec_head_topk(hid1, w_subs[0], remap, k_it)
@@ -638,7 +636,7 @@ def main():
                                    mask_k_range=k_it * d, block_window_size=1024)
                 r = ops.frspec_head_topk(hid_k, w_subs[d % FR_SETS], remap, k_it)
                 dtree.extend(d, r["val"], r["pos"])
-            dtree.finish(T, clen, tree_draft_ids=tree_ids)
+            dtree.finish(Td, clen, tree_draft_ids=tree_ids)
         ms_draft_cold = timed_torch(torch, draft_path, reps, 2)
 
         # the same draft through the library's own model-level calls (drafter state, FR-Spec sub-matrix and the drafter
@@ -672,9 +670,9 @@ def main():
         model.synchronize()
         ms_draft = e0.elapsed_time(e1) / reps
         draft = {"us_per_draft": round(ms_draft * 1e3, 1), "us_per_draft_cold_matrix": round(ms_draft_cold * 1e3, 1),
-                 "rounds": n_it, "topk_per_round": k_it, "tree_size": T,
-                 "operators": "6 x (FR-Spec head + log-softmax + top-10 + id map-back) + 5 x drafter-layer attention "
-                              "(window 1024) + tree bookkeeping (begin, 5 x extend, finish)",
+                 "rounds": n_it, "topk_per_round": k_it, "tree_size": Td,
+                 "operators": "%d x (FR-Spec head + log-softmax + top-%d + id map-back) + %d x drafter-layer attention "
+                              "(window 1024) + tree bookkeeping (begin, %d x extend, finish)" % (n_it, k_it, n_it - 1, n_it - 1),
                  "note": "us_per_draft: cpmcu_draft_round / cpmcu_draft_attention / cpmcu_draft_finish on the library's model, "
                          "replayed as a library graph; us_per_draft_cold_matrix: the same operators with every round reading a "
                          "different copy of the FR-Spec matrix (as after the drafter layer's dense weights)"}

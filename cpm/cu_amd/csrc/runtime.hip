@@ -413,7 +413,7 @@ int init_storage_impl(Model& m, int* max_context) {
         used += bytes;
         return CPMCU_OK;
     };
-    const int max_tree = 64;  // decode_attention / draft_attention accept up to 64 rows whatever the tree size
+    const int max_tree = kMaxTree;  // decode_attention / draft_attention accept up to 64 rows whatever the tree size, verify_step up to kMaxTree
     if ((rc = alloc((void**)&m.lm_head, cpmcu_head_weight_tiled_bytes(m.vocab, m.hidden)))) return rc;  // kept in tiled layout
     if (m.drafter && m.frspec_vocab != m.vocab) {
         if ((rc = alloc((void**)&m.fr_head, cpmcu_head_weight_tiled_bytes(m.frspec_vocab, m.hidden)))) return rc;
@@ -755,9 +755,10 @@ struct StepArgs {
 int enqueue_verify_step(Model& m, const StepArgs& a, hipStream_t st) {
     const int32_t* table = a.block_table ? (const int32_t*)a.block_table : m.block_table;
     const float scale = 1.f / sqrtf((float)kHeadDim);
+    const int mask_words = ceil_div(a.T, 64);  // one uint64 per row up to the reference's 64 nodes, two for wider trees
     for (int l = 0; l < m.layers; ++l) {
         int rc = cpmcu_tree_attention((const void*)a.q[l], m.k_pools[l], m.v_pools[l], table, (const int32_t*)a.kv_length, a.padded_length,
-                                      (const void*)a.k_new[l], (const void*)a.v_new[l], (const uint64_t*)a.attn_mask, 1, 0, a.T, m.q_heads,
+                                      (const void*)a.k_new[l], (const void*)a.v_new[l], (const uint64_t*)a.attn_mask, mask_words, 0, a.T, m.q_heads,
                                       m.kv_heads, scale, (void*)a.attn_out[l], m.attn_ws, m.attn_ws_bytes, 0, st);
         if (rc) return rc;
     }
@@ -767,7 +768,7 @@ int enqueue_verify_step(Model& m, const StepArgs& a, hipStream_t st) {
     if (rc) return rc;
     rc = cpmcu_verify_tail(m.d_k_pools, m.d_v_pools, m.layers, table, m.kv_heads, a.T, (const int32_t*)a.draft_ids, nullptr, m.head_ws,
                            num_partials, stride, (const int32_t*)a.position_ids, (const int32_t*)a.cache_length,
-                           (const uint64_t*)a.attn_mask, 1, (const int32_t*)a.tree_parent, a.prev_hidden ? (const void*)a.hidden : nullptr,
+                           (const uint64_t*)a.attn_mask, mask_words, (const int32_t*)a.tree_parent, a.prev_hidden ? (const void*)a.hidden : nullptr,
                            m.hidden, (void*)a.prev_hidden, (int32_t*)a.gt_out, m.d_best, nullptr, (int32_t*)a.accepted_ids,
                            (int32_t*)a.next_position_ids, (int32_t*)a.result, st);
     if (rc) return rc;
@@ -817,7 +818,7 @@ extern "C" int cpmcu_verify_step(int num_layers, int num_tokens, int padded_leng
     }
     CPMCU_CHECK_ARG(m.lm_head_loaded, "verify_step: lm_head.weight has not been loaded");
     CPMCU_CHECK_ARG(num_layers == m.layers, "verify_step: %d per-layer addresses given, the model has %d layers", num_layers, m.layers);
-    CPMCU_CHECK_ARG(num_tokens >= 1 && num_tokens <= 64, "verify_step: num_tokens=%d outside [1, 64]", num_tokens);
+    CPMCU_CHECK_ARG(num_tokens >= 1 && num_tokens <= kMaxTree, "verify_step: num_tokens=%d outside [1, %d]", num_tokens, kMaxTree);
     CPMCU_CHECK_ARG(padded_length >= num_tokens && padded_length <= m.num_pages * kPage, "verify_step: padded_length=%d outside [%d, %d]",
                     padded_length, num_tokens, m.num_pages * kPage);
     CPMCU_CHECK_ARG(q && k_new && v_new && attn_out, "verify_step: null per-layer address array");

@@ -39,7 +39,8 @@ class PathModel:
         # dtype: 0 = fp16, 1 = bf16 (tensors then hold bfloat16 patterns, whatever 16-bit torch dtype carries them)
         L.init_base_model(ctypes.c_float(memory_limit), vocab, layers, hidden, 4 * hidden, q_heads, kv_heads, HEAD_DIM,
                           ctypes.c_float(1e-5), int(dtype), 2048, ctypes.c_float(1.0), ctypes.c_float(scale_lmhead), ctypes.c_float(1.0))
-        L.init_minicpm4_eagle_model(draft_layers, num_iter, topk, tree_size, int(dtype), 0, 128, eagle_window, frspec_vocab,
+        # the drafter builds trees of up to 64 nodes (src/model/minicpm4/minicpm4_eagle.cuh:69); a wider tree for verify_step is the caller's
+        L.init_minicpm4_eagle_model(draft_layers, num_iter, topk, min(tree_size, 64), int(dtype), 0, 128, eagle_window, frspec_vocab,
                                     ctypes.c_float(1.0), 1, 1)
         ctx = ctypes.c_int(0)
         L.init_storage(ctypes.byref(ctx))

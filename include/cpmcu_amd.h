@@ -161,7 +161,9 @@ int cpmcu_verify_and_fix(int num_tokens, uint64_t pred, uint64_t gt, uint64_t po
  *       k_new[l] / v_new[l] [T][Hkv*128], attn_out[l] like q[l];
  *   hidden [T][hidden_size]; draft_ids int32[T] (read only); position_ids int32[T]; cache_length int32[1] = P;
  *   kv_length int32[1] = P + T (the pre-incremented length of cpmcu/llm.py:272, kept as a scalar of its own so
- *       that neither is rewritten between the calls of a step); attn_mask uint64[T]; tree_parent int32[T];
+ *       that neither is rewritten between the calls of a step); attn_mask uint64[T] for T <= 64 as in the reference,
+ *       uint64[T][2] (word w of a row holds bits 64w..64w+63) for trees of 65 to CPMCU_MAX_TREE nodes, which the reference
+ *       does not have; tree_parent int32[T];
  *   block_table: device int32[] logical -> physical pages to use for this step, or 0 = the model's table;
  *   outputs: gt_out int32[T] (0 = skip), accepted_ids int32[T] (first a entries), prev_hidden [T][hidden_size]
  *       (0 = skip: rows hidden[path[d]], src/model/eagle.cuh:108-115), next_position_ids int32[T] (0 = skip),

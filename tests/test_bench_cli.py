@@ -21,8 +21,6 @@ def test_the_survey_tools_print_their_usage_without_a_gpu():
         assert r.returncode == 2 and "python -m " + mod in r.stdout, r.stdout
 
 
-def test_workloads_the_model_level_step_cannot_take_are_refused_before_the_gpu_is_touched():
-    """An unknown workload, and the 128-node tree (the model-level step takes up to 64 nodes, like the reference's)."""
-    for name, needle in (("nope", "unknown workload"), ("c5_wide_32k", "128-node tree")):
-        res = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--workload", name], capture_output=True, text=True, timeout=120)
-        assert res.returncode == 1 and needle in res.stderr and res.stdout.strip() == "", (res.returncode, res.stderr)
+def test_an_unknown_workload_is_refused_before_the_gpu_is_touched():
+    res = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--workload", "nope"], capture_output=True, text=True, timeout=120)
+    assert res.returncode == 1 and "unknown workload" in res.stderr and res.stdout.strip() == "", (res.returncode, res.stderr)

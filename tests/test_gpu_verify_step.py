@@ -268,6 +268,13 @@ def test_library_graph_replays_equal_eager_steps(gpu, orc):
     _graph_replays_equal_eager_steps(gpu, orc, seed=3, T=24, P0=1000, STEPS=10)
 
 
+@pytest.mark.parametrize("T", [65, 100, 128])
+def test_model_level_steps_with_trees_of_more_than_64_nodes(gpu, orc, T):
+    """cpmcu_verify_step takes trees of up to 128 nodes, masks of two words per row: the same sequence of steps, eagerly and
+    as graph replays, against the oracle."""
+    _graph_replays_equal_eager_steps(gpu, orc, seed=T, T=T, P0=900, STEPS=6, LAYERS=2, min_paddings=1)
+
+
 @pytest.mark.parametrize("hq,hkv", [(32, 8), (8, 1), (40, 8)])
 def test_model_level_steps_with_other_head_counts(gpu, orc, monkeypatch, hq, hkv):
     """The same sequence of steps on models with 4, 8 and 5 query heads per KV head (the configurations all have 16)."""
@@ -412,14 +419,16 @@ def test_model_level_draft_rounds(gpu, orc, frspec):
     assert np.array_equal(to_np(tmask).view(np.uint64), o_mask[:, 0])
 
 
-def test_c2_full_size_step_on_the_library_graph(gpu, orc):
+@pytest.mark.parametrize("config", ["c2_verify_4k", "c5_wide_32k"])
+def test_full_size_step_on_the_library_graph(gpu, orc, config):
     """Config 2 as the benchmark runs it: 32 layers, 4096-token prefix, 60-node tree, the 73448 x 4096 head, one
     cpmcu_verify_step on the library's storage replayed from the library's graph.  Accept length, ids and the compacted
     rows of all 64 caches bit-exact against the oracle, the arg-max staged on the oracle's logits of the same head,
-    attention of two sampled layers within the fp16 tolerance."""
+    attention of two sampled layers within the fp16 tolerance.  And config 5 the same way: a 128-node tree (two mask words
+    per row, beyond the reference's 64 nodes) behind a 32768-token prefix."""
     from cpm.cu_amd.model import PathModel
     torch = gpu
-    cfg, shp = synth.CONFIGS["c2_verify_4k"], synth.MINICPM4_8B
+    cfg, shp = synth.CONFIGS[config], synth.MINICPM4_8B
     L, P, T, V, H = cfg["layers"], cfg["prefix"], cfg["T"], shp["vocab"], shp["hidden"]
     S = P + T
     tree = synth.eagle_tree(cfg["num_iter"], cfg["topk"], T, cfg["seed"])
@@ -475,7 +484,7 @@ def test_c2_full_size_step_on_the_library_graph(gpu, orc):
         for l in sampled:
             kp, vp = before[l]
             ref = orc.tree_attention(to_np(q[l]), np.concatenate([kp, to_np(kn[l])]), np.concatenate([vp, to_np(vn[l])]), tree.mask, P)
-            assert_close_f16(to_np(out[l]), ref, "config 2 step on the library graph, attention of layer %d" % l)
+            assert_close_f16(to_np(out[l]), ref, "%s step on the library graph, attention of layer %d" % (config, l))
             kd, vd = cache.read_logical(l, 0, P)
             assert np.array_equal(to_np(kd).view(np.uint16), kp.view(np.uint16)) and np.array_equal(to_np(vd).view(np.uint16), vp.view(np.uint16))
     finally:
