@@ -160,7 +160,7 @@ def main(argv):
 
     def verify_steps(seed):
         g = synth.rng(seed, 97)
-        T = int(g.integers(2, 65))
+        T = int(g.integers(2, 129))  # beyond 64 nodes: two mask words per row
         t_step._graph_replays_equal_eager_steps(torch, orc, seed, T=T, P0=int(g.integers(0, 3000)), STEPS=int(g.integers(3, 13)), LAYERS=int(g.integers(1, 4)),
                                                 V=int(g.integers(500, 6000)), num_iter=8, topk=min(8, T - 1), min_paddings=1)
 
