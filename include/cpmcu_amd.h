@@ -484,13 +484,15 @@ size_t cpmcu_lm_head_argmax_static_scratch_bytes(void);
 int cpmcu_lm_head_argmax_static(const void* hidden, const void* w, int w_layout, int n, int V, int H, int apply_scale,
                                 float head_scale, void* logits, int32_t* gt, void* stream);
 
-/* log_softmax in place -- src/model/eagle.cuh:29-89.  x [n][dim] fp16;
- * row_stats [n][2] fp32 (max, ln sum) output, may be NULL. */
+/* log_softmax in place -- src/model/eagle.cuh:29-89.  x [n][dim] fp16 (bf16 under the dtype option), any dim, 2-byte
+ * alignment is enough; row_stats [n][2] fp32 (max, ln sum) output, may be NULL. */
 int cpmcu_log_softmax(void* x, int n, int dim, float* row_stats, void* stream);
 
 /* TopK::prefill -- src/model/topk.cuh:255-288: per row the `top` largest values,
- * value descending, ties -> lower index.  top <= min(dim, 128).
- * workspace: at least cpmcu_topk_workspace_bytes(n, dim, top). */
+ * value descending, ties -> lower index.  top <= min(dim, 128); any dim and any 2-byte aligned x (rows of whole
+ * 16-byte pieces -- dim a multiple of 8, x on 16 bytes -- are read fastest); rows of more than 32768 elements need
+ * top x ceil(dim / 32768) <= 1024.  val [n][top] in the element type, pos int32 [n][top].
+ * workspace: at least cpmcu_topk_workspace_bytes(n, dim, top) (used for rows of more than 32768 elements). */
 size_t cpmcu_topk_workspace_bytes(int n, int dim, int top);
 int cpmcu_topk(const void* x, int n, int dim, int top, void* val, int32_t* pos, void* workspace,
                size_t workspace_bytes, void* stream);
