@@ -7,6 +7,8 @@
     python -m cpm.cu_amd.sweep head                   target head (arg-max), rows 1..128 x vocabulary 8K..256K x hidden 2048/4096/8192
     python -m cpm.cu_amd.sweep frspec                 FR-Spec head + log-softmax + top-k + id map-back, vocabulary 8K..73448 x rows x k
     python -m cpm.cu_amd.sweep topk                   top-k of fp16 rows, row length 64..152K x rows 1..60 x k 1..128
+    python -m cpm.cu_amd.sweep window                 the drafter layer's attention (k queries, block window of 1024 tokens): the
+                                                      library's plan beside both kernel shapes and forced split counts
 
 Eager launches on cuda:0, random fp16 data, event-timed; attention rotates over several layers' K/V pools and the heads over
 copies of the weight matrix, so that no pass is served from the last-level cache.  Fractions are of 8 TB/s (heads) and TFLOP/s
@@ -25,6 +27,22 @@ def _time(torch, fn, reps):
     e1.record()
     torch.cuda.synchronize()
     return e0.elapsed_time(e1) / reps * 1e3
+
+
+def _time_graph(torch, fn, reps, inner):
+    """us per call of fn inside a replayed graph of `inner` calls: launch gaps as a decode loop has them, no Python in between."""
+    for _ in range(3):
+        fn()
+    torch.cuda.synchronize()
+    g, side = torch.cuda.CUDAGraph(), torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            for _ in range(inner):
+                fn()
+    for _ in range(3):
+        g.replay()
+    torch.cuda.synchronize()
+    return _time(torch, g.replay, reps) / inner
 
 
 def attention(torch, with_groups, Hq=32, Hkv=2):
@@ -151,8 +169,44 @@ def topk(torch):
             print(line, flush=True)
 
 
+def window(torch):
+    from . import lib, ops
+    from .kvcache import PagedKVCache
+    Hq, Hkv, D = 32, 2, 128
+    L = lib.get()
+    splits = (0, 2, 4, 8, 12, 16)
+    print("drafter-layer attention, %d query / %d KV heads, block window 1024: us per call in a replayed graph (0 = the library's choice)" % (Hq, Hkv))
+    print("%28s" % "shape <G> \\ splits" + "".join("%8d" % ns for ns in splits))
+    for P in (4096, 32768):
+        for k, d in ((10, 1), (10, 5), (16, 3)):
+            S = P + k * d
+            cache = PagedKVCache(4, Hkv, (S + 255) // 256 + 2)
+            for l in range(4):
+                cache.k[l].normal_()
+                cache.v[l].normal_()
+            q = torch.randn(k, Hq, D, device="cuda").half()
+            kn = torch.randn(k, Hkv, D, device="cuda").half()
+            vn = torch.randn_like(kn)
+            kv_len = torch.tensor([S], dtype=torch.int32, device="cuda")
+            mask = torch.from_numpy(np.random.default_rng(0).integers(1, 2 ** min(k * d, 62), size=k, dtype=np.int64)).cuda()
+            out = torch.empty_like(q)
+            pad = (S + 127) // 128 * 128
+            for G in (0, 1, 2):
+                L.set_option(b"attn_kv_groups", G)
+                line = "%28s" % ("P %d, %d queries, round %d, <%d>" % (P, k, d, G))
+                for ns in splits:
+                    def run():
+                        for l in range(4):
+                            ops.tree_attention(q, cache, l, kv_len, pad, mask, out=out, k_new=kn, v_new=vn, mask_k_range=k * d,
+                                               block_window_size=1024, num_splits=ns)
+                    line += "%8.1f" % (_time_graph(torch, run, 20, 2) / 4)
+                print(line, flush=True)
+            L.set_option(b"attn_kv_groups", 0)
+            del cache
+
+
 def main(argv):
-    if not argv or argv[0] not in ("attention", "head", "frspec", "topk"):
+    if not argv or argv[0] not in ("attention", "head", "frspec", "topk", "window"):
         print(__doc__)
         return 2
     import torch
@@ -166,6 +220,8 @@ def main(argv):
         head(torch)
     elif argv[0] == "topk":
         topk(torch)
+    elif argv[0] == "window":
+        window(torch)
     else:
         frspec(torch)
     return 0
