@@ -1,9 +1,11 @@
 """Timings of the operators over ranges of shapes, with the kernels the library picks for each: looks for cliffs in the launch plans.
 
-    python -m cpm.cu_amd.sweep attention [--groups] [--heads Hq,Hkv]
+    python -m cpm.cu_amd.sweep attention [--groups] [--heads Hq,Hkv] [--graph]
                                                       tree attention, prefix 256..131072 x tree rows 1..128 (us per layer);
                                                       --groups: the automatic choice beside both kernel shapes forced;
-                                                      --heads: query / KV head counts other than 32,2
+                                                      --heads: query / KV head counts other than 32,2;
+                                                      --graph: timed inside replayed graphs (short contexts are
+                                                      launch-bound when enqueued from Python)
     python -m cpm.cu_amd.sweep head                   target head (arg-max), rows 1..128 x vocabulary 8K..256K x hidden 2048/4096/8192
     python -m cpm.cu_amd.sweep frspec                 FR-Spec head + log-softmax + top-k + id map-back, vocabulary 8K..73448 x rows x k
     python -m cpm.cu_amd.sweep topk                   top-k of fp16 rows, row length 64..152K x rows 1..60 x k 1..128
@@ -45,7 +47,7 @@ def _time_graph(torch, fn, reps, inner):
     return _time(torch, g.replay, reps) / inner
 
 
-def attention(torch, with_groups, Hq=32, Hkv=2):
+def attention(torch, with_groups, Hq=32, Hkv=2, graph=False):
     from . import lib, ops, synth
     from .kvcache import PagedKVCache
     D = 128
@@ -82,7 +84,7 @@ def attention(torch, with_groups, Hq=32, Hkv=2):
                 for _ in range(3):
                     run()
                 torch.cuda.synchronize()
-                us = _time(torch, run, 12 if P <= 32768 else 6) / nl
+                us = (_time_graph(torch, run, 12, 1) if graph else _time(torch, run, 12 if P <= 32768 else 6)) / nl
                 kernels, splits, groups, _ = ops.attention_plan(T, Hq, Hkv, pad)
                 cell.append("%.1f <%d> s%d%s" % (us, groups, splits, "+c" if "combine" in kernels else ""))
             L.set_option(b"attn_kv_groups", 0)
@@ -215,7 +217,7 @@ def main(argv):
     torch.cuda.set_device(0)
     if argv[0] == "attention":
         heads = argv[argv.index("--heads") + 1].split(",") if "--heads" in argv else (32, 2)
-        attention(torch, "--groups" in argv[1:], int(heads[0]), int(heads[1]))
+        attention(torch, "--groups" in argv[1:], int(heads[0]), int(heads[1]), "--graph" in argv[1:])
     elif argv[0] == "head":
         head(torch)
     elif argv[0] == "topk":
